@@ -1,0 +1,172 @@
+"""ctypes mirror of ``include/adop_raster.h`` and loader of the HIP library ``libadop_raster.so``.
+
+The structs below are field-for-field copies of the C declarations; ``tests/test_capi_symbols.py`` checks
+the sizes and that every declared entry point is exported.  There is no CPU fallback: if the shared library
+has not been built, loading raises.
+"""
+import ctypes as C
+import os
+
+ADOP_MAX_LAYERS = 5
+
+ADOP_OK = 0
+ADOP_INVALID_ARG = 1
+ADOP_UNSUPPORTED_LAYERS = 2
+ADOP_HIP_ERROR = 3
+ADOP_WORKSPACE_TOO_SMALL = 4
+
+CAMERA_PINHOLE_DISTORTION = 0
+CAMERA_OCAM = 1
+
+TEXTURE_F32 = 0
+TEXTURE_F16 = 1
+
+
+class View(C.Structure):
+    _fields_ = [
+        ("w", C.c_int32),
+        ("h", C.c_int32),
+        ("image_index", C.c_int32),
+        ("camera_index", C.c_int32),
+        ("camera_model_type", C.c_int32),
+        ("crop_fx", C.c_float),
+        ("crop_fy", C.c_float),
+        ("crop_cx", C.c_float),
+        ("crop_cy", C.c_float),
+        ("crop_s", C.c_float),
+    ]
+
+
+class RenderParams(C.Structure):
+    _fields_ = [
+        ("test_backward_mode", C.c_int32),
+        ("check_normal", C.c_int32),
+        ("ghost_gradients", C.c_int32),
+        ("drop_out_points_by_radius", C.c_int32),
+        ("depth_accept", C.c_float),
+        ("drop_out_radius_threshold", C.c_float),
+        ("dist_cutoff", C.c_float),
+        ("distortion_gradient_factor", C.c_float),
+        ("K_gradient_factor", C.c_float),
+        ("output_background_mask", C.c_int32),
+        ("output_background_mask_value", C.c_float),
+        ("normalize_mode", C.c_int32),
+    ]
+
+
+class Scene(C.Structure):
+    _fields_ = [
+        ("position", C.c_void_p),
+        ("normal", C.c_void_p),
+        ("index", C.c_void_p),
+        ("num_points", C.c_int32),
+        ("texture", C.c_void_p),
+        ("texture_dtype", C.c_int32),
+        ("num_channels", C.c_int32),
+        ("num_texels", C.c_int32),
+        ("background_color", C.c_void_p),
+        ("poses_se3", C.c_void_p),
+        ("num_poses", C.c_int32),
+        ("intrinsics", C.c_void_p),
+        ("num_cameras", C.c_int32),
+        ("intrinsics_cols", C.c_int32),
+    ]
+
+
+class Layer(C.Structure):
+    _fields_ = [
+        ("w", C.c_int32),
+        ("h", C.c_int32),
+        ("depth_index", C.c_void_p),
+        ("depth", C.c_void_p),
+        ("weight", C.c_void_p),
+        ("out", C.c_void_p),
+        ("mask", C.c_void_p),
+    ]
+
+
+class ForwardBuffers(C.Structure):
+    _fields_ = [
+        ("num_layers", C.c_int32),
+        ("layers", Layer * ADOP_MAX_LAYERS),
+        ("dropout_points", C.c_void_p),
+    ]
+
+
+class BackwardBuffers(C.Structure):
+    _fields_ = [
+        ("grad_out", C.c_void_p * ADOP_MAX_LAYERS),
+        ("grad_texture", C.c_void_p),
+        ("grad_background", C.c_void_p),
+        ("grad_points", C.c_void_p),
+        ("grad_points_count", C.c_void_p),
+        ("grad_pose", C.c_void_p),
+        ("grad_pose_count", C.c_void_p),
+        ("grad_intrinsics", C.c_void_p),
+        ("grad_intrinsics_count", C.c_void_p),
+    ]
+
+
+class Stats(C.Structure):
+    _fields_ = [
+        ("visible", C.c_uint64 * ADOP_MAX_LAYERS),
+        ("accepted", C.c_uint64 * ADOP_MAX_LAYERS),
+        ("spatial", C.c_uint64 * ADOP_MAX_LAYERS),
+        ("bad_index", C.c_uint64),
+    ]
+
+
+# Entry points declared in include/adop_raster.h (name -> (restype, argtypes)).
+ENTRY_POINTS = {
+    "adop_workspace_size": (C.c_size_t, [C.POINTER(Scene), C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
+    "adop_forward": (
+        C.c_int,
+        [C.POINTER(Scene), C.POINTER(View), C.c_int32, C.POINTER(RenderParams), C.POINTER(ForwardBuffers),
+         C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
+    ),
+    "adop_backward": (
+        C.c_int,
+        [C.POINTER(Scene), C.POINTER(View), C.c_int32, C.POINTER(RenderParams), C.POINTER(ForwardBuffers),
+         C.POINTER(BackwardBuffers), C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p],
+    ),
+    "adop_env_sample": (
+        C.c_int,
+        [C.POINTER(Scene), C.POINTER(View), C.c_int32, C.c_void_p, C.c_int32, C.c_int32, C.POINTER(ForwardBuffers),
+         C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_int32, C.c_void_p],
+    ),
+    "adop_env_sample_backward": (
+        C.c_int,
+        [C.POINTER(Scene), C.POINTER(View), C.c_int32, C.c_int32, C.c_int32, C.POINTER(ForwardBuffers),
+         C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p],
+    ),
+    "adop_apply_tangent": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "adop_last_error_string": (C.c_char_p, []),
+    "adop_version": (C.c_char_p, []),
+}
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libadop_raster.so")
+
+_lib = None
+
+
+def load_library(path=None):
+    """Load ``libadop_raster.so`` and bind every entry point.  Raises if the library is missing."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    p = path or LIB_PATH
+    if not os.path.exists(p):
+        raise RuntimeError(
+            f"{p} not found: the HIP rasterizer has not been built "
+            "(run `python -c 'import __graft_entry__ as g; g.build()'` or `make -C adop_amd/csrc`). "
+            "There is no CPU fallback."
+        )
+    lib = C.CDLL(p)
+    for name, (restype, argtypes) in ENTRY_POINTS.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    if path is None:
+        _lib = lib
+    return lib

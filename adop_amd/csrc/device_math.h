@@ -1,0 +1,372 @@
+// device_math.h — per-point camera arithmetic of the rasterizer kernels (gfx950 device code).
+//
+// Every function states the reference routine it stands for (paths inside the darglein/ADOP tree; the saiga
+// routines are named by their call sites).  The operation ORDER written here is part of the contract: the file
+// is compiled with -ffp-contract=off, IEEE division and square root, so depth bits and pixel coordinates are
+// reproducible by any implementation that performs the same + - * / sqrt sequence.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#pragma clang fp contract(off)
+
+namespace adop
+{
+struct V2
+{
+    float x, y;
+};
+struct V3
+{
+    float x, y, z;
+};
+
+// One view, prepared on the device from poses_se3 / intrinsics by prepare_views_kernel.
+struct ViewConst
+{
+    float qx, qy, qz, qw;  // world->camera rotation (unit quaternion, float)
+    float tx, ty, tz;
+    float k[5];     // fx fy cx cy s
+    float d[8];     // k1..k6 p1 p2
+    float crop[5];  // crop_transform fx fy cx cy s
+    int32_t w, h;
+    int32_t image_index, camera_index;
+    int32_t model;        // 0 pinhole+distortion, 1 OCam
+    int32_t intr_offset;  // first float of this camera's row in `intrinsics`
+    int32_t npoly;        // OCam: number of world2cam coefficients
+    int32_t pad;
+};
+
+__device__ __forceinline__ uint32_t f2u(float f)
+{
+    return __float_as_uint(f);
+}
+
+// __float2int_rn semantics (PointRenderer.cu:266): nearest-even, saturating, NaN -> 0.
+__device__ __forceinline__ int f2i_rn(float f)
+{
+    if (f != f) return 0;
+    float r = rintf(f);
+    if (r >= 2147483648.f) return 2147483647;
+    if (r <= -2147483648.f) return (-2147483647 - 1);
+    return (int)r;
+}
+
+// Fixed-polynomial arctangent family (Cephes single precision), + - * / sqrt only.
+#define ADOP_PI 3.14159265358979323846f
+#define ADOP_HALF_PI 1.57079632679489661923f
+#define ADOP_QUART_PI 0.78539816339744830962f
+
+__device__ __forceinline__ float atan_poly(float xx)
+{
+    float x = xx < 0 ? -xx : xx;
+    float y;
+    if (x > 2.414213562373095f)
+    {
+        y = ADOP_HALF_PI;
+        x = -(1.0f / x);
+    }
+    else if (x > 0.4142135623730950f)
+    {
+        y = ADOP_QUART_PI;
+        x = (x - 1.0f) / (x + 1.0f);
+    }
+    else
+        y = 0.0f;
+    float z = x * x;
+    float p = (((8.05374449538e-2f * z - 1.38776856032e-1f) * z + 1.99777106478e-1f) * z - 3.33329491539e-1f);
+    y       = y + (p * z * x + x);
+    return xx < 0 ? -y : y;
+}
+
+__device__ __forceinline__ float atan2_poly(float y, float x)
+{
+    if (x == 0.0f)
+    {
+        if (y > 0.0f) return ADOP_HALF_PI;
+        if (y < 0.0f) return -ADOP_HALF_PI;
+        return 0.0f;
+    }
+    float a = atan_poly(y / x);
+    if (x < 0.0f) return (y < 0.0f) ? a - ADOP_PI : a + ADOP_PI;
+    return a;
+}
+
+__device__ __forceinline__ float asin_poly(float xx)
+{
+    float a = xx < 0 ? -xx : xx;
+    if (a > 1.0f) a = 1.0f;
+    bool flag = a > 0.5f;
+    float z, x;
+    if (flag)
+    {
+        z = 0.5f * (1.0f - a);
+        x = sqrtf(z);
+    }
+    else
+    {
+        x = a;
+        z = x * x;
+    }
+    float p = ((((4.2163199048e-2f * z + 2.4181311049e-2f) * z + 4.5470025998e-2f) * z + 7.4953002686e-2f) * z +
+               1.6666752422e-1f);
+    float r = p * z * x + x;
+    if (flag)
+    {
+        r = r + r;
+        r = ADOP_HALF_PI - r;
+    }
+    return xx < 0 ? -r : r;
+}
+
+__device__ __forceinline__ float acos_poly(float x)
+{
+    if (x < -0.5f) return ADOP_PI - 2.0f * asin_poly(sqrtf(0.5f * (1.0f + x)));
+    if (x > 0.5f) return 2.0f * asin_poly(sqrtf(0.5f * (1.0f - x)));
+    return ADOP_HALF_PI - asin_poly(x);
+}
+
+__device__ __forceinline__ V3 cross3(V3 a, V3 b)
+{
+    return {a.y * b.z - a.z * b.y, a.z * b.x - a.x * b.z, a.x * b.y - a.y * b.x};
+}
+__device__ __forceinline__ float dot3(V3 a, V3 b)
+{
+    return (a.x * b.x + a.y * b.y) + a.z * b.z;
+}
+
+// SO3f * v as Eigen evaluates it (Quaternion::_transformVector), used by Sophus for V.so3()*n and V*p
+// (PointRendererHelper.h:55,63).
+__device__ __forceinline__ V3 quat_rotate(float qx, float qy, float qz, float qw, V3 v)
+{
+    V3 q  = {qx, qy, qz};
+    V3 uv = cross3(q, v);
+    uv.x += uv.x;
+    uv.y += uv.y;
+    uv.z += uv.z;
+    V3 c = cross3(q, uv);
+    return {(v.x + qw * uv.x) + c.x, (v.y + qw * uv.y) + c.y, (v.z + qw * uv.z) + c.z};
+}
+
+// UnpackNormal10Bit (NeuralPointCloudCuda.h:96): three 10-bit fields, x in bits 0..9, mapped to [-1,1].
+__device__ __forceinline__ V3 unpack_normal10(int32_t enc)
+{
+    uint32_t e    = (uint32_t)enc;
+    const float s = 2.0f / 1023.0f;
+    return {(float)(e & 1023u) * s - 1.0f, (float)((e >> 10) & 1023u) * s - 1.0f,
+            (float)((e >> 20) & 1023u) * s - 1.0f};
+}
+
+// IntrinsicsPinhole::normalizedToImage
+__device__ __forceinline__ V2 k_apply(const float* K, V2 p)
+{
+    return {(K[0] * p.x + K[4] * p.y) + K[2], K[1] * p.y + K[3]};
+}
+
+// distortNormalizedPoint (PointRendererHelper.h:72,151): OpenCV rational + tangential model, sentinel
+// (100000,100000) beyond the cutoff radius.  Jp: 2x2, Jd: 2x8 (k1..k6,p1,p2), both row-major, optional.
+template <bool WITH_J>
+__device__ __forceinline__ V2 distort(V2 p, const float* D, float max_r, float* Jp, float* Jd)
+{
+    float k1 = D[0], k2 = D[1], k3 = D[2], k4 = D[3], k5 = D[4], k6 = D[5], p1 = D[6], p2 = D[7];
+    float x = p.x, y = p.y;
+    float x2 = x * x, y2 = y * y;
+    float r2  = x2 + y2;
+    float xy2 = 2.0f * x * y;
+    float r4  = r2 * r2;
+    float r6  = r2 * r4;
+    float U   = 1.0f + k1 * r2 + k2 * r4 + k3 * r6;
+    float Vv  = 1.0f + k4 * r2 + k5 * r4 + k6 * r6;
+    float iV  = 1.0f / Vv;
+    float rad = U * iV;
+    float tx  = p1 * xy2 + p2 * (r2 + 2.0f * x2);
+    float ty  = p1 * (r2 + 2.0f * y2) + p2 * xy2;
+    V2 out    = {x * rad + tx, y * rad + ty};
+    if (WITH_J)
+    {
+        float dU  = k1 + 2.0f * k2 * r2 + 3.0f * k3 * r4;
+        float dV  = k4 + 2.0f * k5 * r2 + 3.0f * k6 * r4;
+        float dr  = (dU * Vv - U * dV) * iV * iV;
+        float drx = dr * 2.0f * x, dry = dr * 2.0f * y;
+        Jp[0]     = rad + x * drx + p1 * 2.0f * y + p2 * 6.0f * x;
+        Jp[1]     = x * dry + p1 * 2.0f * x + p2 * 2.0f * y;
+        Jp[2]     = y * drx + p1 * 2.0f * x + p2 * 2.0f * y;
+        Jp[3]     = rad + y * dry + p1 * 6.0f * y + p2 * 2.0f * x;
+        float a   = -U * iV * iV;
+        float cu0 = r2 * iV, cu1 = r4 * iV, cu2 = r6 * iV;
+        float cv0 = r2 * a, cv1 = r4 * a, cv2 = r6 * a;
+        Jd[0] = x * cu0; Jd[1] = x * cu1; Jd[2] = x * cu2;
+        Jd[3] = x * cv0; Jd[4] = x * cv1; Jd[5] = x * cv2;
+        Jd[6] = xy2;     Jd[7] = r2 + 2.0f * x2;
+        Jd[8] = y * cu0; Jd[9] = y * cu1; Jd[10] = y * cu2;
+        Jd[11] = y * cv0; Jd[12] = y * cv1; Jd[13] = y * cv2;
+        Jd[14] = r2 + 2.0f * y2; Jd[15] = xy2;
+    }
+    if (r2 > max_r * max_r)
+    {
+        out.x = 100000.f;
+        out.y = 100000.f;
+    }
+    return out;
+}
+
+// ProjectOCam (PointRendererHelper.h:95,211): Scaramuzza world2cam polynomial for a camera looking along +z.
+template <bool WITH_J>
+__device__ __forceinline__ void ocam_core(V3 p, const float* aff, const float* poly, int npoly, float cutoff, V2* uv,
+                                          float* z_out, float* Jp, float* Ja)
+{
+    float c = aff[0], d = aff[1], e = aff[2], cx = aff[3], cy = aff[4];
+    float x = p.x, y = p.y, z = p.z;
+    float r2   = x * x + y * y;
+    float norm = sqrtf(r2);
+    float dist = sqrtf(r2 + z * z);
+    if (norm == 0.0f)
+    {
+        *uv    = {cx, cy};
+        *z_out = z > 0 ? dist : 0.0f;
+        if (WITH_J)
+        {
+            for (int i = 0; i < 6; ++i) Jp[i] = 0;
+            for (int i = 0; i < 10; ++i) Ja[i] = 0;
+            Ja[3] = 1;
+            Ja[9] = 1;
+        }
+        return;
+    }
+    float theta = atan_poly(-z / norm);
+    float rho   = poly[0];
+    float drho  = 0;
+    float t_i   = 1;
+    for (int i = 1; i < npoly; ++i)
+    {
+        drho += (float)i * poly[i] * t_i;
+        t_i *= theta;
+        rho += t_i * poly[i];
+    }
+    float inv = 1.0f / norm;
+    float cxn = x * inv, cyn = y * inv;
+    float uu = cxn * rho, vv = cyn * rho;
+    *uv    = {(uu * c + vv * d) + cx, (uu * e + vv) + cy};
+    *z_out = theta > cutoff ? 0.0f : dist;
+    if (WITH_J)
+    {
+        float d2  = r2 + z * z;
+        float tx  = z * x / (norm * d2);
+        float ty  = z * y / (norm * d2);
+        float tz  = -norm / d2;
+        float i3  = inv * inv * inv;
+        float uux = rho * (inv - x * x * i3) + cxn * drho * tx;
+        float uuy = rho * (-x * y * i3) + cxn * drho * ty;
+        float uuz = cxn * drho * tz;
+        float vvx = rho * (-x * y * i3) + cyn * drho * tx;
+        float vvy = rho * (inv - y * y * i3) + cyn * drho * ty;
+        float vvz = cyn * drho * tz;
+        Jp[0] = c * uux + d * vvx; Jp[1] = c * uuy + d * vvy; Jp[2] = c * uuz + d * vvz;
+        Jp[3] = e * uux + vvx;     Jp[4] = e * uuy + vvy;     Jp[5] = e * uuz + vvz;
+        Ja[0] = uu; Ja[1] = vv; Ja[2] = 0;  Ja[3] = 1; Ja[4] = 0;
+        Ja[5] = 0;  Ja[6] = 0;  Ja[7] = uu; Ja[8] = 0; Ja[9] = 1;
+    }
+}
+
+// Head of the three reference point kernels (PointRenderer.cu:227-256, 334-359, 409-438):
+// ProjectPointPinhole / ProjectPointOcam (PointRendererHelper.h:49-106), the LOD radius in pixels and the
+// crop transform.  Returns false when the point is culled (z == 0).
+__device__ __forceinline__ bool project_point(const ViewConst& vc, const float* __restrict__ intrinsics, V3 pos,
+                                              V3 nrm, float radius, bool check_normal, float dist_cutoff, int w0,
+                                              V2* ip, float* z_out, float* radius_pixels, V3* view_p_out)
+{
+    V3 r      = quat_rotate(vc.qx, vc.qy, vc.qz, vc.qw, pos);
+    V3 view_p = {r.x + vc.tx, r.y + vc.ty, r.z + vc.tz};
+    *view_p_out = view_p;
+    V2 image_p;
+    float z;
+    if (vc.model == 0)
+    {
+        z = fmaxf(view_p.z, 0.f);
+        if (check_normal)
+        {
+            V3 view_n = quat_rotate(vc.qx, vc.qy, vc.qz, vc.qw, nrm);
+            if (dot3(view_p, view_n) > 0) z = 0;
+        }
+        float iz  = 1.0f / view_p.z;
+        V2 norm_p = {view_p.x * iz, view_p.y * iz};
+        V2 dist_p = distort<false>(norm_p, vc.d, dist_cutoff, nullptr, nullptr);
+        if (dist_p.x == 100000.f) z = 0;
+        image_p        = k_apply(vc.k, dist_p);
+        *radius_pixels = vc.k[0] * vc.crop[0] * radius / z;
+    }
+    else
+    {
+        const float* row = intrinsics + vc.intr_offset;
+        ocam_core<false>(view_p, row, row + 5, vc.npoly, dist_cutoff, &image_p, &z, nullptr, nullptr);
+        V3 view_n = quat_rotate(vc.qx, vc.qy, vc.qz, vc.qw, nrm);
+        if (check_normal & (dot3(view_p, view_n) > 0)) z = 0;
+        *radius_pixels = (float)w0 * vc.crop[0] * radius / z;
+    }
+    *z_out = z;
+    if (z == 0) return false;
+    *ip = k_apply(vc.crop, image_p);
+    return true;
+}
+
+struct BackwardOut
+{
+    float g_point[3];
+    float g_pose[6];
+    float g_k[5];    // pinhole K (fx,fy,cx,cy,s) or OCam affine (c,d,e,cx,cy)
+    float g_dis[8];  // pinhole distortion
+};
+
+// ProjectPointPinholeBackward / ProjectPointOcamBackward (PointRendererHelper.h:120-170, 184-227):
+// J_point^T J_div^T J_dis^T J_K^T J_crop^T g.  The pose Jacobian is that of a left perturbation
+// exp(eps)*V with translation first: J_pose = [I | -[V p]x], so J_pose^T c = (c, (V p) x c).
+__device__ __forceinline__ void project_point_backward(const ViewConst& vc, const float* __restrict__ intrinsics,
+                                                       V3 view_p, V2 grad, const float* crop, float dist_cutoff,
+                                                       BackwardOut* o)
+{
+    V2 g2 = {crop[0] * grad.x, crop[4] * grad.x + crop[1] * grad.y};
+    V3 c;
+    if (vc.model == 0)
+    {
+        float iz  = 1.0f / view_p.z;
+        V2 norm_p = {view_p.x * iz, view_p.y * iz};
+        float Jp[4], Jd[16];
+        V2 dist_p = distort<true>(norm_p, vc.d, dist_cutoff, Jp, Jd);
+        V2 g1     = {vc.k[0] * g2.x, vc.k[4] * g2.x + vc.k[1] * g2.y};
+        V2 g0     = {Jp[0] * g1.x + Jp[2] * g1.y, Jp[1] * g1.x + Jp[3] * g1.y};
+        c         = {g0.x * iz, g0.y * iz, (-(view_p.x * iz * iz)) * g0.x + (-(view_p.y * iz * iz)) * g0.y};
+        o->g_k[0] = dist_p.x * g2.x;
+        o->g_k[1] = dist_p.y * g2.y;
+        o->g_k[2] = g2.x;
+        o->g_k[3] = g2.y;
+        o->g_k[4] = dist_p.y * g2.x;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o->g_dis[i] = Jd[i] * g1.x + Jd[8 + i] * g1.y;
+    }
+    else
+    {
+        const float* row = intrinsics + vc.intr_offset;
+        float Jp[6], Ja[10];
+        V2 uv;
+        float z;
+        ocam_core<true>(view_p, row, row + 5, vc.npoly, dist_cutoff, &uv, &z, Jp, Ja);
+        c = {Jp[0] * g2.x + Jp[3] * g2.y, Jp[1] * g2.x + Jp[4] * g2.y, Jp[2] * g2.x + Jp[5] * g2.y};
+#pragma unroll
+        for (int i = 0; i < 5; ++i) o->g_k[i] = Ja[i] * g2.x + Ja[5 + i] * g2.y;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o->g_dis[i] = 0;
+    }
+    V3 gp         = quat_rotate(-vc.qx, -vc.qy, -vc.qz, vc.qw, c);
+    o->g_point[0] = gp.x;
+    o->g_point[1] = gp.y;
+    o->g_point[2] = gp.z;
+    V3 rc         = cross3(view_p, c);
+    o->g_pose[0]  = c.x;
+    o->g_pose[1]  = c.y;
+    o->g_pose[2]  = c.z;
+    o->g_pose[3]  = rc.x;
+    o->g_pose[4]  = rc.y;
+    o->g_pose[5]  = rc.z;
+}
+
+}  // namespace adop

@@ -1,0 +1,200 @@
+/*
+ * adop_raster.h — C-ABI of the MI355X (gfx950) one-pixel point rasterizer.
+ *
+ * Torch-free boundary: plain device pointers, explicit shapes, POD structs. Every entry point enqueues
+ * work on the caller's HIP stream and returns without a device-wide synchronisation; nothing here
+ * allocates device memory (the caller passes outputs plus a workspace sized by adop_workspace_size()).
+ *
+ * Each declaration cites the piece of darglein/ADOP it replaces (paths relative to the ADOP source tree).
+ *
+ * Tensor layouts are the reference's:
+ *   t_position [N,4] f32 (x,y,z,drop_out_radius)    src/lib/rendering/NeuralPointCloudCuda.h:35,82-103
+ *   t_normal   [N,1] i32 (3x10-bit packed normal)   NeuralPointCloudCuda.h:37,94-97
+ *   t_index    [N,1] i32 (texel of the point)       NeuralPointCloudCuda.h:41,105
+ *   texture    [C,N_tex] f32 (channel-major)        src/lib/models/NeuralTexture.h:62-65
+ *   background [C] f32
+ *   poses_se3  [F,8] f64  (qx,qy,qz,qw,tx,ty,tz,pad) world->camera  src/lib/data/NeuralStructure.cpp:13-27
+ *   intrinsics [K,13] f32 (fx,fy,cx,cy,s,k1..k6,p1,p2) or [K,5+P] (c,d,e,cx,cy,world2cam poly)
+ *                                                   NeuralStructure.cpp:64-133, PointRenderer.cu:78-96
+ *   per level l: depth_l/weight_l/mask_l [B,1,h_l,w_l] f32, out_l [B,C,h_l,w_l] f32,
+ *                h_l = h>>l, w_l = w>>l             PointRenderer.cu:996-1018,1045-1071
+ */
+#ifndef ADOP_RASTER_H
+#define ADOP_RASTER_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ADOP_MAX_LAYERS 5 /* constexpr int max_layers = 5, PointRenderer.h:20 */
+
+/* Error convention: the reference aborts (SAIGA_ASSERT / device asserts, PointRenderer.cu:1199,362,481).
+ * The C-ABI returns a status and keeps a per-thread message instead. */
+typedef enum adop_status
+{
+    ADOP_OK                 = 0,
+    ADOP_INVALID_ARG        = 1,
+    ADOP_UNSUPPORTED_LAYERS = 2, /* "invalid number of layers", PointRenderer.cu:1199 */
+    ADOP_HIP_ERROR          = 3,
+    ADOP_WORKSPACE_TOO_SMALL = 4
+} adop_status;
+
+/* enum class CameraModel, src/lib/data/SceneData.h:28-32 */
+typedef enum adop_camera_model
+{
+    ADOP_CAMERA_PINHOLE_DISTORTION = 0,
+    ADOP_CAMERA_OCAM               = 1
+} adop_camera_model;
+
+typedef enum adop_texture_dtype
+{
+    ADOP_TEXTURE_F32 = 0, /* the reference's only storage type */
+    ADOP_TEXTURE_F16 = 1  /* half storage, fp32 accumulation (extension for the 100M-point viewer case) */
+} adop_texture_dtype;
+
+/* struct ReducedImageInfo, SceneData.h:37-47 (passed by value to every reference kernel). */
+typedef struct adop_view
+{
+    int32_t w, h;
+    int32_t image_index;       /* row of poses_se3 */
+    int32_t camera_index;      /* row of intrinsics */
+    int32_t camera_model_type; /* adop_camera_model */
+    float crop_fx, crop_fy, crop_cx, crop_cy, crop_s; /* IntrinsicsPinholef crop_transform */
+} adop_view;
+
+/* struct RenderParams (Settings.h:22-52) as consumed by DeviceRenderParams (PointRenderer.cu:47-117). */
+typedef struct adop_render_params
+{
+    int32_t test_backward_mode;        /* only the value 4 changes behaviour, PointRenderer.cu:543-566 */
+    int32_t check_normal;              /* back-face cull, PointRendererHelper.h:59-68 */
+    int32_t ghost_gradients;           /* PointRenderer.cu:487-488 */
+    int32_t drop_out_points_by_radius; /* PointRenderer.cu:261-264 */
+    float depth_accept;                /* fuzzy depth threshold (relative), PointRenderer.cu:380 */
+    float drop_out_radius_threshold;
+    float dist_cutoff;                 /* pinhole: distortion radius cutoff; OCam: theta cutoff */
+    float distortion_gradient_factor;  /* PointRenderer.cu:661 */
+    float K_gradient_factor;           /* PointRenderer.cu:647 */
+    int32_t output_background_mask;    /* CreateMask is run, PointRenderer.cu:1454-1460 */
+    float output_background_mask_value;
+    /* 0: NormalizeGradient exactly as the reference launches it (points normalised through a vec3 view of
+     *    the [N,4] buffer, intrinsics always as 13 floats per row; PointRenderer.cu:1611-1636).
+     * 1: row-wise normalisation (points row i by count i, intrinsics over the real row width). */
+    int32_t normalize_mode;
+} adop_render_params;
+
+/* Inputs owned by NeuralScene: NeuralPointCloudCuda + NeuralTexture + PoseModule + IntrinsicsModule. */
+typedef struct adop_scene
+{
+    const float* position;   /* [N,4] */
+    const int32_t* normal;   /* [N] or NULL (then check_normal must be 0; NeuralScene.cpp:28) */
+    const int32_t* index;    /* [N] */
+    int32_t num_points;
+    const void* texture;     /* [C,N_tex] f32 or f16 */
+    int32_t texture_dtype;   /* adop_texture_dtype */
+    int32_t num_channels;    /* C <= 16 */
+    int32_t num_texels;      /* N_tex */
+    const float* background_color; /* [C] */
+    const double* poses_se3; /* [F,8] */
+    int32_t num_poses;
+    const float* intrinsics; /* [K,intrinsics_cols] */
+    int32_t num_cameras;
+    int32_t intrinsics_cols;
+} adop_scene;
+
+/* struct LayerCuda (PointRenderer.h:65-94) plus the per-level output tensors of PointRendererCache
+ * (output_forward, output_forward_background_mask; PointRenderer.h:131-132). */
+typedef struct adop_layer
+{
+    int32_t w, h;
+    uint64_t* depth_index; /* [B,1,h,w] u64 = (float bits of depth << 32) | point id; PackIndex,
+                              PointRendererHelper.h:30-34. Empty pixel: (bits(100000.f) << 32) | 0xFFFFFFFF */
+    float* depth;          /* [B,1,h,w] high word of depth_index as f32 (saved for backward) */
+    float* weight;         /* [B,1,h,w] */
+    float* out;            /* [B,C,h,w] */
+    float* mask;           /* [B,1,h,w] or NULL */
+} adop_layer;
+
+typedef struct adop_forward_buffers
+{
+    int32_t num_layers;
+    adop_layer layers[ADOP_MAX_LAYERS];
+    /* [B,N] f32 in {0,1}; 1 = point is dropped for that image. NULL = nothing dropped. The reference
+     * draws it with bernoulli_ inside InitializeData (PointRenderer.cu:1081-1088); here it is an input so
+     * that both sides of a parity test see the same mask. */
+    const float* dropout_points;
+} adop_forward_buffers;
+
+/* DeviceBackwardParams (PointRenderer.cu:124-137) + the tensors PointRendererCache::Build(.., false)
+ * creates (PointRenderer.cu:922-949). Every non-NULL gradient buffer is cleared by adop_backward. */
+typedef struct adop_backward_buffers
+{
+    const float* grad_out[ADOP_MAX_LAYERS]; /* upstream [B,C,h_l,w_l] */
+    float* grad_texture;          /* [C,N_tex] */
+    float* grad_background;       /* [C] */
+    float* grad_points;           /* [N,4] or NULL */
+    float* grad_points_count;     /* [N]   (required iff grad_points) */
+    double* grad_pose;            /* [F,6] f64 or NULL */
+    float* grad_pose_count;       /* [F] */
+    float* grad_intrinsics;       /* [K,intrinsics_cols] or NULL */
+    float* grad_intrinsics_count; /* [K] */
+} adop_backward_buffers;
+
+/* Counters filled by the kernels (uint64 each), used for the algorithmic byte model. */
+typedef struct adop_stats
+{
+    uint64_t visible[ADOP_MAX_LAYERS];  /* V_l: point-levels that land inside the image */
+    uint64_t accepted[ADOP_MAX_LAYERS]; /* A_l: ... that also pass the fuzzy depth test and are blended */
+    uint64_t spatial[ADOP_MAX_LAYERS];  /* G_l: ... that receive a ghost / spatial gradient */
+    uint64_t bad_index;                 /* texture index out of range (reference: device assert :362) */
+} adop_stats;
+
+/* Size in bytes of the workspace adop_forward / adop_backward need for B views. */
+size_t adop_workspace_size(const adop_scene* scene, int32_t num_views, int32_t num_layers, int32_t w, int32_t h);
+
+/* Replaces BlendPointCloudForward (PointRenderer.cu:1389-1531): InitializeData (:1039-1090),
+ * DepthPrepassMulti (:203-301,1166-1203), RenderForwardMulti (:303-393,1294-1335),
+ * CombineAndFill (:726-754,1268-1291), CreateMask (:828-847,1371-1387).
+ * `stats` may be NULL; if not, it is a device pointer that receives adop_stats (forward fields). */
+adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_t num_views,
+                         const adop_render_params* params, const adop_forward_buffers* buffers, void* workspace,
+                         size_t workspace_bytes, adop_stats* stats, void* hip_stream);
+
+/* Replaces BlendPointCloudBackward (PointRenderer.cu:1549-1644): CombineAndFillBackward (:851-900),
+ * RenderBackward (:396-724), NormalizeGradient (:1534-1547,1611-1636). `fwd` holds depth/weight/out as
+ * left by adop_forward (the reference's saved variables, :1517-1525). */
+adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32_t num_views,
+                          const adop_render_params* params, const adop_forward_buffers* fwd,
+                          const adop_backward_buffers* grads, void* workspace, size_t workspace_bytes,
+                          adop_stats* stats, void* hip_stream);
+
+/* Replaces EnvironmentMapImpl::Sample (EnvironmentMap.cu:107-157: BuildSphericalUV + grid_sample bilinear /
+ * border / align_corners) fused with the composition images += (1-mask)*env (RenderModule.cpp:121-125).
+ * env_texture [C,eh,ew] f32. For level l: uv_l [B,h_l,w_l,2] (may be NULL), env_l [B,C,h_l,w_l] (may be NULL),
+ * and, if add_to_out != 0, out_l += (1 - mask_l) * env. */
+adop_status adop_env_sample(const adop_scene* scene, const adop_view* views, int32_t num_views,
+                            const float* env_texture, int32_t env_h, int32_t env_w, const adop_forward_buffers* buffers,
+                            float* const* uv_levels, float* const* env_levels, int32_t add_to_out, void* hip_stream);
+
+/* Gradient of adop_env_sample w.r.t. env_texture: grad_env [C,eh,ew] += sum over pixels of
+ * (1-mask) * grad_out * bilinear weights (torch autograd of grid_sample in the reference). */
+adop_status adop_env_sample_backward(const adop_scene* scene, const adop_view* views, int32_t num_views,
+                                     int32_t env_h, int32_t env_w, const adop_forward_buffers* buffers,
+                                     const float* const* grad_out_levels, float* grad_env, void* hip_stream);
+
+/* Replaces ApplyTangentToPose / ApplyTangent (PointRenderer.cu:1646-1665): pose = se3_exp(tangent) * pose,
+ * tangent = 0; f64. tangent [F,6], poses_se3 [F,8]. */
+adop_status adop_apply_tangent(double* tangent, double* poses_se3, int32_t num_poses, void* hip_stream);
+
+/* Message for the last non-OK status returned on the calling thread. */
+const char* adop_last_error_string(void);
+
+/* Library version / build identification. */
+const char* adop_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ADOP_RASTER_H */

@@ -1,0 +1,117 @@
+"""Shared helpers of the GPU parity tests: run a HostScene through the HIP path and compare with the CPU checker."""
+import sys
+
+import numpy as np
+
+
+def announce(msg):
+    print(f"[case] {msg}", flush=True)
+    sys.stdout.flush()
+
+
+def run_hip_forward(hs, collect_stats=True):
+    import torch
+    from adop_amd import render
+
+    scene = render.NeuralScene.from_host(hs, "cuda")
+    cache = render.PointRendererCache()
+    info = render.NeuralRenderInfo(scene=scene, images=list(hs.views), params=hs.params, num_layers=hs.num_layers,
+                                   cache=cache, collect_stats=collect_stats,
+                                   dropout_points=None if hs.dropout is None else torch.from_numpy(hs.dropout))
+
+    class Ctx:
+        def save_for_backward(self, *t):
+            self.saved_tensors = t
+
+    ctx = Ctx()
+    images, masks = render.BlendPointCloudForward(ctx, info)
+    torch.cuda.synchronize()
+    return scene, info, ctx, images, masks
+
+
+def download_forward(hs, info, images, masks):
+    """The HIP forward state (the reference's saved variables) as a checker-side ForwardResult."""
+    import oracle
+
+    res = oracle.ForwardResult(hs)
+    for l, L in enumerate(info.cache.layers_cuda):
+        res.depth_index[l][...] = L.depth_index_tensor.cpu().numpy().view(np.uint64)
+        res.depth[l][...] = L.depth.cpu().numpy()
+        res.weight[l][...] = L.weight.cpu().numpy()
+        res.out[l][...] = images[l].detach().cpu().numpy()
+        if masks:
+            res.mask[l][...] = masks[l].cpu().numpy()
+    return res
+
+
+def assert_norm_close(got, want, tol, what):
+    """tensor-level bound: max|got-want| <= tol * max|want| (for sums whose terms cancel)."""
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    assert np.isfinite(got).all(), what + ": non-finite values"
+    scale = np.abs(want).max()
+    err = np.abs(got - want).max()
+    assert err <= tol * max(scale, 1e-30), f"{what}: max error {err} vs scale {scale}"
+
+
+def rel_err(a, b):
+    a = np.asarray(a, np.float64)
+    b = np.asarray(b, np.float64)
+    return np.abs(a - b) / np.maximum(np.abs(b), 1e-30)
+
+
+def assert_close(got, want, rel, abs_tol, what):
+    """|got-want| <= max(rel*|want|, abs_tol) element-wise."""
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    assert got.shape == want.shape, (what, got.shape, want.shape)
+    assert np.isfinite(got).all(), what + ": non-finite values"
+    err = np.abs(got - want)
+    tol = np.maximum(rel * np.abs(want), abs_tol)
+    bad = err > tol
+    if bad.any():
+        i = np.unravel_index(np.argmax(err - tol), err.shape)
+        raise AssertionError(f"{what}: {bad.sum()} of {bad.size} elements out of tolerance; worst at {i}: "
+                             f"got {got[i]!r} want {want[i]!r}")
+
+
+def check_forward(hs, ref, ctx, images, masks, info):
+    """depth/index bit-exact; weight exact; blended descriptors within 1e-5 relative."""
+    cache = info.cache
+    for l in range(hs.num_layers):
+        L = cache.layers_cuda[l]
+        di = L.depth_index_tensor.cpu().numpy().view(np.uint64)
+        assert np.array_equal(di, ref.depth_index[l]), f"level {l}: packed depth|index differs"
+        d = L.depth.cpu().numpy()
+        assert np.array_equal(d.view(np.uint32), ref.depth[l].view(np.uint32)), f"level {l}: depth bits differ"
+        w = L.weight.cpu().numpy()
+        assert np.array_equal(w, ref.weight[l]), f"level {l}: weight differs"
+        assert_close(images[l].cpu().numpy(), ref.out[l], 1e-5, 1e-7, f"level {l} out")
+        if hs.params.output_background_mask:
+            assert np.array_equal(masks[l].cpu().numpy(), ref.mask[l]), f"level {l}: mask differs"
+    st = cache.read_stats()
+    for l in range(hs.num_layers):
+        assert st.visible[l] == ref.stats.visible[l], ("visible", l, st.visible[l], ref.stats.visible[l])
+        assert st.accepted[l] == ref.stats.accepted[l], ("accepted", l, st.accepted[l], ref.stats.accepted[l])
+
+
+def check_backward(hs, refb, grads, info):
+    """gradients within 1e-4 relative or 1e-6 absolute (float atomics reorder the sums)."""
+    g_tex, g_bg, g_pts, g_pose, g_intr = grads
+    cache = info.cache
+    assert_close(g_tex.cpu().numpy(), refb.grad_texture, 1e-4, 1e-6, "grad_texture")
+    assert_close(g_bg.cpu().numpy(), refb.grad_background, 1e-4, 1e-5, "grad_background")
+    if g_pts is not None:
+        assert np.array_equal(cache.output_gradient_point_count.cpu().numpy(), refb.grad_points_count), "point count"
+        assert_close(g_pts.cpu().numpy(), refb.grad_points, 1e-4, 1e-6, "grad_points")
+    if g_pose is not None:
+        assert np.array_equal(cache.output_gradient_pose_tangent_count.cpu().numpy(), refb.grad_pose_count)
+        scale = np.abs(refb.grad_pose).max() + 1e-30
+        assert_close(g_pose.cpu().numpy(), refb.grad_pose, 1e-4, 1e-6 * max(scale, 1.0), "grad_pose")
+    if g_intr is not None:
+        assert np.array_equal(cache.output_gradient_intrinsics_count.cpu().numpy(), refb.grad_intrinsics_count)
+        scale = np.abs(refb.grad_intrinsics).max() + 1e-30
+        assert_close(g_intr.cpu().numpy(), refb.grad_intrinsics, 1e-4, 1e-6 * max(scale, 1.0), "grad_intrinsics")
+    st = cache.read_stats()
+    for l in range(hs.num_layers):
+        assert st.spatial[l] == refb.stats.spatial[l], ("spatial", l, st.spatial[l], refb.stats.spatial[l])
