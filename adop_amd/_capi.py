@@ -116,6 +116,10 @@ class Stats(C.Structure):
     ]
 
 
+class StageTime(C.Structure):
+    _fields_ = [("name", C.c_char * 32), ("total_ms", C.c_float), ("calls", C.c_int32)]
+
+
 # Entry points declared in include/adop_raster.h (name -> (restype, argtypes)).
 ENTRY_POINTS = {
     "adop_workspace_size": (C.c_size_t, [C.POINTER(Scene), C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
@@ -140,6 +144,8 @@ ENTRY_POINTS = {
          C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p],
     ),
     "adop_apply_tangent": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "adop_profile_enable": (C.c_int, [C.c_int32]),
+    "adop_profile_read": (C.c_int32, [C.POINTER(StageTime), C.c_int32]),
     "adop_last_error_string": (C.c_char_p, []),
     "adop_version": (C.c_char_p, []),
 }

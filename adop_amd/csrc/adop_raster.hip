@@ -22,6 +22,7 @@
 #include <string.h>
 
 #include <string>
+#include <vector>
 
 #include "../../include/adop_raster.h"
 #include "device_math.h"
@@ -974,6 +975,49 @@ adop_status fail(adop_status s, const std::string& msg)
             return fail(ADOP_HIP_ERROR, std::string(#expr) + ": " + hipGetErrorString(e_));              \
     } while (0)
 
+// Stage timers: HIP events recorded on the caller's stream around each kernel launch when profiling is enabled
+// on the calling thread (the reference's SAIGA_OPTIONAL_TIME_MEASURE scopes, PointRenderer.cu:906-1610).
+struct StageEvent
+{
+    const char* name;
+    hipEvent_t start, stop;
+};
+thread_local bool g_profile = false;
+thread_local std::vector<StageEvent> g_stage_events;
+thread_local std::vector<hipEvent_t> g_event_pool;
+
+hipEvent_t take_event()
+{
+    if (!g_event_pool.empty())
+    {
+        hipEvent_t e = g_event_pool.back();
+        g_event_pool.pop_back();
+        return e;
+    }
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) return nullptr;
+    return e;
+}
+
+struct StageScope
+{
+    hipStream_t st;
+    hipEvent_t stop = nullptr;
+    StageScope(const char* name, hipStream_t s) : st(s)
+    {
+        if (!g_profile) return;
+        hipEvent_t a = take_event(), b = take_event();
+        if (!a || !b) return;
+        (void)hipEventRecord(a, st);
+        g_stage_events.push_back({name, a, b});
+        stop = b;
+    }
+    ~StageScope()
+    {
+        if (stop) (void)hipEventRecord(stop, st);
+    }
+};
+
 struct WorkspaceLayout
 {
     size_t views;       // ViewConst[B]
@@ -1184,16 +1228,24 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
         st = fill_async(stats, sizeof(adop_stats), 0, stream);
         if (st != ADOP_OK) return st;
     }
-    hipLaunchKernelGGL(clear_kernel, dim3(pixel_grid(lv)), dim3(kBlock), 0, stream, lv);
+    {
+        StageScope sc("Initialize", stream);
+        hipLaunchKernelGGL(clear_kernel, dim3(pixel_grid(lv)), dim3(kBlock), 0, stream, lv);
+    }
 
     int grid = (scene->num_points + kBlock - 1) / kBlock;
     if (grid > 0)
     {
-        if (stats)
-            hipLaunchKernelGGL((prepass_kernel<true>), dim3(grid), dim3(kBlock), 0, stream, pc, dviews, lv, rp, stats);
-        else
-            hipLaunchKernelGGL((prepass_kernel<false>), dim3(grid), dim3(kBlock), 0, stream, pc, dviews, lv, rp,
-                               stats);
+        {
+            StageScope sc("DepthPrepass", stream);
+            if (stats)
+                hipLaunchKernelGGL((prepass_kernel<true>), dim3(grid), dim3(kBlock), 0, stream, pc, dviews, lv, rp,
+                                   stats);
+            else
+                hipLaunchKernelGGL((prepass_kernel<false>), dim3(grid), dim3(kBlock), 0, stream, pc, dviews, lv, rp,
+                                   stats);
+        }
+        StageScope sc("RenderForward", stream);
         bool half = scene->texture_dtype == ADOP_TEXTURE_F16;
         if (half && stats)
             hipLaunchKernelGGL((blend_kernel<true, true>), dim3(grid), dim3(kBlock), 0, stream, pc, dviews, lv, rp,
@@ -1208,8 +1260,11 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
             hipLaunchKernelGGL((blend_kernel<false, false>), dim3(grid), dim3(kBlock), 0, stream, pc, dviews, lv, rp,
                                stats);
     }
-    hipLaunchKernelGGL(resolve_kernel, dim3(pixel_grid(lv)), dim3(kBlock), 0, stream, lv, scene->background_color,
-                       params->output_background_mask, params->output_background_mask_value);
+    {
+        StageScope sc("CombineAndFill", stream);
+        hipLaunchKernelGGL(resolve_kernel, dim3(pixel_grid(lv)), dim3(kBlock), 0, stream, lv, scene->background_color,
+                           params->output_background_mask, params->output_background_mask_value);
+    }
     ADOP_HIP_CHECK(hipGetLastError());
     return ADOP_OK;
 }
@@ -1246,21 +1301,29 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     const int N = scene->num_points;
 
     // Build(info,false): zero the gradient tensors (:922-949)
-    if ((st = fill_async(grads->grad_texture, sizeof(float) * (size_t)C * scene->num_texels, 0, stream)) != ADOP_OK)
-        return st;
-    if (grads->grad_points)
     {
-        if ((st = fill_async(grads->grad_points, sizeof(float) * 4 * (size_t)N, 0, stream)) != ADOP_OK) return st;
-        if ((st = fill_async(grads->grad_points_count, sizeof(float) * (size_t)N, 0, stream)) != ADOP_OK) return st;
-    }
-    if (stats)
-    {
-        // keep the forward counters, clear only the backward ones
-        if ((st = fill_async(stats->spatial, sizeof(uint64_t) * ADOP_MAX_LAYERS, 0, stream)) != ADOP_OK) return st;
+        StageScope sc("Prepare Backward", stream);
+        if ((st = fill_async(grads->grad_texture, sizeof(float) * (size_t)C * scene->num_texels, 0, stream)) != ADOP_OK)
+            return st;
+        if (grads->grad_points)
+        {
+            if ((st = fill_async(grads->grad_points, sizeof(float) * 4 * (size_t)N, 0, stream)) != ADOP_OK) return st;
+            if ((st = fill_async(grads->grad_points_count, sizeof(float) * (size_t)N, 0, stream)) != ADOP_OK)
+                return st;
+        }
+        if (stats)
+        {
+            // keep the forward counters, clear only the backward ones
+            if ((st = fill_async(stats->spatial, sizeof(uint64_t) * ADOP_MAX_LAYERS, 0, stream)) != ADOP_OK)
+                return st;
+        }
     }
 
     int bg_blocks = pixel_grid(lv) < kPartialBlocks ? pixel_grid(lv) : kPartialBlocks;
-    hipLaunchKernelGGL(background_grad_kernel, dim3(bg_blocks), dim3(kBlock), 0, stream, lv, bg_partial);
+    {
+        StageScope sc("CombineAndFillBackward", stream);
+        hipLaunchKernelGGL(background_grad_kernel, dim3(bg_blocks), dim3(kBlock), 0, stream, lv, bg_partial);
+    }
 
     int want_pose = grads->grad_pose != nullptr;
     int want_intr = grads->grad_intrinsics != nullptr;
@@ -1270,6 +1333,7 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     bool half = scene->texture_dtype == ADOP_TEXTURE_F16;
     for (int b = 0; b < num_views; ++b)
     {
+        StageScope sc("RenderBackward", stream);
 #define ADOP_LAUNCH_BWD(H, S)                                                                                       \
     hipLaunchKernelGGL((render_backward_kernel<H, S>), dim3(pt_blocks), dim3(kBlock), 0, stream, pc, dviews, lv, rp, \
                        grads->grad_texture, grads->grad_points, grads->grad_points_count, want_pose, want_intr, b,   \
@@ -1284,6 +1348,7 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
             ADOP_LAUNCH_BWD(false, false);
 #undef ADOP_LAUNCH_BWD
     }
+    StageScope post("Post Process Gradient", stream);
     hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kBlock), 0, stream, dviews, num_views, C, bg_partial, bg_blocks,
                        pt_partial, pt_blocks, grads->grad_background, grads->grad_pose, grads->grad_pose_count,
                        scene->num_poses, grads->grad_intrinsics, grads->grad_intrinsics_count, scene->num_cameras,
@@ -1389,6 +1454,42 @@ adop_status adop_apply_tangent(double* tangent, double* poses_se3, int32_t num_p
                        tangent, poses_se3, num_poses);
     ADOP_HIP_CHECK(hipGetLastError());
     return ADOP_OK;
+}
+
+adop_status adop_profile_enable(int32_t enable)
+{
+    g_profile = enable != 0;
+    return ADOP_OK;
+}
+
+int32_t adop_profile_read(adop_stage_time* out, int32_t max_entries)
+{
+    int n = 0;
+    for (StageEvent& e : g_stage_events)
+    {
+        float ms = 0.f;
+        if (hipEventSynchronize(e.stop) == hipSuccess && hipEventElapsedTime(&ms, e.start, e.stop) == hipSuccess)
+        {
+            int k = 0;
+            for (; k < n; ++k)
+                if (strcmp(out[k].name, e.name) == 0) break;
+            if (k == n && n < max_entries)
+            {
+                memset(&out[n], 0, sizeof(out[n]));
+                strncpy(out[n].name, e.name, sizeof(out[n].name) - 1);
+                ++n;
+            }
+            if (k < n)
+            {
+                out[k].total_ms += ms;
+                out[k].calls += 1;
+            }
+        }
+        g_event_pool.push_back(e.start);
+        g_event_pool.push_back(e.stop);
+    }
+    g_stage_events.clear();
+    return n;
 }
 
 const char* adop_last_error_string(void)

@@ -1,0 +1,230 @@
+#!/usr/bin/env python3
+"""Benchmark of the point-rasterizer hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config3|config2|config4|config5]
+
+A step is one pass of the hot path over one batch of synthetic input that already sits in HBM:
+``adop_forward`` + ``adop_backward`` through the C-ABI (forward only for the viewer workload config4).
+Prints ONE JSON line.  Default workload: BASELINE config 3 (10 M points, 1920x1080, 4 levels, 8 channels,
+forward + backward with descriptor / point / pose / intrinsics gradients) -> points/s.
+
+``roofline`` describes the slowest kernel of the step: algorithmic bytes of that kernel (byte model below, with
+the point-level counts V/A/G measured by the kernels' own counters in an untimed pass) divided by its average
+duration measured with HIP events on the launch stream, against the 8 TB/s HBM peak.
+``cpu_baseline`` times the CPU checker (OpenMP build) on the host cores for the same workload (or a bounded
+sample of it).
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def byte_model(N, B, C_, S_d, P, V, A, G, has_mask, has_dropout):
+    """Algorithmic bytes per kernel for one step (per-unit figures of the hot-path byte model)."""
+    sv, sa, sg = sum(V), sum(A), sum(G)
+    drop = 4 if has_dropout else 0
+    k = {}
+    k["DepthPrepass"] = B * N * 20 + sv * 8
+    k["RenderForward"] = B * N * (24 + drop) + sa * (C_ * S_d + C_ * 4 + 4)
+    k["CombineAndFill"] = B * P * (8 + 4 + 2 * C_ * 4) + (B * P * 4 if has_mask else 0)
+    k["RenderBackward"] = B * N * (24 + drop) + sa * (4 + 4 + C_ * 4 + C_ * 4) + sg * (4 * (8 + 8 * C_) + C_ * S_d + 16)
+    k["CombineAndFillBackward"] = B * P * (4 + 4 * C_)
+    return k
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="config3", choices=["config2", "config3", "config4", "config5"])
+    ap.add_argument("--points", type=int, default=0, help="override the point count (0 = the configuration's)")
+    ap.add_argument("--point-order", default="morton", choices=["morton", "random"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-points", type=int, default=0, help="point count of the CPU sample (0 = automatic)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (one process, one MI355X); "
+              "a figure at several GPUs is not produced. Use --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from adop_amd import _capi, render, scenes
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    lib = _capi.load_library()
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+
+    t0 = time.time()
+    kw = {"n": args.points} if args.points else {}
+    if args.workload == "config3":
+        hs = scenes.config3(point_order=args.point_order, **kw)
+    elif args.workload == "config2":
+        hs = scenes.config2(**kw)
+    elif args.workload == "config4":
+        hs = scenes.config4(**kw)
+    else:
+        hs = scenes.config5(**kw)
+    backward = args.workload != "config4"
+    gen_s = time.time() - t0
+
+    scene = render.NeuralScene.from_host(hs, dev)
+    cache = render.PointRendererCache()
+    info = render.NeuralRenderInfo(scene=scene, images=list(hs.views), params=hs.params, num_layers=hs.num_layers,
+                                   cache=cache,
+                                   dropout_points=None if hs.dropout is None else torch.from_numpy(hs.dropout))
+    cache.Build(info, True)
+    s = scene.struct()
+    fb = cache.forward_struct()
+    views = cache.views_array()
+    B, N, Cn, L = hs.batch, hs.num_points, hs.num_channels, hs.num_layers
+    ws = C.c_void_p(cache.workspace.data_ptr())
+    ws_n = cache.workspace.numel()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    gb = None
+    keep = []
+    if backward:
+        gout = [torch.from_numpy(g).to(dev) for g in scenes.upstream_grads(hs)]
+        gb = _capi.BackwardBuffers()
+        for l in range(L):
+            gb.grad_out[l] = gout[l].data_ptr()
+        g_tex = torch.empty(scene.texture.shape, dtype=torch.float32, device=dev)
+        g_bg = torch.empty(Cn, dtype=torch.float32, device=dev)
+        g_pts = torch.empty(N, 4, dtype=torch.float32, device=dev)
+        g_pts_c = torch.empty(N, dtype=torch.float32, device=dev)
+        g_pose = torch.empty(scene.poses_se3.shape[0], 6, dtype=torch.float64, device=dev)
+        g_pose_c = torch.empty(scene.poses_se3.shape[0], dtype=torch.float32, device=dev)
+        g_intr = torch.empty_like(scene.intrinsics)
+        g_intr_c = torch.empty(scene.intrinsics.shape[0], dtype=torch.float32, device=dev)
+        keep = [gout, g_tex, g_bg, g_pts, g_pts_c, g_pose, g_pose_c, g_intr, g_intr_c]
+        gb.grad_texture, gb.grad_background = g_tex.data_ptr(), g_bg.data_ptr()
+        gb.grad_points, gb.grad_points_count = g_pts.data_ptr(), g_pts_c.data_ptr()
+        if args.workload in ("config3",):
+            gb.grad_pose, gb.grad_pose_count = g_pose.data_ptr(), g_pose_c.data_ptr()
+            gb.grad_intrinsics, gb.grad_intrinsics_count = g_intr.data_ptr(), g_intr_c.data_ptr()
+
+    frame = [0]
+
+    def step(stats=None):
+        if args.workload == "config4":
+            views[0].image_index = frame[0] % scene.poses_se3.shape[0]  # orbit
+            frame[0] += 1
+        rc = lib.adop_forward(C.byref(s), views, B, C.byref(hs.params), C.byref(fb), ws, ws_n, stats, stream)
+        if rc != 0:
+            raise RuntimeError(lib.adop_last_error_string().decode())
+        if backward:
+            rc = lib.adop_backward(C.byref(s), views, B, C.byref(hs.params), C.byref(fb), C.byref(gb), ws, ws_n,
+                                   stats, stream)
+            if rc != 0:
+                raise RuntimeError(lib.adop_last_error_string().decode())
+
+    # untimed pass with counters: V_l, A_l, G_l of the byte model
+    step(C.c_void_p(cache.stats.data_ptr()))
+    torch.cuda.synchronize()
+    st = cache.read_stats()
+    V, A, G = list(st.visible)[:L], list(st.accepted)[:L], list(st.spatial)[:L]
+
+    frame[0] = 0
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    ms_per_step = (t2 - t1) * 1e3 / args.steps
+
+    # per-stage durations from HIP events on the launch stream
+    lib.adop_profile_enable(1)
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    arr = (_capi.StageTime * 16)()
+    n = lib.adop_profile_read(arr, 16)
+    lib.adop_profile_enable(0)
+    stages = {arr[i].name.decode(): arr[i].total_ms / args.steps for i in range(n)}  # ms per step
+
+    P = sum(w * h for (w, h) in hs.level_sizes())
+    S_d = 2 if hs.texture.dtype == np.float16 else 4
+    model = byte_model(N, B, Cn, S_d, P, V, A, G, bool(hs.params.output_background_mask), hs.dropout is not None)
+    if not backward:
+        model = {k: v for k, v in model.items() if k in ("DepthPrepass", "RenderForward", "CombineAndFill")}
+    total_bytes = sum(model.values())
+    dom = max((k for k in model if k in stages), key=lambda k: stages[k])
+    dom_gbs = model[dom] / (stages[dom] * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "kernel": dom, "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                "kernel_ms": round(stages[dom], 4), "algorithmic_bytes": int(model[dom])}
+    step_gbs = total_bytes / (ms_per_step * 1e-3) / 1e9
+
+    if args.workload == "config4":
+        metric, unit, value = "forward frames/s at 100M points 1920x1080 x5 levels", "frames/s", 1e3 / ms_per_step
+    else:
+        metric, unit = "fwd+bwd points/s", "points/s"
+        value = N * B / (ms_per_step * 1e-3)
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        import oracle
+        cores = min(os.cpu_count() or 1, 16)
+        os.environ["OMP_NUM_THREADS"] = str(cores)
+        chs, sample = hs, "the full workload, one step"
+        cpu_n = args.cpu_points or (20_000_000 if N > 20_000_000 else 0)
+        if cpu_n and cpu_n < N:
+            # bounded sample: the first cpu_n points of the same cloud at the same resolution
+            import copy
+            chs = copy.copy(hs)
+            chs.position, chs.index = hs.position[:cpu_n], hs.index[:cpu_n]
+            chs.normal = None if hs.normal is None else hs.normal[:cpu_n]
+            chs.dropout = None if hs.dropout is None else np.ascontiguousarray(hs.dropout[:, :cpu_n])
+            sample = f"first {cpu_n} of {N} points, same resolution, one step"
+        tc0 = time.perf_counter()
+        ref = oracle.forward(chs, omp=True)
+        if backward:
+            oracle.backward(chs, ref, scenes.upstream_grads(chs), omp=True)
+        tc = time.perf_counter() - tc0
+        nthreads = oracle.lib(True).oracle_num_threads()
+        if args.workload == "config4":
+            cpu_val, cpu_unit = (chs.num_points / N) / tc, "frames/s"
+            sample += " (frames/s scaled linearly to the full point count)"
+        else:
+            cpu_val, cpu_unit = chs.num_points * B / tc, "points/s"
+        cpu = {"value": cpu_val, "unit": cpu_unit, "cores": nthreads, "kind": "port", "sample": sample,
+               "seconds": round(tc, 3)}
+
+    out = {
+        "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if S_d == 4 else "f16-stored/f32-accumulated", "data": "synthetic",
+        "config": {"workload": f"BASELINE {hs.name}: {N} points, B={B}, {hs.views[0].w}x{hs.views[0].h}, "
+                               f"{L} levels, C={Cn}, " + ("forward+backward" if backward else "forward only"),
+                   "point_order": hs.meta.get("point_order", "as generated"), "lod_radius_test": False,
+                   "dropout": 0.25 if hs.dropout is not None else 0.0,
+                   "ghost_gradients": bool(hs.params.ghost_gradients)},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "step": {"algorithmic_bytes": int(total_bytes), "achieved_GBps": round(step_gbs, 1),
+                 "hbm_frac": round(step_gbs / HBM_PEAK_GBS, 4),
+                 "stage_ms": {k: round(v, 4) for k, v in stages.items()},
+                 "stage_GBps": {k: round(model[k] / (stages[k] * 1e-3) / 1e9, 1) for k in model if k in stages},
+                 "visible": V, "accepted": A, "spatial": G, "scene_gen_s": round(gen_s, 1)},
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

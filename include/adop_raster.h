@@ -188,6 +188,23 @@ adop_status adop_env_sample_backward(const adop_scene* scene, const adop_view* v
  * tangent = 0; f64. tangent [F,6], poses_se3 [F,8]. */
 adop_status adop_apply_tangent(double* tangent, double* poses_se3, int32_t num_poses, void* hip_stream);
 
+/* Stage timers.  The reference wraps each stage in SAIGA_OPTIONAL_TIME_MEASURE(name, info->timer_system)
+ * (PointRenderer.cu:906,913,919,1095,1414,1430,1447,1565,1594,1602,1610); here HIP events are recorded on the
+ * caller's stream around each stage while profiling is enabled on the calling thread.  Stage names are the
+ * reference's: "Initialize", "DepthPrepass", "RenderForward", "CombineAndFill", "Prepare Backward",
+ * "CombineAndFillBackward", "RenderBackward", "Post Process Gradient". */
+typedef struct adop_stage_time
+{
+    char name[32];
+    float total_ms; /* summed over calls since the last read */
+    int32_t calls;
+} adop_stage_time;
+
+adop_status adop_profile_enable(int32_t enable);
+/* Waits for the recorded events, aggregates them by stage name into out[0..max_entries) and clears the
+ * recording.  Returns the number of entries written. */
+int32_t adop_profile_read(adop_stage_time* out, int32_t max_entries);
+
 /* Message for the last non-OK status returned on the calling thread. */
 const char* adop_last_error_string(void);
 

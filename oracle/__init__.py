@@ -173,12 +173,12 @@ class BackwardResult:
         return gb
 
 
-def backward(hs, fwd, grad_out, points=True, pose=True, intrinsics=True):
+def backward(hs, fwd, grad_out, points=True, pose=True, intrinsics=True, omp=False):
     res = BackwardResult(hs, points, pose, intrinsics)
     s = scene_struct(hs)
     fb = fwd.struct(hs)
     gb = res.struct(grad_out)
-    rc = lib(False).oracle_backward(C.byref(s), views_array(hs), hs.batch, C.byref(hs.params), C.byref(fb),
+    rc = lib(omp).oracle_backward(C.byref(s), views_array(hs), hs.batch, C.byref(hs.params), C.byref(fb),
                                     C.byref(gb), C.byref(res.stats))
     if rc != 0:
         raise RuntimeError(f"oracle_backward returned {rc}")

@@ -841,6 +841,7 @@ int oracle_backward(const adop_scene* s, const adop_view* views, int B, const ad
             for (int c = 0; c < C; ++c)
             {
                 double a = 0;
+#pragma omp parallel for reduction(+ : a) schedule(static)
                 for (int y = 0; y < Ly.h; ++y)
                     for (int x = 0; x < Ly.w; ++x)
                         if (Ly.weight[pix(Ly, b, y, x)] == 0) a += gb->grad_out[l][pixc(Ly, C, b, c, y, x)];
@@ -855,6 +856,13 @@ int oracle_backward(const adop_scene* s, const adop_view* views, int B, const ad
         Cam cam              = make_cam(s, views[b]);
         const adop_view& vw  = views[b];
         const float* dropout = fb->dropout_points ? fb->dropout_points + (size_t)b * N : nullptr;
+#pragma omp parallel
+        {
+        // per-thread partial sums (single-threaded build: the only copy)
+        std::vector<double> l_pose(acc_pose.size(), 0.0), l_cnt_pose(cnt_pose.size(), 0.0);
+        std::vector<double> l_intr(acc_intr.size(), 0.0), l_cnt_intr(cnt_intr.size(), 0.0);
+        uint64_t l_spatial[ADOP_MAX_LAYERS] = {0, 0, 0, 0, 0};
+#pragma omp for schedule(static)
         for (int i = 0; i < N; ++i)
         {
             bool drop_out = dropout && dropout[i] == 1;
@@ -885,13 +893,15 @@ int oracle_backward(const adop_scene* s, const adop_view* views, int B, const ad
                     for (int c = 0; c < C; ++c)
                     {
                         float g = iw * gin[pixc(Ly, C, b, c, py, px)];
-                        gb->grad_texture[(size_t)c * s->num_texels + texture_index] += g;
+                        float* gt = &gb->grad_texture[(size_t)c * s->num_texels + texture_index];
+#pragma omp atomic
+                        *gt += g;
                     }
                 }
 
                 bool point_grad = (rp->ghost_gradients && drop_out) | (!rp->ghost_gradients && !drop_out);
                 if (!(point_grad && distance_from_edge(Ly, py, px) > 2)) continue;
-                if (stats) stats->spatial[l]++;
+                l_spatial[l]++;
 
                 const int nx[4] = {px - 1, px + 1, px, px};
                 const int ny[4] = {py, py, py - 1, py + 1};
@@ -947,12 +957,12 @@ int oracle_backward(const adop_scene* s, const adop_view* views, int B, const ad
                 }
                 if (gb->grad_pose)
                 {
-                    for (int k = 0; k < 6; ++k) acc_pose[6 * (size_t)vw.image_index + k] += (double)bo.g_pose[k];
-                    cnt_pose[vw.image_index] += 1;
+                    for (int k = 0; k < 6; ++k) l_pose[6 * (size_t)vw.image_index + k] += (double)bo.g_pose[k];
+                    l_cnt_pose[vw.image_index] += 1;
                 }
                 if (gb->grad_intrinsics_count && gb->grad_intrinsics)
                 {
-                    double* gi = &acc_intr[(size_t)cols * vw.camera_index];
+                    double* gi = &l_intr[(size_t)cols * vw.camera_index];
                     if (cam.model == ADOP_CAMERA_PINHOLE_DISTORTION)
                     {
                         float k_factor = rp->K_gradient_factor;
@@ -967,16 +977,26 @@ int oracle_backward(const adop_scene* s, const adop_view* views, int B, const ad
                         bo.g_dis[6] *= 0.1f;
                         bo.g_dis[7] *= 0.1f;
                         for (int k = 0; k < 8; ++k) gi[5 + k] += (double)(df * bo.g_dis[k]);
-                        cnt_intr[vw.camera_index] += 1.0 / 1024.0;  // :680-681
+                        l_cnt_intr[vw.camera_index] += 1.0 / 1024.0;  // :680-681
                     }
                     else
                     {
                         for (int k = 0; k < 5; ++k) gi[k] += (double)bo.g_k[k];
-                        cnt_intr[vw.camera_index] += 1.0;  // :718
+                        l_cnt_intr[vw.camera_index] += 1.0;  // :718
                     }
                 }
             }
         }
+#pragma omp critical
+        {
+            for (size_t k = 0; k < acc_pose.size(); ++k) acc_pose[k] += l_pose[k];
+            for (size_t k = 0; k < cnt_pose.size(); ++k) cnt_pose[k] += l_cnt_pose[k];
+            for (size_t k = 0; k < acc_intr.size(); ++k) acc_intr[k] += l_intr[k];
+            for (size_t k = 0; k < cnt_intr.size(); ++k) cnt_intr[k] += l_cnt_intr[k];
+            if (stats)
+                for (int l = 0; l < ADOP_MAX_LAYERS; ++l) stats->spatial[l] += l_spatial[l];
+        }
+        }  // omp parallel
     }
 
     // NormalizeGradient, :1534-1547 and its three launches :1611-1636
