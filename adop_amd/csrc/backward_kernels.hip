@@ -1,0 +1,564 @@
+// backward_kernels.hip — background gradient + gradient/image interleave, RenderBackward, finalize, normalise.
+//
+// The ghost gradient of one point-level reads the image I and the upstream gradient G at four neighbour pixels for
+// every channel.  In the planar [B,C,h,w] layout that is 8C scattered 4-byte loads (plus C for the centre); the
+// interleave kernel therefore first builds a pixel-major array IG[pixel][I_0..I_{C-1}, G_0..G_{C-1}] in the
+// workspace (one 64-byte line per pixel for C = 8), while it sums the background gradient in the same pass.
+#include "common.h"
+#include "launch.h"
+
+#pragma clang fp contract(off)
+
+namespace adop
+{
+// CombineAndFillBackward (:851-900) fused with the I/G interleave.  One thread per pixel of every level/image.
+// Background gradient: per-thread fp32 partial over a handful of pixels, wave/block reduction in f64, one f64
+// partial row per block.
+template <int CT>
+__global__ __launch_bounds__(kBlock) void interleave_kernel(Levels lv, float* __restrict__ ig,
+                                                            double* __restrict__ partial)
+{
+    constexpr int CMAX = CT ? CT : kMaxChannels;
+    const int C        = CT ? CT : lv.C;
+    __shared__ double red[kBlock / 64][kMaxChannels];
+    float acc[CMAX];
+#pragma unroll
+    for (int c = 0; c < CMAX; ++c) acc[c] = 0;
+    int per_image = lv.pix_prefix[lv.num];
+    size_t total  = (size_t)per_image * lv.B;
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride)
+    {
+        int b             = (int)(t / per_image);
+        int r             = (int)(t - (size_t)b * per_image);
+        int l             = level_of(lv, r);
+        const LevelArg& L = lv.l[l];
+        int p             = r - lv.pix_prefix[l];
+        size_t hw         = (size_t)L.w * L.h;
+        bool empty        = L.weight[(size_t)b * hw + p] == 0;
+        const float* g    = L.gin + (size_t)b * C * hw + p;
+        const float* im   = L.out + (size_t)b * C * hw + p;
+        float* dst        = ig + (size_t)ws_pixel(lv, l, b, (uint32_t)p) * (2 * C);
+        float I[CMAX], G[CMAX];
+#pragma unroll
+        for (int c = 0; c < CMAX; ++c)
+            if (c < C)
+            {
+                I[c] = im[(size_t)c * hw];
+                G[c] = g[(size_t)c * hw];
+                if (empty) acc[c] += G[c];
+            }
+        if (CT == 8 || CT == 4)
+        {
+            float4* d4 = (float4*)dst;
+#pragma unroll
+            for (int q = 0; q < CT / 4; ++q) d4[q] = make_float4(I[4 * q], I[4 * q + 1], I[4 * q + 2], I[4 * q + 3]);
+#pragma unroll
+            for (int q = 0; q < CT / 4; ++q)
+                d4[CT / 4 + q] = make_float4(G[4 * q], G[4 * q + 1], G[4 * q + 2], G[4 * q + 3]);
+        }
+        else
+        {
+#pragma unroll
+            for (int c = 0; c < CMAX; ++c)
+                if (c < C)
+                {
+                    dst[c]     = I[c];
+                    dst[C + c] = G[c];
+                }
+        }
+    }
+    int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+#pragma unroll
+    for (int c = 0; c < CMAX; ++c)
+    {
+        double v = wave_sum<double>((double)acc[c]);
+        if (lane == 0) red[wave][c] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x < kMaxChannels)
+    {
+        double v = 0;
+        if ((int)threadIdx.x < CMAX)
+            for (int w = 0; w < kBlock / 64; ++w) v += red[w][threadIdx.x];
+        partial[(size_t)blockIdx.x * kMaxChannels + threadIdx.x] = v;
+    }
+}
+
+template <int CT>
+__device__ __forceinline__ void load_channels(const float* __restrict__ src, int C, float* dst)
+{
+    if (CT == 8 || CT == 4)
+    {
+        const float4* s4 = (const float4*)src;
+#pragma unroll
+        for (int q = 0; q < CT / 4; ++q)
+        {
+            float4 v       = s4[q];
+            dst[4 * q]     = v.x;
+            dst[4 * q + 1] = v.y;
+            dst[4 * q + 2] = v.z;
+            dst[4 * q + 3] = v.w;
+        }
+    }
+    else
+    {
+#pragma unroll
+        for (int c = 0; c < kMaxChannels; ++c)
+            if (c < C) dst[c] = src[c];
+    }
+}
+
+// RenderBackward (PointRenderer.cu:396-724).  Grid-stride over points so that the pose / intrinsics sums can live
+// in registers (f64) for the whole kernel; they leave the block as one partial row per (block, view).
+// Descriptor gradients of one point are summed over the levels in registers and added once per channel.
+template <int CT, bool HALF>
+__global__ __launch_bounds__(kBlock) void render_backward_kernel(CloudArg pc, const ViewConst* __restrict__ views,
+                                                                  Levels lv, ParamArg rp, const float* __restrict__ ig,
+                                                                  float* __restrict__ gtex,
+                                                                  float* __restrict__ gpoints,
+                                                                  float* __restrict__ gpoints_count, int want_pose,
+                                                                  int want_intr, int view_b,
+                                                                  double* __restrict__ partial, adop_stats* stats)
+{
+    constexpr int CMAX = CT ? CT : 1;  // register arrays exist only for compile-time channel counts
+    __shared__ double red[kBlock / 64][kPartialStride];
+    const bool STATS    = stats != nullptr;  // counter pass (uniform branch)
+    const int b         = view_b;
+    const ViewConst& vc = views[b];
+    const float accept  = rp.depth_accept + 1;
+    const int C         = CT ? CT : lv.C;
+
+    double acc[kAcc];
+#pragma unroll
+    for (int k = 0; k < kAcc; ++k) acc[k] = 0;
+
+    const int n_round = ((pc.n + kBlock - 1) / kBlock) * kBlock;
+    for (int i = blockIdx.x * kBlock + threadIdx.x; i < n_round; i += gridDim.x * kBlock)
+    {
+        bool valid = i < pc.n;
+        float4 P   = valid ? pc.position[i] : make_float4(0, 0, 0, 0);
+        V3 pos     = {P.x, P.y, P.z};
+        V3 nrm     = {0, 0, 0};
+        if (valid && pc.normal) nrm = unpack_normal10(pc.normal[i]);
+        bool drop_out = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;
+        V2 ip;
+        V3 view_p;
+        float z, radius_pixels;
+        bool ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff,
+                                         lv.l[0].w, &ip, &z, &radius_pixels, &view_p);
+        int tex_index = valid ? pc.index[i] : 0;
+        ok            = ok && (unsigned)tex_index < (unsigned)pc.num_texels;
+        if (!STATS && !ok) continue;
+
+        float scale = 1;
+        bool alive  = ok;
+        // running value of grad_points[i] / count[i]; loaded at the first contribution so that the additions
+        // happen in the reference's order (view after view, level after level)
+        float gp[3]  = {0, 0, 0};
+        float gp_n   = 0;
+        bool gp_live = false;
+        float gt[CMAX];  // descriptor gradient of this point, summed over the levels
+#pragma unroll
+        for (int c = 0; c < CMAX; ++c) gt[c] = 0;
+        bool gt_live = false;
+        float T[CMAX];
+        bool T_live = false;
+#pragma unroll 1
+        for (int l = 0; l < lv.num; ++l)
+        {
+            const LevelArg& L = lv.l[l];
+            int px = f2i_rn(ip.x), py = f2i_rn(ip.y);
+            bool lod_skip = rp.drop_by_radius && radius_pixels < rp.drop_threshold;  // continue, :451-454
+            bool in       = alive && !lod_skip && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h;
+            bool spatial  = false;
+            if (in)
+            {
+                size_t hw = (size_t)L.w * L.h;
+                size_t p  = (size_t)py * L.w + px;
+                float image_depth = L.depth[(size_t)b * hw + p];
+                if (z > image_depth * accept)
+                {
+                    alive = false;  // break, :462
+                }
+                else
+                {
+                    float w         = L.weight[(size_t)b * hw + p];
+                    const float* pg = ig + (size_t)ws_pixel(lv, l, b, (uint32_t)p) * (2 * C);  // [I | G] of the pixel
+                    bool go         = true;
+                    if (!drop_out)
+                    {
+                        if (w == 0)
+                            go = false;  // continue, :473
+                        else
+                        {
+                            float iw = 1.f / w;
+                            if (CT == 0)
+                            {
+                                // any channel count: one atomic per channel and level (:478-484)
+#pragma unroll 1
+                                for (int c = 0; c < C; ++c)
+                                    unsafeAtomicAdd(gtex + (size_t)c * pc.num_texels + tex_index, iw * pg[C + c]);
+                            }
+                            else
+                            {
+                                float G[CMAX];
+                                load_channels<CT>(pg + C, C, G);
+#pragma unroll
+                                for (int c = 0; c < CMAX; ++c) gt[c] += iw * G[c];
+                                gt_live = true;
+                            }
+                        }
+                    }
+                    bool point_grad = (rp.ghost_gradients && drop_out) | (!rp.ghost_gradients && !drop_out);
+                    int ex          = min(px, L.w - 1 - px);
+                    int ey          = min(py, L.h - 1 - py);
+                    if (go && point_grad && min(ex, ey) > 2)  // distanceFromEdge > 2, :489
+                    {
+                        spatial = true;
+                        const ptrdiff_t nb[4] = {-1, 1, -(ptrdiff_t)L.w, (ptrdiff_t)L.w};
+                        const float* Wp       = L.weight + (size_t)b * hw + p;
+                        const float* Dp       = L.depth + (size_t)b * hw + p;
+                        float Wn[4] = {0, 0, 0, 0}, Dn[4] = {0, 0, 0, 0};
+                        if (rp.test_backward_mode == 4)
+                        {
+#pragma unroll
+                            for (int k = 0; k < 4; ++k)
+                            {
+                                Wn[k] = Wp[nb[k]];
+                                Dn[k] = Dp[nb[k]];
+                            }
+                        }
+                        auto dI_of = [&](float T_c, float I_x, float W_x, float D_x) -> float
+                        {
+                            if (rp.test_backward_mode == 4)
+                            {
+                                if (W_x == 0 || z * accept < D_x) return T_c - I_x;  // full override
+                                if (z > D_x * accept) return 0.f;                    // discard
+                                return (W_x / (W_x + 1) * I_x + 1 / (W_x + 1) * T_c - I_x);  // blend
+                            }
+                            return T_c - I_x;
+                        };
+                        float dR_dpx = 0, dR_dpy = 0;
+                        if (CT == 0)
+                        {
+#pragma unroll 1
+                            for (int c = 0; c < C; ++c)
+                            {
+                                float T_c = tex_fetch<HALF>(pc.texture, (size_t)c * pc.num_texels + tex_index);
+                                float v[4];
+#pragma unroll
+                                for (int k = 0; k < 4; ++k)
+                                {
+                                    const float* q = pg + nb[k] * (2 * C);
+                                    v[k]           = dI_of(T_c, q[c], Wn[k], Dn[k]) * q[C + c];
+                                }
+                                float a0 = -v[0], a1 = v[1], b0 = -v[2], b1 = v[3];
+                                dR_dpx += 0.5f * (a0 + a1);
+                                dR_dpy += 0.5f * (b0 + b1);
+                            }
+                        }
+                        else
+                        {
+                            if (!T_live)
+                            {
+#pragma unroll
+                                for (int c = 0; c < CMAX; ++c)
+                                    T[c] = tex_fetch<HALF>(pc.texture, (size_t)c * pc.num_texels + tex_index);
+                                T_live = true;
+                            }
+                            float v[4][CMAX];  // dI * G per neighbour and channel
+#pragma unroll
+                            for (int k = 0; k < 4; ++k)
+                            {
+                                const float* q = pg + nb[k] * (2 * C);
+                                float In[CMAX], Gn[CMAX];
+                                load_channels<CT>(q, C, In);
+                                load_channels<CT>(q + C, C, Gn);
+#pragma unroll
+                                for (int c = 0; c < CMAX; ++c) v[k][c] = dI_of(T[c], In[c], Wn[k], Dn[k]) * Gn[c];
+                            }
+#pragma unroll
+                            for (int c = 0; c < CMAX; ++c)
+                            {
+                                float a0 = -v[0][c], a1 = v[1][c], b0 = -v[2][c], b1 = v[3][c];
+                                dR_dpx += 0.5f * (a0 + a1);
+                                dR_dpy += 0.5f * (b0 + b1);
+                            }
+                        }
+                        V2 dR_dp       = {dR_dpx / (float)C, dR_dpy / (float)C};
+                        float crop2[5] = {vc.crop[0] * scale, vc.crop[1] * scale, vc.crop[2] * scale,
+                                          vc.crop[3] * scale, vc.crop[4] * scale};  // crop.scale(scale), :616
+                        BackwardOut bo;
+                        project_point_backward(vc, pc.intrinsics, view_p, dR_dp, crop2, rp.dist_cutoff, &bo);
+                        if (gpoints)
+                        {
+                            if (!gp_live)
+                            {
+                                const float* g = gpoints + 4 * (size_t)i;
+                                gp[0]          = g[0];
+                                gp[1]          = g[1];
+                                gp[2]          = g[2];
+                                gp_n           = gpoints_count[i];
+                                gp_live        = true;
+                            }
+                            gp[0] += bo.g_point[0];
+                            gp[1] += bo.g_point[1];
+                            gp[2] += bo.g_point[2];
+                            gp_n += 1.f;
+                        }
+                        if (want_pose)
+                        {
+#pragma unroll
+                            for (int k = 0; k < 6; ++k) acc[k] += (double)bo.g_pose[k];
+                            acc[6] += 1.0;
+                        }
+                        if (want_intr)
+                        {
+                            if (vc.model == 0)
+                            {
+                                float kf = rp.K_gradient_factor;
+                                bo.g_k[4] *= 0.1f;
+                                bo.g_k[4] *= 0;  // :653-654
+#pragma unroll
+                                for (int k = 0; k < 5; ++k) acc[8 + k] += (double)(kf * bo.g_k[k]);
+                                float df = rp.distortion_gradient_factor;
+                                bo.g_dis[2] *= 0.25f;
+                                bo.g_dis[3] *= 0.1f;
+                                bo.g_dis[4] *= 0.1f;
+                                bo.g_dis[5] *= 0.1f;
+                                bo.g_dis[6] *= 0.1f;
+                                bo.g_dis[7] *= 0.1f;
+#pragma unroll
+                                for (int k = 0; k < 8; ++k) acc[13 + k] += (double)(df * bo.g_dis[k]);
+                                acc[7] += 1.0 / 1024.0;  // :680-681
+                            }
+                            else
+                            {
+#pragma unroll
+                                for (int k = 0; k < 5; ++k) acc[8 + k] += (double)bo.g_k[k];
+                                acc[7] += 1.0;  // :718
+                            }
+                        }
+                    }
+                }
+            }
+            if (STATS) stat_add(&stats->spatial[l], spatial);
+            scale *= 0.5f;
+            radius_pixels *= 0.5f;
+            ip.x *= 0.5f;
+            ip.y *= 0.5f;
+        }
+        if (gt_live)
+        {
+#pragma unroll
+            for (int c = 0; c < CMAX; ++c) unsafeAtomicAdd(gtex + (size_t)c * pc.num_texels + tex_index, gt[c]);
+        }
+        if (gp_live)
+        {
+            // one thread owns point i for this view; views are launched one after another on the stream
+            float* g         = gpoints + 4 * (size_t)i;
+            g[0]             = gp[0];
+            g[1]             = gp[1];
+            g[2]             = gp[2];
+            gpoints_count[i] = gp_n;
+        }
+    }
+
+    if (want_pose || want_intr)
+    {
+        int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+#pragma unroll
+        for (int k = 0; k < kAcc; ++k)
+        {
+            double v = wave_sum<double>(acc[k]);
+            if (lane == 0) red[wave][k] = v;
+        }
+        __syncthreads();
+        if (threadIdx.x < kAcc)
+        {
+            double v = 0;
+            for (int w = 0; w < kBlock / 64; ++w) v += red[w][threadIdx.x];
+            partial[((size_t)b * gridDim.x + blockIdx.x) * kPartialStride + threadIdx.x] = v;
+        }
+    }
+}
+
+// Reduces the per-block partial rows and runs NormalizeGradient (:1534-1547, launches :1611-1636) for the
+// background / pose / intrinsics outputs.  One block.
+__global__ __launch_bounds__(kBlock) void finalize_kernel(const ViewConst* __restrict__ views, int B, int C,
+                                                          const double* __restrict__ bg_partial, int bg_blocks,
+                                                          const double* __restrict__ pt_partial, int pt_blocks,
+                                                          float* __restrict__ gbg, double* __restrict__ gpose,
+                                                          float* __restrict__ gpose_count, int num_poses,
+                                                          float* __restrict__ gintr, float* __restrict__ gintr_count,
+                                                          int num_cameras, int cols, int normalize_mode,
+                                                          double* __restrict__ scratch)
+{
+    __shared__ double sh[kBlock];
+    // background
+    for (int c = 0; c < C; ++c)
+    {
+        double v = 0;
+        for (int k = threadIdx.x; k < bg_blocks; k += kBlock) v += bg_partial[(size_t)k * kMaxChannels + c];
+        sh[threadIdx.x] = v;
+        __syncthreads();
+        for (int s = kBlock / 2; s > 0; s >>= 1)
+        {
+            if (threadIdx.x < s) sh[threadIdx.x] += sh[threadIdx.x + s];
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) gbg[c] = (float)sh[0];
+        __syncthreads();
+    }
+    if (!gpose && !gintr) return;
+
+    // scratch: [num_poses*7] pose sums + count, then [num_cameras*(cols+1)] intrinsics sums + count
+    double* sp = scratch;
+    double* si = scratch + (size_t)num_poses * 7;
+    for (int k = threadIdx.x; k < num_poses * 7 + num_cameras * (cols + 1); k += kBlock) scratch[k] = 0;
+    __syncthreads();
+    for (int b = 0; b < B; ++b)
+    {
+        for (int q = 0; q < 21; ++q)
+        {
+            double v = 0;
+            for (int k = threadIdx.x; k < pt_blocks; k += kBlock)
+                v += pt_partial[((size_t)b * pt_blocks + k) * kPartialStride + q];
+            sh[threadIdx.x] = v;
+            __syncthreads();
+            for (int s = kBlock / 2; s > 0; s >>= 1)
+            {
+                if (threadIdx.x < s) sh[threadIdx.x] += sh[threadIdx.x + s];
+                __syncthreads();
+            }
+            if (threadIdx.x == 0)
+            {
+                const ViewConst& vc = views[b];
+                double t            = sh[0];
+                if (q < 6)
+                    sp[(size_t)vc.image_index * 7 + q] += t;
+                else if (q == 6)
+                    sp[(size_t)vc.image_index * 7 + 6] += t;
+                else if (q == 7)
+                    si[(size_t)vc.camera_index * (cols + 1) + cols] += t;
+                else if (q - 8 < cols)
+                    si[(size_t)vc.camera_index * (cols + 1) + (q - 8)] += t;
+            }
+            __syncthreads();
+        }
+    }
+    if (gpose)
+    {
+        for (int f = threadIdx.x; f < num_poses; f += kBlock)
+        {
+            float c        = (float)sp[(size_t)f * 7 + 6];
+            gpose_count[f] = c;
+            for (int k = 0; k < 6; ++k)
+            {
+                double t                   = sp[(size_t)f * 7 + k];
+                gpose[(size_t)f * 6 + k] = (c > 0) ? t / (double)c : t;
+            }
+        }
+    }
+    if (gintr)
+    {
+        for (int k = threadIdx.x; k < num_cameras * cols; k += kBlock)
+            gintr[k] = (float)si[(size_t)(k / cols) * (cols + 1) + (k % cols)];
+        for (int k = threadIdx.x; k < num_cameras; k += kBlock) gintr_count[k] = (float)si[(size_t)k * (cols + 1) + cols];
+        __syncthreads();
+        if (threadIdx.x == 0)
+        {
+            int total = num_cameras * cols;
+            if (normalize_mode == 0)
+            {
+                // NormalizeGradient<float,13> whatever the row width (:1633)
+                for (int t = 0; t < num_cameras; ++t)
+                {
+                    float c = gintr_count[t];
+                    if (c > 0)
+                        for (int k = 0; k < 13; ++k)
+                            if (13 * t + k < total) gintr[13 * t + k] = gintr[13 * t + k] / c;
+                }
+            }
+            else
+            {
+                for (int t = 0; t < num_cameras; ++t)
+                {
+                    float c = gintr_count[t];
+                    if (c > 0)
+                        for (int k = 0; k < cols; ++k) gintr[cols * t + k] = gintr[cols * t + k] / c;
+                }
+            }
+        }
+    }
+}
+
+// NormalizeGradient<float,3> on the [N,4] point-gradient buffer (:1620-1627).  mode 0 reproduces the reference's
+// vec3 view (element t = floats 3t..3t+2 divided by count[t]); mode 1 normalises row t by count[t].
+__global__ __launch_bounds__(kBlock) void normalize_points_kernel(float* __restrict__ g, const float* __restrict__ count,
+                                                                  int n, int mode)
+{
+    int t = blockIdx.x * kBlock + threadIdx.x;
+    if (t >= n) return;
+    float c = count[t];
+    if (!(c > 0)) return;
+    size_t o = (mode == 0) ? 3 * (size_t)t : 4 * (size_t)t;
+    g[o + 0] = g[o + 0] / c;
+    g[o + 1] = g[o + 1] / c;
+    g[o + 2] = g[o + 2] / c;
+}
+
+
+// ------------------------------------------------------------------------------------------------
+// launchers
+// ------------------------------------------------------------------------------------------------
+void launch_interleave(const Levels& lv, int blocks, float* ig, double* partial, hipStream_t st)
+{
+    if (lv.C == 8)
+        hipLaunchKernelGGL((interleave_kernel<8>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, partial);
+    else if (lv.C == 4)
+        hipLaunchKernelGGL((interleave_kernel<4>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, partial);
+    else
+        hipLaunchKernelGGL((interleave_kernel<0>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, partial);
+}
+
+template <int CT, bool HALF>
+static void launch_bwd_t(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp,
+                         const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr, int b,
+                         int blocks, double* partial, adop_stats* stats, hipStream_t st)
+{
+    hipLaunchKernelGGL((render_backward_kernel<CT, HALF>), dim3(blocks), dim3(kBlock), 0, st, pc, views, lv, rp, ig,
+                       g->grad_texture, g->grad_points, g->grad_points_count, want_pose, want_intr, b, partial, stats);
+}
+
+void launch_render_backward(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
+                            const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr, int b,
+                            int blocks, double* partial, adop_stats* stats, hipStream_t st)
+{
+#define ADOP_ARGS pc, views, lv, rp, ig, g, want_pose, want_intr, b, blocks, partial, stats, st
+    if (lv.C == 8)
+        half ? launch_bwd_t<8, true>(ADOP_ARGS) : launch_bwd_t<8, false>(ADOP_ARGS);
+    else if (lv.C == 4)
+        half ? launch_bwd_t<4, true>(ADOP_ARGS) : launch_bwd_t<4, false>(ADOP_ARGS);
+    else
+        half ? launch_bwd_t<0, true>(ADOP_ARGS) : launch_bwd_t<0, false>(ADOP_ARGS);
+#undef ADOP_ARGS
+}
+
+void launch_finalize(const ViewConst* views, int B, int C, const double* bg_partial, int bg_blocks,
+                     const double* pt_partial, int pt_blocks, const adop_backward_buffers* g, int num_poses,
+                     int num_cameras, int cols, int normalize_mode, double* scratch, hipStream_t st)
+{
+    hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kBlock), 0, st, views, B, C, bg_partial, bg_blocks, pt_partial,
+                       pt_blocks, g->grad_background, g->grad_pose, g->grad_pose_count, num_poses, g->grad_intrinsics,
+                       g->grad_intrinsics_count, num_cameras, cols, normalize_mode, scratch);
+}
+
+void launch_normalize_points(float* g, const float* count, int n, int mode, hipStream_t st)
+{
+    if (n < 1) return;
+    hipLaunchKernelGGL(normalize_points_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, g, count, n, mode);
+}
+
+}  // namespace adop

@@ -1,0 +1,183 @@
+// common.h — kernel argument structs and small device helpers shared by the rasterizer kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "../../include/adop_raster.h"
+#include "device_math.h"
+
+#pragma clang fp contract(off)
+
+namespace adop
+{
+constexpr int kBlock         = 256;
+constexpr int kMaxChannels   = 16;
+constexpr int kPartialBlocks = 2048;  // grid of the grid-stride kernels that write per-block partial sums
+constexpr int kPartialStride = 24;    // doubles per (block, view), 21 used: 6 pose, pose count, intr count, 13 intr
+constexpr int kAcc           = 21;
+constexpr int kMaxIntrinsicsCols = 24;  // 13 pinhole / 5 affine + up to 19 polynomial coefficients
+constexpr uint64_t kClearPacked = (uint64_t(0x47C35000u) << 32) | 0xFFFFFFFFull;  // bits(100000.f), PointRenderer.cu:1045
+
+// Workgroup-local pre-reduction table (LDS): open addressing, linear probing.
+constexpr int kMaxProbe       = 24;
+constexpr uint32_t kEmptyKey  = 0xFFFFFFFFu;
+
+struct LevelArg
+{
+    int32_t w, h;
+    uint64_t* depth_index;
+    float* depth;
+    float* weight;
+    float* out;
+    float* mask;
+    const float* gin;  // upstream gradient (backward only)
+};
+
+struct Levels
+{
+    int32_t num;
+    int32_t B;
+    int32_t C;
+    int32_t pix_prefix[ADOP_MAX_LAYERS + 1];  // prefix sum of w*h over levels (one image)
+    LevelArg l[ADOP_MAX_LAYERS];
+};
+
+struct CloudArg
+{
+    const float4* position;
+    const int32_t* normal;
+    const int32_t* index;
+    int32_t n;
+    const void* texture;
+    int32_t num_texels;
+    const float* intrinsics;
+    const float* dropout;  // [B,N] or null
+};
+
+struct ParamArg
+{
+    int32_t test_backward_mode;
+    int32_t check_normal;
+    int32_t ghost_gradients;
+    int32_t drop_by_radius;
+    float depth_accept;
+    float drop_threshold;
+    float dist_cutoff;
+    float distortion_gradient_factor;
+    float K_gradient_factor;
+};
+
+struct ViewChunk
+{
+    adop_view v[32];
+};
+
+// Workspace pixel index of pixel p of level l of image b: all levels and images of a call form one array
+// (B images of level 0, then B images of level 1, ...).
+__device__ __forceinline__ uint32_t ws_pixel(const Levels& lv, int l, int b, uint32_t p)
+{
+    return (uint32_t)lv.pix_prefix[l] * (uint32_t)lv.B + (uint32_t)b * (uint32_t)(lv.l[l].w * lv.l[l].h) + p;
+}
+
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+    return v;
+}
+
+// counter += number of lanes with pred (one atomic per wavefront; counter passes only)
+__device__ __forceinline__ void stat_add(uint64_t* dst, bool pred)
+{
+    unsigned long long m = __ballot(pred);
+    if (m && (threadIdx.x & 63) == (__ffsll((long long)m) - 1))
+        atomicAdd((unsigned long long*)dst, (unsigned long long)__popcll(m));
+}
+
+template <bool HALF>
+__device__ __forceinline__ float tex_fetch(const void* tex, size_t o)
+{
+    if (HALF) return __half2float(((const __half*)tex)[o]);
+    return ((const float*)tex)[o];
+}
+
+template <int BITS>
+__device__ __forceinline__ uint32_t table_hash(uint32_t key)
+{
+    return (key * 0x9E3779B1u) >> (32 - BITS);
+}
+
+// Finds or creates the slot of `key`.  New slots are appended to used[] (count in *used_count).
+// Returns -1 when no slot is found within kMaxProbe probes (caller falls back to a direct global atomic).
+template <int BITS>
+__device__ __forceinline__ int table_insert(uint32_t* keys, uint16_t* used, uint32_t* used_count, uint32_t key)
+{
+    uint32_t slot = table_hash<BITS>(key);
+#pragma unroll 1
+    for (int probe = 0; probe < kMaxProbe; ++probe)
+    {
+        uint32_t old = atomicCAS(&keys[slot], kEmptyKey, key);
+        if (old == kEmptyKey)
+        {
+            uint32_t e = atomicAdd(used_count, 1u);
+            used[e]    = (uint16_t)slot;
+            return (int)slot;
+        }
+        if (old == key) return (int)slot;
+        slot = (slot + 1) & ((1u << BITS) - 1);
+    }
+    return -1;
+}
+
+// d_render_params.Pose() / PinholeIntrinsics() / OcamIntrinsics() (PointRenderer.cu:73-96) for one view.
+__device__ __forceinline__ ViewConst make_view_const(const adop_view& v, const double* __restrict__ poses,
+                                                     const float* __restrict__ intrinsics, int cols)
+{
+    ViewConst c;
+    const double* p = poses + 8 * (size_t)v.image_index;
+    float x = (float)p[0], y = (float)p[1], z = (float)p[2], w = (float)p[3];
+    float n = sqrtf(((x * x + y * y) + z * z) + w * w);  // Sophus SO3f(quaternion) normalises
+    c.qx    = x / n;
+    c.qy    = y / n;
+    c.qz    = z / n;
+    c.qw    = w / n;
+    c.tx    = (float)p[4];
+    c.ty    = (float)p[5];
+    c.tz    = (float)p[6];
+    const float* row = intrinsics + (size_t)cols * v.camera_index;
+    for (int i = 0; i < 5; ++i) c.k[i] = 0;
+    for (int i = 0; i < 8; ++i) c.d[i] = 0;
+    if (v.camera_model_type == ADOP_CAMERA_PINHOLE_DISTORTION)
+    {
+        for (int i = 0; i < 5; ++i) c.k[i] = row[i];
+        for (int i = 0; i < 8; ++i) c.d[i] = row[5 + i];
+    }
+    c.crop[0]      = v.crop_fx;
+    c.crop[1]      = v.crop_fy;
+    c.crop[2]      = v.crop_cx;
+    c.crop[3]      = v.crop_cy;
+    c.crop[4]      = v.crop_s;
+    c.w            = v.w;
+    c.h            = v.h;
+    c.image_index  = v.image_index;
+    c.camera_index = v.camera_index;
+    c.model        = v.camera_model_type;
+    c.intr_offset  = cols * v.camera_index;
+    c.npoly        = cols - 5;
+    c.pad          = 0;
+    return c;
+}
+
+// level of flattened per-image pixel index r (pix_prefix is increasing)
+__device__ __forceinline__ int level_of(const Levels& lv, int r)
+{
+    int l = 0;
+#pragma unroll
+    for (int k = 1; k < ADOP_MAX_LAYERS; ++k)
+        if (k < lv.num && r >= lv.pix_prefix[k]) l = k;
+    return l;
+}
+
+}  // namespace adop

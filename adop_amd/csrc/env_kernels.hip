@@ -1,0 +1,249 @@
+// env_kernels.hip — environment-map kernels (EnvironmentMap.cu:41-157, RenderModule.cpp:106-127) and ApplyTangent.
+#include "common.h"
+#include "launch.h"
+
+#pragma clang fp contract(off)
+
+namespace adop
+{
+// ------------------------------------------------------------------------------------------------
+// environment map (EnvironmentMap.cu:41-157) and its composition (RenderModule.cpp:106-127)
+// ------------------------------------------------------------------------------------------------
+
+__device__ __forceinline__ V2 k_unproject2(const float* K, V2 ip)
+{
+    float y = (ip.y - K[3]) / K[1];
+    float x = ((ip.x - K[2]) - K[4] * y) / K[0];
+    return {x, y};
+}
+
+// undistortNormalizedPointSimple: OpenCV fixed-point iteration, 5 rounds.
+__device__ __forceinline__ V2 undistort_simple(V2 p, const float* D)
+{
+    float k1 = D[0], k2 = D[1], k3 = D[2], k4 = D[3], k5 = D[4], k6 = D[5], p1 = D[6], p2 = D[7];
+    float x0 = p.x, y0 = p.y, x = p.x, y = p.y;
+    for (int it = 0; it < 5; ++it)
+    {
+        float r2     = x * x + y * y;
+        float icdist = (1.0f + ((k6 * r2 + k5) * r2 + k4) * r2) / (1.0f + ((k3 * r2 + k2) * r2 + k1) * r2);
+        float dx     = 2.0f * p1 * x * y + p2 * (r2 + 2.0f * x * x);
+        float dy     = p1 * (r2 + 2.0f * y * y) + 2.0f * p2 * x * y;
+        x            = (x0 - dx) * icdist;
+        y            = (y0 - dy) * icdist;
+    }
+    return {x, y};
+}
+
+// BuildSphericalUV + SphericalCoordinates for pixel (gx,gy) of a level whose crop is scaled by `sc`.
+__device__ __forceinline__ V2 spherical_uv(const ViewConst& vc, float sc, int gx, int gy)
+{
+    float cr[5] = {vc.crop[0] * sc, vc.crop[1] * sc, vc.crop[2] * sc, vc.crop[3] * sc, vc.crop[4] * sc};
+    V3 t    = {vc.tx, vc.ty, vc.tz};
+    V3 rt   = quat_rotate(-vc.qx, -vc.qy, -vc.qz, vc.qw, t);
+    V3 tinv = {-rt.x, -rt.y, -rt.z};
+    V2 ip   = {(float)gx, (float)gy};
+    V2 dist_p = k_unproject2(vc.k, k_unproject2(cr, ip));
+    V2 np     = undistort_simple(dist_p, vc.d);
+    V3 inp    = {np.x, np.y, 1};
+    V3 r      = quat_rotate(-vc.qx, -vc.qy, -vc.qz, vc.qw, inp);
+    V3 wp     = {r.x + tinv.x, r.y + tinv.y, r.z + tinv.z};
+    V3 d      = {wp.x - tinv.x, wp.y - tinv.y, wp.z - tinv.z};
+    float n   = sqrtf(dot3(d, d));
+    d         = {d.x / n, d.y / n, d.z / n};
+    float phi = atan2_poly(-d.z, d.x);
+    float x   = phi / (2.0f * ADOP_PI);
+    x         = x - floorf(x);
+    float th  = acos_poly(d.y);
+    float y   = 1 - th / ADOP_PI;
+    return {x * 2 - 1, y * 2 - 1};
+}
+
+struct Bilinear
+{
+    int x0, y0;
+    float w00, w01, w10, w11;
+    bool x1ok, y1ok;
+};
+
+// grid_sample(bilinear, padding border, align_corners=true) addressing
+__device__ __forceinline__ Bilinear bilinear_setup(V2 uv, int ew, int eh)
+{
+    float fx = (uv.x + 1) * 0.5f * (float)(ew - 1);
+    float fy = (uv.y + 1) * 0.5f * (float)(eh - 1);
+    fx       = fminf(fmaxf(fx, 0.f), (float)(ew - 1));
+    fy       = fminf(fmaxf(fy, 0.f), (float)(eh - 1));
+    Bilinear s;
+    s.x0     = (int)floorf(fx);
+    s.y0     = (int)floorf(fy);
+    float ax = fx - (float)s.x0, ay = fy - (float)s.y0;
+    s.w00    = (1 - ax) * (1 - ay);
+    s.w01    = ax * (1 - ay);
+    s.w10    = (1 - ax) * ay;
+    s.w11    = ax * ay;
+    s.x1ok   = s.x0 + 1 < ew;
+    s.y1ok   = s.y0 + 1 < eh;
+    return s;
+}
+
+
+__global__ __launch_bounds__(kBlock) void env_sample_kernel(ViewChunk chunk, const double* __restrict__ poses,
+                                                            const float* __restrict__ intrinsics, Levels lv,
+                                                            EnvLevels ev, const float* __restrict__ tex, int eh, int ew,
+                                                            int add_to_out)
+{
+    int per_image = lv.pix_prefix[lv.num];
+    size_t total  = (size_t)per_image * lv.B;
+    size_t t      = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total) return;
+    int b = (int)(t / per_image);
+    int r = (int)(t - (size_t)b * per_image);
+    int l = 0;
+#pragma unroll
+    for (int k = 1; k < ADOP_MAX_LAYERS; ++k)
+        if (k < lv.num && r >= lv.pix_prefix[k]) l = k;
+    const LevelArg& L = lv.l[l];
+    int p             = r - lv.pix_prefix[l];
+    int gy = p / L.w, gx = p - gy * L.w;
+    size_t hw   = (size_t)L.w * L.h;
+    float sc    = 1;
+    for (int k = 0; k < l; ++k) sc /= 2;
+    float bgw = 1.f;
+    if (add_to_out && L.mask) bgw = 1.f - L.mask[(size_t)b * hw + p];
+    bool need = ev.uv[l] || ev.env[l] || (add_to_out && bgw != 0.f);
+    if (!need) return;
+    V2 uv = spherical_uv(make_view_const(chunk.v[b], poses, intrinsics, 13), sc, gx, gy);
+    if (ev.uv[l])
+    {
+        ev.uv[l][((size_t)b * hw + p) * 2 + 0] = uv.x;
+        ev.uv[l][((size_t)b * hw + p) * 2 + 1] = uv.y;
+    }
+    if (!ev.env[l] && !(add_to_out && bgw != 0.f)) return;
+    Bilinear s = bilinear_setup(uv, ew, eh);
+    for (int c = 0; c < lv.C; ++c)
+    {
+        const float* tc = tex + (size_t)c * eh * ew;
+        float a         = 0;
+        a += tc[(size_t)s.y0 * ew + s.x0] * s.w00;
+        if (s.x1ok) a += tc[(size_t)s.y0 * ew + s.x0 + 1] * s.w01;
+        if (s.y1ok) a += tc[(size_t)(s.y0 + 1) * ew + s.x0] * s.w10;
+        if (s.x1ok && s.y1ok) a += tc[(size_t)(s.y0 + 1) * ew + s.x0 + 1] * s.w11;
+        size_t o = ((size_t)b * lv.C + c) * hw + p;
+        if (ev.env[l]) ev.env[l][o] = a;
+        if (add_to_out) L.out[o] = L.out[o] + bgw * a;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void env_backward_kernel(ViewChunk chunk, const double* __restrict__ poses,
+                                                              const float* __restrict__ intrinsics, Levels lv,
+                                                              EnvLevels ev, float* __restrict__ genv, int eh, int ew)
+{
+    int per_image = lv.pix_prefix[lv.num];
+    size_t total  = (size_t)per_image * lv.B;
+    size_t t      = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total) return;
+    int b = (int)(t / per_image);
+    int r = (int)(t - (size_t)b * per_image);
+    int l = 0;
+#pragma unroll
+    for (int k = 1; k < ADOP_MAX_LAYERS; ++k)
+        if (k < lv.num && r >= lv.pix_prefix[k]) l = k;
+    const LevelArg& L = lv.l[l];
+    int p             = r - lv.pix_prefix[l];
+    int gy = p / L.w, gx = p - gy * L.w;
+    size_t hw = (size_t)L.w * L.h;
+    float sc  = 1;
+    for (int k = 0; k < l; ++k) sc /= 2;
+    float bgw = 1.f;
+    if (L.mask) bgw = 1.f - L.mask[(size_t)b * hw + p];
+    if (bgw == 0.f) return;
+    V2 uv      = spherical_uv(make_view_const(chunk.v[b], poses, intrinsics, 13), sc, gx, gy);
+    Bilinear s = bilinear_setup(uv, ew, eh);
+    for (int c = 0; c < lv.C; ++c)
+    {
+        float g   = bgw * ev.gout[l][((size_t)b * lv.C + c) * hw + p];
+        float* tc = genv + (size_t)c * eh * ew;
+        unsafeAtomicAdd(tc + (size_t)s.y0 * ew + s.x0, g * s.w00);
+        if (s.x1ok) unsafeAtomicAdd(tc + (size_t)s.y0 * ew + s.x0 + 1, g * s.w01);
+        if (s.y1ok) unsafeAtomicAdd(tc + (size_t)(s.y0 + 1) * ew + s.x0, g * s.w10);
+        if (s.x1ok && s.y1ok) unsafeAtomicAdd(tc + (size_t)(s.y0 + 1) * ew + s.x0 + 1, g * s.w11);
+    }
+}
+
+// ApplyTangent (PointRenderer.cu:1646-1657): pose = Sophus::se3_expd(tangent) * pose; tangent = 0.  f64.
+__global__ void apply_tangent_kernel(double* __restrict__ tangent, double* __restrict__ poses, int n)
+{
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    double* t = tangent + 6 * (size_t)i;
+    double* p = poses + 8 * (size_t)i;
+    double ux = t[0], uy = t[1], uz = t[2], wx = t[3], wy = t[4], wz = t[5];
+    double th2 = wx * wx + wy * wy + wz * wz;
+    double th  = sqrt(th2);
+    double im, re, a, bb;
+    if (th < 1e-10)
+    {
+        double th4 = th2 * th2;
+        im         = 0.5 - th2 / 48.0 + th4 / 3840.0;
+        re         = 1.0 - th2 / 8.0 + th4 / 384.0;
+        a          = 0.5;
+        bb         = 1.0 / 6.0;
+    }
+    else
+    {
+        im = sin(0.5 * th) / th;
+        re = cos(0.5 * th);
+        a  = (1.0 - cos(th)) / th2;
+        bb = (th - sin(th)) / (th2 * th);
+    }
+    double ex = im * wx, ey = im * wy, ez = im * wz, ew = re;
+    double c1x = wy * uz - wz * uy, c1y = wz * ux - wx * uz, c1z = wx * uy - wy * ux;
+    double c2x = wy * c1z - wz * c1y, c2y = wz * c1x - wx * c1z, c2z = wx * c1y - wy * c1x;
+    double etx = ux + a * c1x + bb * c2x, ety = uy + a * c1y + bb * c2y, etz = uz + a * c1z + bb * c2z;
+    double qx = p[0], qy = p[1], qz = p[2], qw = p[3];
+    double nx = ew * qx + ex * qw + ey * qz - ez * qy;
+    double ny = ew * qy - ex * qz + ey * qw + ez * qx;
+    double nz = ew * qz + ex * qy - ey * qx + ez * qw;
+    double nw = ew * qw - ex * qx - ey * qy - ez * qz;
+    double tx = p[4], ty = p[5], tz = p[6];
+    double uvx = 2 * (ey * tz - ez * ty), uvy = 2 * (ez * tx - ex * tz), uvz = 2 * (ex * ty - ey * tx);
+    double rx = tx + ew * uvx + (ey * uvz - ez * uvy);
+    double ry = ty + ew * uvy + (ez * uvx - ex * uvz);
+    double rz = tz + ew * uvz + (ex * uvy - ey * uvx);
+    double qn = sqrt(nx * nx + ny * ny + nz * nz + nw * nw);
+    p[0]      = nx / qn;
+    p[1]      = ny / qn;
+    p[2]      = nz / qn;
+    p[3]      = nw / qn;
+    p[4]      = rx + etx;
+    p[5]      = ry + ety;
+    p[6]      = rz + etz;
+    for (int k = 0; k < 6; ++k) t[k] = 0;
+}
+
+
+void launch_env_sample(const ViewChunk& chunk, const double* poses, const float* intrinsics, const Levels& lv,
+                       const EnvLevels& ev, const float* tex, int eh, int ew, int add_to_out, hipStream_t st)
+{
+    size_t total = (size_t)lv.pix_prefix[lv.num] * lv.B;
+    int grid     = (int)((total + kBlock - 1) / kBlock);
+    if (grid > 0)
+        hipLaunchKernelGGL(env_sample_kernel, dim3(grid), dim3(kBlock), 0, st, chunk, poses, intrinsics, lv, ev, tex, eh,
+                           ew, add_to_out);
+}
+
+void launch_env_backward(const ViewChunk& chunk, const double* poses, const float* intrinsics, const Levels& lv,
+                         const EnvLevels& ev, float* genv, int eh, int ew, hipStream_t st)
+{
+    size_t total = (size_t)lv.pix_prefix[lv.num] * lv.B;
+    int grid     = (int)((total + kBlock - 1) / kBlock);
+    if (grid > 0)
+        hipLaunchKernelGGL(env_backward_kernel, dim3(grid), dim3(kBlock), 0, st, chunk, poses, intrinsics, lv, ev, genv,
+                           eh, ew);
+}
+
+void launch_apply_tangent(double* tangent, double* poses, int n, hipStream_t st)
+{
+    hipLaunchKernelGGL(apply_tangent_kernel, dim3((n + 127) / 128), dim3(128), 0, st, tangent, poses, n);
+}
+
+}  // namespace adop

@@ -1,0 +1,39 @@
+// launch.h — host-callable launchers of the kernels (one translation unit per kernel family).
+#pragma once
+#include "common.h"
+
+namespace adop
+{
+struct EnvLevels
+{
+    float* uv[ADOP_MAX_LAYERS];
+    float* env[ADOP_MAX_LAYERS];
+    const float* gout[ADOP_MAX_LAYERS];
+};
+
+void launch_prepare_views(const ViewChunk& ch, int first, int count, const double* poses, const float* intrinsics,
+                          int cols, ViewConst* out, hipStream_t st);
+void launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t st);
+void launch_clear(const Levels& lv, int grid, float* accum, size_t accum_floats, hipStream_t st);
+void launch_prepass(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, adop_stats* stats,
+                    hipStream_t st);
+void launch_blend(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
+                  float* accum, int S, adop_stats* stats, hipStream_t st);
+void launch_resolve(const Levels& lv, int grid, const float* accum, int S, const float* background, int write_mask,
+                    float mask_value, hipStream_t st);
+
+void launch_interleave(const Levels& lv, int blocks, float* ig, double* partial, hipStream_t st);
+void launch_render_backward(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
+                            const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr, int b,
+                            int blocks, double* partial, adop_stats* stats, hipStream_t st);
+void launch_finalize(const ViewConst* views, int B, int C, const double* bg_partial, int bg_blocks,
+                     const double* pt_partial, int pt_blocks, const adop_backward_buffers* g, int num_poses,
+                     int num_cameras, int cols, int normalize_mode, double* scratch, hipStream_t st);
+void launch_normalize_points(float* g, const float* count, int n, int mode, hipStream_t st);
+
+void launch_env_sample(const ViewChunk& chunk, const double* poses, const float* intrinsics, const Levels& lv,
+                       const EnvLevels& ev, const float* tex, int eh, int ew, int add_to_out, hipStream_t st);
+void launch_env_backward(const ViewChunk& chunk, const double* poses, const float* intrinsics, const Levels& lv,
+                         const EnvLevels& ev, float* genv, int eh, int ew, hipStream_t st);
+void launch_apply_tangent(double* tangent, double* poses, int n, hipStream_t st);
+}  // namespace adop

@@ -50,6 +50,8 @@ def main():
     ap.add_argument("--point-order", default="morton", choices=["morton", "random"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-points", type=int, default=0, help="point count of the CPU sample (0 = automatic)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (one process, one MI355X); "
@@ -130,6 +132,14 @@ def main():
                                    stats, stream)
             if rc != 0:
                 raise RuntimeError(lib.adop_last_error_string().decode())
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # untimed pass with counters: V_l, A_l, G_l of the byte model
     step(C.c_void_p(cache.stats.data_ptr()))

@@ -58,8 +58,11 @@ def test_struct_sizes_match_the_c_header(tmp_path):
 def test_workspace_query_needs_no_gpu():
     lib = _capi.load_library()
     s = _capi.Scene()
-    s.num_poses, s.num_cameras, s.intrinsics_cols = 3, 1, 13
+    s.num_poses, s.num_cameras, s.intrinsics_cols, s.num_channels = 3, 1, 13, 8
     n1 = lib.adop_workspace_size(C.byref(s), 1, 4, 640, 480)
     n4 = lib.adop_workspace_size(C.byref(s), 4, 4, 640, 480)
-    assert 0 < n1 < n4 < 64 << 20
+    pixels = 640 * 480 + 320 * 240 + 160 * 120 + 80 * 60
+    assert 64 * pixels < n1 < 64 * pixels + (4 << 20)  # 16 floats per pixel + partial sums
+    assert n1 < n4 < 4 * n1
     assert lib.adop_workspace_size(None, 1, 4, 640, 480) == 0
+    assert lib.adop_workspace_size(C.byref(s), 1, 9, 640, 480) == 0
