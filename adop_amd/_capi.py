@@ -70,6 +70,7 @@ class Scene(C.Structure):
         ("intrinsics", C.c_void_p),
         ("num_cameras", C.c_int32),
         ("intrinsics_cols", C.c_int32),
+        ("index_is_identity", C.c_int32),
     ]
 
 

@@ -98,6 +98,10 @@ struct WorkspaceLayout
     size_t pt_partial;  // double[B * kPartialBlocks * kPartialStride]
     size_t scratch;     // double[num_poses*7 + num_cameras*(cols+1)]
     size_t pixels;      // float[B * P * max(S, 2C)]: blend accumulators (forward) / [I|G] array (backward)
+    size_t q_counts;    // uint32[kNumQueues]
+    size_t q_prefix;    // uint32[kNumQueues + 1]
+    size_t q_items;     // uint64[kNumQueues * q_cap]
+    uint32_t q_cap;
     size_t total;
 };
 
@@ -143,7 +147,17 @@ WorkspaceLayout layout(const adop_scene* s, int B, int L, int w0, int h0)
     w.pixels = o;
     int per  = accum_stride(s->num_channels) > 2 * s->num_channels ? accum_stride(s->num_channels) : 2 * s->num_channels;
     o        = align_up(o + sizeof(float) * (size_t)B * pyramid_pixels(L, w0, h0) * (size_t)per, 256);
-    w.total  = o;
+    // backward work queue: workgroup k of backward_tex_kernel appends to sub-queue k % kNumQueues
+    size_t blocks = ((size_t)(s->num_points > 0 ? s->num_points : 0) + kBlock - 1) / kBlock;
+    w.q_cap       = (uint32_t)(((blocks + kNumQueues - 1) / kNumQueues) * kBlock);
+    if (w.q_cap == 0) w.q_cap = kBlock;
+    w.q_counts = o;
+    o          = align_up(o + sizeof(uint32_t) * kNumQueues, 256);
+    w.q_prefix = o;
+    o          = align_up(o + sizeof(uint32_t) * (kNumQueues + 1), 256);
+    w.q_items  = o;
+    o          = align_up(o + sizeof(unsigned long long) * (size_t)kNumQueues * w.q_cap, 256);
+    w.total    = o;
     return w;
 }
 
@@ -166,6 +180,8 @@ adop_status validate(const adop_scene* s, const adop_view* views, int B, const a
         return fail(ADOP_INVALID_ARG, "poses / intrinsics missing");
     if (s->intrinsics_cols < 5 || s->intrinsics_cols > kMaxIntrinsicsCols)
         return fail(ADOP_INVALID_ARG, "intrinsics_cols out of range");
+    if (s->index_is_identity && s->num_texels != s->num_points)
+        return fail(ADOP_INVALID_ARG, "index_is_identity needs num_texels == num_points");
     int w = views[0].w, h = views[0].h;
     for (int b = 0; b < B; ++b)
     {
@@ -387,7 +403,10 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     // Build(info,false): zero the gradient tensors (:922-949)
     {
         StageScope sc("Prepare Backward", stream);
-        if ((st = fill_async(grads->grad_texture, sizeof(float) * (size_t)C * scene->num_texels, 0, stream)) != ADOP_OK)
+        // with an identity index and a vectorised channel count backward_tex_kernel writes every texel itself
+        const bool tex_self_clearing = scene->index_is_identity && (C == 4 || C == 8) && N > 0;
+        if (!tex_self_clearing &&
+            (st = fill_async(grads->grad_texture, sizeof(float) * (size_t)C * scene->num_texels, 0, stream)) != ADOP_OK)
             return st;
         if (grads->grad_points)
         {
@@ -415,11 +434,23 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     if (pt_blocks > kPartialBlocks) pt_blocks = kPartialBlocks;
     if (pt_blocks < 1) pt_blocks = 1;
     bool half = scene->texture_dtype == ADOP_TEXTURE_F16;
+    QueueArg q;
+    q.counts = (uint32_t*)((char*)workspace + wl.q_counts);
+    q.prefix = (uint32_t*)((char*)workspace + wl.q_prefix);
+    q.items  = (unsigned long long*)((char*)workspace + wl.q_items);
+    q.cap    = wl.q_cap;
+    if (N < 1)
+    {
+        // nothing writes the partial rows: clear them for finalize
+        if ((st = fill_async(pt_partial, sizeof(double) * (size_t)num_views * kPartialBlocks * kPartialStride, 0,
+                             stream)) != ADOP_OK)
+            return st;
+    }
     for (int b = 0; b < num_views; ++b)
     {
         StageScope sc("RenderBackward", stream);
-        launch_render_backward(pc, dviews, lv, rp, half, ig, grads, want_pose, want_intr, b, pt_blocks, pt_partial,
-                               stats, stream);
+        launch_render_backward(pc, dviews, lv, rp, half, ig, grads, want_pose, want_intr, scene->index_is_identity, b,
+                               b == 0, q, pt_blocks, pt_partial, stats, stream);
     }
     StageScope post("Post Process Gradient", stream);
     launch_finalize(dviews, num_views, C, bg_partial, bg_blocks, pt_partial, pt_blocks, grads, scene->num_poses,

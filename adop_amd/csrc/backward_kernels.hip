@@ -11,6 +11,12 @@
 
 namespace adop
 {
+__global__ void fill_zero_u32_kernel(uint32_t* __restrict__ p, int n)
+{
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
 // CombineAndFillBackward (:851-900) fused with the I/G interleave.  One thread per pixel of every level/image.
 // Background gradient: per-thread fp32 partial over a handful of pixels, wave/block reduction in f64, one f64
 // partial row per block.
@@ -86,277 +92,417 @@ __global__ __launch_bounds__(kBlock) void interleave_kernel(Levels lv, float* __
 }
 
 template <int CT>
-__device__ __forceinline__ void load_channels(const float* __restrict__ src, int C, float* dst)
+__device__ __forceinline__ void load_channels(const float* __restrict__ src, float* dst)
 {
-    if (CT == 8 || CT == 4)
-    {
-        const float4* s4 = (const float4*)src;
+    static_assert(CT == 4 || CT == 8, "vector path");
+    const float4* s4 = (const float4*)src;
 #pragma unroll
-        for (int q = 0; q < CT / 4; ++q)
-        {
-            float4 v       = s4[q];
-            dst[4 * q]     = v.x;
-            dst[4 * q + 1] = v.y;
-            dst[4 * q + 2] = v.z;
-            dst[4 * q + 3] = v.w;
-        }
-    }
-    else
+    for (int q = 0; q < CT / 4; ++q)
     {
-#pragma unroll
-        for (int c = 0; c < kMaxChannels; ++c)
-            if (c < C) dst[c] = src[c];
+        float4 v       = s4[q];
+        dst[4 * q]     = v.x;
+        dst[4 * q + 1] = v.y;
+        dst[4 * q + 2] = v.z;
+        dst[4 * q + 3] = v.w;
     }
 }
 
-// RenderBackward (PointRenderer.cu:396-724).  Grid-stride over points so that the pose / intrinsics sums can live
-// in registers (f64) for the whole kernel; they leave the block as one partial row per (block, view).
-// Descriptor gradients of one point are summed over the levels in registers and added once per channel.
+// RenderBackward (PointRenderer.cu:396-724) is split in two kernels.
+//
+// backward_tex_kernel — one thread per point: projection, the per-level depth test (`break` at the first failed
+// level, :462), the descriptor gradient (:469-485, summed over the levels in registers) and the decision which
+// levels receive a ghost / spatial gradient (:487-489).  Points with at least one such level are appended to a
+// work queue as (point id | level mask << 32).  The queue is split in kNumQueues sub-queues with their own counters
+// (one returning atomic per workgroup; a single counter would serialise ~40 k same-address atomics).
+//
+// backward_ghost_kernel — one thread per queue item, all lanes busy: the four-neighbour gather from the
+// pixel-major [I|G] array, the approximate image-space gradient (:491-611) and ProjectPoint*Backward.
 template <int CT, bool HALF>
-__global__ __launch_bounds__(kBlock) void render_backward_kernel(CloudArg pc, const ViewConst* __restrict__ views,
-                                                                  Levels lv, ParamArg rp, const float* __restrict__ ig,
-                                                                  float* __restrict__ gtex,
-                                                                  float* __restrict__ gpoints,
-                                                                  float* __restrict__ gpoints_count, int want_pose,
-                                                                  int want_intr, int view_b,
-                                                                  double* __restrict__ partial, adop_stats* stats)
+__global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const ViewConst* __restrict__ views,
+                                                               Levels lv, ParamArg rp, const float* __restrict__ ig,
+                                                               float* __restrict__ gtex, int identity_index,
+                                                               int view_b, int first_view,
+                                                               uint32_t* __restrict__ q_counts,
+                                                               unsigned long long* __restrict__ q_items,
+                                                               uint32_t q_cap, adop_stats* stats)
 {
     constexpr int CMAX = CT ? CT : 1;  // register arrays exist only for compile-time channel counts
-    __shared__ double red[kBlock / 64][kPartialStride];
+    __shared__ uint32_t s_wave_count[kBlock / 64];
+    __shared__ uint32_t s_base;
     const bool STATS    = stats != nullptr;  // counter pass (uniform branch)
     const int b         = view_b;
     const ViewConst& vc = views[b];
     const float accept  = rp.depth_accept + 1;
     const int C         = CT ? CT : lv.C;
+    const int lane      = threadIdx.x & 63;
+    const int wave      = threadIdx.x >> 6;
+
+    const int i  = blockIdx.x * kBlock + threadIdx.x;
+    bool valid   = i < pc.n;
+    float4 P     = valid ? pc.position[i] : make_float4(0, 0, 0, 0);
+    V3 pos       = {P.x, P.y, P.z};
+    V3 nrm       = {0, 0, 0};
+    if (valid && pc.normal) nrm = unpack_normal10(pc.normal[i]);
+    bool drop_out = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;
+    V2 ip;
+    V3 view_p;
+    float z, radius_pixels;
+    bool ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff, lv.l[0].w,
+                                     &ip, &z, &radius_pixels, &view_p);
+    int tex_index = identity_index ? i : (valid ? pc.index[i] : 0);
+    ok            = ok && (unsigned)tex_index < (unsigned)pc.num_texels;
+
+    // phase 1: pixel of every level, depth loads (independent)
+    uint32_t pix[ADOP_MAX_LAYERS];
+    bool in[ADOP_MAX_LAYERS];
+    bool edge_ok[ADOP_MAX_LAYERS];
+    float dep[ADOP_MAX_LAYERS];
+#pragma unroll
+    for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+    {
+        in[l]      = false;
+        edge_ok[l] = false;
+        pix[l]     = 0;
+        dep[l]     = 0.f;
+        if (l < lv.num)
+        {
+            const LevelArg& L = lv.l[l];
+            int px = f2i_rn(ip.x), py = f2i_rn(ip.y);
+            bool lod_skip = rp.drop_by_radius && radius_pixels < rp.drop_threshold;  // continue, :451-454
+            in[l]         = ok && !lod_skip && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h;
+            if (in[l])
+            {
+                pix[l]     = (uint32_t)py * (uint32_t)L.w + (uint32_t)px;
+                dep[l]     = L.depth[(size_t)b * L.w * L.h + pix[l]];
+                int ex     = min(px, L.w - 1 - px);
+                int ey     = min(py, L.h - 1 - py);
+                edge_ok[l] = min(ex, ey) > 2;  // distanceFromEdge > 2, :489
+            }
+            radius_pixels *= 0.5f;
+            ip.x *= 0.5f;
+            ip.y *= 0.5f;
+        }
+    }
+    // phase 2: depth test in level order, `break` at the first failure (:462); weight loads
+    bool pass[ADOP_MAX_LAYERS];
+    float wgt[ADOP_MAX_LAYERS];
+    {
+        bool alive = true;
+#pragma unroll
+        for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+        {
+            pass[l] = false;
+            wgt[l]  = 0.f;
+            if (in[l] && alive)
+            {
+                if (z > dep[l] * accept)
+                    alive = false;
+                else
+                    pass[l] = true;
+            }
+            if (pass[l]) wgt[l] = lv.l[l].weight[(size_t)b * lv.l[l].w * lv.l[l].h + pix[l]];
+        }
+    }
+    // phase 3: descriptor gradient of the rendered (not dropped) points; spatial-gradient eligibility
+    const bool point_grad = (rp.ghost_gradients && drop_out) | (!rp.ghost_gradients && !drop_out);
+    uint32_t mask         = 0;
+    float gt[CMAX];
+#pragma unroll
+    for (int c = 0; c < CMAX; ++c) gt[c] = 0.f;
+    bool gt_live = false;
+#pragma unroll
+    for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+    {
+        bool go = pass[l];
+        if (pass[l] && !drop_out)
+        {
+            if (wgt[l] == 0)
+                go = false;  // continue, :473
+            else
+            {
+                float iw        = 1.f / wgt[l];
+                const float* pg = ig + (size_t)ws_pixel(lv, l, b, pix[l]) * (2 * C) + C;  // G of the pixel
+                if (CT == 0)
+                {
+                    // any channel count: one atomic per channel and level (:478-484)
+#pragma unroll 1
+                    for (int c = 0; c < C; ++c)
+                        unsafeAtomicAdd(gtex + (size_t)c * pc.num_texels + tex_index, iw * pg[c]);
+                }
+                else
+                {
+                    float G[CMAX];
+                    load_channels<CT ? CT : 4>(pg, G);
+#pragma unroll
+                    for (int c = 0; c < CMAX; ++c) gt[c] += iw * G[c];
+                    gt_live = true;
+                }
+            }
+        }
+        bool spatial = go && point_grad && edge_ok[l];
+        if (spatial) mask |= 1u << l;
+        if (STATS && l < lv.num) stat_add(&stats->spatial[l], spatial);
+    }
+    if (CT != 0)
+    {
+        if (identity_index)
+        {
+            // texel i belongs to this thread alone: plain coalesced stores, which also clear the buffer on the first view
+            if (valid)
+            {
+#pragma unroll
+                for (int c = 0; c < CMAX; ++c)
+                {
+                    float* dst = gtex + (size_t)c * pc.num_texels + i;
+                    *dst       = first_view ? gt[c] : (*dst + gt[c]);
+                }
+            }
+        }
+        else if (gt_live)
+        {
+#pragma unroll
+            for (int c = 0; c < CMAX; ++c) unsafeAtomicAdd(gtex + (size_t)c * pc.num_texels + tex_index, gt[c]);
+        }
+    }
+
+    // queue push: rank inside the workgroup, one returning atomic per workgroup on the sub-queue counter
+    bool has               = mask != 0;
+    unsigned long long bal = __ballot(has);
+    uint32_t rank_in_wave  = (uint32_t)__popcll(bal & ((1ull << lane) - 1ull));
+    if (lane == 0) s_wave_count[wave] = (uint32_t)__popcll(bal);
+    __syncthreads();
+    uint32_t before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < kBlock / 64; ++w)
+    {
+        uint32_t c = s_wave_count[w];
+        if (w < wave) before += c;
+        total += c;
+    }
+    const uint32_t q = blockIdx.x % kNumQueues;
+    if (threadIdx.x == 0) s_base = total ? atomicAdd(&q_counts[q], total) : 0u;
+    __syncthreads();
+    if (has)
+        q_items[(size_t)q * q_cap + s_base + before + rank_in_wave] =
+            (unsigned long long)(uint32_t)i | ((unsigned long long)mask << 32);
+}
+
+// exclusive prefix over the sub-queue counters: prefix[0..kNumQueues], prefix[kNumQueues] = number of items
+__global__ __launch_bounds__(kBlock) void queue_scan_kernel(const uint32_t* __restrict__ counts,
+                                                            uint32_t* __restrict__ prefix)
+{
+    constexpr int PER = kNumQueues / kBlock;
+    __shared__ uint32_t s_sum[kBlock];
+    uint32_t local[PER];
+    uint32_t acc = 0;
+#pragma unroll
+    for (int k = 0; k < PER; ++k)
+    {
+        local[k] = acc;
+        acc += counts[threadIdx.x * PER + k];
+    }
+    s_sum[threadIdx.x] = acc;
+    __syncthreads();
+    uint32_t base = 0;
+    for (int t = 0; t < (int)threadIdx.x; ++t) base += s_sum[t];
+#pragma unroll
+    for (int k = 0; k < PER; ++k) prefix[threadIdx.x * PER + k] = base + local[k];
+    if (threadIdx.x == kBlock - 1) prefix[kNumQueues] = base + acc;
+}
+
+template <int CT, bool HALF>
+__global__ __launch_bounds__(kBlock) void backward_ghost_kernel(CloudArg pc, const ViewConst* __restrict__ views,
+                                                                 Levels lv, ParamArg rp, const float* __restrict__ ig,
+                                                                 float* __restrict__ gpoints,
+                                                                 float* __restrict__ gpoints_count, int want_pose,
+                                                                 int want_intr, int identity_index, int view_b,
+                                                                 const uint32_t* __restrict__ q_prefix,
+                                                                 const unsigned long long* __restrict__ q_items,
+                                                                 uint32_t q_cap, double* __restrict__ partial)
+{
+    constexpr int CMAX = CT ? CT : 1;
+    __shared__ double red[kBlock / 64][kPartialStride];
+    __shared__ uint32_t s_prefix[kNumQueues + 1];
+    const int b         = view_b;
+    const ViewConst& vc = views[b];
+    const float accept  = rp.depth_accept + 1;
+    const int C         = CT ? CT : lv.C;
+
+    for (int k = threadIdx.x; k <= kNumQueues; k += kBlock) s_prefix[k] = q_prefix[k];
+    __syncthreads();
+    const uint32_t total = s_prefix[kNumQueues];
 
     double acc[kAcc];
 #pragma unroll
     for (int k = 0; k < kAcc; ++k) acc[k] = 0;
 
-    const int n_round = ((pc.n + kBlock - 1) / kBlock) * kBlock;
-    for (int i = blockIdx.x * kBlock + threadIdx.x; i < n_round; i += gridDim.x * kBlock)
+    for (uint32_t t = blockIdx.x * kBlock + threadIdx.x; t < total; t += gridDim.x * kBlock)
     {
-        bool valid = i < pc.n;
-        float4 P   = valid ? pc.position[i] : make_float4(0, 0, 0, 0);
-        V3 pos     = {P.x, P.y, P.z};
-        V3 nrm     = {0, 0, 0};
-        if (valid && pc.normal) nrm = unpack_normal10(pc.normal[i]);
-        bool drop_out = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;
+        // sub-queue of item t: largest q with prefix[q] <= t
+        uint32_t lo = 0, hi = kNumQueues;
+        while (hi - lo > 1)
+        {
+            uint32_t mid = (lo + hi) >> 1;
+            if (s_prefix[mid] <= t)
+                lo = mid;
+            else
+                hi = mid;
+        }
+        unsigned long long item = q_items[(size_t)lo * q_cap + (t - s_prefix[lo])];
+        const int i             = (int)(uint32_t)item;
+        const uint32_t mask     = (uint32_t)(item >> 32);
+
+        float4 P = pc.position[i];
+        V3 pos   = {P.x, P.y, P.z};
+        V3 nrm   = {0, 0, 0};
+        if (pc.normal) nrm = unpack_normal10(pc.normal[i]);
         V2 ip;
         V3 view_p;
         float z, radius_pixels;
-        bool ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff,
-                                         lv.l[0].w, &ip, &z, &radius_pixels, &view_p);
-        int tex_index = valid ? pc.index[i] : 0;
-        ok            = ok && (unsigned)tex_index < (unsigned)pc.num_texels;
-        if (!STATS && !ok) continue;
-
-        float scale = 1;
-        bool alive  = ok;
-        // running value of grad_points[i] / count[i]; loaded at the first contribution so that the additions
-        // happen in the reference's order (view after view, level after level)
-        float gp[3]  = {0, 0, 0};
-        float gp_n   = 0;
-        bool gp_live = false;
-        float gt[CMAX];  // descriptor gradient of this point, summed over the levels
-#pragma unroll
-        for (int c = 0; c < CMAX; ++c) gt[c] = 0;
-        bool gt_live = false;
+        project_point(vc, pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff, lv.l[0].w, &ip, &z,
+                      &radius_pixels, &view_p);
+        const int tex_index = identity_index ? i : pc.index[i];
         float T[CMAX];
-        bool T_live = false;
+        if (CT != 0)
+        {
+#pragma unroll
+            for (int c = 0; c < CMAX; ++c) T[c] = tex_fetch<HALF>(pc.texture, (size_t)c * pc.num_texels + tex_index);
+        }
+        // running value of grad_points[i] / count[i]: the additions happen in the reference's order (view after
+        // view, level after level); this thread owns point i for this view
+        float gp[3] = {0, 0, 0};
+        float gp_n  = 0;
+        if (gpoints)
+        {
+            const float* g = gpoints + 4 * (size_t)i;
+            gp[0]          = g[0];
+            gp[1]          = g[1];
+            gp[2]          = g[2];
+            gp_n           = gpoints_count[i];
+        }
+        float scale = 1;
 #pragma unroll 1
         for (int l = 0; l < lv.num; ++l)
         {
-            const LevelArg& L = lv.l[l];
-            int px = f2i_rn(ip.x), py = f2i_rn(ip.y);
-            bool lod_skip = rp.drop_by_radius && radius_pixels < rp.drop_threshold;  // continue, :451-454
-            bool in       = alive && !lod_skip && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h;
-            bool spatial  = false;
-            if (in)
+            if (mask & (1u << l))
             {
-                size_t hw = (size_t)L.w * L.h;
-                size_t p  = (size_t)py * L.w + px;
-                float image_depth = L.depth[(size_t)b * hw + p];
-                if (z > image_depth * accept)
+                const LevelArg& L = lv.l[l];
+                int px = f2i_rn(ip.x), py = f2i_rn(ip.y);
+                size_t hw             = (size_t)L.w * L.h;
+                size_t p              = (size_t)py * L.w + px;
+                const float* pg       = ig + (size_t)ws_pixel(lv, l, b, (uint32_t)p) * (2 * C);  // [I | G] of the pixel
+                const ptrdiff_t nb[4] = {-1, 1, -(ptrdiff_t)L.w, (ptrdiff_t)L.w};
+                float Wn[4] = {0, 0, 0, 0}, Dn[4] = {0, 0, 0, 0};
+                if (rp.test_backward_mode == 4)
                 {
-                    alive = false;  // break, :462
+                    const float* Wp = L.weight + (size_t)b * hw + p;
+                    const float* Dp = L.depth + (size_t)b * hw + p;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+                    {
+                        Wn[k] = Wp[nb[k]];
+                        Dn[k] = Dp[nb[k]];
+                    }
+                }
+                auto dI_of = [&](float T_c, float I_x, float W_x, float D_x) -> float
+                {
+                    if (rp.test_backward_mode == 4)
+                    {
+                        if (W_x == 0 || z * accept < D_x) return T_c - I_x;          // full override
+                        if (z > D_x * accept) return 0.f;                            // discard
+                        return (W_x / (W_x + 1) * I_x + 1 / (W_x + 1) * T_c - I_x);  // blend
+                    }
+                    return T_c - I_x;
+                };
+                float dR_dpx = 0, dR_dpy = 0;
+                if (CT == 0)
+                {
+#pragma unroll 1
+                    for (int c = 0; c < C; ++c)
+                    {
+                        float T_c = tex_fetch<HALF>(pc.texture, (size_t)c * pc.num_texels + tex_index);
+                        float v[4];
+#pragma unroll
+                        for (int k = 0; k < 4; ++k)
+                        {
+                            const float* q = pg + nb[k] * (2 * C);
+                            v[k]           = dI_of(T_c, q[c], Wn[k], Dn[k]) * q[C + c];
+                        }
+                        float a0 = -v[0], a1 = v[1], b0 = -v[2], b1 = v[3];
+                        dR_dpx += 0.5f * (a0 + a1);
+                        dR_dpy += 0.5f * (b0 + b1);
+                    }
                 }
                 else
                 {
-                    float w         = L.weight[(size_t)b * hw + p];
-                    const float* pg = ig + (size_t)ws_pixel(lv, l, b, (uint32_t)p) * (2 * C);  // [I | G] of the pixel
-                    bool go         = true;
-                    if (!drop_out)
-                    {
-                        if (w == 0)
-                            go = false;  // continue, :473
-                        else
-                        {
-                            float iw = 1.f / w;
-                            if (CT == 0)
-                            {
-                                // any channel count: one atomic per channel and level (:478-484)
-#pragma unroll 1
-                                for (int c = 0; c < C; ++c)
-                                    unsafeAtomicAdd(gtex + (size_t)c * pc.num_texels + tex_index, iw * pg[C + c]);
-                            }
-                            else
-                            {
-                                float G[CMAX];
-                                load_channels<CT>(pg + C, C, G);
+                    float v[4][CMAX];  // dI * G per neighbour and channel
 #pragma unroll
-                                for (int c = 0; c < CMAX; ++c) gt[c] += iw * G[c];
-                                gt_live = true;
-                            }
-                        }
+                    for (int k = 0; k < 4; ++k)
+                    {
+                        const float* q = pg + nb[k] * (2 * C);
+                        float In[CMAX], Gn[CMAX];
+                        load_channels<CT ? CT : 4>(q, In);
+                        load_channels<CT ? CT : 4>(q + C, Gn);
+#pragma unroll
+                        for (int c = 0; c < CMAX; ++c) v[k][c] = dI_of(T[c], In[c], Wn[k], Dn[k]) * Gn[c];
                     }
-                    bool point_grad = (rp.ghost_gradients && drop_out) | (!rp.ghost_gradients && !drop_out);
-                    int ex          = min(px, L.w - 1 - px);
-                    int ey          = min(py, L.h - 1 - py);
-                    if (go && point_grad && min(ex, ey) > 2)  // distanceFromEdge > 2, :489
+#pragma unroll
+                    for (int c = 0; c < CMAX; ++c)
                     {
-                        spatial = true;
-                        const ptrdiff_t nb[4] = {-1, 1, -(ptrdiff_t)L.w, (ptrdiff_t)L.w};
-                        const float* Wp       = L.weight + (size_t)b * hw + p;
-                        const float* Dp       = L.depth + (size_t)b * hw + p;
-                        float Wn[4] = {0, 0, 0, 0}, Dn[4] = {0, 0, 0, 0};
-                        if (rp.test_backward_mode == 4)
-                        {
+                        float a0 = -v[0][c], a1 = v[1][c], b0 = -v[2][c], b1 = v[3][c];
+                        dR_dpx += 0.5f * (a0 + a1);
+                        dR_dpy += 0.5f * (b0 + b1);
+                    }
+                }
+                V2 dR_dp       = {dR_dpx / (float)C, dR_dpy / (float)C};
+                float crop2[5] = {vc.crop[0] * scale, vc.crop[1] * scale, vc.crop[2] * scale, vc.crop[3] * scale,
+                                  vc.crop[4] * scale};  // crop.scale(scale), :616
+                BackwardOut bo;
+                project_point_backward(vc, pc.intrinsics, view_p, dR_dp, crop2, rp.dist_cutoff, &bo);
+                gp[0] += bo.g_point[0];
+                gp[1] += bo.g_point[1];
+                gp[2] += bo.g_point[2];
+                gp_n += 1.f;
+                if (want_pose)
+                {
 #pragma unroll
-                            for (int k = 0; k < 4; ++k)
-                            {
-                                Wn[k] = Wp[nb[k]];
-                                Dn[k] = Dp[nb[k]];
-                            }
-                        }
-                        auto dI_of = [&](float T_c, float I_x, float W_x, float D_x) -> float
-                        {
-                            if (rp.test_backward_mode == 4)
-                            {
-                                if (W_x == 0 || z * accept < D_x) return T_c - I_x;  // full override
-                                if (z > D_x * accept) return 0.f;                    // discard
-                                return (W_x / (W_x + 1) * I_x + 1 / (W_x + 1) * T_c - I_x);  // blend
-                            }
-                            return T_c - I_x;
-                        };
-                        float dR_dpx = 0, dR_dpy = 0;
-                        if (CT == 0)
-                        {
-#pragma unroll 1
-                            for (int c = 0; c < C; ++c)
-                            {
-                                float T_c = tex_fetch<HALF>(pc.texture, (size_t)c * pc.num_texels + tex_index);
-                                float v[4];
+                    for (int k = 0; k < 6; ++k) acc[k] += (double)bo.g_pose[k];
+                    acc[6] += 1.0;
+                }
+                if (want_intr)
+                {
+                    if (vc.model == 0)
+                    {
+                        float kf = rp.K_gradient_factor;
+                        bo.g_k[4] *= 0.1f;
+                        bo.g_k[4] *= 0;  // :653-654
 #pragma unroll
-                                for (int k = 0; k < 4; ++k)
-                                {
-                                    const float* q = pg + nb[k] * (2 * C);
-                                    v[k]           = dI_of(T_c, q[c], Wn[k], Dn[k]) * q[C + c];
-                                }
-                                float a0 = -v[0], a1 = v[1], b0 = -v[2], b1 = v[3];
-                                dR_dpx += 0.5f * (a0 + a1);
-                                dR_dpy += 0.5f * (b0 + b1);
-                            }
-                        }
-                        else
-                        {
-                            if (!T_live)
-                            {
+                        for (int k = 0; k < 5; ++k) acc[8 + k] += (double)(kf * bo.g_k[k]);
+                        float df = rp.distortion_gradient_factor;
+                        bo.g_dis[2] *= 0.25f;
+                        bo.g_dis[3] *= 0.1f;
+                        bo.g_dis[4] *= 0.1f;
+                        bo.g_dis[5] *= 0.1f;
+                        bo.g_dis[6] *= 0.1f;
+                        bo.g_dis[7] *= 0.1f;
 #pragma unroll
-                                for (int c = 0; c < CMAX; ++c)
-                                    T[c] = tex_fetch<HALF>(pc.texture, (size_t)c * pc.num_texels + tex_index);
-                                T_live = true;
-                            }
-                            float v[4][CMAX];  // dI * G per neighbour and channel
+                        for (int k = 0; k < 8; ++k) acc[13 + k] += (double)(df * bo.g_dis[k]);
+                        acc[7] += 1.0 / 1024.0;  // :680-681
+                    }
+                    else
+                    {
 #pragma unroll
-                            for (int k = 0; k < 4; ++k)
-                            {
-                                const float* q = pg + nb[k] * (2 * C);
-                                float In[CMAX], Gn[CMAX];
-                                load_channels<CT>(q, C, In);
-                                load_channels<CT>(q + C, C, Gn);
-#pragma unroll
-                                for (int c = 0; c < CMAX; ++c) v[k][c] = dI_of(T[c], In[c], Wn[k], Dn[k]) * Gn[c];
-                            }
-#pragma unroll
-                            for (int c = 0; c < CMAX; ++c)
-                            {
-                                float a0 = -v[0][c], a1 = v[1][c], b0 = -v[2][c], b1 = v[3][c];
-                                dR_dpx += 0.5f * (a0 + a1);
-                                dR_dpy += 0.5f * (b0 + b1);
-                            }
-                        }
-                        V2 dR_dp       = {dR_dpx / (float)C, dR_dpy / (float)C};
-                        float crop2[5] = {vc.crop[0] * scale, vc.crop[1] * scale, vc.crop[2] * scale,
-                                          vc.crop[3] * scale, vc.crop[4] * scale};  // crop.scale(scale), :616
-                        BackwardOut bo;
-                        project_point_backward(vc, pc.intrinsics, view_p, dR_dp, crop2, rp.dist_cutoff, &bo);
-                        if (gpoints)
-                        {
-                            if (!gp_live)
-                            {
-                                const float* g = gpoints + 4 * (size_t)i;
-                                gp[0]          = g[0];
-                                gp[1]          = g[1];
-                                gp[2]          = g[2];
-                                gp_n           = gpoints_count[i];
-                                gp_live        = true;
-                            }
-                            gp[0] += bo.g_point[0];
-                            gp[1] += bo.g_point[1];
-                            gp[2] += bo.g_point[2];
-                            gp_n += 1.f;
-                        }
-                        if (want_pose)
-                        {
-#pragma unroll
-                            for (int k = 0; k < 6; ++k) acc[k] += (double)bo.g_pose[k];
-                            acc[6] += 1.0;
-                        }
-                        if (want_intr)
-                        {
-                            if (vc.model == 0)
-                            {
-                                float kf = rp.K_gradient_factor;
-                                bo.g_k[4] *= 0.1f;
-                                bo.g_k[4] *= 0;  // :653-654
-#pragma unroll
-                                for (int k = 0; k < 5; ++k) acc[8 + k] += (double)(kf * bo.g_k[k]);
-                                float df = rp.distortion_gradient_factor;
-                                bo.g_dis[2] *= 0.25f;
-                                bo.g_dis[3] *= 0.1f;
-                                bo.g_dis[4] *= 0.1f;
-                                bo.g_dis[5] *= 0.1f;
-                                bo.g_dis[6] *= 0.1f;
-                                bo.g_dis[7] *= 0.1f;
-#pragma unroll
-                                for (int k = 0; k < 8; ++k) acc[13 + k] += (double)(df * bo.g_dis[k]);
-                                acc[7] += 1.0 / 1024.0;  // :680-681
-                            }
-                            else
-                            {
-#pragma unroll
-                                for (int k = 0; k < 5; ++k) acc[8 + k] += (double)bo.g_k[k];
-                                acc[7] += 1.0;  // :718
-                            }
-                        }
+                        for (int k = 0; k < 5; ++k) acc[8 + k] += (double)bo.g_k[k];
+                        acc[7] += 1.0;  // :718
                     }
                 }
             }
-            if (STATS) stat_add(&stats->spatial[l], spatial);
             scale *= 0.5f;
-            radius_pixels *= 0.5f;
             ip.x *= 0.5f;
             ip.y *= 0.5f;
         }
-        if (gt_live)
+        if (gpoints)
         {
-#pragma unroll
-            for (int c = 0; c < CMAX; ++c) unsafeAtomicAdd(gtex + (size_t)c * pc.num_texels + tex_index, gt[c]);
-        }
-        if (gp_live)
-        {
-            // one thread owns point i for this view; views are launched one after another on the stream
             float* g         = gpoints + 4 * (size_t)i;
             g[0]             = gp[0];
             g[1]             = gp[1];
@@ -525,18 +671,27 @@ void launch_interleave(const Levels& lv, int blocks, float* ig, double* partial,
 
 template <int CT, bool HALF>
 static void launch_bwd_t(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp,
-                         const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr, int b,
-                         int blocks, double* partial, adop_stats* stats, hipStream_t st)
+                         const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr,
+                         int identity_index, int b, int first_view, const QueueArg& q, int ghost_blocks,
+                         double* partial, adop_stats* stats, hipStream_t st)
 {
-    hipLaunchKernelGGL((render_backward_kernel<CT, HALF>), dim3(blocks), dim3(kBlock), 0, st, pc, views, lv, rp, ig,
-                       g->grad_texture, g->grad_points, g->grad_points_count, want_pose, want_intr, b, partial, stats);
+    int grid = (pc.n + kBlock - 1) / kBlock;
+    hipLaunchKernelGGL(fill_zero_u32_kernel, dim3(kNumQueues / kBlock), dim3(kBlock), 0, st, q.counts, kNumQueues);
+    hipLaunchKernelGGL((backward_tex_kernel<CT, HALF>), dim3(grid), dim3(kBlock), 0, st, pc, views, lv, rp, ig,
+                       g->grad_texture, identity_index, b, first_view, q.counts, q.items, q.cap, stats);
+    hipLaunchKernelGGL(queue_scan_kernel, dim3(1), dim3(kBlock), 0, st, q.counts, q.prefix);
+    hipLaunchKernelGGL((backward_ghost_kernel<CT, HALF>), dim3(ghost_blocks), dim3(kBlock), 0, st, pc, views, lv, rp,
+                       ig, g->grad_points, g->grad_points_count, want_pose, want_intr, identity_index, b, q.prefix,
+                       q.items, q.cap, partial);
 }
 
 void launch_render_backward(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
-                            const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr, int b,
-                            int blocks, double* partial, adop_stats* stats, hipStream_t st)
+                            const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr,
+                            int identity_index, int b, int first_view, const QueueArg& q, int ghost_blocks,
+                            double* partial, adop_stats* stats, hipStream_t st)
 {
-#define ADOP_ARGS pc, views, lv, rp, ig, g, want_pose, want_intr, b, blocks, partial, stats, st
+    if (pc.n < 1) return;
+#define ADOP_ARGS pc, views, lv, rp, ig, g, want_pose, want_intr, identity_index, b, first_view, q, ghost_blocks, partial, stats, st
     if (lv.C == 8)
         half ? launch_bwd_t<8, true>(ADOP_ARGS) : launch_bwd_t<8, false>(ADOP_ARGS);
     else if (lv.C == 4)

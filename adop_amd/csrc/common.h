@@ -16,6 +16,7 @@ constexpr int kMaxChannels   = 16;
 constexpr int kPartialBlocks = 2048;  // grid of the grid-stride kernels that write per-block partial sums
 constexpr int kPartialStride = 24;    // doubles per (block, view), 21 used: 6 pose, pose count, intr count, 13 intr
 constexpr int kAcc           = 21;
+constexpr int kNumQueues     = 2048;  // sub-queues of the backward work queue (multiple of kBlock)
 constexpr int kMaxIntrinsicsCols = 24;  // 13 pinhole / 5 affine + up to 19 polynomial coefficients
 constexpr uint64_t kClearPacked = (uint64_t(0x47C35000u) << 32) | 0xFFFFFFFFull;  // bits(100000.f), PointRenderer.cu:1045
 

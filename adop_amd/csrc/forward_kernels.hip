@@ -5,9 +5,10 @@
 // one transaction.  Hence:
 //   * the blend accumulates into a pixel-major workspace array (S floats per pixel: C sums + the weight, padded to
 //     a power of two), so the C+1 adds of one point-level are ONE transaction instead of C+1;
-//   * every workgroup first merges its point-levels per pixel in an LDS hash table (ds_add_f32 / ds_min_u64) and
-//     flushes each distinct pixel once; clouds stored in Morton-ordered 256-point blocks (the reference's
-//     preprocessing order) collide heavily at the coarse levels.
+//   * every wavefront first merges its point-levels per pixel (ballot grouping + plain LDS reads, no LDS atomics:
+//     an LDS hash table with ds_add_f32 / ds_cmpst was measured to be latency-bound at ~370 cycles per LDS
+//     instruction) and issues one transaction per distinct pixel; clouds stored in Morton-ordered 256-point blocks
+//     (the reference's preprocessing order) collide heavily at the coarse levels.
 #include "common.h"
 #include "launch.h"
 
@@ -51,16 +52,6 @@ __global__ __launch_bounds__(kBlock) void clear_kernel(Levels lv, float4* __rest
     for (size_t t = t0; t < accum_vec4; t += stride) accum[t] = z;
 }
 
-__device__ __forceinline__ uint64_t* depth_index_ptr(const Levels& lv, int l)
-{
-    uint64_t* p = lv.l[0].depth_index;
-    if (l == 1) p = lv.l[1].depth_index;
-    if (l == 2) p = lv.l[2].depth_index;
-    if (l == 3) p = lv.l[3].depth_index;
-    if (l == 4) p = lv.l[4].depth_index;
-    return p;
-}
-
 __device__ __forceinline__ void depth_min_global(uint64_t* dst, uint64_t pk)
 {
     // early-z (PointRenderer.cu:278): a stale value only costs a redundant atomic
@@ -68,19 +59,56 @@ __device__ __forceinline__ void depth_min_global(uint64_t* dst, uint64_t pk)
     if (pk < cur) atomicMin((unsigned long long*)dst, (unsigned long long)pk);
 }
 
+// LDS written by some lanes of a wavefront is read by other lanes of the same wavefront: DS operations of one
+// wavefront execute in order, so only the compiler has to be kept from moving accesses across this point.
+__device__ __forceinline__ void wave_lds_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Groups the lanes of a wavefront by key.  Lanes with active == false are ignored.  For every distinct key, in
+// order of its first lane, writes gkey[g] and the 64-bit lane mask gmask[g]; returns the number of groups.
+// (gfx950 has no match-any instruction: one ballot per distinct key.)
+__device__ __forceinline__ int wave_group_by_key(bool active, uint32_t key, uint32_t* gkey, unsigned long long* gmask)
+{
+    const int lane                 = threadIdx.x & 63;
+    unsigned long long remaining = __ballot(active);
+    int g                          = 0;
+    while (remaining)
+    {
+        int leader            = __ffsll((long long)remaining) - 1;
+        uint32_t k            = (uint32_t)__builtin_amdgcn_readlane((int)key, leader);
+        unsigned long long m = __ballot(active && key == k);
+        if (lane == leader)
+        {
+            gkey[g]  = k;
+            gmask[g] = m;
+        }
+        remaining &= ~m;
+        ++g;
+    }
+    return g;
+}
+
 // DepthPrepassMulti (PointRenderer.cu:203-301) on the packed buffer the reference keeps as "old rendering"
 // (LayerCuda::depth_index_tensor, PackIndex): min over (depth bits << 32 | point id).
-// Key of the LDS table: level << 28 | pixel.
-template <int BITS>
+// Per level every wavefront groups its lanes by pixel, one lane per distinct pixel takes the minimum of the group
+// from LDS and issues the (early-z guarded) 64-bit atomicMin: clouds stored in Morton-ordered blocks collide heavily
+// at the coarse levels, and a device-scope atomic costs one memory transaction whatever it carries.
 __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const ViewConst* __restrict__ views, Levels lv,
                                                          ParamArg rp, adop_stats* stats)
 {
-    constexpr int T = 1 << BITS;
-    __shared__ uint32_t keys[T];
-    __shared__ unsigned long long mins[T];
-    __shared__ uint16_t used[T];
-    __shared__ uint32_t used_count;
+    __shared__ unsigned long long s_pk[kBlock];
+    __shared__ unsigned long long s_gmask[kBlock];
+    __shared__ uint32_t s_gkey[kBlock];
     const bool STATS = stats != nullptr;  // counter pass (uniform branch)
+    const int lane   = threadIdx.x & 63;
+    const int wbase  = threadIdx.x & ~63;
+    unsigned long long* pk_w    = s_pk + wbase;
+    unsigned long long* gmask_w = s_gmask + wbase;
+    uint32_t* gkey_w            = s_gkey + wbase;
 
     int i      = blockIdx.x * kBlock + threadIdx.x;
     bool valid = i < pc.n;
@@ -91,83 +119,107 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
 
     for (int b = 0; b < lv.B; ++b)
     {
-        for (int k = threadIdx.x; k < T; k += kBlock)
-        {
-            keys[k] = kEmptyKey;
-            mins[k] = ~0ull;
-        }
-        if (threadIdx.x == 0) used_count = 0;
-        __syncthreads();
-
         const ViewConst& vc = views[b];
         V2 ip;
         V3 view_p;
         float z, radius_pixels;
         bool ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff,
                                          lv.l[0].w, &ip, &z, &radius_pixels, &view_p);
-        bool alive = ok;
-        if (STATS || ok)
+        if (!__ballot(ok) && !STATS) continue;  // wavefront-uniform
+        const uint64_t pk = ((uint64_t)f2u(z) << 32) | (uint32_t)i;
+
+        // phase 1: pixel of every level and the early-z read (PointRenderer.cu:278); the loads are independent.
+        // A stale value only costs a redundant atomic.
+        uint32_t pix[ADOP_MAX_LAYERS];
+        bool cand[ADOP_MAX_LAYERS];
         {
+            uint64_t cur[ADOP_MAX_LAYERS];
+            bool in[ADOP_MAX_LAYERS];
+            bool alive = ok;
 #pragma unroll
             for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
             {
-                if (l >= lv.num) break;
-                if (rp.drop_by_radius && radius_pixels < rp.drop_threshold) alive = false;  // break, :261-264
-                const LevelArg& L = lv.l[l];
-                int px = f2i_rn(ip.x), py = f2i_rn(ip.y);
-                bool in = alive && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h;
-                if (STATS) stat_add(&stats->visible[l], in);
-                if (in)
+                in[l]  = false;
+                pix[l] = 0;
+                cur[l] = 0;
+                if (l < lv.num)
                 {
-                    uint64_t pk  = ((uint64_t)f2u(z) << 32) | (uint32_t)i;
-                    uint32_t pix = (uint32_t)py * (uint32_t)L.w + (uint32_t)px;
-                    int slot     = table_insert<BITS>(keys, used, &used_count, ((uint32_t)l << 28) | pix);
-                    if (slot >= 0)
-                        atomicMin(&mins[slot], (unsigned long long)pk);
-                    else
-                        depth_min_global(L.depth_index + (size_t)b * L.w * L.h + pix, pk);
+                    if (rp.drop_by_radius && radius_pixels < rp.drop_threshold) alive = false;  // break, :261-264
+                    const LevelArg& L = lv.l[l];
+                    int px = f2i_rn(ip.x), py = f2i_rn(ip.y);
+                    in[l] = alive && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h;
+                    if (STATS) stat_add(&stats->visible[l], in[l]);
+                    if (in[l])
+                    {
+                        pix[l] = (uint32_t)py * (uint32_t)L.w + (uint32_t)px;
+                        cur[l] = __builtin_nontemporal_load(L.depth_index + (size_t)b * L.w * L.h + pix[l]);
+                    }
+                    radius_pixels *= 0.5f;
+                    ip.x *= 0.5f;
+                    ip.y *= 0.5f;
                 }
-                radius_pixels *= 0.5f;
-                ip.x *= 0.5f;
-                ip.y *= 0.5f;
+            }
+#pragma unroll
+            for (int l = 0; l < ADOP_MAX_LAYERS; ++l) cand[l] = in[l] && pk < cur[l];
+        }
+        bool any = false;
+#pragma unroll
+        for (int l = 0; l < ADOP_MAX_LAYERS; ++l) any |= cand[l];
+        if (!__ballot(any)) continue;  // wavefront-uniform
+        wave_lds_sync();               // previous view's readers are done
+        pk_w[lane] = pk;
+
+        // phase 2: per level, the surviving lanes are grouped by pixel; one atomicMin per distinct pixel
+#pragma unroll
+        for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+        {
+            if (l >= lv.num) break;
+            if (!__ballot(cand[l])) continue;
+            const LevelArg& L = lv.l[l];
+            wave_lds_sync();
+            int G = wave_group_by_key(cand[l], pix[l], gkey_w, gmask_w);
+            wave_lds_sync();
+            if (lane < G)
+            {
+                unsigned long long m  = gmask_w[lane];
+                unsigned long long mn = ~0ull;
+                while (m)
+                {
+                    int bit = __ffsll((long long)m) - 1;
+                    m &= m - 1;
+                    unsigned long long v = pk_w[bit];
+                    mn                   = v < mn ? v : mn;
+                }
+                atomicMin((unsigned long long*)(L.depth_index + (size_t)b * L.w * L.h + gkey_w[lane]), mn);
             }
         }
-        __syncthreads();
-        uint32_t n = used_count;
-        for (uint32_t e = threadIdx.x; e < n; e += kBlock)
-        {
-            uint32_t slot = used[e];
-            uint32_t key  = keys[slot];
-            int l         = (int)(key >> 28);
-            uint32_t pix  = key & 0x0FFFFFFFu;
-            size_t hw     = (size_t)lv.l[0].w * lv.l[0].h;
-            if (l == 1) hw = (size_t)lv.l[1].w * lv.l[1].h;
-            if (l == 2) hw = (size_t)lv.l[2].w * lv.l[2].h;
-            if (l == 3) hw = (size_t)lv.l[3].w * lv.l[3].h;
-            if (l == 4) hw = (size_t)lv.l[4].w * lv.l[4].h;
-            depth_min_global(depth_index_ptr(lv, l) + (size_t)b * hw + pix, (uint64_t)mins[slot]);
-        }
-        __syncthreads();
     }
 }
 
 // RenderForwardMulti (PointRenderer.cu:303-393).  CT = compile-time channel count (0: runtime lv.C <= 16).
-// Key of the LDS table: workspace pixel index (ws_pixel).  accum: S floats per workspace pixel.
-template <int CT, int BITS, bool HALF>
+// accum: S floats per workspace pixel (C sums + weight, padded to a power of two).
+// Per level every wavefront groups its accepted lanes by pixel; LG = max(S,8) consecutive lanes then sum the
+// staged descriptors of one group (lane j = channel j, lane C = the count) and add them with ONE cache-line atomic.
+template <int CT, bool HALF>
 __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewConst* __restrict__ views, Levels lv,
                                                        ParamArg rp, float* __restrict__ accum, int S,
                                                        adop_stats* stats)
 {
-    constexpr int T    = 1 << BITS;
     constexpr int CMAX = CT ? CT : kMaxChannels;
-    __shared__ uint32_t keys[T];
-    __shared__ uint16_t used[T];
-    __shared__ uint32_t used_count;
-    extern __shared__ float vals[];  // T * (C+1)
+    __shared__ unsigned long long s_gmask[kBlock];
+    __shared__ uint32_t s_gkey[kBlock];
+    extern __shared__ float s_stage[];  // kBlock * C descriptors of the block's points
     const bool STATS = stats != nullptr;  // counter pass (uniform branch)
-
-    const int C  = CT ? CT : lv.C;
-    const int C1 = C + 1;
+    const int C      = CT ? CT : lv.C;
+    const int lane   = threadIdx.x & 63;
+    const int wbase  = threadIdx.x & ~63;
+    unsigned long long* gmask_w = s_gmask + wbase;
+    uint32_t* gkey_w            = s_gkey + wbase;
+    float* stage_w              = s_stage + wbase * C;
+    const int LG                = S < 8 ? 8 : S;  // lanes per group in the accumulate phase
+    const int sub               = lane / LG;
+    const int j                 = lane - sub * LG;
+    const int subs              = 64 / LG;
 
     int i      = blockIdx.x * kBlock + threadIdx.x;
     bool valid = i < pc.n;
@@ -178,17 +230,10 @@ __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewCo
     int tex_index = valid ? pc.index[i] : 0;
     bool tex_ok   = (unsigned)tex_index < (unsigned)pc.num_texels;  // device assert :362
     const float accept = rp.depth_accept + 1;
-
-    float t[CMAX];
-    bool t_loaded = false;
+    bool staged = false;
 
     for (int b = 0; b < lv.B; ++b)
     {
-        for (int k = threadIdx.x; k < T; k += kBlock) keys[k] = kEmptyKey;
-        for (int k = threadIdx.x; k < T * C1; k += kBlock) vals[k] = 0.f;
-        if (threadIdx.x == 0) used_count = 0;
-        __syncthreads();
-
         bool dropped = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;  // :314-315
         const ViewConst& vc = views[b];
         V2 ip;
@@ -198,74 +243,93 @@ __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewCo
                   project_point(vc, pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff, lv.l[0].w, &ip,
                                 &z, &radius_pixels, &view_p);
         if (STATS) stat_add(&stats->bad_index, ok && !tex_ok);
-        ok         = ok && tex_ok;
-        bool alive = ok;
-        if (STATS || ok)
+        ok = ok && tex_ok;
+        if (!__ballot(ok) && !STATS) continue;  // wavefront-uniform
+
+        // phase 1: pixel of every level and the depth test (all depth loads are independent)
+        uint32_t gp[ADOP_MAX_LAYERS];
+        bool acc[ADOP_MAX_LAYERS];
         {
+            uint32_t dw[ADOP_MAX_LAYERS];
+            bool in[ADOP_MAX_LAYERS];
+            bool alive = ok;
 #pragma unroll
             for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
             {
-                if (l >= lv.num) break;
-                if (rp.drop_by_radius && radius_pixels < rp.drop_threshold) alive = false;
-                const LevelArg& L = lv.l[l];
-                int px = f2i_rn(ip.x), py = f2i_rn(ip.y);
-                bool in  = alive && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h;
-                bool acc = false;
-                if (in)
+                in[l] = false;
+                gp[l] = 0;
+                dw[l] = 0;
+                if (l < lv.num)
                 {
-                    size_t hw    = (size_t)L.w * L.h;
-                    uint32_t pix = (uint32_t)py * (uint32_t)L.w + (uint32_t)px;
-                    // high word of the packed pixel = depth
-                    float image_depth = __uint_as_float((uint32_t)(L.depth_index[(size_t)b * hw + pix] >> 32));
-                    acc               = !(z > image_depth * accept);  // :380
-                    if (acc)
+                    if (rp.drop_by_radius && radius_pixels < rp.drop_threshold) alive = false;
+                    const LevelArg& L = lv.l[l];
+                    int px = f2i_rn(ip.x), py = f2i_rn(ip.y);
+                    in[l] = alive && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h;
+                    if (in[l])
                     {
-                        if (!t_loaded)
-                        {
-#pragma unroll
-                            for (int c = 0; c < CMAX; ++c)
-                                if (c < C) t[c] = tex_fetch<HALF>(pc.texture, (size_t)c * pc.num_texels + tex_index);
-                            t_loaded = true;
-                        }
-                        uint32_t gp = ws_pixel(lv, l, b, pix);
-                        int slot    = table_insert<BITS>(keys, used, &used_count, gp);
-                        if (slot >= 0)
-                        {
-                            float* v = vals + slot * C1;
-#pragma unroll
-                            for (int c = 0; c < CMAX; ++c)
-                                if (c < C) atomicAdd(v + c, t[c]);
-                            atomicAdd(v + C, 1.f);
-                        }
-                        else
-                        {
-                            float* g = accum + (size_t)gp * S;
-#pragma unroll
-                            for (int c = 0; c < CMAX; ++c)
-                                if (c < C) unsafeAtomicAdd(g + c, t[c]);
-                            unsafeAtomicAdd(g + C, 1.f);
-                        }
+                        uint32_t pix = (uint32_t)py * (uint32_t)L.w + (uint32_t)px;
+                        size_t o     = (size_t)b * L.w * L.h + pix;
+                        dw[l]        = ((const uint32_t*)L.depth_index)[2 * o + 1];  // high word = depth bits
+                        gp[l]        = ws_pixel(lv, l, b, pix);
                     }
+                    radius_pixels *= 0.5f;
+                    ip.x *= 0.5f;
+                    ip.y *= 0.5f;
                 }
-                if (STATS) stat_add(&stats->accepted[l], acc);
-                radius_pixels *= 0.5f;
-                ip.x *= 0.5f;
-                ip.y *= 0.5f;
+            }
+#pragma unroll
+            for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+            {
+                acc[l] = in[l] && !(z > __uint_as_float(dw[l]) * accept);  // :380
+                if (STATS && l < lv.num) stat_add(&stats->accepted[l], acc[l]);
             }
         }
-        __syncthreads();
-        // flush: S consecutive lanes add the C+1 sums of one pixel into one cache line
-        uint32_t n    = used_count;
-        int lane      = threadIdx.x % S;
-        int group     = threadIdx.x / S;
-        int groups    = kBlock / S;
-        for (uint32_t e = group; e < n; e += groups)
+        bool any = false;
+#pragma unroll
+        for (int l = 0; l < ADOP_MAX_LAYERS; ++l) any |= acc[l];
+        if (!__ballot(any)) continue;  // wavefront-uniform
+
+        // phase 2: stage the descriptors of this point (the same for every level and view)
+        if (any && !staged)
         {
-            uint32_t slot = used[e];
-            uint32_t gp   = keys[slot];
-            if (lane < C1) unsafeAtomicAdd(accum + (size_t)gp * S + lane, vals[slot * C1 + lane]);
+#pragma unroll
+            for (int c = 0; c < CMAX; ++c)
+                if (c < C) stage_w[lane * C + c] = tex_fetch<HALF>(pc.texture, (size_t)c * pc.num_texels + tex_index);
+            staged = true;
         }
-        __syncthreads();
+
+        // phase 3: per level, one cache-line atomic per distinct pixel of the wavefront
+#pragma unroll
+        for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+        {
+            if (l >= lv.num) break;
+            if (!__ballot(acc[l])) continue;
+            wave_lds_sync();
+            int G = wave_group_by_key(acc[l], gp[l], gkey_w, gmask_w);
+            wave_lds_sync();
+            for (int g0 = 0; g0 < G; g0 += subs)
+            {
+                int g = g0 + sub;
+                if (g < G && j <= C)
+                {
+                    unsigned long long m = gmask_w[g];
+                    float sum;
+                    if (j < C)
+                    {
+                        sum = 0.f;
+                        while (m)
+                        {
+                            int bit = __ffsll((long long)m) - 1;
+                            m &= m - 1;
+                            sum += stage_w[bit * C + j];
+                        }
+                    }
+                    else
+                        sum = (float)__popcll(m);
+                    unsafeAtomicAdd(accum + (size_t)gkey_w[g] * S + j, sum);
+                }
+            }
+        }
     }
 }
 
@@ -328,9 +392,6 @@ __global__ __launch_bounds__(kBlock) void resolve_kernel(Levels lv, const float*
 // ------------------------------------------------------------------------------------------------
 // launchers
 // ------------------------------------------------------------------------------------------------
-constexpr int kPrepassBits = 10;  // LDS table of the prepass: 1024 slots x 14 B
-constexpr int kBlendBits   = 9;   // LDS table of the blend: 512 slots x (6 + 4(C+1)) B
-
 void launch_prepare_views(const ViewChunk& ch, int first, int count, const double* poses, const float* intrinsics,
                           int cols, ViewConst* out, hipStream_t st)
 {
@@ -354,7 +415,7 @@ void launch_prepass(const CloudArg& pc, const ViewConst* views, const Levels& lv
 {
     int grid = (pc.n + kBlock - 1) / kBlock;
     if (grid < 1) return;
-    hipLaunchKernelGGL((prepass_kernel<kPrepassBits>), dim3(grid), dim3(kBlock), 0, st, pc, views, lv, rp, stats);
+    hipLaunchKernelGGL(prepass_kernel, dim3(grid), dim3(kBlock), 0, st, pc, views, lv, rp, stats);
 }
 
 template <int CT, bool HALF>
@@ -362,8 +423,8 @@ static void launch_blend_t(const CloudArg& pc, const ViewConst* views, const Lev
                            float* accum, int S, adop_stats* stats, hipStream_t st)
 {
     int grid   = (pc.n + kBlock - 1) / kBlock;
-    size_t lds = sizeof(float) * ((size_t)1 << kBlendBits) * (size_t)(lv.C + 1);
-    hipLaunchKernelGGL((blend_kernel<CT, kBlendBits, HALF>), dim3(grid), dim3(kBlock), lds, st, pc, views, lv, rp,
+    size_t lds = sizeof(float) * (size_t)kBlock * (size_t)lv.C;
+    hipLaunchKernelGGL((blend_kernel<CT, HALF>), dim3(grid), dim3(kBlock), lds, st, pc, views, lv, rp,
                        accum, S, stats);
 }
 

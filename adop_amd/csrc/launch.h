@@ -23,9 +23,19 @@ void launch_resolve(const Levels& lv, int grid, const float* accum, int S, const
                     float mask_value, hipStream_t st);
 
 void launch_interleave(const Levels& lv, int blocks, float* ig, double* partial, hipStream_t st);
+// Work queue of the backward pass (points that receive a ghost / spatial gradient), split in kNumQueues sub-queues
+// of `cap` items each.
+struct QueueArg
+{
+    uint32_t* counts;           // [kNumQueues]
+    uint32_t* prefix;           // [kNumQueues + 1]
+    unsigned long long* items;  // [kNumQueues * cap]
+    uint32_t cap;
+};
 void launch_render_backward(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
-                            const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr, int b,
-                            int blocks, double* partial, adop_stats* stats, hipStream_t st);
+                            const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr,
+                            int identity_index, int b, int first_view, const QueueArg& q, int ghost_blocks,
+                            double* partial, adop_stats* stats, hipStream_t st);
 void launch_finalize(const ViewConst* views, int B, int C, const double* bg_partial, int bg_blocks,
                      const double* pt_partial, int pt_blocks, const adop_backward_buffers* g, int num_poses,
                      int num_cameras, int cols, int normalize_mode, double* scratch, hipStream_t st);

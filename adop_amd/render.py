@@ -44,6 +44,15 @@ class NeuralPointCloud:
         self.t_index = torch.as_tensor(index, dtype=torch.int32).to(device).reshape(-1, 1).contiguous()
         assert self.t_position.dim() == 2 and self.t_position.shape[1] == 4
         assert self.t_index.shape[0] == self.t_position.shape[0]
+        self._index_is_identity = None
+
+    def index_is_identity(self):
+        """True if t_index[i] == i for all i (how the reference builds it); evaluated once and cached."""
+        if self._index_is_identity is None:
+            n = self.Size()
+            ar = torch.arange(n, dtype=torch.int32, device=self.t_index.device)
+            self._index_is_identity = bool((self.t_index.view(-1) == ar).all().item())
+        return self._index_is_identity
 
     def Size(self):
         return int(self.t_position.shape[0])
@@ -88,6 +97,7 @@ class NeuralScene:
         s.intrinsics = _ptr(self.intrinsics)
         s.num_cameras = int(self.intrinsics.shape[0])
         s.intrinsics_cols = int(self.intrinsics.shape[1])
+        s.index_is_identity = 1 if (pc.index_is_identity() and s.num_texels == s.num_points) else 0
         return s
 
 

@@ -102,6 +102,10 @@ typedef struct adop_scene
     const float* intrinsics; /* [K,intrinsics_cols] */
     int32_t num_cameras;
     int32_t intrinsics_cols;
+    /* Caller's promise that index[i] == i for every point and num_texels == num_points (how the reference
+     * builds t_index, NeuralPointCloud.h:31).  Lets the backward write grad_texture with plain coalesced stores
+     * instead of atomics.  0 = make no assumption. */
+    int32_t index_is_identity;
 } adop_scene;
 
 /* struct LayerCuda (PointRenderer.h:65-94) plus the per-level output tensors of PointRendererCache

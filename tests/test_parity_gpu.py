@@ -109,6 +109,20 @@ def test_distortion_crop_lod_mask(oracle_mod):
     _fwd_bwd(hs, oracle_mod)
 
 
+def test_shared_texels_use_the_atomic_path(oracle_mod):
+    """index is not the identity: two points share a texel, a permutation for the rest."""
+    from adop_amd import scenes
+
+    announce("shared texels / permuted index (atomic descriptor-gradient path), C=8 and C=3")
+    for channels in (8, 3):
+        hs = scenes.config3(n=200_000, w=320, h=180, channels=channels)
+        n = hs.num_points
+        idx = np.random.default_rng(5).permutation(n).astype(np.int32) // 2
+        hs.index = idx
+        hs.texture = np.ascontiguousarray(hs.texture[:, : n // 2 + 1])
+        _fwd_bwd(hs, oracle_mod)
+
+
 def test_ocam_forward_backward(oracle_mod):
     from adop_amd import scenes
 
