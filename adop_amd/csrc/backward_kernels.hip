@@ -157,6 +157,7 @@ __global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const
     bool in[ADOP_MAX_LAYERS];
     bool edge_ok[ADOP_MAX_LAYERS];
     float dep[ADOP_MAX_LAYERS];
+    float wgt[ADOP_MAX_LAYERS];
 #pragma unroll
     for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
     {
@@ -164,6 +165,7 @@ __global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const
         edge_ok[l] = false;
         pix[l]     = 0;
         dep[l]     = 0.f;
+        wgt[l]     = 0.f;
         if (l < lv.num)
         {
             const LevelArg& L = lv.l[l];
@@ -174,6 +176,7 @@ __global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const
             {
                 pix[l]     = (uint32_t)py * (uint32_t)L.w + (uint32_t)px;
                 dep[l]     = L.depth[(size_t)b * L.w * L.h + pix[l]];
+                wgt[l]     = L.weight[(size_t)b * L.w * L.h + pix[l]];  // same round trip as the depth
                 int ex     = min(px, L.w - 1 - px);
                 int ey     = min(py, L.h - 1 - py);
                 edge_ok[l] = min(ex, ey) > 2;  // distanceFromEdge > 2, :489
@@ -183,16 +186,14 @@ __global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const
             ip.y *= 0.5f;
         }
     }
-    // phase 2: depth test in level order, `break` at the first failure (:462); weight loads
+    // phase 2: depth test in level order, `break` at the first failure (:462)
     bool pass[ADOP_MAX_LAYERS];
-    float wgt[ADOP_MAX_LAYERS];
     {
         bool alive = true;
 #pragma unroll
         for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
         {
             pass[l] = false;
-            wgt[l]  = 0.f;
             if (in[l] && alive)
             {
                 if (z > dep[l] * accept)
@@ -200,7 +201,6 @@ __global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const
                 else
                     pass[l] = true;
             }
-            if (pass[l]) wgt[l] = lv.l[l].weight[(size_t)b * lv.l[l].w * lv.l[l].h + pix[l]];
         }
     }
     // phase 3: descriptor gradient of the rendered (not dropped) points; spatial-gradient eligibility
@@ -542,19 +542,21 @@ __global__ __launch_bounds__(kBlock) void finalize_kernel(const ViewConst* __res
                                                           double* __restrict__ scratch)
 {
     __shared__ double sh[kBlock];
-    // background
-    for (int c = 0; c < C; ++c)
+    // background: thread t sums channel t%16 over the partial rows t/16, t/16+16, ...
     {
+        const int c = threadIdx.x % kMaxChannels, k0 = threadIdx.x / kMaxChannels;
+        constexpr int GR = kBlock / kMaxChannels;
         double v = 0;
-        for (int k = threadIdx.x; k < bg_blocks; k += kBlock) v += bg_partial[(size_t)k * kMaxChannels + c];
+#pragma unroll 16
+        for (int k = k0; k < bg_blocks; k += GR) v += bg_partial[(size_t)k * kMaxChannels + c];
         sh[threadIdx.x] = v;
         __syncthreads();
-        for (int s = kBlock / 2; s > 0; s >>= 1)
+        if (threadIdx.x < kMaxChannels)
         {
-            if (threadIdx.x < s) sh[threadIdx.x] += sh[threadIdx.x + s];
-            __syncthreads();
+            double t = 0;
+            for (int g = 0; g < GR; ++g) t += sh[g * kMaxChannels + threadIdx.x];
+            if ((int)threadIdx.x < C) gbg[threadIdx.x] = (float)t;
         }
-        if (threadIdx.x == 0) gbg[c] = (float)sh[0];
         __syncthreads();
     }
     if (!gpose && !gintr) return;
@@ -566,33 +568,32 @@ __global__ __launch_bounds__(kBlock) void finalize_kernel(const ViewConst* __res
     __syncthreads();
     for (int b = 0; b < B; ++b)
     {
-        for (int q = 0; q < 21; ++q)
+        // thread t sums value t%32 (21 used) over the partial rows t/32, t/32+8, ...
+        const int q = threadIdx.x % 32, k0 = threadIdx.x / 32;
+        constexpr int GR = kBlock / 32;
+        double v = 0;
+        if (q < kAcc)
+#pragma unroll 16
+            for (int k = k0; k < pt_blocks; k += GR) v += pt_partial[((size_t)b * pt_blocks + k) * kPartialStride + q];
+        sh[threadIdx.x] = v;
+        __syncthreads();
+        if (threadIdx.x < kAcc)
         {
-            double v = 0;
-            for (int k = threadIdx.x; k < pt_blocks; k += kBlock)
-                v += pt_partial[((size_t)b * pt_blocks + k) * kPartialStride + q];
-            sh[threadIdx.x] = v;
-            __syncthreads();
-            for (int s = kBlock / 2; s > 0; s >>= 1)
-            {
-                if (threadIdx.x < s) sh[threadIdx.x] += sh[threadIdx.x + s];
-                __syncthreads();
-            }
-            if (threadIdx.x == 0)
-            {
-                const ViewConst& vc = views[b];
-                double t            = sh[0];
-                if (q < 6)
-                    sp[(size_t)vc.image_index * 7 + q] += t;
-                else if (q == 6)
-                    sp[(size_t)vc.image_index * 7 + 6] += t;
-                else if (q == 7)
-                    si[(size_t)vc.camera_index * (cols + 1) + cols] += t;
-                else if (q - 8 < cols)
-                    si[(size_t)vc.camera_index * (cols + 1) + (q - 8)] += t;
-            }
-            __syncthreads();
+            double t = 0;
+            for (int g = 0; g < GR; ++g) t += sh[g * 32 + threadIdx.x];
+            const ViewConst& vc = views[b];
+            const int qq        = threadIdx.x;
+            // distinct threads write distinct addresses; views are processed one after another
+            if (qq < 6)
+                sp[(size_t)vc.image_index * 7 + qq] += t;
+            else if (qq == 6)
+                sp[(size_t)vc.image_index * 7 + 6] += t;
+            else if (qq == 7)
+                si[(size_t)vc.camera_index * (cols + 1) + cols] += t;
+            else if (qq - 8 < cols)
+                si[(size_t)vc.camera_index * (cols + 1) + (qq - 8)] += t;
         }
+        __syncthreads();
     }
     if (gpose)
     {

@@ -13,7 +13,7 @@ namespace adop
 {
 constexpr int kBlock         = 256;
 constexpr int kMaxChannels   = 16;
-constexpr int kPartialBlocks = 2048;  // grid of the grid-stride kernels that write per-block partial sums
+constexpr int kPartialBlocks = 1024;  // grid of the grid-stride kernels that write per-block partial sums
 constexpr int kPartialStride = 24;    // doubles per (block, view), 21 used: 6 pose, pose count, intr count, 13 intr
 constexpr int kAcc           = 21;
 constexpr int kNumQueues     = 2048;  // sub-queues of the backward work queue (multiple of kBlock)

@@ -6,9 +6,11 @@
 //   * the blend accumulates into a pixel-major workspace array (S floats per pixel: C sums + the weight, padded to
 //     a power of two), so the C+1 adds of one point-level are ONE transaction instead of C+1;
 //   * every wavefront first merges its point-levels per pixel (ballot grouping + plain LDS reads, no LDS atomics:
-//     an LDS hash table with ds_add_f32 / ds_cmpst was measured to be latency-bound at ~370 cycles per LDS
-//     instruction) and issues one transaction per distinct pixel; clouds stored in Morton-ordered 256-point blocks
+//     two variants built on ds_add_f32 / ds_cmpst - a workgroup hash table and a per-wavefront leader election -
+//     were measured 1.8-2.2x slower) and issues one transaction per distinct pixel; clouds stored in Morton-ordered 256-point blocks
 //     (the reference's preprocessing order) collide heavily at the coarse levels.
+#include <stdlib.h>
+
 #include "common.h"
 #include "launch.h"
 
@@ -94,11 +96,14 @@ __device__ __forceinline__ int wave_group_by_key(bool active, uint32_t key, uint
 
 // DepthPrepassMulti (PointRenderer.cu:203-301) on the packed buffer the reference keeps as "old rendering"
 // (LayerCuda::depth_index_tensor, PackIndex): min over (depth bits << 32 | point id).
-// Per level every wavefront groups its lanes by pixel, one lane per distinct pixel takes the minimum of the group
-// from LDS and issues the (early-z guarded) 64-bit atomicMin: clouds stored in Morton-ordered blocks collide heavily
-// at the coarse levels, and a device-scope atomic costs one memory transaction whatever it carries.
+// Every thread handles PPT points (all their loads are issued before anything waits: the kernel is bound by memory
+// latency, not by arithmetic).  Per level and 64-point run the lanes that survive the early-z read are grouped by
+// pixel, one lane per distinct pixel takes the minimum of its group from LDS and issues the 64-bit atomicMin:
+// clouds stored in Morton-ordered blocks collide heavily at the coarse levels, and a device-scope atomic costs one
+// memory transaction whatever it carries.
+template <int PPT>
 __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const ViewConst* __restrict__ views, Levels lv,
-                                                         ParamArg rp, adop_stats* stats)
+                                                         ParamArg rp, int group_from, adop_stats* stats)
 {
     __shared__ unsigned long long s_pk[kBlock];
     __shared__ unsigned long long s_gmask[kBlock];
@@ -110,87 +115,109 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
     unsigned long long* gmask_w = s_gmask + wbase;
     uint32_t* gkey_w            = s_gkey + wbase;
 
-    int i      = blockIdx.x * kBlock + threadIdx.x;
-    bool valid = i < pc.n;
-    float4 P   = valid ? pc.position[i] : make_float4(0, 0, 0, 0);
-    V3 pos     = {P.x, P.y, P.z};
-    V3 nrm     = {0, 0, 0};
-    if (valid && pc.normal) nrm = unpack_normal10(pc.normal[i]);
+    const int base = blockIdx.x * (kBlock * PPT) + threadIdx.x;
+    float4 P[PPT];
+    int32_t nenc[PPT];
+#pragma unroll
+    for (int k = 0; k < PPT; ++k)
+    {
+        int i   = base + k * kBlock;
+        P[k]    = i < pc.n ? pc.position[i] : make_float4(0, 0, 0, 0);
+        nenc[k] = (i < pc.n && pc.normal) ? pc.normal[i] : 0;
+    }
 
     for (int b = 0; b < lv.B; ++b)
     {
         const ViewConst& vc = views[b];
-        V2 ip;
-        V3 view_p;
-        float z, radius_pixels;
-        bool ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff,
-                                         lv.l[0].w, &ip, &z, &radius_pixels, &view_p);
-        if (!__ballot(ok) && !STATS) continue;  // wavefront-uniform
-        const uint64_t pk = ((uint64_t)f2u(z) << 32) | (uint32_t)i;
-
-        // phase 1: pixel of every level and the early-z read (PointRenderer.cu:278); the loads are independent.
-        // A stale value only costs a redundant atomic.
-        uint32_t pix[ADOP_MAX_LAYERS];
-        bool cand[ADOP_MAX_LAYERS];
+        // phase 1: projection, pixel of every level and the early-z read (PointRenderer.cu:278) of the depth word;
+        // the loads are independent.  A stale value only costs a redundant atomic.
+        uint32_t pix[PPT][ADOP_MAX_LAYERS];
+        uint32_t cur[PPT][ADOP_MAX_LAYERS];
+        uint32_t inmask[PPT];
+        float zz[PPT];
+#pragma unroll
+        for (int k = 0; k < PPT; ++k)
         {
-            uint64_t cur[ADOP_MAX_LAYERS];
-            bool in[ADOP_MAX_LAYERS];
+            int i      = base + k * kBlock;
+            bool valid = i < pc.n;
+            V3 pos     = {P[k].x, P[k].y, P[k].z};
+            V3 nrm     = unpack_normal10(nenc[k]);
+            V2 ip;
+            V3 view_p;
+            float z, radius_pixels;
+            bool ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P[k].w, rp.check_normal != 0, rp.dist_cutoff,
+                                             lv.l[0].w, &ip, &z, &radius_pixels, &view_p);
+            zz[k]      = z;
+            inmask[k]  = 0;
             bool alive = ok;
 #pragma unroll
             for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
             {
-                in[l]  = false;
-                pix[l] = 0;
-                cur[l] = 0;
+                pix[k][l] = 0;
+                cur[k][l] = 0;
                 if (l < lv.num)
                 {
                     if (rp.drop_by_radius && radius_pixels < rp.drop_threshold) alive = false;  // break, :261-264
                     const LevelArg& L = lv.l[l];
                     int px = f2i_rn(ip.x), py = f2i_rn(ip.y);
-                    in[l] = alive && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h;
-                    if (STATS) stat_add(&stats->visible[l], in[l]);
-                    if (in[l])
+                    bool in = alive && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h;
+                    if (STATS) stat_add(&stats->visible[l], in);
+                    if (in)
                     {
-                        pix[l] = (uint32_t)py * (uint32_t)L.w + (uint32_t)px;
-                        cur[l] = __builtin_nontemporal_load(L.depth_index + (size_t)b * L.w * L.h + pix[l]);
+                        inmask[k] |= 1u << l;
+                        pix[k][l] = (uint32_t)py * (uint32_t)L.w + (uint32_t)px;
+                        size_t o  = (size_t)b * L.w * L.h + pix[k][l];
+                        cur[k][l] = __builtin_nontemporal_load((const uint32_t*)L.depth_index + 2 * o + 1);
                     }
                     radius_pixels *= 0.5f;
                     ip.x *= 0.5f;
                     ip.y *= 0.5f;
                 }
             }
-#pragma unroll
-            for (int l = 0; l < ADOP_MAX_LAYERS; ++l) cand[l] = in[l] && pk < cur[l];
         }
-        bool any = false;
+        // phase 2: per 64-point run and level, the surviving lanes are grouped by pixel; one atomicMin per group
 #pragma unroll
-        for (int l = 0; l < ADOP_MAX_LAYERS; ++l) any |= cand[l];
-        if (!__ballot(any)) continue;  // wavefront-uniform
-        wave_lds_sync();               // previous view's readers are done
-        pk_w[lane] = pk;
-
-        // phase 2: per level, the surviving lanes are grouped by pixel; one atomicMin per distinct pixel
-#pragma unroll
-        for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+        for (int k = 0; k < PPT; ++k)
         {
-            if (l >= lv.num) break;
-            if (!__ballot(cand[l])) continue;
-            const LevelArg& L = lv.l[l];
-            wave_lds_sync();
-            int G = wave_group_by_key(cand[l], pix[l], gkey_w, gmask_w);
-            wave_lds_sync();
-            if (lane < G)
+            const uint32_t zbits = f2u(zz[k]);
+            uint32_t cmask       = 0;
+#pragma unroll
+            for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+                if ((inmask[k] >> l & 1u) && zbits <= cur[k][l]) cmask |= 1u << l;  // equal depth: the index decides
+            if (!__ballot(cmask != 0)) continue;  // wavefront-uniform
+            const uint64_t pk = ((uint64_t)zbits << 32) | (uint32_t)(base + k * kBlock);
+            wave_lds_sync();  // readers of the previous run are done
+            pk_w[lane] = pk;
+#pragma unroll
+            for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
             {
-                unsigned long long m  = gmask_w[lane];
-                unsigned long long mn = ~0ull;
-                while (m)
+                if (l >= lv.num) break;
+                const bool cand = cmask >> l & 1u;
+                if (!__ballot(cand)) continue;
+                const LevelArg& L = lv.l[l];
+                uint64_t* dst     = L.depth_index + (size_t)b * L.w * L.h;
+                if (l < group_from)
                 {
-                    int bit = __ffsll((long long)m) - 1;
-                    m &= m - 1;
-                    unsigned long long v = pk_w[bit];
-                    mn                   = v < mn ? v : mn;
+                    // fine levels: few lanes of a wavefront share a pixel, grouping would cost more than it saves
+                    if (cand) atomicMin((unsigned long long*)(dst + pix[k][l]), (unsigned long long)pk);
+                    continue;
                 }
-                atomicMin((unsigned long long*)(L.depth_index + (size_t)b * L.w * L.h + gkey_w[lane]), mn);
+                wave_lds_sync();
+                int G = wave_group_by_key(cand, pix[k][l], gkey_w, gmask_w);
+                wave_lds_sync();
+                if (lane < G)
+                {
+                    unsigned long long m  = gmask_w[lane];
+                    unsigned long long mn = ~0ull;
+                    while (m)
+                    {
+                        int bit = __ffsll((long long)m) - 1;
+                        m &= m - 1;
+                        unsigned long long v = pk_w[bit];
+                        mn                   = v < mn ? v : mn;
+                    }
+                    atomicMin((unsigned long long*)(dst + gkey_w[lane]), mn);
+                }
             }
         }
     }
@@ -246,6 +273,16 @@ __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewCo
         ok = ok && tex_ok;
         if (!__ballot(ok) && !STATS) continue;  // wavefront-uniform
 
+        // The descriptors are requested together with the depth words (one memory round trip instead of two); points
+        // that end up rejected at every level fetch them in vain, which costs less than the extra latency.
+        float t[CMAX];
+        const bool want_t = ok && !staged;
+        if (want_t)
+        {
+#pragma unroll
+            for (int c = 0; c < CMAX; ++c)
+                if (c < C) t[c] = tex_fetch<HALF>(pc.texture, (size_t)c * pc.num_texels + tex_index);
+        }
         // phase 1: pixel of every level and the depth test (all depth loads are independent)
         uint32_t gp[ADOP_MAX_LAYERS];
         bool acc[ADOP_MAX_LAYERS];
@@ -290,11 +327,11 @@ __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewCo
         if (!__ballot(any)) continue;  // wavefront-uniform
 
         // phase 2: stage the descriptors of this point (the same for every level and view)
-        if (any && !staged)
+        if (want_t)
         {
 #pragma unroll
             for (int c = 0; c < CMAX; ++c)
-                if (c < C) stage_w[lane * C + c] = tex_fetch<HALF>(pc.texture, (size_t)c * pc.num_texels + tex_index);
+                if (c < C) stage_w[lane * C + c] = t[c];
             staged = true;
         }
 
@@ -413,9 +450,18 @@ void launch_clear(const Levels& lv, int grid, float* accum, size_t accum_floats,
 void launch_prepass(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, adop_stats* stats,
                     hipStream_t st)
 {
-    int grid = (pc.n + kBlock - 1) / kBlock;
-    if (grid < 1) return;
-    hipLaunchKernelGGL(prepass_kernel, dim3(grid), dim3(kBlock), 0, st, pc, views, lv, rp, stats);
+    if (pc.n < 1) return;
+    static const int group_from = getenv("ADOP_PREPASS_GROUP_FROM") ? atoi(getenv("ADOP_PREPASS_GROUP_FROM")) : 1;
+    static const int ppt        = getenv("ADOP_PREPASS_PPT") ? atoi(getenv("ADOP_PREPASS_PPT")) : 2;
+    if (ppt == 4)
+        hipLaunchKernelGGL((prepass_kernel<4>), dim3((pc.n + kBlock * 4 - 1) / (kBlock * 4)), dim3(kBlock), 0, st, pc,
+                           views, lv, rp, group_from, stats);
+    else if (ppt == 2)
+        hipLaunchKernelGGL((prepass_kernel<2>), dim3((pc.n + kBlock * 2 - 1) / (kBlock * 2)), dim3(kBlock), 0, st, pc,
+                           views, lv, rp, group_from, stats);
+    else
+        hipLaunchKernelGGL((prepass_kernel<1>), dim3((pc.n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, pc, views, lv,
+                           rp, group_from, stats);
 }
 
 template <int CT, bool HALF>
