@@ -1,0 +1,108 @@
+"""GPU parity of the environment-map entry points (EnvironmentMap.cu:41-157 + RenderModule.cpp:106-127) and of
+ApplyTangentToPose (PointRenderer.cu:1646-1665), through the C-ABI."""
+import numpy as np
+import pytest
+
+from helpers import announce, assert_close, assert_norm_close, run_hip_forward
+
+pytestmark = pytest.mark.gpu
+
+
+def _env_scene():
+    from adop_amd import scenes
+
+    hs = scenes.config3(n=100_000, w=200, h=120, channels=4, levels=3)
+    hs.intrinsics[0, 5:] = [0.03, -0.01, 0.002, 0.005, 0.001, -0.0005, 0.0008, -0.001]
+    hs.params.output_background_mask = 1
+    hs.params.output_background_mask_value = 0.0
+    hs.env_texture = scenes.rng(17).random((4, 64, 128), dtype=np.float32)
+    # a second view from another pose, cropped
+    hs.poses_se3 = np.stack([hs.poses_se3[0], scenes.look_at_view((2.0, 1.5, 1.8))])
+    hs.views.append(scenes.make_view(200, 120, image_index=1, crop=(0.8, 0.8, 10.0, -5.0, 0.0)))
+    hs.dropout = scenes.bernoulli_mask(3, 2, hs.num_points, 0.25)
+    return hs
+
+
+def test_env_uv_sample_and_composition(oracle_mod):
+    import torch
+    from adop_amd import render
+
+    announce("environment map: uv, bilinear sample, out += (1-mask)*env")
+    hs = _env_scene()
+    scene, info, ctx, images, masks = run_hip_forward(hs)
+    before = [im.clone() for im in images]
+    uv, env = render.EnvironmentMapSample(info, add_to_out=True, want_uv=True, want_env=True)
+    torch.cuda.synchronize()
+    for l in range(hs.num_layers):
+        for b in range(hs.batch):
+            want_uv = oracle_mod.env_uv(hs, b, l)
+            got_uv = uv[l][b].cpu().numpy()
+            assert np.abs(got_uv - want_uv).max() <= 1e-6, (l, b)
+            # sampling of the HIP uv with the checker's bilinear rule
+            want_env = oracle_mod.grid_sample(hs.env_texture, got_uv)
+            assert_close(env[l][b].cpu().numpy(), want_env, 1e-5, 1e-6, f"env level {l} view {b}")
+        m = masks[l].cpu().numpy()
+        want = before[l].cpu().numpy() + (1 - m) * env[l].cpu().numpy()
+        assert_close(images[l].cpu().numpy(), want, 1e-6, 1e-7, f"composition level {l}")
+        # library cross-check: torch grid_sample on the same uv
+        ref = torch.nn.functional.grid_sample(torch.from_numpy(hs.env_texture)[None].repeat(hs.batch, 1, 1, 1),
+                                              uv[l].cpu(), mode="bilinear", padding_mode="border", align_corners=True)
+        assert_close(env[l].cpu().numpy(), ref.numpy(), 1e-5, 2e-6, f"env vs torch level {l}")
+
+
+def test_env_backward_matches_autograd_of_grid_sample():
+    import torch
+    from adop_amd import render, scenes
+
+    announce("environment map: gradient w.r.t. the texture")
+    hs = _env_scene()
+    scene, info, ctx, images, masks = run_hip_forward(hs)
+    uv, env = render.EnvironmentMapSample(info, add_to_out=False, want_uv=True, want_env=False)
+    gout = [torch.from_numpy(g).cuda() for g in scenes.upstream_grads(hs, 9)]
+    g_env = render.EnvironmentMapSampleBackward(info, gout)
+    torch.cuda.synchronize()
+    tex = torch.from_numpy(hs.env_texture).double().requires_grad_(True)
+    loss = 0
+    for l in range(hs.num_layers):
+        s = torch.nn.functional.grid_sample(tex[None].repeat(hs.batch, 1, 1, 1), uv[l].cpu().double(), mode="bilinear",
+                                            padding_mode="border", align_corners=True)
+        loss = loss + (s * (1 - masks[l].cpu().double()) * gout[l].cpu().double()).sum()
+    loss.backward()
+    # every texel sums hundreds of N(0,1)-weighted terms with fp32 atomics; autograd here runs in f64:
+    # bound the error against the size of the sums (tensor-level), not against each cancelled result
+    assert_norm_close(g_env.cpu().numpy(), tex.grad.numpy(), 2e-5, "grad env texture")
+
+
+def test_env_rejects_ocam():
+    import ctypes as C
+    from adop_amd import _capi, scenes
+
+    announce("environment map: OCam views are rejected (reference asserts pinhole)")
+    hs = scenes.config5(n=1000, w=44, h=30, batch=1, patches=10)
+    scene, info, ctx, images, masks = run_hip_forward(hs)
+    cache = info.cache
+    s = scene.struct()
+    fb = cache.forward_struct()
+    rc = cache.lib.adop_env_sample(C.byref(s), cache.views_array(), 1, C.c_void_p(scene.environment_map.data_ptr()),
+                                   512, 1024, C.byref(fb), None, None, 1, None)
+    assert rc == _capi.ADOP_INVALID_ARG
+
+
+def test_apply_tangent(oracle_mod):
+    import torch
+    from adop_amd import render, scenes
+
+    announce("ApplyTangentToPose")
+    g = scenes.rng(4)
+    F = 300
+    q = g.standard_normal((F, 4))
+    q /= np.linalg.norm(q, axis=1, keepdims=True)
+    poses = np.concatenate([q, g.uniform(-3, 3, (F, 3)), np.zeros((F, 1))], axis=1)
+    tang = g.standard_normal((F, 6)) * g.choice([1e-12, 1e-4, 0.1, 1.5], (F, 1))
+    t_ref, p_ref = oracle_mod.apply_tangent(tang, poses)
+    t = torch.from_numpy(tang.copy()).cuda()
+    p = torch.from_numpy(poses.copy()).cuda()
+    render.ApplyTangentToPose(t, p)
+    torch.cuda.synchronize()
+    assert (t == 0).all()
+    assert np.abs(p.cpu().numpy() - p_ref).max() < 1e-12
