@@ -215,15 +215,30 @@ def reference_point_order(xyz, seed, block=256):
     return order[idx]
 
 
+def apply_point_order(xyz, nrm, seed, point_order):
+    """``morton``: the reference's preprocessing order (Morton curve + shuffled 256-point blocks, which every ADOP
+    cloud goes through, SceneData.cpp:101-102); ``random``: a random permutation; ``generated``: unchanged."""
+    if point_order == "morton":
+        order = reference_point_order(xyz, seed + 7)
+    elif point_order == "random":
+        order = rng(seed + 8).permutation(len(xyz))
+    elif point_order == "generated":
+        return xyz, nrm
+    else:
+        raise ValueError(point_order)
+    return xyz[order], (None if nrm is None else nrm[order])
+
+
 # ---------------------------------------------------------------------------------------------------
 # the five benchmark configurations
 # ---------------------------------------------------------------------------------------------------
 
-def config1(n=100_000, w=256, h=256, levels=4, seed=0):
+def config1(n=100_000, w=256, h=256, levels=4, seed=0, point_order="generated"):
     """Forward only; points uniform in [-1,1]^3, pinhole 256x256, camera at (0,0,-3) looking +z."""
     g = rng(seed)
     xyz = g.uniform(-1.0, 1.0, (n, 3)).astype(np.float32)
     nrm = _unit(g.standard_normal((n, 3))).astype(np.float32)
+    xyz, nrm = apply_point_order(xyz, nrm, seed, point_order)
     pos = np.concatenate([xyz, np.zeros((n, 1), np.float32)], axis=1)
     tex = g.random((4, n), dtype=np.float32)
     f = float(w)
@@ -233,14 +248,16 @@ def config1(n=100_000, w=256, h=256, levels=4, seed=0):
         poses_se3=look_at_view((0, 0, -3), (0, 0, 0), world_up=(0, -1, 0))[None, :],
         intrinsics=pinhole_row(f, f, w / 2, h / 2)[None, :],
         views=[make_view(w, h)], params=default_params(), num_layers=levels, name="config1",
+        meta={"point_order": point_order},
     )
 
 
-def config2(n=1_000_000, w=512, h=512, levels=4, batch=4, seed=0, ghost=True):
+def config2(n=1_000_000, w=512, h=512, levels=4, batch=4, seed=0, ghost=True, point_order="morton"):
     """Forward+backward, batch of views on a radius-3 sphere; Gaussian cloud, outward normals."""
     g = rng(seed)
     xyz = (g.standard_normal((n, 3)) * 0.5).astype(np.float32)
     nrm = _unit(xyz.astype(np.float64) + 1e-12).astype(np.float32)
+    xyz, nrm = apply_point_order(xyz, nrm, seed, point_order)
     pos = np.concatenate([xyz, np.zeros((n, 1), np.float32)], axis=1)
     tex = np.clip(0.5 + 0.2 * g.standard_normal((4, n)), 0.0, 1.0).astype(np.float32)
     dirs = _unit(g.standard_normal((batch, 3)))
@@ -253,6 +270,7 @@ def config2(n=1_000_000, w=512, h=512, levels=4, batch=4, seed=0, ghost=True):
         intrinsics=pinhole_row(f, f, w / 2, h / 2)[None, :],
         views=[make_view(w, h, image_index=b) for b in range(batch)], params=params, num_layers=levels,
         dropout=bernoulli_mask(seed + 1, batch, n, 0.25) if ghost else None, name="config2",
+        meta={"point_order": point_order},
     )
 
 
@@ -266,14 +284,7 @@ def config3(n=10_000_000, w=1920, h=1080, levels=4, channels=8, seed=0, point_or
     pl = np.stack([g.uniform(-2, 2, npl), np.full(npl, -1.0), g.uniform(-2, 2, npl)], axis=1)
     xyz = np.concatenate([sph, pl]).astype(np.float32)
     nrm = np.concatenate([sph, np.tile(np.array([[0.0, 1.0, 0.0]]), (npl, 1))]).astype(np.float32)
-    if point_order == "morton":
-        order = reference_point_order(xyz, seed + 7)
-        xyz, nrm = xyz[order], nrm[order]
-    elif point_order != "random":
-        raise ValueError(point_order)
-    else:
-        order = g.permutation(n)
-        xyz, nrm = xyz[order], nrm[order]
+    xyz, nrm = apply_point_order(xyz, nrm, seed, point_order)
     pos = np.concatenate([xyz, np.zeros((n, 1), np.float32)], axis=1)
     tex = g.random((channels, n), dtype=np.float32)
     el, az = np.deg2rad(20.0), np.deg2rad(30.0)
@@ -294,7 +305,7 @@ def orbit_pose(frame, radius=12.0, deg_per_frame=1.2):
     return look_at_view((radius * np.sin(a), 0.0, -radius * np.cos(a)))
 
 
-def config4(n=100_000_000, w=1920, h=1080, levels=5, frames=300, seed=0):
+def config4(n=100_000_000, w=1920, h=1080, levels=5, frames=300, seed=0, point_order="morton"):
     """Viewer path: uniform points in a 10^3 volume, fp16-stored descriptors, 300-frame orbit of radius 12."""
     g = rng(seed)
     pos = np.empty((n, 4), np.float32)
@@ -303,6 +314,10 @@ def config4(n=100_000_000, w=1920, h=1080, levels=5, frames=300, seed=0):
         e = min(n, s + chunk)
         pos[s:e, :3] = g.uniform(-5.0, 5.0, (e - s, 3)).astype(np.float32)
     pos[:, 3] = 0
+    if point_order != "generated":
+        xyz, _ = apply_point_order(pos[:, :3], None, seed, point_order)
+        pos[:, :3] = xyz
+        del xyz
     tex = np.empty((4, n), np.float16)
     for s in range(0, n, chunk):
         e = min(n, s + chunk)
@@ -315,6 +330,7 @@ def config4(n=100_000_000, w=1920, h=1080, levels=5, frames=300, seed=0):
         background=np.zeros(4, np.float32), poses_se3=poses,
         intrinsics=pinhole_row(1400.0 * scale, 1400.0 * scale, w / 2, h / 2)[None, :],
         views=[make_view(w, h)], params=params, num_layers=levels, name="config4",
+        meta={"point_order": point_order},
     )
 
 
@@ -329,7 +345,8 @@ def ocam_row(w, h, seed=0, max_angle_deg=95.0):
     return np.concatenate([[1.0, 0.0, 0.0, w / 2.0, h / 2.0], poly]).astype(np.float32)
 
 
-def config5(n=20_000_000, w=2200, h=1500, levels=4, batch=8, patches=1000, seed=0, env_hw=(512, 1024)):
+def config5(n=20_000_000, w=2200, h=1500, levels=4, batch=8, patches=1000, seed=0, env_hw=(512, 1024),
+            point_order="morton"):
     """Forward+backward, OCam fisheye, random planar patches, spherical environment map."""
     g = rng(seed)
     centers = g.uniform(-3.0, 3.0, (patches, 3))
@@ -341,6 +358,7 @@ def config5(n=20_000_000, w=2200, h=1500, levels=4, batch=8, patches=1000, seed=
     v = g.uniform(-0.25, 0.25, (n, 1))
     xyz = (centers[pid] + u * a[pid] + v * b[pid]).astype(np.float32)
     nrm = normals[pid].astype(np.float32)
+    xyz, nrm = apply_point_order(xyz, nrm, seed, point_order)
     pos = np.concatenate([xyz, np.zeros((n, 1), np.float32)], axis=1)
     tex = g.random((4, n), dtype=np.float32)
     dirs = _unit(g.standard_normal((batch, 3)))
@@ -351,7 +369,7 @@ def config5(n=20_000_000, w=2200, h=1500, levels=4, batch=8, patches=1000, seed=
         position=pos, normal=pack_normals(nrm), index=np.arange(n, dtype=np.int32), texture=tex,
         background=np.zeros(4, np.float32), poses_se3=poses, intrinsics=ocam_row(w, h, seed)[None, :],
         views=[make_view(w, h, image_index=i, model=_capi.CAMERA_OCAM) for i in range(batch)],
-        params=params, num_layers=levels, env_texture=env, name="config5",
+        params=params, num_layers=levels, env_texture=env, name="config5", meta={"point_order": point_order},
     )
 
 

@@ -74,11 +74,11 @@ def main():
     if args.workload == "config3":
         hs = scenes.config3(point_order=args.point_order, **kw)
     elif args.workload == "config2":
-        hs = scenes.config2(**kw)
+        hs = scenes.config2(point_order=args.point_order, **kw)
     elif args.workload == "config4":
-        hs = scenes.config4(**kw)
+        hs = scenes.config4(point_order=args.point_order, **kw)
     else:
-        hs = scenes.config5(**kw)
+        hs = scenes.config5(point_order=args.point_order, **kw)
     backward = args.workload != "config4"
     gen_s = time.time() - t0
 
