@@ -1,0 +1,102 @@
+// bindings.cpp — pybind11 front end of the libTorch wrapper, used by the tests to drive PointRender /
+// PointRenderModuleForward exactly as the C++ pipeline would (same objects, same autograd function).
+#include <torch/extension.h>
+
+#include "PointRendererHip.h"
+
+namespace py = pybind11;
+
+struct PyScene
+{
+    NeuralScene scene;
+    PointRendererCache cache;
+
+    PyScene(torch::Tensor position, c10::optional<torch::Tensor> normal, torch::Tensor index, torch::Tensor texture,
+            torch::Tensor background, torch::Tensor poses_se3, torch::Tensor tangent_poses, torch::Tensor intrinsics,
+            c10::optional<torch::Tensor> env)
+    {
+        scene.point_cloud_cuda = NeuralPointCloudCuda(position, normal.has_value() ? *normal : torch::Tensor(), index);
+        // the leaf tensors stay the caller's objects so that autograd delivers the gradients to them
+        scene.point_cloud_cuda->t_position = position;
+        scene.texture                      = std::make_shared<NeuralTextureHolder>();
+        scene.texture->texture             = texture;
+        scene.texture->background_color    = background;
+        scene.poses                        = std::make_shared<PoseModuleHolder>();
+        scene.poses->poses_se3             = poses_se3;
+        scene.poses->tangent_poses         = tangent_poses;
+        scene.intrinsics                   = std::make_shared<IntrinsicsModuleHolder>();
+        scene.intrinsics->intrinsics       = intrinsics;
+        if (env.has_value())
+        {
+            scene.environment_map          = std::make_shared<EnvironmentMapHolder>();
+            scene.environment_map->texture = *env;
+        }
+    }
+};
+
+static RenderParams ParamsFromDict(const py::dict& d)
+{
+    RenderParams p;
+    p.drop_out_points_by_radius = false;
+    p.dropout                   = 0;
+    p.dist_cutoff               = 1e4f;
+#define GET(name, type) \
+    if (d.contains(#name)) p.name = d[#name].cast<type>()
+    GET(test_backward_mode, int);
+    GET(check_normal, bool);
+    GET(super_sampling, bool);
+    GET(dropout, float);
+    GET(depth_accept, float);
+    GET(ghost_gradients, bool);
+    GET(drop_out_radius_threshold, float);
+    GET(drop_out_points_by_radius, bool);
+    GET(distortion_gradient_factor, float);
+    GET(K_gradient_factor, float);
+    GET(dist_cutoff, float);
+    GET(output_background_mask, bool);
+    GET(output_background_mask_value, float);
+    GET(normalize_mode, int);
+#undef GET
+    return p;
+}
+
+// views: (w, h, image_index, camera_index, camera_model, crop_fx, crop_fy, crop_cx, crop_cy, crop_s)
+using ViewTuple = std::tuple<int, int, int, int, int, float, float, float, float, float>;
+
+static std::vector<torch::Tensor> Render(PyScene& s, const std::vector<ViewTuple>& views, const py::dict& params,
+                                         int num_layers, bool training, bool through_module)
+{
+    NeuralRenderInfo nri;
+    nri.scene      = &s.scene;
+    nri.num_layers = num_layers;
+    nri.params     = ParamsFromDict(params);
+    nri.cache      = &s.cache;
+    for (auto& v : views)
+    {
+        ReducedImageInfo i;
+        i.w                 = std::get<0>(v);
+        i.h                 = std::get<1>(v);
+        i.image_index       = std::get<2>(v);
+        i.camera_index      = std::get<3>(v);
+        i.camera_model_type = (CameraModel)std::get<4>(v);
+        i.crop_transform    = {std::get<5>(v), std::get<6>(v), std::get<7>(v), std::get<8>(v), std::get<9>(v)};
+        nri.images.push_back(i);
+    }
+    if (!through_module) return BlendPointCloud(&nri);
+    auto [images, masks] = PointRenderModuleForward(&nri, &s.cache, PointRenderModuleOptions(), training);
+    images.insert(images.end(), masks.begin(), masks.end());
+    return images;
+}
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
+{
+    py::class_<PyScene>(m, "Scene")
+        .def(py::init<torch::Tensor, c10::optional<torch::Tensor>, torch::Tensor, torch::Tensor, torch::Tensor,
+                      torch::Tensor, torch::Tensor, torch::Tensor, c10::optional<torch::Tensor>>(),
+             py::arg("position"), py::arg("normal"), py::arg("index"), py::arg("texture"), py::arg("background"),
+             py::arg("poses_se3"), py::arg("tangent_poses"), py::arg("intrinsics"), py::arg("env") = py::none())
+        .def("apply_tangent", [](PyScene& s) { s.scene.poses->ApplyTangent(); });
+    m.def("render", &Render, py::arg("scene"), py::arg("views"), py::arg("params"), py::arg("num_layers"),
+          py::arg("training") = true, py::arg("through_module") = false);
+    m.def("apply_tangent_to_pose", &ApplyTangentToPose);
+}

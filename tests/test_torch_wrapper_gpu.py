@@ -1,0 +1,164 @@
+"""The C++ libTorch wrapper (adop_amd/csrc/torch: PointRendererCache, PointRender autograd function, BlendPointCloud,
+PointRenderModuleForward, ApplyTangentToPose) driven through its pybind front end, against the CPU checker."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+from helpers import announce, assert_close, assert_norm_close
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _module():
+    sys.path.insert(0, os.path.join(ROOT, "adop_amd", "csrc", "torch"))
+    import torch  # noqa: F401  (libtorch must be loaded first)
+    import adop_torch
+
+    return adop_torch
+
+
+def _views(hs):
+    return [(v.w, v.h, v.image_index, v.camera_index, v.camera_model_type, v.crop_fx, v.crop_fy, v.crop_cx, v.crop_cy,
+             v.crop_s) for v in hs.views]
+
+
+def _params(hs, **extra):
+    p = hs.params
+    d = dict(test_backward_mode=p.test_backward_mode, check_normal=bool(p.check_normal),
+             ghost_gradients=bool(p.ghost_gradients), drop_out_points_by_radius=bool(p.drop_out_points_by_radius),
+             depth_accept=p.depth_accept, drop_out_radius_threshold=p.drop_out_radius_threshold,
+             dist_cutoff=p.dist_cutoff, distortion_gradient_factor=p.distortion_gradient_factor,
+             K_gradient_factor=p.K_gradient_factor, output_background_mask=bool(p.output_background_mask),
+             output_background_mask_value=p.output_background_mask_value, normalize_mode=p.normalize_mode)
+    d.update(extra)
+    return d
+
+
+def _scene(mod, hs, env=None):
+    import torch
+
+    t = dict(
+        position=torch.from_numpy(hs.position).cuda().requires_grad_(True),
+        normal=None if hs.normal is None else torch.from_numpy(hs.normal).cuda().reshape(-1, 1),
+        index=torch.from_numpy(hs.index).cuda().reshape(-1, 1),
+        texture=torch.from_numpy(hs.texture).cuda().requires_grad_(True),
+        background=torch.from_numpy(hs.background).cuda().requires_grad_(True),
+        poses_se3=torch.from_numpy(hs.poses_se3).cuda(),
+        tangent_poses=torch.zeros(hs.poses_se3.shape[0], 6, dtype=torch.float64, device="cuda").requires_grad_(True),
+        intrinsics=torch.from_numpy(hs.intrinsics).cuda().requires_grad_(True),
+    )
+    s = mod.Scene(t["position"], t["normal"], t["index"], t["texture"], t["background"], t["poses_se3"],
+                  t["tangent_poses"], t["intrinsics"], env)
+    return s, t
+
+
+def test_point_render_autograd_matches_checker(oracle_mod):
+    import torch
+    from adop_amd import scenes
+
+    announce("libTorch wrapper: PointRender forward + autograd backward, no dropout, spatial gradients of rendered points")
+    mod = _module()
+    hs = scenes.config3(n=200_000, w=320, h=180, channels=8)
+    hs.dropout = None
+    hs.params.ghost_gradients = 0
+    hs.params.output_background_mask = 1
+    ref = oracle_mod.forward(hs)
+    s, t = _scene(mod, hs)
+    outs = mod.render(s, _views(hs), _params(hs, dropout=0.0), hs.num_layers)
+    L = hs.num_layers
+    assert len(outs) == 2 * L  # images then masks (RenderInfo.cpp:39-41)
+    for l in range(L):
+        assert_close(outs[l].detach().cpu().numpy(), ref.out[l], 1e-5, 1e-7, f"out {l}")
+        # the masks leave PointRender as graph outputs (RenderModule.cpp:77-81 detaches them afterwards)
+        assert np.array_equal(outs[L + l].detach().cpu().numpy(), ref.mask[l])
+    gout = scenes.upstream_grads(hs, 3)
+    loss = sum((o * torch.from_numpy(g).cuda()).sum() for o, g in zip(outs[:L], gout))
+    loss.backward()
+    refb = oracle_mod.backward(hs, ref, gout)
+    assert_close(t["texture"].grad.cpu().numpy(), refb.grad_texture, 1e-4, 1e-5, "grad texture")
+    assert_close(t["background"].grad.cpu().numpy(), refb.grad_background, 1e-4, 1e-4, "grad background")
+    assert_norm_close(t["position"].grad.cpu().numpy(), refb.grad_points, 1e-4, "grad points")
+    assert_norm_close(t["tangent_poses"].grad.cpu().numpy(), refb.grad_pose, 1e-4, "grad pose")
+    assert_norm_close(t["intrinsics"].grad.cpu().numpy(), refb.grad_intrinsics, 1e-4, "grad intrinsics")
+
+
+def test_dropout_is_drawn_like_the_reference_and_eval_disables_it(oracle_mod):
+    import torch
+    from adop_amd import scenes
+
+    announce("libTorch wrapper: bernoulli_ dropout mask, eval mode -> no dropout")
+    mod = _module()
+    hs = scenes.config2(n=100_000, w=128, h=128, batch=2)
+    s, t = _scene(mod, hs)
+    torch.manual_seed(1234)
+    outs = mod.render(s, _views(hs), _params(hs, dropout=0.25), hs.num_layers)
+    torch.manual_seed(1234)
+    mask = torch.empty(2, hs.num_points, device="cuda").bernoulli_(0.25)  # PointRenderer.cu:1083
+    hs.dropout = mask.cpu().numpy()
+    ref = oracle_mod.forward(hs)
+    for l in range(hs.num_layers):
+        assert_close(outs[l].detach().cpu().numpy(), ref.out[l], 1e-5, 1e-7, f"out {l}")
+    # through the module in eval mode: dropout forced to 0 (RenderModule.cpp:25-28)
+    outs = mod.render(s, _views(hs), _params(hs, dropout=0.25), hs.num_layers, training=False, through_module=True)
+    hs.dropout = None
+    ref = oracle_mod.forward(hs)
+    for l in range(hs.num_layers):
+        assert_close(outs[l].detach().cpu().numpy(), ref.out[l], 1e-5, 1e-7, f"eval out {l}")
+
+
+def test_module_forward_supersampling_and_environment_map(oracle_mod):
+    import torch
+    from adop_amd import scenes
+
+    announce("libTorch wrapper: PointRenderModuleForward with super-sampling and the environment map")
+    mod = _module()
+    hs = scenes.config3(n=100_000, w=160, h=96, channels=4, levels=3)
+    hs.dropout = None
+    hs.params.ghost_gradients = 0
+    hs.params.output_background_mask = 1
+    env_np = scenes.rng(5).random((4, 32, 64), dtype=np.float32)
+    env = torch.from_numpy(env_np).cuda().requires_grad_(True)
+    s, t = _scene(mod, hs, env)
+    outs = mod.render(s, _views(hs), _params(hs, dropout=0.0, super_sampling=True), hs.num_layers, training=True,
+                      through_module=True)
+    L = hs.num_layers
+    assert [tuple(o.shape[2:]) for o in outs[:L]] == [(96, 160), (48, 80), (24, 40)]
+    # reference composition on the host: render at 2x, 2x2 average pool, + (1-mask)*env (RenderModule.cpp:54-127)
+    import copy
+    hs2 = copy.copy(hs)
+    v = hs.views[0]
+    hs2.views = [scenes.make_view(2 * v.w, 2 * v.h, v.image_index, v.camera_index, v.camera_model_type,
+                                  (2 * v.crop_fx, 2 * v.crop_fy, 2 * v.crop_cx, 2 * v.crop_cy, 2 * v.crop_s))]
+    ref = oracle_mod.forward(hs2)
+    for l in range(L):
+        img = torch.nn.functional.avg_pool2d(torch.from_numpy(ref.out[l]), 2)
+        m = torch.nn.functional.avg_pool2d(torch.from_numpy(ref.mask[l]), 2)
+        uv = torch.from_numpy(oracle_mod.env_uv(hs, 0, l))[None]
+        e = torch.nn.functional.grid_sample(torch.from_numpy(env_np)[None], uv, mode="bilinear", padding_mode="border",
+                                            align_corners=True)
+        want = img + (1 - m) * e
+        assert_close(outs[l].detach().cpu().numpy(), want.numpy(), 2e-5, 2e-6, f"module out {l}")
+        assert_close(outs[L + l].cpu().numpy(), m.numpy(), 1e-6, 1e-7, f"module mask {l}")
+    sum(o.sum() for o in outs[:L]).backward()
+    assert env.grad is not None and float(env.grad.abs().sum()) > 0  # texture gradient through torch's grid_sample
+
+
+def test_apply_tangent(oracle_mod):
+    import torch
+    from adop_amd import scenes
+
+    announce("libTorch wrapper: PoseModule::ApplyTangent")
+    mod = _module()
+    hs = scenes.config1(n=10, w=16, h=16, levels=1)
+    s, t = _scene(mod, hs)
+    with torch.no_grad():
+        t["tangent_poses"][0] = torch.tensor([0.1, -0.2, 0.05, 0.02, 0.01, -0.03], dtype=torch.float64)
+    tang, want = oracle_mod.apply_tangent(t["tangent_poses"].detach().cpu().numpy(), hs.poses_se3)
+    with torch.no_grad():
+        s.apply_tangent()
+    torch.cuda.synchronize()
+    assert np.abs(t["poses_se3"].cpu().numpy() - want).max() < 1e-12
+    assert float(t["tangent_poses"].detach().abs().sum()) == 0
