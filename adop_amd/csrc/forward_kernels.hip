@@ -230,7 +230,7 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
 template <int CT, bool HALF>
 __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewConst* __restrict__ views, Levels lv,
                                                        ParamArg rp, float* __restrict__ accum, int S,
-                                                       adop_stats* stats)
+                                                       adop_stats* stats, int group_from)
 {
     constexpr int CMAX = CT ? CT : kMaxChannels;
     __shared__ unsigned long long s_gmask[kBlock];
@@ -340,9 +340,23 @@ __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewCo
         for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
         {
             if (l >= lv.num) break;
-            if (!__ballot(acc[l])) continue;
+            const unsigned long long bal = __ballot(acc[l]);
+            if (!bal) continue;
             wave_lds_sync();
-            int G = wave_group_by_key(acc[l], gp[l], gkey_w, gmask_w);
+            int G;
+            if (l < group_from)
+            {
+                // fine level: few lanes of a wavefront share a pixel; every accepted lane is its own entry
+                G = __popcll(bal);
+                if (acc[l])
+                {
+                    int e      = __popcll(bal & ((1ull << lane) - 1ull));
+                    gkey_w[e]  = gp[l];
+                    gmask_w[e] = 1ull << lane;
+                }
+            }
+            else
+                G = wave_group_by_key(acc[l], gp[l], gkey_w, gmask_w);
             wave_lds_sync();
             for (int g0 = 0; g0 < G; g0 += subs)
             {
@@ -470,8 +484,9 @@ static void launch_blend_t(const CloudArg& pc, const ViewConst* views, const Lev
 {
     int grid   = (pc.n + kBlock - 1) / kBlock;
     size_t lds = sizeof(float) * (size_t)kBlock * (size_t)lv.C;
+    static const int group_from = getenv("ADOP_BLEND_GROUP_FROM") ? atoi(getenv("ADOP_BLEND_GROUP_FROM")) : 0;  // 0: group at every level
     hipLaunchKernelGGL((blend_kernel<CT, HALF>), dim3(grid), dim3(kBlock), lds, st, pc, views, lv, rp,
-                       accum, S, stats);
+                       accum, S, stats, group_from);
 }
 
 void launch_blend(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
