@@ -332,7 +332,9 @@ __global__ __launch_bounds__(kBlock) void backward_ghost_kernel(CloudArg pc, con
     __syncthreads();
     const uint32_t total = s_prefix[kNumQueues];
 
-    double acc[kAcc];
+    // per-thread sums of the pose / intrinsics gradients: a thread sees a few dozen contributions at most, so fp32
+    // here costs ~1e-7 relative; everything beyond the thread (wavefront, block, grid) is summed in f64
+    float acc[kAcc];
 #pragma unroll
     for (int k = 0; k < kAcc; ++k) acc[k] = 0;
 
@@ -466,8 +468,8 @@ __global__ __launch_bounds__(kBlock) void backward_ghost_kernel(CloudArg pc, con
                 if (want_pose)
                 {
 #pragma unroll
-                    for (int k = 0; k < 6; ++k) acc[k] += (double)bo.g_pose[k];
-                    acc[6] += 1.0;
+                    for (int k = 0; k < 6; ++k) acc[k] += bo.g_pose[k];
+                    acc[6] += 1.0f;
                 }
                 if (want_intr)
                 {
@@ -477,7 +479,7 @@ __global__ __launch_bounds__(kBlock) void backward_ghost_kernel(CloudArg pc, con
                         bo.g_k[4] *= 0.1f;
                         bo.g_k[4] *= 0;  // :653-654
 #pragma unroll
-                        for (int k = 0; k < 5; ++k) acc[8 + k] += (double)(kf * bo.g_k[k]);
+                        for (int k = 0; k < 5; ++k) acc[8 + k] += kf * bo.g_k[k];
                         float df = rp.distortion_gradient_factor;
                         bo.g_dis[2] *= 0.25f;
                         bo.g_dis[3] *= 0.1f;
@@ -486,14 +488,14 @@ __global__ __launch_bounds__(kBlock) void backward_ghost_kernel(CloudArg pc, con
                         bo.g_dis[6] *= 0.1f;
                         bo.g_dis[7] *= 0.1f;
 #pragma unroll
-                        for (int k = 0; k < 8; ++k) acc[13 + k] += (double)(df * bo.g_dis[k]);
-                        acc[7] += 1.0 / 1024.0;  // :680-681
+                        for (int k = 0; k < 8; ++k) acc[13 + k] += df * bo.g_dis[k];
+                        acc[7] += 1.0f / 1024.0f;  // :680-681
                     }
                     else
                     {
 #pragma unroll
-                        for (int k = 0; k < 5; ++k) acc[8 + k] += (double)bo.g_k[k];
-                        acc[7] += 1.0;  // :718
+                        for (int k = 0; k < 5; ++k) acc[8 + k] += bo.g_k[k];
+                        acc[7] += 1.0f;  // :718
                     }
                 }
             }
@@ -517,7 +519,7 @@ __global__ __launch_bounds__(kBlock) void backward_ghost_kernel(CloudArg pc, con
 #pragma unroll
         for (int k = 0; k < kAcc; ++k)
         {
-            double v = wave_sum<double>(acc[k]);
+            double v = wave_sum<double>((double)acc[k]);
             if (lane == 0) red[wave][k] = v;
         }
         __syncthreads();
