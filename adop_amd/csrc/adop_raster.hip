@@ -448,9 +448,14 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     }
     for (int b = 0; b < num_views; ++b)
     {
-        StageScope sc("RenderBackward", stream);
-        launch_render_backward(pc, dviews, lv, rp, half, ig, grads, want_pose, want_intr, scene->index_is_identity, b,
-                               b == 0, q, pt_blocks, pt_partial, stats, stream);
+        {
+            StageScope sc("RenderBackward/descriptor", stream);
+            launch_backward_tex(pc, dviews, lv, rp, half, ig, grads, scene->index_is_identity, b, b == 0, q, stats,
+                                stream);
+        }
+        StageScope sc("RenderBackward/spatial", stream);
+        launch_backward_ghost(pc, dviews, lv, rp, half, ig, grads, want_pose, want_intr, scene->index_is_identity, b,
+                              q, pt_blocks, pt_partial, stream);
     }
     StageScope post("Post Process Gradient", stream);
     launch_finalize(dviews, num_views, C, bg_partial, bg_blocks, pt_partial, pt_blocks, grads, scene->num_poses,

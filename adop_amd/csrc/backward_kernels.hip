@@ -673,36 +673,59 @@ void launch_interleave(const Levels& lv, int blocks, float* ig, double* partial,
 }
 
 template <int CT, bool HALF>
-static void launch_bwd_t(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp,
-                         const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr,
-                         int identity_index, int b, int first_view, const QueueArg& q, int ghost_blocks,
-                         double* partial, adop_stats* stats, hipStream_t st)
+static void launch_bwd_tex_t(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp,
+                             const float* ig, const adop_backward_buffers* g, int identity_index, int b,
+                             int first_view, const QueueArg& q, adop_stats* stats, hipStream_t st)
 {
     int grid = (pc.n + kBlock - 1) / kBlock;
     hipLaunchKernelGGL(fill_zero_u32_kernel, dim3(kNumQueues / kBlock), dim3(kBlock), 0, st, q.counts, kNumQueues);
     hipLaunchKernelGGL((backward_tex_kernel<CT, HALF>), dim3(grid), dim3(kBlock), 0, st, pc, views, lv, rp, ig,
                        g->grad_texture, identity_index, b, first_view, q.counts, q.items, q.cap, stats);
+}
+
+template <int CT, bool HALF>
+static void launch_bwd_ghost_t(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp,
+                               const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr,
+                               int identity_index, int b, const QueueArg& q, int ghost_blocks, double* partial,
+                               hipStream_t st)
+{
     hipLaunchKernelGGL(queue_scan_kernel, dim3(1), dim3(kBlock), 0, st, q.counts, q.prefix);
     hipLaunchKernelGGL((backward_ghost_kernel<CT, HALF>), dim3(ghost_blocks), dim3(kBlock), 0, st, pc, views, lv, rp,
                        ig, g->grad_points, g->grad_points_count, want_pose, want_intr, identity_index, b, q.prefix,
                        q.items, q.cap, partial);
 }
 
-void launch_render_backward(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
-                            const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr,
-                            int identity_index, int b, int first_view, const QueueArg& q, int ghost_blocks,
-                            double* partial, adop_stats* stats, hipStream_t st)
+#define ADOP_DISPATCH_C_HALF(FN, ...)                                   \
+    do                                                                  \
+    {                                                                   \
+        if (lv.C == 8)                                                  \
+            half ? FN<8, true>(__VA_ARGS__) : FN<8, false>(__VA_ARGS__); \
+        else if (lv.C == 4)                                             \
+            half ? FN<4, true>(__VA_ARGS__) : FN<4, false>(__VA_ARGS__); \
+        else                                                            \
+            half ? FN<0, true>(__VA_ARGS__) : FN<0, false>(__VA_ARGS__); \
+    } while (0)
+
+// descriptor gradient of one view + the work queue of its ghost / spatial gradients
+void launch_backward_tex(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
+                         const float* ig, const adop_backward_buffers* g, int identity_index, int b, int first_view,
+                         const QueueArg& q, adop_stats* stats, hipStream_t st)
 {
     if (pc.n < 1) return;
-#define ADOP_ARGS pc, views, lv, rp, ig, g, want_pose, want_intr, identity_index, b, first_view, q, ghost_blocks, partial, stats, st
-    if (lv.C == 8)
-        half ? launch_bwd_t<8, true>(ADOP_ARGS) : launch_bwd_t<8, false>(ADOP_ARGS);
-    else if (lv.C == 4)
-        half ? launch_bwd_t<4, true>(ADOP_ARGS) : launch_bwd_t<4, false>(ADOP_ARGS);
-    else
-        half ? launch_bwd_t<0, true>(ADOP_ARGS) : launch_bwd_t<0, false>(ADOP_ARGS);
-#undef ADOP_ARGS
+    ADOP_DISPATCH_C_HALF(launch_bwd_tex_t, pc, views, lv, rp, ig, g, identity_index, b, first_view, q, stats, st);
 }
+
+// ghost / spatial gradients of the queued points of one view
+void launch_backward_ghost(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
+                           const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr,
+                           int identity_index, int b, const QueueArg& q, int ghost_blocks, double* partial,
+                           hipStream_t st)
+{
+    if (pc.n < 1) return;
+    ADOP_DISPATCH_C_HALF(launch_bwd_ghost_t, pc, views, lv, rp, ig, g, want_pose, want_intr, identity_index, b, q,
+                         ghost_blocks, partial, st);
+}
+#undef ADOP_DISPATCH_C_HALF
 
 void launch_finalize(const ViewConst* views, int B, int C, const double* bg_partial, int bg_blocks,
                      const double* pt_partial, int pt_blocks, const adop_backward_buffers* g, int num_poses,

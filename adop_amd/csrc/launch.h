@@ -32,10 +32,13 @@ struct QueueArg
     unsigned long long* items;  // [kNumQueues * cap]
     uint32_t cap;
 };
-void launch_render_backward(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
-                            const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr,
-                            int identity_index, int b, int first_view, const QueueArg& q, int ghost_blocks,
-                            double* partial, adop_stats* stats, hipStream_t st);
+void launch_backward_tex(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
+                         const float* ig, const adop_backward_buffers* g, int identity_index, int b, int first_view,
+                         const QueueArg& q, adop_stats* stats, hipStream_t st);
+void launch_backward_ghost(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
+                           const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr,
+                           int identity_index, int b, const QueueArg& q, int ghost_blocks, double* partial,
+                           hipStream_t st);
 void launch_finalize(const ViewConst* views, int B, int C, const double* bg_partial, int bg_blocks,
                      const double* pt_partial, int pt_blocks, const adop_backward_buffers* g, int num_poses,
                      int num_cameras, int cols, int normalize_mode, double* scratch, hipStream_t st);

@@ -25,6 +25,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+KERNEL_OF_STAGE = {"DepthPrepass": "prepass_kernel", "RenderForward": "blend_kernel", "CombineAndFill": "resolve_kernel",
+                   "CombineAndFillBackward": "interleave_kernel", "RenderBackward/descriptor": "backward_tex_kernel",
+                   "RenderBackward/spatial": "backward_ghost_kernel"}
 
 
 def byte_model(N, B, C_, S_d, P, V, A, G, has_mask, has_dropout):
@@ -35,7 +38,9 @@ def byte_model(N, B, C_, S_d, P, V, A, G, has_mask, has_dropout):
     k["DepthPrepass"] = B * N * 20 + sv * 8
     k["RenderForward"] = B * N * (24 + drop) + sa * (C_ * S_d + C_ * 4 + 4)
     k["CombineAndFill"] = B * P * (8 + 4 + 2 * C_ * 4) + (B * P * 4 if has_mask else 0)
-    k["RenderBackward"] = B * N * (24 + drop) + sa * (4 + 4 + C_ * 4 + C_ * 4) + sg * (4 * (8 + 8 * C_) + C_ * S_d + 16)
+    # RenderBackward runs as two kernels: descriptor gradient (+ work queue) and ghost / spatial gradient
+    k["RenderBackward/descriptor"] = B * N * (24 + drop) + sa * (4 + 4 + C_ * 4 + C_ * 4)
+    k["RenderBackward/spatial"] = sg * (4 * (8 + 8 * C_) + C_ * S_d + 16)
     k["CombineAndFillBackward"] = B * P * (4 + 4 * C_)
     return k
 
@@ -176,8 +181,13 @@ def main():
     total_bytes = sum(model.values())
     dom = max((k for k in model if k in stages), key=lambda k: stages[k])
     dom_gbs = model[dom] / (stages[dom] * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "kernel": dom, "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+    # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
+    # FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 after calibration with a plain 1 GiB copy); measured for the default
+    # workload only
+    measured_traffic = {("config3", "RenderForward"): 691.9e6} if not args.points and args.point_order == "morton" else {}
+    roofline = {"bound": "hbm", "kernel": KERNEL_OF_STAGE.get(dom, dom), "stage": dom, "achieved": round(dom_gbs, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
+                "traffic": measured_traffic.get((args.workload, dom)),
                 "kernel_ms": round(stages[dom], 4), "algorithmic_bytes": int(model[dom])}
     step_gbs = total_bytes / (ms_per_step * 1e-3) / 1e9
 

@@ -196,7 +196,8 @@ adop_status adop_apply_tangent(double* tangent, double* poses_se3, int32_t num_p
  * (PointRenderer.cu:906,913,919,1095,1414,1430,1447,1565,1594,1602,1610); here HIP events are recorded on the
  * caller's stream around each stage while profiling is enabled on the calling thread.  Stage names are the
  * reference's: "Initialize", "DepthPrepass", "RenderForward", "CombineAndFill", "Prepare Backward",
- * "CombineAndFillBackward", "RenderBackward", "Post Process Gradient". */
+ * "CombineAndFillBackward", "RenderBackward/descriptor" and "RenderBackward/spatial" (the two kernels RenderBackward is
+ * split into), "Post Process Gradient". */
 typedef struct adop_stage_time
 {
     char name[32];
