@@ -51,6 +51,7 @@ class RenderParams(C.Structure):
         ("output_background_mask", C.c_int32),
         ("output_background_mask_value", C.c_float),
         ("normalize_mode", C.c_int32),
+        ("forward_path", C.c_int32),
     ]
 
 
@@ -91,6 +92,7 @@ class ForwardBuffers(C.Structure):
         ("num_layers", C.c_int32),
         ("layers", Layer * ADOP_MAX_LAYERS),
         ("dropout_points", C.c_void_p),
+        ("point_cache", C.c_void_p),
     ]
 
 

@@ -19,6 +19,7 @@
 
 #include <stdint.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <string>
@@ -94,7 +95,7 @@ struct StageScope
 struct WorkspaceLayout
 {
     size_t views;       // ViewConst[B]
-    size_t bg_partial;  // double[kPartialBlocks * kMaxChannels]
+    size_t bg_partial;  // double[kBgBlocks * kMaxChannels]
     size_t pt_partial;  // double[B * kPartialBlocks * kPartialStride]
     size_t scratch;     // double[num_poses*7 + num_cameras*(cols+1)]
     size_t pixels;      // float[B * P * max(S, 2C)]: blend accumulators (forward) / [I|G] array (backward)
@@ -102,8 +103,25 @@ struct WorkspaceLayout
     size_t q_prefix;    // uint32[kNumQueues + 1]
     size_t q_items;     // uint64[kNumQueues * q_cap]
     uint32_t q_cap;
+    size_t proj;        // float4[B * N]: projected points of the forward pass when the caller keeps no point_cache
+    size_t bin_count;   // uint32[max tiles]           tile bins of the forward pass
+    size_t bin_offset;  // uint32[max tiles + 1]
+    size_t bin_cursor;  // uint32[max tiles]
+    size_t bin_entries; // float4[kTileLevels * B * N]
+    size_t bin_cap;     // entries
     size_t total;
 };
+
+constexpr int kTileLevels = 2;  // levels the tile path renders in LDS (a point has at most one bin entry per such level)
+constexpr int kMinTileShift = 4;
+constexpr int kTilePathMinPoints = 1 << 16;
+
+size_t max_tiles(int B, int w0, int h0)
+{
+    size_t tx = ((size_t)(w0 > 0 ? w0 : 1) - 1 >> kMinTileShift) + 1;
+    size_t ty = ((size_t)(h0 > 0 ? h0 : 1) - 1 >> kMinTileShift) + 1;
+    return tx * ty * (size_t)B;
+}
 
 // floats per pixel of the blend accumulators: C sums + the weight, padded to a power of two so that the group
 // of lanes flushing one pixel never straddles a cache line
@@ -138,7 +156,7 @@ WorkspaceLayout layout(const adop_scene* s, int B, int L, int w0, int h0)
     w.views      = o;
     o            = align_up(o + sizeof(ViewConst) * (size_t)B, 256);
     w.bg_partial = o;
-    o            = align_up(o + sizeof(double) * kPartialBlocks * kMaxChannels, 256);
+    o            = align_up(o + sizeof(double) * kBgBlocks * kMaxChannels, 256);
     w.pt_partial = o;
     o            = align_up(o + sizeof(double) * (size_t)B * kPartialBlocks * kPartialStride, 256);
     w.scratch    = o;
@@ -157,7 +175,19 @@ WorkspaceLayout layout(const adop_scene* s, int B, int L, int w0, int h0)
     o          = align_up(o + sizeof(uint32_t) * (kNumQueues + 1), 256);
     w.q_items  = o;
     o          = align_up(o + sizeof(unsigned long long) * (size_t)kNumQueues * w.q_cap, 256);
-    w.total    = o;
+    w.proj       = o;
+    o            = align_up(o + sizeof(float4) * (size_t)B * (size_t)(s->num_points > 0 ? s->num_points : 0), 256);
+    size_t T     = max_tiles(B, w0, h0);
+    w.bin_count  = o;
+    o            = align_up(o + sizeof(uint32_t) * T * kBinStride, 256);
+    w.bin_offset = o;
+    o            = align_up(o + sizeof(uint32_t) * (T + 1), 256);
+    w.bin_cursor = o;
+    o            = align_up(o + sizeof(uint32_t) * T * kBinStride, 256);
+    w.bin_cap    = (size_t)kTileLevels * (size_t)B * (size_t)(s->num_points > 0 ? s->num_points : 0);
+    w.bin_entries = o;
+    o            = align_up(o + sizeof(float4) * w.bin_cap, 256);
+    w.total      = o;
     return w;
 }
 
@@ -255,6 +285,7 @@ CloudArg make_cloud(const adop_scene* s, const adop_forward_buffers* fb)
     c.num_texels = s->num_texels;
     c.intrinsics = s->intrinsics;
     c.dropout    = fb->dropout_points;
+    c.cache      = (float4*)fb->point_cache;
     return c;
 }
 
@@ -295,9 +326,9 @@ adop_status fill_async(void* p, size_t bytes, uint32_t v, hipStream_t st)
     return ADOP_OK;
 }
 
-int pixel_grid(const Levels& lv)
+int pixel_grid(const Levels& lv, int first_level = 0)
 {
-    size_t total = (size_t)lv.pix_prefix[lv.num] * lv.B;
+    size_t total = (size_t)(lv.pix_prefix[lv.num] - lv.pix_prefix[first_level]) * lv.B;
     size_t want  = (total + kBlock - 1) / kBlock;
     return (int)(want < 16384 ? (want ? want : 1) : 16384);
 }
@@ -331,6 +362,7 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
     Levels lv   = make_levels(scene, num_views, buffers, nullptr);
     CloudArg pc = make_cloud(scene, buffers);
     ParamArg rp = make_params(params);
+    if (!pc.cache) pc.cache = (float4*)((char*)workspace + wl.proj);
 
     if (stats)
     {
@@ -340,18 +372,85 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
     const int C      = scene->num_channels;
     const int S      = accum_stride(C);
     float* accum     = (float*)((char*)workspace + wl.pixels);
+    const bool half  = scene->texture_dtype == ADOP_TEXTURE_F16;
+
+    // Tile path: point ids need 28 bits of the bin entry; a handful of points is faster through the direct path.
+    static const int env_path = getenv("ADOP_FORWARD_PATH") ? atoi(getenv("ADOP_FORWARD_PATH")) : 0;
+    int path = params->forward_path ? params->forward_path : env_path;
+    if (path < 0 || path > 2) return fail(ADOP_INVALID_ARG, "forward_path must be 0, 1 or 2");
+    const bool can_bin = scene->num_points > 0 && scene->num_points < (1 << 28);
+    if (path == 0) path = scene->num_points >= kTilePathMinPoints ? 2 : 1;
+    if (path == 2 && !can_bin) path = 1;
+
+    if (path == 2)
+    {
+        BinArg bin;
+        bin.ts      = kMinTileShift;
+        bin.lt      = kTileLevels < lv.num ? kTileLevels : lv.num;
+        bin.tiles_x = ((views[0].w - 1) >> bin.ts) + 1;
+        bin.tiles_y = ((views[0].h - 1) >> bin.ts) + 1;
+        bin.count   = (uint32_t*)((char*)workspace + wl.bin_count);
+        bin.offset  = (uint32_t*)((char*)workspace + wl.bin_offset);
+        bin.cursor  = (uint32_t*)((char*)workspace + wl.bin_cursor);
+        bin.entries = (float4*)((char*)workspace + wl.bin_entries);
+        const int T = bin.tiles_x * bin.tiles_y * num_views;
+        {
+            StageScope sc("Initialize", stream);
+            if ((st = fill_async(bin.count, sizeof(uint32_t) * (size_t)T * kBinStride, 0, stream)) != ADOP_OK) return st;
+            if (bin.lt < lv.num)
+            {
+                // coarse levels: packed depth and global accumulators as in the direct path
+                size_t first  = (size_t)lv.pix_prefix[bin.lt] * lv.B * S;
+                size_t accum_n = (size_t)lv.pix_prefix[lv.num] * lv.B * S - first;
+                if (S % 4 == 0)
+                    launch_clear(lv, bin.lt, pixel_grid(lv, bin.lt), accum + first, accum_n, stream);
+                else
+                {
+                    launch_clear(lv, bin.lt, pixel_grid(lv, bin.lt), accum, 0, stream);
+                    if ((st = fill_async(accum + first, accum_n * sizeof(float), 0, stream)) != ADOP_OK) return st;
+                }
+            }
+        }
+        {
+            StageScope sc("BinCount", stream);
+            launch_bin(0, pc, dviews, lv, rp, bin, stats, stream);
+        }
+        {
+            StageScope sc("BinScatter", stream);
+            launch_tile_scan(bin, T, stream);
+            launch_bin(1, pc, dviews, lv, rp, bin, nullptr, stream);
+        }
+        {
+            StageScope sc("TileDepth", stream);
+            launch_tile_depth(lv, bin, T, stream);
+        }
+        {
+            StageScope sc("TileBlend", stream);
+            ADOP_HIP_CHECK(launch_tile_blend(pc, lv, rp, bin, T, half, accum, S, scene->background_color,
+                                             params->output_background_mask, params->output_background_mask_value,
+                                             scene->index_is_identity, stats, stream));
+        }
+        if (bin.lt < lv.num)
+        {
+            StageScope sc("CombineAndFill", stream);
+            launch_resolve(lv, bin.lt, pixel_grid(lv, bin.lt), accum, S, scene->background_color,
+                           params->output_background_mask, params->output_background_mask_value, stream);
+        }
+        ADOP_HIP_CHECK(hipGetLastError());
+        return ADOP_OK;
+    }
+
     size_t accum_n   = (size_t)lv.pix_prefix[lv.num] * lv.B * S;  // floats, multiple of 4 unless S < 4
     {
         StageScope sc("Initialize", stream);
         if (S % 4 == 0)
-            launch_clear(lv, pixel_grid(lv), accum, accum_n, stream);
+            launch_clear(lv, 0, pixel_grid(lv), accum, accum_n, stream);
         else
         {
-            launch_clear(lv, pixel_grid(lv), accum, 0, stream);
+            launch_clear(lv, 0, pixel_grid(lv), accum, 0, stream);
             if ((st = fill_async(accum, accum_n * sizeof(float), 0, stream)) != ADOP_OK) return st;
         }
     }
-    const bool half = scene->texture_dtype == ADOP_TEXTURE_F16;
     {
         StageScope sc("DepthPrepass", stream);
         launch_prepass(pc, dviews, lv, rp, stats, stream);
@@ -362,7 +461,7 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
     }
     {
         StageScope sc("CombineAndFill", stream);
-        launch_resolve(lv, pixel_grid(lv), accum, S, scene->background_color, params->output_background_mask,
+        launch_resolve(lv, 0, pixel_grid(lv), accum, S, scene->background_color, params->output_background_mask,
                        params->output_background_mask_value, stream);
     }
     ADOP_HIP_CHECK(hipGetLastError());
@@ -423,7 +522,7 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     }
 
     float* ig     = (float*)((char*)workspace + wl.pixels);
-    int bg_blocks = pixel_grid(lv) < kPartialBlocks ? pixel_grid(lv) : kPartialBlocks;
+    int bg_blocks = pixel_grid(lv) < kBgBlocks ? pixel_grid(lv) : kBgBlocks;
     {
         StageScope sc("CombineAndFillBackward", stream);
         launch_interleave(lv, bg_blocks, ig, bg_partial, stream);

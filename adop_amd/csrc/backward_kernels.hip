@@ -27,6 +27,7 @@ __global__ __launch_bounds__(kBlock) void interleave_kernel(Levels lv, float* __
     constexpr int CMAX = CT ? CT : kMaxChannels;
     const int C        = CT ? CT : lv.C;
     __shared__ double red[kBlock / 64][kMaxChannels];
+    __shared__ float4 s_tr[kBlock / 64][(CT == 8 || CT == 4) ? 64 * (CT / 2) : 1];
     float acc[CMAX];
 #pragma unroll
     for (int c = 0; c < CMAX; ++c) acc[c] = 0;
@@ -56,12 +57,40 @@ __global__ __launch_bounds__(kBlock) void interleave_kernel(Levels lv, float* __
             }
         if (CT == 8 || CT == 4)
         {
-            float4* d4 = (float4*)dst;
+            // The 64 pixels of a wavefront are 64 consecutive records of the pixel-major array when they lie in one
+            // level of one image: transposed through LDS, every store instruction then writes 1 KB of consecutive
+            // bytes instead of a quarter (half) of 64 separate lines.
+            constexpr int V     = CT / 2;  // float4 per record
+            const int lane      = threadIdx.x & 63;
+            const size_t t_wave = t - lane;
+            const int r_last    = (int)((t_wave + 63) - (size_t)b * per_image);
+            const bool whole    = t_wave + 63 < total && (t_wave / per_image) == (size_t)b &&
+                               (t_wave + 63) / per_image == (size_t)b && level_of(lv, r_last) == l &&
+                               level_of(lv, r - lane) == l;
+            if (whole)  // wavefront-uniform
+            {
+                float4* sw = s_tr[threadIdx.x >> 6];
+                wave_lds_sync();
 #pragma unroll
-            for (int q = 0; q < CT / 4; ++q) d4[q] = make_float4(I[4 * q], I[4 * q + 1], I[4 * q + 2], I[4 * q + 3]);
+                for (int q = 0; q < CT / 4; ++q)
+                {
+                    sw[lane * V + q]          = make_float4(I[4 * q], I[4 * q + 1], I[4 * q + 2], I[4 * q + 3]);
+                    sw[lane * V + CT / 4 + q] = make_float4(G[4 * q], G[4 * q + 1], G[4 * q + 2], G[4 * q + 3]);
+                }
+                wave_lds_sync();
+                float4* d4 = (float4*)(dst - (size_t)lane * (2 * CT));  // record of the wavefront's first pixel
 #pragma unroll
-            for (int q = 0; q < CT / 4; ++q)
-                d4[CT / 4 + q] = make_float4(G[4 * q], G[4 * q + 1], G[4 * q + 2], G[4 * q + 3]);
+                for (int k = 0; k < V; ++k) d4[k * 64 + lane] = sw[k * 64 + lane];
+            }
+            else
+            {
+                float4* d4 = (float4*)dst;
+#pragma unroll
+                for (int q = 0; q < CT / 4; ++q) d4[q] = make_float4(I[4 * q], I[4 * q + 1], I[4 * q + 2], I[4 * q + 3]);
+#pragma unroll
+                for (int q = 0; q < CT / 4; ++q)
+                    d4[CT / 4 + q] = make_float4(G[4 * q], G[4 * q + 1], G[4 * q + 2], G[4 * q + 3]);
+            }
         }
         else
         {
@@ -139,16 +168,28 @@ __global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const
 
     const int i  = blockIdx.x * kBlock + threadIdx.x;
     bool valid   = i < pc.n;
-    float4 P     = valid ? pc.position[i] : make_float4(0, 0, 0, 0);
-    V3 pos       = {P.x, P.y, P.z};
-    V3 nrm       = {0, 0, 0};
-    if (valid && pc.normal) nrm = unpack_normal10(pc.normal[i]);
     bool drop_out = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;
-    V2 ip;
-    V3 view_p;
-    float z, radius_pixels;
-    bool ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff, lv.l[0].w,
-                                     &ip, &z, &radius_pixels, &view_p);
+    V2 ip = {0.f, 0.f};
+    float z = 0.f, radius_pixels = 0.f;
+    bool ok;
+    if (pc.cache)  // kernel-uniform: the forward pass left the projected points with the caller
+    {
+        const float4 R = valid ? pc.cache[(size_t)b * pc.n + i] : make_float4(0, 0, 0, 0);
+        ip             = {R.x, R.y};
+        z              = R.z;
+        radius_pixels  = R.w;
+        ok             = valid && z != 0;
+    }
+    else
+    {
+        float4 P = valid ? pc.position[i] : make_float4(0, 0, 0, 0);
+        V3 pos   = {P.x, P.y, P.z};
+        V3 nrm   = {0, 0, 0};
+        if (valid && pc.normal) nrm = unpack_normal10(pc.normal[i]);
+        V3 view_p;
+        ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff, lv.l[0].w,
+                                    &ip, &z, &radius_pixels, &view_p);
+    }
     int tex_index = identity_index ? i : (valid ? pc.index[i] : 0);
     ok            = ok && (unsigned)tex_index < (unsigned)pc.num_texels;
 
@@ -310,8 +351,10 @@ __global__ __launch_bounds__(kBlock) void queue_scan_kernel(const uint32_t* __re
     if (threadIdx.x == kBlock - 1) prefix[kNumQueues] = base + acc;
 }
 
+// 4 waves per SIMD (<= 128 VGPRs): the grid of kPartialBlocks = 4 workgroups x 256 CUs is then resident at once; with
+// the 151 VGPRs the compiler takes by itself only 3 fit and a quarter of the grid runs as a second, mostly idle round.
 template <int CT, bool HALF>
-__global__ __launch_bounds__(kBlock) void backward_ghost_kernel(CloudArg pc, const ViewConst* __restrict__ views,
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) void backward_ghost_kernel(CloudArg pc, const ViewConst* __restrict__ views,
                                                                  Levels lv, ParamArg rp, const float* __restrict__ ig,
                                                                  float* __restrict__ gpoints,
                                                                  float* __restrict__ gpoints_count, int want_pose,

@@ -1,0 +1,254 @@
+// binned_kernels.hip — forward pass through screen-space tile bins (gfx950).
+//
+// The direct forward (prepass_kernel + blend_kernel) issues ~5 M device-scope atomics per 10 M-point frame and spends
+// most of its vector instructions merging lanes by pixel.  Here every point is first sorted into the bin of the
+// screen tile it falls in; the per-tile kernels (tile_kernels.hip) then work in LDS.
+//
+//   bin_count       per point: projection (kept in the point cache), number of bin entries per screen tile
+//   tile_scan       exclusive prefix sum of the tile counts
+//   bin_scatter     per point: reads the point cache, writes a 16-byte entry (level-0 image point, depth, point id |
+//                   flags) into the bin of the tile that owns its level-0 pixel, and into the tile that owns its
+//                   level-1 pixel when that is another one (levels are not nested: pixel = rint(ip * 0.5^l))
+// The entries of a wavefront are appended with one returning atomic per distinct tile (Morton-ordered clouds put a
+// wavefront's points into one to three tiles), so the bins hold runs of consecutive point ids.
+#include <stdlib.h>
+
+#include "common.h"
+#include "launch.h"
+
+#pragma clang fp contract(off)
+
+namespace adop
+{
+constexpr uint32_t kNoTile       = 0xFFFFFFFFu;
+
+// Pixels of every level -> does the point touch the image at all, how many levels precede the LOD break, the tile
+// of its primary entry (tile of the level-0 pixel, clamped into the image; the primary entry also carries the
+// coarse levels) and the tile of a second entry when the level-1 pixel belongs to another tile.
+__device__ __forceinline__ void entry_tiles(const Levels& lv, const ParamArg& rp, const BinArg& bin, int b, bool ok,
+                                            V2 ip, float radius_pixels, bool* in_out, bool* any_in, uint32_t* nlev,
+                                            uint32_t* ptile, uint32_t* xtile)
+{
+    int px[ADOP_MAX_LAYERS], py[ADOP_MAX_LAYERS];
+    bool in[ADOP_MAX_LAYERS];
+    bool alive = ok;
+    *any_in    = false;
+    *nlev      = 0;
+#pragma unroll
+    for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+    {
+        px[l] = py[l] = 0;
+        in[l]         = false;
+        if (l < lv.num)
+        {
+            if (rp.drop_by_radius && radius_pixels < rp.drop_threshold) alive = false;  // break, :261-264
+            if (alive) *nlev = l + 1;
+            const LevelArg& L = lv.l[l];
+            px[l]             = f2i_rn(ip.x);
+            py[l]             = f2i_rn(ip.y);
+            in[l] = alive && (unsigned)px[l] < (unsigned)L.w && (unsigned)py[l] < (unsigned)L.h;
+            *any_in |= in[l];
+            radius_pixels *= 0.5f;
+            ip.x *= 0.5f;
+            ip.y *= 0.5f;
+        }
+        if (in_out) in_out[l] = in[l];
+    }
+    const int tiles_per_view = bin.tiles_x * bin.tiles_y;
+    const int ts             = bin.ts;
+    int cx = px[0] < 0 ? 0 : (px[0] >= lv.l[0].w ? lv.l[0].w - 1 : px[0]);
+    int cy = py[0] < 0 ? 0 : (py[0] >= lv.l[0].h ? lv.l[0].h - 1 : py[0]);
+    *ptile = (uint32_t)(b * tiles_per_view + (cy >> ts) * bin.tiles_x + (cx >> ts));
+    *xtile = kNoTile;
+    if (bin.lt > 1 && in[1])
+    {
+        uint32_t t1 = (uint32_t)(b * tiles_per_view + (py[1] >> (ts - 1)) * bin.tiles_x + (px[1] >> (ts - 1)));
+        if (t1 != *ptile) *xtile = t1;
+    }
+}
+
+// First pass over the points: projection (kept in the point cache) and the number of entries per tile.
+__global__ __launch_bounds__(kBlock) void bin_count_kernel(CloudArg pc, const ViewConst* __restrict__ views, Levels lv,
+                                                           ParamArg rp, BinArg bin, adop_stats* stats)
+{
+    __shared__ unsigned long long s_gmask[kBlock];
+    __shared__ uint32_t s_gkey[kBlock];
+    const bool STATS = stats != nullptr;  // counter pass (uniform branch)
+    const int lane   = threadIdx.x & 63;
+    const int wbase  = threadIdx.x & ~63;
+    unsigned long long* gmask_w = s_gmask + wbase;
+    uint32_t* gkey_w            = s_gkey + wbase;
+
+    const int i      = blockIdx.x * kBlock + threadIdx.x;
+    const bool valid = i < pc.n;
+    float4 P         = valid ? pc.position[i] : make_float4(0, 0, 0, 0);
+    int32_t nenc     = (valid && pc.normal) ? pc.normal[i] : 0;
+    V3 pos           = {P.x, P.y, P.z};
+    V3 nrm           = unpack_normal10(nenc);
+    bool tex_ok      = true;
+    if (STATS)
+    {
+        int tex_index = valid ? pc.index[i] : 0;
+        tex_ok        = (unsigned)tex_index < (unsigned)pc.num_texels;
+    }
+
+    for (int b = 0; b < lv.B; ++b)
+    {
+        const ViewConst& vc = views[b];
+        V2 ip = {0.f, 0.f};
+        V3 view_p;
+        float z = 0.f, radius_pixels = 0.f;
+        bool ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff,
+                                         lv.l[0].w, &ip, &z, &radius_pixels, &view_p);
+        // the second pass (and the backward pass, if the caller keeps the buffer) read this instead of projecting
+        if (valid) pc.cache[(size_t)b * pc.n + i] = ok ? make_float4(ip.x, ip.y, z, radius_pixels) : make_float4(0, 0, 0, 0);
+        if (STATS)
+        {
+            bool dropped = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;
+            stat_add(&stats->bad_index, ok && !dropped && !tex_ok);
+        }
+        if (!__ballot(ok) && !STATS) continue;  // wavefront-uniform
+
+        bool in[ADOP_MAX_LAYERS];
+        bool any_in;
+        uint32_t nlev, ptile, xtile;
+        entry_tiles(lv, rp, bin, b, ok, ip, radius_pixels, in, &any_in, &nlev, &ptile, &xtile);
+        if (STATS)
+        {
+#pragma unroll
+            for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+                if (l < lv.num) stat_add(&stats->visible[l], in[l]);
+        }
+        if (!__ballot(any_in)) continue;
+        wave_lds_sync();
+        int G = wave_group_by_key(any_in, ptile, gkey_w, gmask_w);
+        wave_lds_sync();
+        if (lane < G) atomicAdd(&bin.count[(size_t)gkey_w[lane] * kBinStride], (uint32_t)__popcll(gmask_w[lane]));
+        if (xtile != kNoTile) atomicAdd(&bin.count[(size_t)xtile * kBinStride], 1u);
+    }
+}
+
+// Second pass: PPT points per thread, so that the cache loads, the slot reservations (one returning atomic per
+// distinct tile of a wavefront) and the entry stores of PPT runs of 64 points are in flight together — the kernel
+// is a chain of three dependent memory round trips.
+template <int PPT>
+__global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels lv, ParamArg rp, BinArg bin)
+{
+    __shared__ unsigned long long s_gmask[PPT][kBlock];
+    __shared__ uint32_t s_gkey[PPT][kBlock];
+    __shared__ uint32_t s_gbase[PPT][kBlock];
+    const int lane  = threadIdx.x & 63;
+    const int wbase = threadIdx.x & ~63;
+    const int base  = blockIdx.x * (kBlock * PPT) + threadIdx.x;
+
+    for (int b = 0; b < lv.B; ++b)
+    {
+        float4 R[PPT];
+        float drop[PPT];
+#pragma unroll
+        for (int k = 0; k < PPT; ++k)
+        {
+            const int i = base + k * kBlock;
+            R[k]        = i < pc.n ? pc.cache[(size_t)b * pc.n + i] : make_float4(0, 0, 0, 0);
+            drop[k]     = (i < pc.n && pc.dropout) ? pc.dropout[(size_t)b * pc.n + i] : 0.f;
+        }
+        bool any_in[PPT];
+        uint32_t nlev[PPT], ptile[PPT], xtile[PPT], gslot[PPT], xslot[PPT];
+        int mine[PPT], G[PPT];
+#pragma unroll
+        for (int k = 0; k < PPT; ++k)
+        {
+            V2 ip = {R[k].x, R[k].y};
+            entry_tiles(lv, rp, bin, b, R[k].z != 0, ip, R[k].w, nullptr, &any_in[k], &nlev[k], &ptile[k], &xtile[k]);
+            G[k]     = wave_group_by_key(any_in[k], ptile[k], s_gkey[k] + wbase, s_gmask[k] + wbase, &mine[k]);
+            gslot[k] = 0;
+            xslot[k] = 0;
+        }
+        wave_lds_sync();
+#pragma unroll
+        for (int k = 0; k < PPT; ++k)
+        {
+            if (lane < G[k])
+                gslot[k] = atomicAdd(&bin.cursor[(size_t)s_gkey[k][wbase + lane] * kBinStride],
+                                     (uint32_t)__popcll(s_gmask[k][wbase + lane]));
+            if (xtile[k] != kNoTile) xslot[k] = atomicAdd(&bin.cursor[(size_t)xtile[k] * kBinStride], 1u);
+        }
+#pragma unroll
+        for (int k = 0; k < PPT; ++k)
+            if (lane < G[k]) s_gbase[k][wbase + lane] = gslot[k];
+        wave_lds_sync();
+#pragma unroll
+        for (int k = 0; k < PPT; ++k)
+        {
+            const int i         = base + k * kBlock;
+            const float z       = R[k].z;
+            const float zs      = drop[k] == 1.f ? -z : z;  // z > 0: the sign carries the dropout flag (:314-315)
+            const uint32_t word = (uint32_t)i | (nlev[k] << 28);
+            if (any_in[k])
+            {
+                const unsigned long long m = s_gmask[k][wbase + mine[k]];
+                const uint32_t slot        = s_gbase[k][wbase + mine[k]] + (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
+                bin.entries[slot] = make_float4(R[k].x, R[k].y, zs, __uint_as_float(word | kEntryPrimary));
+            }
+            if (xtile[k] != kNoTile) bin.entries[xslot[k]] = make_float4(R[k].x, R[k].y, zs, __uint_as_float(word));
+        }
+        wave_lds_sync();  // the group tables are reused by the next view
+    }
+}
+
+// Exclusive prefix sum of the tile counts (one workgroup): offset[0..T], cursor[t] = offset[t].
+__global__ __launch_bounds__(1024) void tile_scan_kernel(const uint32_t* __restrict__ count, uint32_t* __restrict__ offset,
+                                                         uint32_t* __restrict__ cursor, int T)
+{
+    __shared__ uint32_t s_wave[16];
+    const int tid = threadIdx.x;
+    const int per = (T + 1023) / 1024;
+    const int t0  = tid * per;
+    uint32_t sum  = 0;
+    for (int k = 0; k < per; ++k)
+        if (t0 + k < T) sum += count[(size_t)(t0 + k) * kBinStride];
+    // inclusive scan inside the wavefront, then over the 16 wavefronts
+    uint32_t inc = sum;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1)
+    {
+        uint32_t v = __shfl_up(inc, off, 64);
+        if ((tid & 63) >= off) inc += v;
+    }
+    if ((tid & 63) == 63) s_wave[tid >> 6] = inc;
+    __syncthreads();
+    uint32_t base = 0;
+    for (int w = 0; w < (tid >> 6); ++w) base += s_wave[w];
+    uint32_t run = base + inc - sum;
+    for (int k = 0; k < per; ++k)
+        if (t0 + k < T)
+        {
+            offset[t0 + k]                      = run;
+            cursor[(size_t)(t0 + k) * kBinStride] = run;
+            run += count[(size_t)(t0 + k) * kBinStride];
+        }
+    if (tid == 1023) offset[T] = base + inc;
+}
+
+// ------------------------------------------------------------------------------------------------
+// launchers
+// ------------------------------------------------------------------------------------------------
+void launch_bin(int pass, const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp,
+                const BinArg& bin, adop_stats* stats, hipStream_t st)
+{
+    if (pc.n < 1) return;
+    constexpr int PPT = 4;
+    if (pass == 0)
+        hipLaunchKernelGGL(bin_count_kernel, dim3((pc.n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, pc, views, lv, rp,
+                           bin, stats);
+    else
+        hipLaunchKernelGGL((bin_scatter_kernel<PPT>), dim3((pc.n + kBlock * PPT - 1) / (kBlock * PPT)), dim3(kBlock), 0,
+                           st, pc, lv, rp, bin);
+}
+
+void launch_tile_scan(const BinArg& bin, int num_tiles, hipStream_t st)
+{
+    hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, st, bin.count, bin.offset, bin.cursor, num_tiles);
+}
+
+}  // namespace adop

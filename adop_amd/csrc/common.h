@@ -13,16 +13,13 @@ namespace adop
 {
 constexpr int kBlock         = 256;
 constexpr int kMaxChannels   = 16;
-constexpr int kPartialBlocks = 1024;  // grid of the grid-stride kernels that write per-block partial sums
+constexpr int kPartialBlocks = 1024;  // grid of backward_ghost_kernel: per-block partial sums of the pose / intrinsics gradients
+constexpr int kBgBlocks      = 2048;  // grid of interleave_kernel: per-block partial sums of the background gradient
 constexpr int kPartialStride = 24;    // doubles per (block, view), 21 used: 6 pose, pose count, intr count, 13 intr
 constexpr int kAcc           = 21;
 constexpr int kNumQueues     = 2048;  // sub-queues of the backward work queue (multiple of kBlock)
 constexpr int kMaxIntrinsicsCols = 24;  // 13 pinhole / 5 affine + up to 19 polynomial coefficients
 constexpr uint64_t kClearPacked = (uint64_t(0x47C35000u) << 32) | 0xFFFFFFFFull;  // bits(100000.f), PointRenderer.cu:1045
-
-// Workgroup-local pre-reduction table (LDS): open addressing, linear probing.
-constexpr int kMaxProbe       = 24;
-constexpr uint32_t kEmptyKey  = 0xFFFFFFFFu;
 
 struct LevelArg
 {
@@ -54,6 +51,7 @@ struct CloudArg
     int32_t num_texels;
     const float* intrinsics;
     const float* dropout;  // [B,N] or null
+    float4* cache;         // [B,N] projected points (ip.x, ip.y, depth or 0, LOD radius in pixels) or null
 };
 
 struct ParamArg
@@ -104,32 +102,43 @@ __device__ __forceinline__ float tex_fetch(const void* tex, size_t o)
     return ((const float*)tex)[o];
 }
 
-template <int BITS>
-__device__ __forceinline__ uint32_t table_hash(uint32_t key)
+// LDS written by some lanes of a wavefront is read by other lanes of the same wavefront: DS operations of one
+// wavefront execute in order, so only the compiler has to be kept from moving accesses across this point.
+__device__ __forceinline__ void wave_lds_sync()
 {
-    return (key * 0x9E3779B1u) >> (32 - BITS);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// Finds or creates the slot of `key`.  New slots are appended to used[] (count in *used_count).
-// Returns -1 when no slot is found within kMaxProbe probes (caller falls back to a direct global atomic).
-template <int BITS>
-__device__ __forceinline__ int table_insert(uint32_t* keys, uint16_t* used, uint32_t* used_count, uint32_t key)
+// Groups the lanes of a wavefront by key.  Lanes with active == false are ignored.  For every distinct key, in
+// order of its first lane, writes gkey[g] and the 64-bit lane mask gmask[g]; returns the number of groups.
+// *mine (if not null) receives the group of the calling lane (-1 for inactive lanes).
+// (gfx950 has no match-any instruction: one ballot per distinct key.)
+__device__ __forceinline__ int wave_group_by_key(bool active, uint32_t key, uint32_t* gkey, unsigned long long* gmask,
+                                                 int* mine = nullptr)
 {
-    uint32_t slot = table_hash<BITS>(key);
-#pragma unroll 1
-    for (int probe = 0; probe < kMaxProbe; ++probe)
+    const int lane               = threadIdx.x & 63;
+    unsigned long long remaining = __ballot(active);
+    int g                        = 0;
+    int my                       = -1;
+    while (remaining)
     {
-        uint32_t old = atomicCAS(&keys[slot], kEmptyKey, key);
-        if (old == kEmptyKey)
+        int leader           = __ffsll((long long)remaining) - 1;
+        uint32_t k           = (uint32_t)__builtin_amdgcn_readlane((int)key, leader);
+        bool hit             = active && key == k;
+        unsigned long long m = __ballot(hit);
+        if (hit) my = g;
+        if (lane == leader)
         {
-            uint32_t e = atomicAdd(used_count, 1u);
-            used[e]    = (uint16_t)slot;
-            return (int)slot;
+            gkey[g]  = k;
+            gmask[g] = m;
         }
-        if (old == key) return (int)slot;
-        slot = (slot + 1) & ((1u << BITS) - 1);
+        remaining &= ~m;
+        ++g;
     }
-    return -1;
+    if (mine) *mine = my;
+    return g;
 }
 
 // d_render_params.Pose() / PinholeIntrinsics() / OcamIntrinsics() (PointRenderer.cu:73-96) for one view.

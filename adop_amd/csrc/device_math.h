@@ -288,6 +288,13 @@ __device__ __forceinline__ bool project_point(const ViewConst& vc, const float* 
             V3 view_n = quat_rotate(vc.qx, vc.qy, vc.qz, vc.qw, nrm);
             if (dot3(view_p, view_n) > 0) z = 0;
         }
+        // culled: nothing below can bring the point back; Morton-ordered clouds cull whole wavefronts here
+        if (z == 0)
+        {
+            *z_out         = 0;
+            *radius_pixels = 0;
+            return false;
+        }
         float iz  = 1.0f / view_p.z;
         V2 norm_p = {view_p.x * iz, view_p.y * iz};
         V2 dist_p = distort<false>(norm_p, vc.d, dist_cutoff, nullptr, nullptr);

@@ -35,16 +35,19 @@ __global__ void fill_u32_kernel(uint32_t* __restrict__ p, size_t n, uint32_t v)
 }
 
 // InitializeData (PointRenderer.cu:1039-1090): packed depth|index of every level, and the blend accumulators.
-__global__ __launch_bounds__(kBlock) void clear_kernel(Levels lv, float4* __restrict__ accum, size_t accum_vec4)
+// Levels below first_level are left alone (the tile path writes them itself).
+__global__ __launch_bounds__(kBlock) void clear_kernel(Levels lv, int first_level, float4* __restrict__ accum,
+                                                       size_t accum_vec4)
 {
-    int per_image = lv.pix_prefix[lv.num];
+    int r0        = lv.pix_prefix[first_level];
+    int per_image = lv.pix_prefix[lv.num] - r0;
     size_t total  = (size_t)per_image * lv.B;
     size_t stride = (size_t)gridDim.x * blockDim.x;
     size_t t0     = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     for (size_t t = t0; t < total; t += stride)
     {
         int b             = (int)(t / per_image);
-        int r             = (int)(t - (size_t)b * per_image);
+        int r             = r0 + (int)(t - (size_t)b * per_image);
         int l             = level_of(lv, r);
         const LevelArg& L = lv.l[l];
         int p             = r - lv.pix_prefix[l];
@@ -59,39 +62,6 @@ __device__ __forceinline__ void depth_min_global(uint64_t* dst, uint64_t pk)
     // early-z (PointRenderer.cu:278): a stale value only costs a redundant atomic
     uint64_t cur = __builtin_nontemporal_load(dst);
     if (pk < cur) atomicMin((unsigned long long*)dst, (unsigned long long)pk);
-}
-
-// LDS written by some lanes of a wavefront is read by other lanes of the same wavefront: DS operations of one
-// wavefront execute in order, so only the compiler has to be kept from moving accesses across this point.
-__device__ __forceinline__ void wave_lds_sync()
-{
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
-// Groups the lanes of a wavefront by key.  Lanes with active == false are ignored.  For every distinct key, in
-// order of its first lane, writes gkey[g] and the 64-bit lane mask gmask[g]; returns the number of groups.
-// (gfx950 has no match-any instruction: one ballot per distinct key.)
-__device__ __forceinline__ int wave_group_by_key(bool active, uint32_t key, uint32_t* gkey, unsigned long long* gmask)
-{
-    const int lane                 = threadIdx.x & 63;
-    unsigned long long remaining = __ballot(active);
-    int g                          = 0;
-    while (remaining)
-    {
-        int leader            = __ffsll((long long)remaining) - 1;
-        uint32_t k            = (uint32_t)__builtin_amdgcn_readlane((int)key, leader);
-        unsigned long long m = __ballot(active && key == k);
-        if (lane == leader)
-        {
-            gkey[g]  = k;
-            gmask[g] = m;
-        }
-        remaining &= ~m;
-        ++g;
-    }
-    return g;
 }
 
 // DepthPrepassMulti (PointRenderer.cu:203-301) on the packed buffer the reference keeps as "old rendering"
@@ -142,11 +112,13 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
             bool valid = i < pc.n;
             V3 pos     = {P[k].x, P[k].y, P[k].z};
             V3 nrm     = unpack_normal10(nenc[k]);
-            V2 ip;
+            V2 ip = {0.f, 0.f};
             V3 view_p;
-            float z, radius_pixels;
+            float z = 0.f, radius_pixels = 0.f;
             bool ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P[k].w, rp.check_normal != 0, rp.dist_cutoff,
                                              lv.l[0].w, &ip, &z, &radius_pixels, &view_p);
+            // the blend (and the backward pass, if the caller keeps the buffer) read this instead of projecting again
+            if (valid) pc.cache[(size_t)b * pc.n + i] = ok ? make_float4(ip.x, ip.y, z, radius_pixels) : make_float4(0, 0, 0, 0);
             zz[k]      = z;
             inmask[k]  = 0;
             bool alive = ok;
@@ -250,10 +222,6 @@ __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewCo
 
     int i      = blockIdx.x * kBlock + threadIdx.x;
     bool valid = i < pc.n;
-    float4 P   = valid ? pc.position[i] : make_float4(0, 0, 0, 0);
-    V3 pos     = {P.x, P.y, P.z};
-    V3 nrm     = {0, 0, 0};
-    if (valid && pc.normal) nrm = unpack_normal10(pc.normal[i]);
     int tex_index = valid ? pc.index[i] : 0;
     bool tex_ok   = (unsigned)tex_index < (unsigned)pc.num_texels;  // device assert :362
     const float accept = rp.depth_accept + 1;
@@ -262,13 +230,12 @@ __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewCo
     for (int b = 0; b < lv.B; ++b)
     {
         bool dropped = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;  // :314-315
-        const ViewConst& vc = views[b];
-        V2 ip;
-        V3 view_p;
-        float z, radius_pixels;
-        bool ok = valid && !dropped &&
-                  project_point(vc, pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff, lv.l[0].w, &ip,
-                                &z, &radius_pixels, &view_p);
+        // projected by the depth prepass of this call
+        const float4 R = valid ? pc.cache[(size_t)b * pc.n + i] : make_float4(0, 0, 0, 0);
+        V2 ip          = {R.x, R.y};
+        const float z  = R.z;
+        float radius_pixels = R.w;
+        bool ok = valid && !dropped && z != 0;
         if (STATS) stat_add(&stats->bad_index, ok && !tex_ok);
         ok = ok && tex_ok;
         if (!__ballot(ok) && !STATS) continue;  // wavefront-uniform
@@ -387,19 +354,20 @@ __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewCo
 // CombineAndFill (:726-754) + CreateMask (:828-847) + the f32 depth the reference saves for backward.
 // Reads the pixel-major accumulators, writes the planar [B,C,h,w] image, weight, depth and mask.
 template <int CT>
-__global__ __launch_bounds__(kBlock) void resolve_kernel(Levels lv, const float* __restrict__ accum, int S,
-                                                         const float* __restrict__ background, int write_mask,
+__global__ __launch_bounds__(kBlock) void resolve_kernel(Levels lv, int first_level, const float* __restrict__ accum,
+                                                         int S, const float* __restrict__ background, int write_mask,
                                                          float mask_value)
 {
     constexpr int CMAX = CT ? CT : kMaxChannels;
     const int C        = CT ? CT : lv.C;
-    int per_image      = lv.pix_prefix[lv.num];
+    int r0             = lv.pix_prefix[first_level];
+    int per_image      = lv.pix_prefix[lv.num] - r0;
     size_t total       = (size_t)per_image * lv.B;
     size_t stride      = (size_t)gridDim.x * blockDim.x;
     for (size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride)
     {
         int b             = (int)(t / per_image);
-        int r             = (int)(t - (size_t)b * per_image);
+        int r             = r0 + (int)(t - (size_t)b * per_image);
         int l             = level_of(lv, r);
         const LevelArg& L = lv.l[l];
         int p             = r - lv.pix_prefix[l];
@@ -456,9 +424,9 @@ void launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t st)
     hipLaunchKernelGGL(fill_u32_kernel, dim3(grid), dim3(kBlock), 0, st, p, n, v);
 }
 
-void launch_clear(const Levels& lv, int grid, float* accum, size_t accum_floats, hipStream_t st)
+void launch_clear(const Levels& lv, int first_level, int grid, float* accum, size_t accum_floats, hipStream_t st)
 {
-    hipLaunchKernelGGL(clear_kernel, dim3(grid), dim3(kBlock), 0, st, lv, (float4*)accum, accum_floats / 4);
+    hipLaunchKernelGGL(clear_kernel, dim3(grid), dim3(kBlock), 0, st, lv, first_level, (float4*)accum, accum_floats / 4);
 }
 
 void launch_prepass(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, adop_stats* stats,
@@ -504,18 +472,18 @@ void launch_blend(const CloudArg& pc, const ViewConst* views, const Levels& lv, 
              : launch_blend_t<0, false>(pc, views, lv, rp, accum, S, stats, st);
 }
 
-void launch_resolve(const Levels& lv, int grid, const float* accum, int S, const float* background, int write_mask,
-                    float mask_value, hipStream_t st)
+void launch_resolve(const Levels& lv, int first_level, int grid, const float* accum, int S, const float* background,
+                    int write_mask, float mask_value, hipStream_t st)
 {
     if (lv.C == 8)
-        hipLaunchKernelGGL((resolve_kernel<8>), dim3(grid), dim3(kBlock), 0, st, lv, accum, S, background, write_mask,
-                           mask_value);
+        hipLaunchKernelGGL((resolve_kernel<8>), dim3(grid), dim3(kBlock), 0, st, lv, first_level, accum, S, background,
+                           write_mask, mask_value);
     else if (lv.C == 4)
-        hipLaunchKernelGGL((resolve_kernel<4>), dim3(grid), dim3(kBlock), 0, st, lv, accum, S, background, write_mask,
-                           mask_value);
+        hipLaunchKernelGGL((resolve_kernel<4>), dim3(grid), dim3(kBlock), 0, st, lv, first_level, accum, S, background,
+                           write_mask, mask_value);
     else
-        hipLaunchKernelGGL((resolve_kernel<0>), dim3(grid), dim3(kBlock), 0, st, lv, accum, S, background, write_mask,
-                           mask_value);
+        hipLaunchKernelGGL((resolve_kernel<0>), dim3(grid), dim3(kBlock), 0, st, lv, first_level, accum, S, background,
+                           write_mask, mask_value);
 }
 
 }  // namespace adop

@@ -14,13 +14,36 @@ struct EnvLevels
 void launch_prepare_views(const ViewChunk& ch, int first, int count, const double* poses, const float* intrinsics,
                           int cols, ViewConst* out, hipStream_t st);
 void launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t st);
-void launch_clear(const Levels& lv, int grid, float* accum, size_t accum_floats, hipStream_t st);
+void launch_clear(const Levels& lv, int first_level, int grid, float* accum, size_t accum_floats, hipStream_t st);
 void launch_prepass(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, adop_stats* stats,
                     hipStream_t st);
 void launch_blend(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
                   float* accum, int S, adop_stats* stats, hipStream_t st);
-void launch_resolve(const Levels& lv, int grid, const float* accum, int S, const float* background, int write_mask,
-                    float mask_value, hipStream_t st);
+void launch_resolve(const Levels& lv, int first_level, int grid, const float* accum, int S, const float* background,
+                    int write_mask, float mask_value, hipStream_t st);
+
+// Forward pass through screen-space tile bins (binned_kernels.hip).
+constexpr int kBinStride = 16;  // uint32 per tile counter
+struct BinArg
+{
+    uint32_t* count;   // [T * kBinStride] entries per tile; one counter per 64-byte line: atomics that share a
+                       // line are serialised at the memory side (~25 ns each)
+    uint32_t* offset;  // [T + 1] exclusive prefix sum
+    uint32_t* cursor;  // [T * kBinStride] next free slot while the bins are filled
+    float4* entries;   // (ip.x, ip.y, +-depth, point id | flags), at most lt per point and view
+    int32_t tiles_x, tiles_y;  // tiles of one view
+    int32_t ts;                // log2 of the tile width in level-0 pixels
+    int32_t lt;                // levels rendered in the tile's LDS (1 or 2); the others go through global atomics
+};
+constexpr uint32_t kEntryIdMask  = 0x0FFFFFFFu;  // entry word: point id; bits 28..30: levels before the LOD break;
+constexpr uint32_t kEntryPrimary = 0x80000000u;  // bit 31: entry of the tile that owns the (clamped) level-0 pixel
+void launch_bin(int pass, const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp,
+                const BinArg& bin, adop_stats* stats, hipStream_t st);
+void launch_tile_scan(const BinArg& bin, int num_tiles, hipStream_t st);
+void launch_tile_depth(const Levels& lv, const BinArg& bin, int num_tiles, hipStream_t st);
+hipError_t launch_tile_blend(const CloudArg& pc, const Levels& lv, const ParamArg& rp, const BinArg& bin, int num_tiles,
+                             bool half, float* accum, int S, const float* background, int write_mask,
+                             float mask_value, int identity_index, adop_stats* stats, hipStream_t st);
 
 void launch_interleave(const Levels& lv, int blocks, float* ig, double* partial, hipStream_t st);
 // Work queue of the backward pass (points that receive a ghost / spatial gradient), split in kNumQueues sub-queues

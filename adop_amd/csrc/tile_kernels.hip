@@ -1,0 +1,571 @@
+// tile_kernels.hip — the two per-tile kernels of the binned forward pass (gfx950).
+//
+// One workgroup owns one screen tile of 16 x 16 level-0 pixels and the bin of 16-byte entries bin_kernel<1> wrote for
+// it.  Counters on MI355X show the direct forward (prepass_kernel, blend_kernel) to be bound by vector instruction
+// issue — the per-wavefront ballot loops that merge lanes by pixel — not by memory.  Here the merge needs no ballots and
+// no float atomics: integer LDS atomics run at 12-25 clocks per wavefront instruction and tolerate lanes that share
+// an address (the native LDS float add takes ~200 clocks, a compare-and-swap add 34 and up).
+//
+//   tile_depth_kernel   ds_min_u64 of (depth bits | point id) into the tile's pixels of every level; the levels < lt
+//                       (owned by the tile) are stored to depth_index, the coarse levels (a window of a few pixels
+//                       shared with the neighbouring tiles) are merged with one global atomicMin per touched pixel
+//   tile_blend_kernel   per batch of entries: fuzzy depth test against the final depth; every accepted (entry, level)
+//                       is pushed on the linked list of its pixel (one LDS exchange), the descriptors are staged in
+//                       LDS, then one thread per pixel walks its list and sums in registers; the levels < lt are
+//                       resolved straight to the output tensors, the coarse windows are added to the global
+//                       pixel-major accumulators (one cache-line atomic per pixel) and resolved by resolve_kernel
+#include <stdlib.h>
+
+#include "common.h"
+#include "launch.h"
+
+#pragma clang fp contract(off)
+
+namespace adop
+{
+// Local layout of the pixels a tile touches: levels < lt are the tile's own 2^(ts-l) squares; a coarser level is
+// the window of ((2^ts - 1) >> l) + 2 pixels per axis that rint(ip * 0.5^l) can reach from the tile.
+struct TileLayout
+{
+    int ox[ADOP_MAX_LAYERS], oy[ADOP_MAX_LAYERS], w[ADOP_MAX_LAYERS], base[ADOP_MAX_LAYERS + 1];
+};
+
+__device__ __forceinline__ TileLayout tile_layout(int tx, int ty, int ts, int lt, int num)
+{
+    TileLayout t;
+    int base = 0;
+#pragma unroll
+    for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+    {
+        t.ox[l] = t.oy[l] = t.w[l] = 0;
+        t.base[l]                  = base;
+        if (l < num)
+        {
+            if (l < lt)
+            {
+                t.ox[l] = tx << (ts - l);
+                t.oy[l] = ty << (ts - l);
+                t.w[l]  = 1 << (ts - l);
+            }
+            else
+            {
+                t.ox[l] = (tx << ts) >> l;
+                t.oy[l] = (ty << ts) >> l;
+                t.w[l]  = (((1 << ts) - 1) >> l) + 2;
+            }
+            base += t.w[l] * t.w[l];
+        }
+    }
+    t.base[ADOP_MAX_LAYERS] = base;
+    return t;
+}
+
+__host__ __device__ inline int tile_pixels(int ts, int lt, int num)
+{
+    int n = 0;
+    for (int l = 0; l < num; ++l)
+    {
+        int w = l < lt ? 1 << (ts - l) : (((1 << ts) - 1) >> l) + 2;
+        n += w * w;
+    }
+    return n;
+}
+
+constexpr int kTileMaxPixels = 1408;  // ts = 5, lt = 2, five levels: 1024 + 256 + 81 + 25 + 9
+
+__global__ __launch_bounds__(kBlock) void tile_depth_kernel(Levels lv, BinArg bin)
+{
+    __shared__ unsigned long long s_depth[kTileMaxPixels];
+    const int tiles_per_view = bin.tiles_x * bin.tiles_y;
+    const int tile           = blockIdx.x;
+    const int b              = tile / tiles_per_view;
+    const int tr             = tile - b * tiles_per_view;
+    const int ty             = tr / bin.tiles_x;
+    const int tx             = tr - ty * bin.tiles_x;
+    const uint32_t start     = bin.offset[tile];
+    const uint32_t end       = bin.offset[tile + 1];
+    const TileLayout T       = tile_layout(tx, ty, bin.ts, bin.lt, lv.num);
+    const int npix           = T.base[ADOP_MAX_LAYERS];
+
+    for (int p = threadIdx.x; p < npix; p += kBlock) s_depth[p] = kClearPacked;
+    __syncthreads();
+
+    for (uint32_t e = start + threadIdx.x; e < end; e += kBlock)
+    {
+        const float4 E       = bin.entries[e];
+        const uint32_t word  = __float_as_uint(E.w);
+        const uint32_t id    = word & kEntryIdMask;
+        const int nlev       = (int)(word >> 28 & 7u);
+        const bool primary   = (word & kEntryPrimary) != 0;
+        const uint32_t zbits = f2u(E.z) & 0x7FFFFFFFu;  // the sign carries the dropout flag
+        const uint64_t pk    = ((uint64_t)zbits << 32) | id;
+        float x = E.x, y = E.y;
+#pragma unroll
+        for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+        {
+            if (l < lv.num)
+            {
+                const LevelArg& L = lv.l[l];
+                int px = f2i_rn(x), py = f2i_rn(y);
+                bool in = l < nlev && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h &&
+                          (l < bin.lt || primary);
+                int cx = px - T.ox[l], cy = py - T.oy[l];
+                bool local = (unsigned)cx < (unsigned)T.w[l] && (unsigned)cy < (unsigned)T.w[l];
+                if (in && local)
+                    atomicMin(&s_depth[T.base[l] + cy * T.w[l] + cx], (unsigned long long)pk);
+                else if (in && l >= bin.lt)  // outside the window (does not happen for in-image points): straight to memory
+                    atomicMin((unsigned long long*)(L.depth_index + (size_t)b * L.w * L.h + (size_t)py * L.w + px),
+                              (unsigned long long)pk);
+                x *= 0.5f;
+                y *= 0.5f;
+            }
+        }
+    }
+    __syncthreads();
+
+#pragma unroll
+    for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+    {
+        if (l < lv.num)
+        {
+            const LevelArg& L = lv.l[l];
+            const int W       = T.w[l];
+            for (int q = threadIdx.x; q < W * W; q += kBlock)
+            {
+                const int cy = q / W, cx = q - cy * W;
+                const int px = T.ox[l] + cx, py = T.oy[l] + cy;
+                if (px < L.w && py < L.h)
+                {
+                    unsigned long long v = s_depth[T.base[l] + q];
+                    uint64_t* dst        = L.depth_index + (size_t)b * L.w * L.h + (size_t)py * L.w + px;
+                    if (l < bin.lt)
+                        *dst = v;  // the tile owns the pixel
+                    else if (v != kClearPacked)
+                        atomicMin((unsigned long long*)dst, v);
+                }
+            }
+        }
+    }
+}
+
+// Buckets of the gather (tile of 16 x 16 level-0 pixels = kBlock threads): bucket p < 256 is level-0 pixel p; the
+// level-1 pixels and the pixels of the coarse windows collect many more entries each, so their lists are split
+// in 2 and 3 parts (an entry picks the part by its batch slot): buckets 256 + 2*q + part and 384 + 3*c + part.
+constexpr int kTileShift    = 4;
+constexpr int kL1Parts      = 2;
+constexpr int kCoarseParts  = 3;
+constexpr int kL1Bucket0    = 256;
+constexpr int kCoarseBucket0 = 384;
+constexpr uint32_t kListEnd = 0xFFFFu;
+
+template <int CT>
+__device__ __forceinline__ void add_staged(float* acc, const float* s_stage, int slot, int C)
+{
+    constexpr int CMAX = CT ? CT : kMaxChannels;
+    if (CT == 8)
+    {
+        const float4* d = (const float4*)(s_stage + slot * 8);
+        float4 u = d[0], v = d[1];
+        acc[0] += u.x; acc[1] += u.y; acc[2] += u.z; acc[3] += u.w;
+        acc[4] += v.x; acc[5] += v.y; acc[6] += v.z; acc[7] += v.w;
+    }
+    else if (CT == 4)
+    {
+        float4 u = *(const float4*)(s_stage + slot * 4);
+        acc[0] += u.x; acc[1] += u.y; acc[2] += u.z; acc[3] += u.w;
+    }
+    else
+    {
+#pragma unroll
+        for (int c = 0; c < CMAX; ++c)
+            if (c < C) acc[c] += s_stage[slot * C + c];
+    }
+}
+
+// K entries per thread and batch (BATCH = K * kBlock, a power of two).
+template <int CT, bool HALF, int K>
+__global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels lv, ParamArg rp, BinArg bin,
+                                                            float* __restrict__ accum, int S,
+                                                            const float* __restrict__ background, int write_mask,
+                                                            float mask_value, int identity_index, adop_stats* stats, int dbg)
+{
+    constexpr int CMAX  = CT ? CT : kMaxChannels;
+    constexpr int BATCH = K * kBlock;
+    constexpr int T0    = 1 << kTileShift;
+    extern __shared__ __align__(16) unsigned char smem[];
+    const bool STATS = stats != nullptr;
+    const int C      = CT ? CT : lv.C;
+    const int tid    = threadIdx.x;
+
+    const int tiles_per_view = bin.tiles_x * bin.tiles_y;
+    const int tile           = blockIdx.x;
+    const int b              = tile / tiles_per_view;
+    const int tr             = tile - b * tiles_per_view;
+    const int ty             = tr / bin.tiles_x;
+    const int tx             = tr - ty * bin.tiles_x;
+    const uint32_t start     = bin.offset[tile];
+    const uint32_t end       = bin.offset[tile + 1];
+    const int lt             = bin.lt;
+    const TileLayout T       = tile_layout(tx, ty, kTileShift, lt, lv.num);
+    const int npix           = T.base[ADOP_MAX_LAYERS];
+    const int first_coarse   = lt > 1 ? T0 * T0 + T0 * T0 / 4 : T0 * T0;  // local pixel index of the first coarse pixel
+    const int ncoarse        = npix - first_coarse;
+
+    float* s_stage   = (float*)smem;                     // [BATCH * C]
+    float* s_depth   = s_stage + BATCH * C;              // [npix] f32 depth of the local pixels
+    uint32_t* s_head = (uint32_t*)(s_depth + npix);      // [2 * kBlock] list heads of the buckets
+    uint16_t* s_next = (uint16_t*)(s_head + 2 * kBlock); // [BATCH * num levels] node = level * BATCH + slot
+
+    float acc0[CMAX + 1], acc1[CMAX + 1];  // bucket tid, bucket kBlock + tid
+#pragma unroll
+    for (int c = 0; c <= CMAX; ++c) acc0[c] = acc1[c] = 0.f;
+
+    if (dbg & 32) return;
+    if (end > start && !(dbg & 64))  // workgroup-uniform
+    {
+        // entries of the first batch: requested together with the depth values below
+        float4 Enext[K];
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+        {
+            const uint32_t e = start + k * kBlock + tid;
+            Enext[k]         = e < end ? bin.entries[e] : make_float4(0, 0, -1.f, 0);
+        }
+        // final depth of the local pixels (tile_depth_kernel has completed)
+#pragma unroll
+        for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+        {
+            if (l < lv.num)
+            {
+                const LevelArg& L = lv.l[l];
+                const int W       = T.w[l];
+                for (int q = tid; q < W * W; q += kBlock)
+                {
+                    const int cy = q / W, cx = q - cy * W;
+                    const int px = T.ox[l] + cx, py = T.oy[l] + cy;
+                    float d = 0.f;
+                    if (px < L.w && py < L.h)
+                        d = __uint_as_float(
+                            ((const uint32_t*)(L.depth_index + (size_t)b * L.w * L.h + (size_t)py * L.w + px))[1]);
+                    s_depth[T.base[l] + q] = d;
+                }
+            }
+        }
+        s_head[tid]          = kListEnd;
+        s_head[kBlock + tid] = kListEnd;
+        __syncthreads();
+
+        const float accept = rp.depth_accept + 1;
+        for (uint32_t b0 = start; b0 < end && !(dbg & 8); b0 += BATCH)  // workgroup-uniform
+        {
+            // -- entries of this thread, their descriptors, and the entries of the next batch (all requested before
+            //    anything waits: a batch is a chain of dependent memory round trips) --------------------------------
+            float4 E[K];
+            float t[K][CMAX];
+            bool ok[K];
+#pragma unroll
+            for (int k = 0; k < K; ++k) E[k] = Enext[k];
+#pragma unroll
+            for (int k = 0; k < K; ++k)
+            {
+                const uint32_t id = __float_as_uint(E[k].w) & kEntryIdMask;
+                ok[k]             = E[k].z > 0;  // dropped points carry -z (:314-315), padding too
+                int tex_index     = 0;
+                if (ok[k]) tex_index = identity_index ? (int)id : pc.index[id];
+                ok[k] = ok[k] && (unsigned)tex_index < (unsigned)pc.num_texels;  // device assert :362
+#pragma unroll
+                for (int c = 0; c < CMAX; ++c) t[k][c] = 0.f;
+                if (ok[k] && !(dbg & 4))
+                {
+#pragma unroll
+                    for (int c = 0; c < CMAX; ++c)
+                        if (c < C) t[k][c] = tex_fetch<HALF>(pc.texture, (size_t)c * pc.num_texels + tex_index);
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < K; ++k)
+            {
+                const uint32_t e = b0 + BATCH + k * kBlock + tid;
+                Enext[k]         = e < end ? bin.entries[e] : make_float4(0, 0, -1.f, 0);
+            }
+            // -- fuzzy depth test per level (:380); an accepted (entry, level) is pushed on the list of its bucket ----
+#pragma unroll
+            for (int k = 0; k < K; ++k)
+            {
+                const int slot      = k * kBlock + tid;
+                const uint32_t word = __float_as_uint(E[k].w);
+                const int nlev      = (int)(word >> 28 & 7u);
+                const bool primary  = (word & kEntryPrimary) != 0;
+                const float z       = E[k].z;
+                float x = E[k].x, y = E[k].y;
+#pragma unroll
+                for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+                {
+                    if (l < lv.num)
+                    {
+                        const LevelArg& L = lv.l[l];
+                        int px = f2i_rn(x), py = f2i_rn(y);
+                        bool in = ok[k] && l < nlev && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h &&
+                                  (l < lt || primary);
+                        int cx = px - T.ox[l], cy = py - T.oy[l];
+                        bool local = (unsigned)cx < (unsigned)T.w[l] && (unsigned)cy < (unsigned)T.w[l];
+                        bool accepted = false;
+                        if (in && local)
+                        {
+                            const int q = cy * T.w[l] + cx;
+                            accepted    = !(z > s_depth[T.base[l] + q] * accept);
+                            if (accepted && !(dbg & 2))
+                            {
+                                int bucket;
+                                if (l == 0)
+                                    bucket = q;
+                                else if (l < lt)
+                                    bucket = kL1Bucket0 + q * kL1Parts + (slot & (kL1Parts - 1));
+                                else
+                                    bucket = kCoarseBucket0 + (T.base[l] - first_coarse + q) * kCoarseParts + slot % kCoarseParts;
+                                const uint32_t node = (uint32_t)(l * BATCH + slot);
+                                uint32_t old = atomicExch(s_head + bucket, node);
+                                s_next[node] = (uint16_t)old;
+                            }
+                        }
+                        else if (in && l >= lt)
+                        {
+                            // outside the window (does not happen for in-image points): blend straight to memory
+                            size_t pix = (size_t)py * L.w + px;
+                            float d    = __uint_as_float(((const uint32_t*)(L.depth_index + (size_t)b * L.w * L.h + pix))[1]);
+                            accepted   = !(z > d * accept);
+                            if (accepted)
+                            {
+                                float* a = accum + (size_t)ws_pixel(lv, l, b, (uint32_t)pix) * S;
+#pragma unroll
+                                for (int c = 0; c < CMAX; ++c)
+                                    if (c < C) unsafeAtomicAdd(a + c, t[k][c]);
+                                unsafeAtomicAdd(a + C, 1.f);
+                            }
+                        }
+                        if (STATS) stat_add(&stats->accepted[l], accepted);
+                        x *= 0.5f;
+                        y *= 0.5f;
+                    }
+                }
+            }
+            // -- descriptors staged by batch slot ----------------------------------------------------------------
+#pragma unroll
+            for (int k = 0; k < K; ++k)
+            {
+                const int slot = k * kBlock + tid;
+                if (ok[k])
+                {
+                    if (CT == 8)
+                    {
+                        float4* d = (float4*)(s_stage + slot * 8);
+                        d[0]      = make_float4(t[k][0], t[k][1], t[k][2], t[k][3]);
+                        d[1]      = make_float4(t[k][4], t[k][5], t[k][6], t[k][7]);
+                    }
+                    else if (CT == 4)
+                        *(float4*)(s_stage + slot * 4) = make_float4(t[k][0], t[k][1], t[k][2], t[k][3]);
+                    else
+                    {
+#pragma unroll
+                        for (int c = 0; c < CMAX; ++c)
+                            if (c < C) s_stage[slot * C + c] = t[k][c];
+                    }
+                }
+            }
+            __syncthreads();
+            // -- gather: every thread walks the lists of its two buckets and empties them ------------------------------
+            {
+                uint32_t node = (dbg & 1) ? kListEnd : s_head[tid];
+                float n       = 0.f;
+                while (node != kListEnd)
+                {
+                    add_staged<CT>(acc0, s_stage, (int)(node & (BATCH - 1)), C);
+                    n += 1.f;
+                    node = s_next[node];
+                }
+                acc0[CMAX] += n;
+                s_head[tid] = kListEnd;
+                node        = (dbg & 1) ? kListEnd : s_head[kBlock + tid];
+                n           = 0.f;
+                while (node != kListEnd)
+                {
+                    add_staged<CT>(acc1, s_stage, (int)(node & (BATCH - 1)), C);
+                    n += 1.f;
+                    node = s_next[node];
+                }
+                acc1[CMAX] += n;
+                s_head[kBlock + tid] = kListEnd;
+            }
+            __syncthreads();
+        }
+    }
+
+    // -- resolve (CombineAndFill :726-754, CreateMask :828-847) ----------------------------------------------------
+    // level 0: bucket tid is pixel tid of the tile
+    if (dbg & 16) return;
+    {
+        const LevelArg& L = lv.l[0];
+        const int px = T.ox[0] + (tid & (T0 - 1)), py = T.oy[0] + (tid >> kTileShift);
+        if (px < L.w && py < L.h)
+        {
+            const float cou  = acc0[CMAX];
+            const size_t hw  = (size_t)L.w * L.h;
+            const size_t pix = (size_t)py * L.w + px;
+            const size_t o   = (size_t)b * hw + pix;
+            L.weight[o]      = cou;
+            L.depth[o]       = end > start ? s_depth[tid] : 100000.f;  // high word of the packed pixel
+            float* out       = L.out + (size_t)b * C * hw + pix;
+#pragma unroll
+            for (int c = 0; c < CMAX; ++c)
+                if (c < C) out[(size_t)c * hw] = (cou == 0) ? background[c] : acc0[c] / cou;
+            if (write_mask && L.mask) L.mask[o] = (cou == 0) ? mask_value : 1.f;
+        }
+    }
+    // level 1: buckets kBlock + 2*q and kBlock + 2*q + 1 (adjacent lanes) are the two parts of pixel q
+    if (lt > 1)
+    {
+#pragma unroll
+        for (int c = 0; c <= CMAX; ++c) acc1[c] += (tid < kCoarseBucket0 - kL1Bucket0) ? __shfl_xor(acc1[c], 1, 64) : 0.f;
+        if (tid < kCoarseBucket0 - kL1Bucket0 && (tid & 1) == 0)
+        {
+            constexpr int T1  = T0 / 2;
+            const LevelArg& L = lv.l[1];
+            const int q       = tid >> 1;
+            const int px = T.ox[1] + (q & (T1 - 1)), py = T.oy[1] + q / T1;
+            if (px < L.w && py < L.h)
+            {
+                const float cou  = acc1[CMAX];
+                const size_t hw  = (size_t)L.w * L.h;
+                const size_t pix = (size_t)py * L.w + px;
+                const size_t o   = (size_t)b * hw + pix;
+                L.weight[o]      = cou;
+                L.depth[o]       = end > start ? s_depth[T0 * T0 + q] : 100000.f;
+                float* out       = L.out + (size_t)b * C * hw + pix;
+#pragma unroll
+                for (int c = 0; c < CMAX; ++c)
+                    if (c < C) out[(size_t)c * hw] = (cou == 0) ? background[c] : acc1[c] / cou;
+                if (write_mask && L.mask) L.mask[o] = (cou == 0) ? mask_value : 1.f;
+            }
+        }
+    }
+    // coarse windows: the parts of a pixel are summed through LDS, then S consecutive lanes add the C sums and the
+    // weight of one pixel to the global accumulators with ONE cache-line atomic
+    if (lt < lv.num && end > start)
+    {
+        float* s_flush = (float*)smem;  // [ncoarse * kCoarseParts * S], reuses the stage: all threads are past the gather
+        const int u    = tid - (kCoarseBucket0 - kL1Bucket0);
+        if (u >= 0 && u < ncoarse * kCoarseParts)
+        {
+            float* f = s_flush + u * S;
+#pragma unroll
+            for (int c = 0; c < CMAX; ++c)
+                if (c < C) f[c] = acc1[c];
+            f[C] = acc1[CMAX];
+        }
+        __syncthreads();
+        for (int i = tid; i < ncoarse * S; i += kBlock)
+        {
+            const int cp = i / S, j = i - cp * S;
+            if (j <= C)
+            {
+                const float* f = s_flush + cp * kCoarseParts * S;
+                const float cou = (f[C] + f[S + C]) + f[2 * S + C];
+                if (cou != 0.f)
+                {
+                    const float v = (f[j] + f[S + j]) + f[2 * S + j];
+                    // level and pixel of coarse pixel cp
+                    int l = lt, r = cp;
+#pragma unroll
+                    for (int k = 2; k < ADOP_MAX_LAYERS; ++k)
+                        if (k > lt && k < lv.num && cp >= T.base[k] - first_coarse)
+                        {
+                            l = k;
+                            r = cp - (T.base[k] - first_coarse);
+                        }
+                    int W = 0, ox = 0, oy = 0, Lw = 0;
+#pragma unroll
+                    for (int k = 1; k < ADOP_MAX_LAYERS; ++k)
+                        if (k == l)
+                        {
+                            W  = T.w[k];
+                            ox = T.ox[k];
+                            oy = T.oy[k];
+                            Lw = lv.l[k].w;
+                        }
+                    const int cy = r / W, cx = r - cy * W;
+                    const uint32_t pix = (uint32_t)((oy + cy) * Lw + (ox + cx));  // in the image: something was blended
+                    unsafeAtomicAdd(accum + (size_t)ws_pixel(lv, l, b, pix) * S + j, v);
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// launchers
+// ------------------------------------------------------------------------------------------------
+void launch_tile_depth(const Levels& lv, const BinArg& bin, int num_tiles, hipStream_t st)
+{
+    hipLaunchKernelGGL(tile_depth_kernel, dim3(num_tiles), dim3(kBlock), 0, st, lv, bin);
+}
+
+template <int K>
+static size_t tile_blend_lds(const Levels& lv, const BinArg& bin, int S)
+{
+    size_t npix   = (size_t)tile_pixels(bin.ts, bin.lt, lv.num);
+    size_t stage  = (size_t)K * kBlock * lv.C * 4;
+    size_t rest   = npix * 4 + 2 * kBlock * 4 + (size_t)K * kBlock * lv.num * 2 + 16;
+    size_t flush  = npix * kCoarseParts * (size_t)S * 4;  // upper bound of the flush area (reuses the LDS from its start)
+    return stage + rest > flush ? stage + rest : flush;
+}
+
+template <int CT, bool HALF, int K>
+static hipError_t launch_tile_blend_k(const CloudArg& pc, const Levels& lv, const ParamArg& rp, const BinArg& bin,
+                                      int num_tiles, float* accum, int S, const float* background, int write_mask,
+                                      float mask_value, int identity_index, adop_stats* stats, hipStream_t st)
+{
+    if (bin.ts != kTileShift || bin.lt > 2) return hipErrorInvalidValue;
+    size_t lds = tile_blend_lds<K>(lv, bin, S);
+    static const int dbg = getenv("ADOP_TILE_DBG") ? atoi(getenv("ADOP_TILE_DBG")) : 0;
+    static size_t allowed = 0;  // largest dynamic LDS size this instantiation has been enabled for
+    if (lds > 65536 && lds > allowed)
+    {
+        hipError_t e = hipFuncSetAttribute((const void*)tile_blend_kernel<CT, HALF, K>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        allowed = lds;
+    }
+    hipLaunchKernelGGL((tile_blend_kernel<CT, HALF, K>), dim3(num_tiles), dim3(kBlock), lds, st, pc, lv, rp, bin,
+                       accum, S, background, write_mask, mask_value, identity_index, stats, dbg);
+    return hipSuccess;
+}
+
+template <int CT, bool HALF>
+static hipError_t launch_tile_blend_t(const CloudArg& pc, const Levels& lv, const ParamArg& rp, const BinArg& bin,
+                                      int num_tiles, float* accum, int S, const float* background, int write_mask,
+                                      float mask_value, int identity_index, adop_stats* stats, hipStream_t st)
+{
+    static const int k = getenv("ADOP_TILE_K") ? atoi(getenv("ADOP_TILE_K")) : 2;
+    if (k == 1)
+        return launch_tile_blend_k<CT, HALF, 1>(pc, lv, rp, bin, num_tiles, accum, S, background, write_mask, mask_value,
+                                                identity_index, stats, st);
+    if (k == 4)
+        return launch_tile_blend_k<CT, HALF, 4>(pc, lv, rp, bin, num_tiles, accum, S, background, write_mask, mask_value,
+                                                identity_index, stats, st);
+    return launch_tile_blend_k<CT, HALF, 2>(pc, lv, rp, bin, num_tiles, accum, S, background, write_mask, mask_value,
+                                            identity_index, stats, st);
+}
+
+hipError_t launch_tile_blend(const CloudArg& pc, const Levels& lv, const ParamArg& rp, const BinArg& bin, int num_tiles,
+                             bool half, float* accum, int S, const float* background, int write_mask,
+                             float mask_value, int identity_index, adop_stats* stats, hipStream_t st)
+{
+#define ADOP_TILE(CT, H) \
+    launch_tile_blend_t<CT, H>(pc, lv, rp, bin, num_tiles, accum, S, background, write_mask, mask_value, identity_index, stats, st)
+    if (lv.C == 8) return half ? ADOP_TILE(8, true) : ADOP_TILE(8, false);
+    if (lv.C == 4) return half ? ADOP_TILE(4, true) : ADOP_TILE(4, false);
+    return half ? ADOP_TILE(0, true) : ADOP_TILE(0, false);
+#undef ADOP_TILE
+}
+
+}  // namespace adop

@@ -223,6 +223,13 @@ std::pair<std::vector<torch::Tensor>, std::vector<torch::Tensor>> BlendPointClou
     adop_render_params rp = MakeParams(info->params);
     adop_forward_buffers fb =
         MakeForwardBuffers(info, di, d, w, cache.output_forward, cache.output_forward_background_mask, cache.dropout_points);
+    // projected points: a saved tensor of the backward pass (no counterpart in the reference, which projects again)
+    torch::Tensor point_cache;
+    if (ctx)
+    {
+        point_cache    = torch::empty({(long)views.size(), (long)scene.num_points, 4}, d[0].options());
+        fb.point_cache = point_cache.data_ptr<float>();
+    }
     Check(adop_forward(&scene, views.data(), (int)views.size(), &rp, &fb, cache.workspace.data_ptr(),
                        (size_t)cache.workspace.numel(), nullptr, CurrentStream()));
 
@@ -239,6 +246,7 @@ std::pair<std::vector<torch::Tensor>, std::vector<torch::Tensor>> BlendPointClou
         save.insert(save.end(), cache.output_forward.begin(), cache.output_forward.end());
         save.push_back(cache.dropout_points.defined() ? cache.dropout_points : torch::empty({0}, d[0].options()));
         for (auto& l : cache.layers_cuda) save.push_back(l.depth_index_tensor);
+        save.push_back(point_cache);
         ctx->save_for_backward(save);
         ctx->saved_data["num_masks"] = (int64_t)cache.output_forward_background_mask.size();
         // the cache buffers are handed to the graph: allocate fresh ones on the next forward
@@ -266,7 +274,7 @@ torch::autograd::variable_list BlendPointCloudBackward(torch::autograd::Autograd
         cache.image_gradients.push_back(_image_gradients[i].contiguous());
     }
     auto saved = ctx->get_saved_variables();
-    TORCH_CHECK((int)saved.size() == L * 4 + 1);
+    TORCH_CHECK((int)saved.size() == L * 4 + 2);
     std::vector<torch::Tensor> di, d, w, out;
     for (int i = 0; i < L; ++i)
     {
@@ -328,6 +336,7 @@ torch::autograd::variable_list BlendPointCloudBackward(torch::autograd::Autograd
     adop_render_params rp = MakeParams(info->params);
     std::vector<torch::Tensor> no_mask;
     adop_forward_buffers fb = MakeForwardBuffers(info, di, d, w, out, no_mask, dropout);
+    fb.point_cache          = saved[L * 4 + 1].data_ptr<float>();
     if (!cache.workspace.defined() ||
         (size_t)cache.workspace.numel() < adop_workspace_size(&s, (int)views.size(), L, views[0].w, views[0].h))
         cache.workspace = torch::empty({(long)adop_workspace_size(&s, (int)views.size(), L, views[0].w, views[0].h)},

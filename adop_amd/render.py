@@ -123,6 +123,9 @@ class NeuralRenderInfo:
     dropout_points: Optional[torch.Tensor] = None
     dropout: float = 0.0
     collect_stats: bool = False
+    # NeuralRenderInfo::train (RenderInfo.h): a backward pass may follow, so the forward pass leaves the projected
+    # points in a tensor of its own (saved like depth / weight) instead of the workspace
+    train: bool = True
 
 
 class PointRendererCache:
@@ -134,6 +137,7 @@ class PointRendererCache:
         self.layers_cuda: List[LayerCuda] = []
         self.cache_size = None
         self.dropout_points = None
+        self.point_cache = None
         self.output_forward = []
         self.output_forward_background_mask = []
         self.workspace = None
@@ -198,6 +202,10 @@ class PointRendererCache:
             self.dropout_points = torch.empty(B, N, dtype=torch.float32, device=dev).bernoulli_(info.dropout)
         else:
             self.dropout_points = None  # zero_() in the reference; nothing is dropped
+        # projected points, saved for the backward pass (handed to the autograd context like the outputs);
+        # without a backward pass the library keeps them in its workspace
+        self.point_cache = (torch.empty(B, N, 4, dtype=torch.float32, device=dev)
+                            if (forward and info.train) else None)
 
     # -- C-ABI structs -----------------------------------------------------------------------
     def forward_struct(self):
@@ -212,6 +220,7 @@ class PointRendererCache:
             S.out = _ptr(self.output_forward[l])
             S.mask = _ptr(self.output_forward_background_mask[l]) if self.output_forward_background_mask else None
         fb.dropout_points = _ptr(self.dropout_points)
+        fb.point_cache = _ptr(self.point_cache)
         return fb
 
     def views_array(self):
@@ -246,6 +255,7 @@ def BlendPointCloudForward(ctx, info):
         save += list(cache.output_forward)
         ctx.save_for_backward(*save)
         ctx.dropout_points = cache.dropout_points
+        ctx.point_cache = cache.point_cache
         ctx.depth_index = [L.depth_index_tensor for L in cache.layers_cuda]
         ctx.masks = list(cache.output_forward_background_mask)
     return list(cache.output_forward), list(cache.output_forward_background_mask)
@@ -275,6 +285,7 @@ def BlendPointCloudBackward(ctx, info, image_gradients, needs=(True, True, True)
         S.depth_index = _ptr(ctx.depth_index[l])
         S.mask = _ptr(ctx.masks[l]) if ctx.masks else None
     fb.dropout_points = _ptr(ctx.dropout_points)
+    fb.point_cache = _ptr(getattr(ctx, "point_cache", None))
 
     need_points, need_pose, need_intr = needs
     N = scene.point_cloud_cuda.Size()

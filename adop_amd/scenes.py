@@ -121,6 +121,7 @@ def default_params(**kw):
     p.output_background_mask = 0
     p.output_background_mask_value = 0.0
     p.normalize_mode = 0
+    p.forward_path = 0
     for k, v in kw.items():
         if not hasattr(p, k):
             raise AttributeError(k)

@@ -25,7 +25,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-KERNEL_OF_STAGE = {"DepthPrepass": "prepass_kernel", "RenderForward": "blend_kernel", "CombineAndFill": "resolve_kernel",
+KERNEL_OF_STAGE = {"BinCount": "bin_count_kernel", "BinScatter": "bin_scatter_kernel", "TileDepth": "tile_depth_kernel", "TileBlend": "tile_blend_kernel",
+                   "DepthPrepass": "prepass_kernel", "RenderForward": "blend_kernel", "CombineAndFill": "resolve_kernel",
                    "CombineAndFillBackward": "interleave_kernel", "RenderBackward/descriptor": "backward_tex_kernel",
                    "RenderBackward/spatial": "backward_ghost_kernel"}
 
@@ -45,6 +46,23 @@ def byte_model(N, B, C_, S_d, P, V, A, G, has_mask, has_dropout):
     return k
 
 
+def tile_path_model(k, N, B, C_, P_levels, V, has_dropout, lt=2):
+    """The same forward bytes attributed to the kernels of the tile-bin path: bin_kernel<0> reads the points,
+    bin_kernel<1> re-reads them (the blend's read), tile_depth_kernel does the depth prepass, tile_blend_kernel
+    the blend and the resolve of the fine levels, resolve_kernel the coarse levels."""
+    drop = 4 if has_dropout else 0
+    lt = min(lt, len(V))
+    frac_coarse = sum(P_levels[lt:]) / float(sum(P_levels))
+    prepass, blend, caf = k.pop("DepthPrepass"), k.pop("RenderForward"), k.pop("CombineAndFill")
+    k["BinCount"] = B * N * 20
+    k["BinScatter"] = B * N * (24 + drop)
+    k["TileDepth"] = sum(V) * 8
+    k["TileBlend"] = (blend - B * N * (24 + drop)) + caf * (1 - frac_coarse)
+    k["CombineAndFill"] = caf * frac_coarse
+    assert abs(sum((k[n] for n in ("BinCount", "BinScatter", "TileDepth", "TileBlend", "CombineAndFill"))) - (prepass + blend + caf)) < 1
+    return k
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -54,6 +72,8 @@ def main():
     ap.add_argument("--points", type=int, default=0, help="override the point count (0 = the configuration's)")
     ap.add_argument("--point-order", default="morton", choices=["morton", "random"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-point-cache", action="store_true",
+                    help="do not keep the projected points for the backward pass (it projects again)")
     ap.add_argument("--cpu-points", type=int, default=0, help="point count of the CPU sample (0 = automatic)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
@@ -90,7 +110,7 @@ def main():
     scene = render.NeuralScene.from_host(hs, dev)
     cache = render.PointRendererCache()
     info = render.NeuralRenderInfo(scene=scene, images=list(hs.views), params=hs.params, num_layers=hs.num_layers,
-                                   cache=cache,
+                                   cache=cache, train=backward and not args.no_point_cache,
                                    dropout_points=None if hs.dropout is None else torch.from_numpy(hs.dropout))
     cache.Build(info, True)
     s = scene.struct()
@@ -176,8 +196,11 @@ def main():
     P = sum(w * h for (w, h) in hs.level_sizes())
     S_d = 2 if hs.texture.dtype == np.float16 else 4
     model = byte_model(N, B, Cn, S_d, P, V, A, G, bool(hs.params.output_background_mask), hs.dropout is not None)
+    if "TileBlend" in stages:
+        model = tile_path_model(model, N, B, Cn, [w * h for (w, h) in hs.level_sizes()], V, hs.dropout is not None)
     if not backward:
-        model = {k: v for k, v in model.items() if k in ("DepthPrepass", "RenderForward", "CombineAndFill")}
+        model = {k: v for k, v in model.items() if k in ("DepthPrepass", "RenderForward", "CombineAndFill", "BinCount",
+                                                         "BinScatter", "TileDepth", "TileBlend")}
     total_bytes = sum(model.values())
     dom = max((k for k in model if k in stages), key=lambda k: stages[k])
     dom_gbs = model[dom] / (stages[dom] * 1e-3) / 1e9
@@ -185,6 +208,8 @@ def main():
     # FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 after calibration with a plain 1 GiB copy); measured for the default
     # workload only
     measured_traffic = {("config3", "RenderForward"): 691.9e6} if not args.points and args.point_order == "morton" else {}
+    if os.environ.get("ADOP_FORWARD_PATH"):
+        measured_traffic = {}
     roofline = {"bound": "hbm", "kernel": KERNEL_OF_STAGE.get(dom, dom), "stage": dom, "achieved": round(dom_gbs, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
                 "traffic": measured_traffic.get((args.workload, dom)),

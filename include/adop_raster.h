@@ -83,6 +83,10 @@ typedef struct adop_render_params
      *    the [N,4] buffer, intrinsics always as 13 floats per row; PointRenderer.cu:1611-1636).
      * 1: row-wise normalisation (points row i by count i, intrinsics over the real row width). */
     int32_t normalize_mode;
+    /* How adop_forward renders (same results either way; no counterpart in the reference):
+     * 0: the library chooses; 1: direct (depth prepass and blend with global atomics, PointRenderer.cu:203-393
+     * as written); 2: through screen-space tile bins (the fine levels are rendered in LDS). */
+    int32_t forward_path;
 } adop_render_params;
 
 /* Inputs owned by NeuralScene: NeuralPointCloudCuda + NeuralTexture + PoseModule + IntrinsicsModule. */
@@ -129,6 +133,12 @@ typedef struct adop_forward_buffers
      * draws it with bernoulli_ inside InitializeData (PointRenderer.cu:1081-1088); here it is an input so
      * that both sides of a parity test see the same mask. */
     const float* dropout_points;
+    /* Optional [B,N,4] f32 (no counterpart in the reference, which projects every point again in each of its
+     * three kernels): per view and point the level-0 image point (x,y), the depth (0 = culled) and the LOD
+     * radius in pixels.  adop_forward writes it; adop_backward reads it instead of projecting when the same
+     * buffer is passed back in `fwd`.  NULL: adop_forward keeps the records in the workspace, adop_backward
+     * projects again. */
+    float* point_cache;
 } adop_forward_buffers;
 
 /* DeviceBackwardParams (PointRenderer.cu:124-137) + the tensors PointRendererCache::Build(.., false)

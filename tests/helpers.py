@@ -9,9 +9,16 @@ def announce(msg):
     sys.stdout.flush()
 
 
-def run_hip_forward(hs, collect_stats=True):
+# adop_render_params.forward_path used by run_hip_forward (0: the library chooses, 1: direct, 2: tile bins);
+# the GPU test modules run every case with 1 and 2.
+FORWARD_PATH = 0
+
+
+def run_hip_forward(hs, collect_stats=True, forward_path=None):
     import torch
     from adop_amd import render
+
+    hs.params.forward_path = FORWARD_PATH if forward_path is None else forward_path
 
     scene = render.NeuralScene.from_host(hs, "cuda")
     cache = render.PointRendererCache()

@@ -9,12 +9,33 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.fixture(scope="module")
-def full():
+def full_scene():
     from adop_amd import scenes
 
-    announce("config3 full size: generate + forward")
-    hs = scenes.config3()
-    return hs, run_hip_forward(hs)
+    announce("config3 full size: generate")
+    return scenes.config3()
+
+
+@pytest.fixture(scope="module", params=[1, 2], ids=["direct", "tiles"])
+def full(request, full_scene):
+    announce(f"config3 full size: forward, forward_path={request.param}")
+    return full_scene, run_hip_forward(full_scene, forward_path=request.param)
+
+
+def test_both_forward_paths_agree(full_scene):
+    """direct and tile-bin forward: packed depth|index, depth and weight bit-identical, images within 1e-5."""
+    import torch
+
+    a = run_hip_forward(full_scene, forward_path=1)
+    b = run_hip_forward(full_scene, forward_path=2)
+    for l, (La, Lb) in enumerate(zip(a[1].cache.layers_cuda, b[1].cache.layers_cuda)):
+        assert bool((La.depth_index_tensor == Lb.depth_index_tensor).all()), l
+        assert bool((La.depth.view(torch.int32) == Lb.depth.view(torch.int32)).all()), l
+        assert bool((La.weight == Lb.weight).all()), l
+        ia, ib = a[3][l], b[3][l]
+        assert float((ia - ib).abs().max()) <= 1e-5 * float(ia.abs().max()), l
+    sa, sb = a[1].cache.read_stats(), b[1].cache.read_stats()
+    assert list(sa.visible) == list(sb.visible) and list(sa.accepted) == list(sb.accepted)
 
 
 def test_counts_and_depth_invariants(full):

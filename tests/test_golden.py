@@ -28,16 +28,17 @@ def test_checker_reproduces_fixture(oracle_mod, name):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("path", [1, 2], ids=["direct", "tiles"])
 @pytest.mark.parametrize("name", NAMES)
-def test_hip_path_matches_fixture(name):
+def test_hip_path_matches_fixture(name, path):
     import torch
     from adop_amd import render, scenes
     from helpers import announce, assert_close, assert_norm_close, run_hip_forward
 
-    announce(f"golden {name}")
+    announce(f"golden {name} forward_path={path}")
     hs = make_golden.golden_scenes()[name]
     want = load(name)
-    scene, info, ctx, images, masks = run_hip_forward(hs)
+    scene, info, ctx, images, masks = run_hip_forward(hs, forward_path=path)
     for l in range(hs.num_layers):
         L = info.cache.layers_cuda[l]
         assert np.array_equal(L.depth_index_tensor.cpu().numpy().view(np.uint64), want[f"depth_index_{l}"])

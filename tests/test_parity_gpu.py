@@ -12,6 +12,16 @@ from helpers import (announce, assert_norm_close, check_backward, check_forward,
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True, params=[1, 2], ids=["direct", "tiles"])
+def forward_path(request):
+    """Every case runs through both forward paths of the library."""
+    import helpers
+
+    helpers.FORWARD_PATH = request.param
+    yield request.param
+    helpers.FORWARD_PATH = 0
+
+
 def _torch_grads(grads):
     import torch
 
