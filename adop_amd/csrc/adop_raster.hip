@@ -106,20 +106,20 @@ struct WorkspaceLayout
     size_t proj;        // float4[B * N]: projected points of the forward pass when the caller keeps no point_cache
     size_t bin_count;   // uint32[max tiles]           tile bins of the forward pass
     size_t bin_offset;  // uint32[max tiles + 1]
-    size_t bin_cursor;  // uint32[max tiles]
+    size_t bin_info;    // uint32[B * N]
     size_t bin_entries; // float4[kTileLevels * B * N]
     size_t bin_cap;     // entries
     size_t total;
 };
 
 constexpr int kTileLevels = 2;  // levels the tile path renders in LDS (a point has at most one bin entry per such level)
-constexpr int kMinTileShift = 4;
 constexpr int kTilePathMinPoints = 1 << 16;
+constexpr int kTilePathMaxPointsPerPixel = 16;
 
 size_t max_tiles(int B, int w0, int h0)
 {
-    size_t tx = ((size_t)(w0 > 0 ? w0 : 1) - 1 >> kMinTileShift) + 1;
-    size_t ty = ((size_t)(h0 > 0 ? h0 : 1) - 1 >> kMinTileShift) + 1;
+    size_t tx = ((size_t)(w0 > 0 ? w0 : 1) - 1 >> kTileShiftX) + 1;
+    size_t ty = ((size_t)(h0 > 0 ? h0 : 1) - 1 >> kTileShiftY) + 1;
     return tx * ty * (size_t)B;
 }
 
@@ -179,12 +179,12 @@ WorkspaceLayout layout(const adop_scene* s, int B, int L, int w0, int h0)
     o            = align_up(o + sizeof(float4) * (size_t)B * (size_t)(s->num_points > 0 ? s->num_points : 0), 256);
     size_t T     = max_tiles(B, w0, h0);
     w.bin_count  = o;
-    o            = align_up(o + sizeof(uint32_t) * T * kBinStride, 256);
+    o            = align_up(o + sizeof(uint32_t) * T, 256);
     w.bin_offset = o;
     o            = align_up(o + sizeof(uint32_t) * (T + 1), 256);
-    w.bin_cursor = o;
-    o            = align_up(o + sizeof(uint32_t) * T * kBinStride, 256);
     w.bin_cap    = (size_t)kTileLevels * (size_t)B * (size_t)(s->num_points > 0 ? s->num_points : 0);
+    w.bin_info   = o;
+    o            = align_up(o + sizeof(uint32_t) * (size_t)B * (size_t)(s->num_points > 0 ? s->num_points : 0), 256);
     w.bin_entries = o;
     o            = align_up(o + sizeof(float4) * w.bin_cap, 256);
     w.total      = o;
@@ -362,7 +362,6 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
     Levels lv   = make_levels(scene, num_views, buffers, nullptr);
     CloudArg pc = make_cloud(scene, buffers);
     ParamArg rp = make_params(params);
-    if (!pc.cache) pc.cache = (float4*)((char*)workspace + wl.proj);
 
     if (stats)
     {
@@ -378,25 +377,32 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
     static const int env_path = getenv("ADOP_FORWARD_PATH") ? atoi(getenv("ADOP_FORWARD_PATH")) : 0;
     int path = params->forward_path ? params->forward_path : env_path;
     if (path < 0 || path > 2) return fail(ADOP_INVALID_ARG, "forward_path must be 0, 1 or 2");
-    const bool can_bin = scene->num_points > 0 && scene->num_points < (1 << 28);
-    if (path == 0) path = scene->num_points >= kTilePathMinPoints ? 2 : 1;
+    const bool can_bin = scene->num_points > 0 && scene->num_points < (1 << 28) &&
+                         max_tiles(num_views, views[0].w, views[0].h) < ((size_t)1 << 24);
+    // The tile path bins every projected point; a cloud with very many points per pixel is faster through the direct
+    // path, whose early depth test drops most of them before they cost anything.
+    if (path == 0)
+        path = (scene->num_points >= kTilePathMinPoints &&
+                (size_t)scene->num_points <= (size_t)kTilePathMaxPointsPerPixel * views[0].w * views[0].h)
+                   ? 2
+                   : 1;
     if (path == 2 && !can_bin) path = 1;
 
     if (path == 2)
     {
+        if (!pc.cache) pc.cache = (float4*)((char*)workspace + wl.proj);
         BinArg bin;
-        bin.ts      = kMinTileShift;
         bin.lt      = kTileLevels < lv.num ? kTileLevels : lv.num;
-        bin.tiles_x = ((views[0].w - 1) >> bin.ts) + 1;
-        bin.tiles_y = ((views[0].h - 1) >> bin.ts) + 1;
+        bin.tiles_x = ((views[0].w - 1) >> kTileShiftX) + 1;
+        bin.tiles_y = ((views[0].h - 1) >> kTileShiftY) + 1;
         bin.count   = (uint32_t*)((char*)workspace + wl.bin_count);
         bin.offset  = (uint32_t*)((char*)workspace + wl.bin_offset);
-        bin.cursor  = (uint32_t*)((char*)workspace + wl.bin_cursor);
         bin.entries = (float4*)((char*)workspace + wl.bin_entries);
+        bin.info    = (uint32_t*)((char*)workspace + wl.bin_info);
         const int T = bin.tiles_x * bin.tiles_y * num_views;
         {
             StageScope sc("Initialize", stream);
-            if ((st = fill_async(bin.count, sizeof(uint32_t) * (size_t)T * kBinStride, 0, stream)) != ADOP_OK) return st;
+            if ((st = fill_async(bin.count, sizeof(uint32_t) * (size_t)T, 0, stream)) != ADOP_OK) return st;
             if (bin.lt < lv.num)
             {
                 // coarse levels: packed depth and global accumulators as in the direct path

@@ -21,6 +21,10 @@
 namespace adop
 {
 constexpr uint32_t kNoTile       = 0xFFFFFFFFu;
+constexpr uint32_t kInfoTileMask = 0x00FFFFFFu;
+constexpr uint32_t kInfoRight    = 1u << 27;
+constexpr uint32_t kInfoBelow    = 1u << 28;
+constexpr uint32_t kInfoValid    = 1u << 31;
 
 // Pixels of every level -> does the point touch the image at all, how many levels precede the LOD break, the tile
 // of its primary entry (tile of the level-0 pixel, clamped into the image; the primary entry also carries the
@@ -55,14 +59,13 @@ __device__ __forceinline__ void entry_tiles(const Levels& lv, const ParamArg& rp
         if (in_out) in_out[l] = in[l];
     }
     const int tiles_per_view = bin.tiles_x * bin.tiles_y;
-    const int ts             = bin.ts;
     int cx = px[0] < 0 ? 0 : (px[0] >= lv.l[0].w ? lv.l[0].w - 1 : px[0]);
     int cy = py[0] < 0 ? 0 : (py[0] >= lv.l[0].h ? lv.l[0].h - 1 : py[0]);
-    *ptile = (uint32_t)(b * tiles_per_view + (cy >> ts) * bin.tiles_x + (cx >> ts));
+    *ptile = (uint32_t)(b * tiles_per_view + (cy >> kTileShiftY) * bin.tiles_x + (cx >> kTileShiftX));
     *xtile = kNoTile;
     if (bin.lt > 1 && in[1])
     {
-        uint32_t t1 = (uint32_t)(b * tiles_per_view + (py[1] >> (ts - 1)) * bin.tiles_x + (px[1] >> (ts - 1)));
+        uint32_t t1 = (uint32_t)(b * tiles_per_view + (py[1] >> (kTileShiftY - 1)) * bin.tiles_x + (px[1] >> (kTileShiftX - 1)));
         if (t1 != *ptile) *xtile = t1;
     }
 }
@@ -107,12 +110,32 @@ __global__ __launch_bounds__(kBlock) void bin_count_kernel(CloudArg pc, const Vi
             bool dropped = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;
             stat_add(&stats->bad_index, ok && !dropped && !tex_ok);
         }
-        if (!__ballot(ok) && !STATS) continue;  // wavefront-uniform
+        if (!__ballot(ok) && !STATS)  // wavefront-uniform
+        {
+            if (valid) bin.info[(size_t)b * pc.n + i] = 0;
+            continue;
+        }
 
         bool in[ADOP_MAX_LAYERS];
         bool any_in;
         uint32_t nlev, ptile, xtile;
         entry_tiles(lv, rp, bin, b, ok, ip, radius_pixels, in, &any_in, &nlev, &ptile, &xtile);
+        if (valid)
+        {
+            uint32_t word = 0;
+            if (any_in)
+            {
+                word = kInfoValid | ptile | (nlev << 24);
+                if (xtile != kNoTile)
+                {
+                    const uint32_t d = xtile - ptile;  // 1, tiles_x or tiles_x + 1
+                    const bool below = d >= (uint32_t)bin.tiles_x;
+                    if (below) word |= kInfoBelow;
+                    if (d - (below ? (uint32_t)bin.tiles_x : 0u) == 1u) word |= kInfoRight;
+                }
+            }
+            bin.info[(size_t)b * pc.n + i] = word;
+        }
         if (STATS)
         {
 #pragma unroll
@@ -123,8 +146,8 @@ __global__ __launch_bounds__(kBlock) void bin_count_kernel(CloudArg pc, const Vi
         wave_lds_sync();
         int G = wave_group_by_key(any_in, ptile, gkey_w, gmask_w);
         wave_lds_sync();
-        if (lane < G) atomicAdd(&bin.count[(size_t)gkey_w[lane] * kBinStride], (uint32_t)__popcll(gmask_w[lane]));
-        if (xtile != kNoTile) atomicAdd(&bin.count[(size_t)xtile * kBinStride], 1u);
+        if (lane < G) atomicAdd(&bin.count[gkey_w[lane]], (uint32_t)__popcll(gmask_w[lane]));
+        if (xtile != kNoTile) atomicAdd(&bin.count[xtile], 1u);
     }
 }
 
@@ -143,14 +166,26 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels
 
     for (int b = 0; b < lv.B; ++b)
     {
+        uint32_t info[PPT];
+#pragma unroll
+        for (int k = 0; k < PPT; ++k)
+        {
+            const int i = base + k * kBlock;
+            info[k]     = i < pc.n ? bin.info[(size_t)b * pc.n + i] : 0u;
+        }
         float4 R[PPT];
         float drop[PPT];
 #pragma unroll
         for (int k = 0; k < PPT; ++k)
         {
             const int i = base + k * kBlock;
-            R[k]        = i < pc.n ? pc.cache[(size_t)b * pc.n + i] : make_float4(0, 0, 0, 0);
-            drop[k]     = (i < pc.n && pc.dropout) ? pc.dropout[(size_t)b * pc.n + i] : 0.f;
+            R[k]        = make_float4(0, 0, 0, 0);
+            drop[k]     = 0.f;
+            if (info[k] & kInfoValid)
+            {
+                R[k] = pc.cache[(size_t)b * pc.n + i];
+                if (pc.dropout) drop[k] = pc.dropout[(size_t)b * pc.n + i];
+            }
         }
         bool any_in[PPT];
         uint32_t nlev[PPT], ptile[PPT], xtile[PPT], gslot[PPT], xslot[PPT];
@@ -158,8 +193,12 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels
 #pragma unroll
         for (int k = 0; k < PPT; ++k)
         {
-            V2 ip = {R[k].x, R[k].y};
-            entry_tiles(lv, rp, bin, b, R[k].z != 0, ip, R[k].w, nullptr, &any_in[k], &nlev[k], &ptile[k], &xtile[k]);
+            any_in[k] = (info[k] & kInfoValid) != 0;
+            nlev[k]   = info[k] >> 24 & 7u;
+            ptile[k]  = info[k] & kInfoTileMask;
+            xtile[k]  = kNoTile;
+            if (info[k] & (kInfoRight | kInfoBelow))
+                xtile[k] = ptile[k] + ((info[k] & kInfoRight) ? 1u : 0u) + ((info[k] & kInfoBelow) ? (uint32_t)bin.tiles_x : 0u);
             G[k]     = wave_group_by_key(any_in[k], ptile[k], s_gkey[k] + wbase, s_gmask[k] + wbase, &mine[k]);
             gslot[k] = 0;
             xslot[k] = 0;
@@ -168,10 +207,14 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels
 #pragma unroll
         for (int k = 0; k < PPT; ++k)
         {
+            // slots are handed out from the end of the bin: the tile's counter runs down from its count to zero
             if (lane < G[k])
-                gslot[k] = atomicAdd(&bin.cursor[(size_t)s_gkey[k][wbase + lane] * kBinStride],
-                                     (uint32_t)__popcll(s_gmask[k][wbase + lane]));
-            if (xtile[k] != kNoTile) xslot[k] = atomicAdd(&bin.cursor[(size_t)xtile[k] * kBinStride], 1u);
+            {
+                const uint32_t t = s_gkey[k][wbase + lane];
+                const uint32_t n = (uint32_t)__popcll(s_gmask[k][wbase + lane]);
+                gslot[k]         = bin.offset[t] + atomicSub(&bin.count[t], n) - n;
+            }
+            if (xtile[k] != kNoTile) xslot[k] = bin.offset[xtile[k]] + atomicSub(&bin.count[xtile[k]], 1u) - 1u;
         }
 #pragma unroll
         for (int k = 0; k < PPT; ++k)
@@ -196,38 +239,50 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels
     }
 }
 
-// Exclusive prefix sum of the tile counts (one workgroup): offset[0..T], cursor[t] = offset[t].
+// Exclusive prefix sum of the tile counts (one workgroup): offset[0..T].  Chunks of 8192 tiles; the eight counts of a
+// thread are consecutive (two 16-byte loads, one memory round trip per chunk).
 __global__ __launch_bounds__(1024) void tile_scan_kernel(const uint32_t* __restrict__ count, uint32_t* __restrict__ offset,
-                                                         uint32_t* __restrict__ cursor, int T)
+                                                         int T)
 {
+    constexpr int PER = 8;
     __shared__ uint32_t s_wave[16];
+    __shared__ uint32_t s_carry;
     const int tid = threadIdx.x;
-    const int per = (T + 1023) / 1024;
-    const int t0  = tid * per;
-    uint32_t sum  = 0;
-    for (int k = 0; k < per; ++k)
-        if (t0 + k < T) sum += count[(size_t)(t0 + k) * kBinStride];
-    // inclusive scan inside the wavefront, then over the 16 wavefronts
-    uint32_t inc = sum;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1)
-    {
-        uint32_t v = __shfl_up(inc, off, 64);
-        if ((tid & 63) >= off) inc += v;
-    }
-    if ((tid & 63) == 63) s_wave[tid >> 6] = inc;
+    if (tid == 0) s_carry = 0;
     __syncthreads();
-    uint32_t base = 0;
-    for (int w = 0; w < (tid >> 6); ++w) base += s_wave[w];
-    uint32_t run = base + inc - sum;
-    for (int k = 0; k < per; ++k)
-        if (t0 + k < T)
+    for (int c0 = 0; c0 < T; c0 += 1024 * PER)
+    {
+        const int t0 = c0 + tid * PER;
+        uint32_t v[PER];
+#pragma unroll
+        for (int k = 0; k < PER; ++k) v[k] = t0 + k < T ? count[t0 + k] : 0u;
+        uint32_t sum = 0;
+#pragma unroll
+        for (int k = 0; k < PER; ++k) sum += v[k];
+        // inclusive scan inside the wavefront, then over the 16 wavefronts
+        uint32_t inc = sum;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1)
         {
-            offset[t0 + k]                      = run;
-            cursor[(size_t)(t0 + k) * kBinStride] = run;
-            run += count[(size_t)(t0 + k) * kBinStride];
+            uint32_t u = __shfl_up(inc, off, 64);
+            if ((tid & 63) >= off) inc += u;
         }
-    if (tid == 1023) offset[T] = base + inc;
+        if ((tid & 63) == 63) s_wave[tid >> 6] = inc;
+        __syncthreads();
+        uint32_t run = s_carry + inc - sum;
+        for (int w = 0; w < (tid >> 6); ++w) run += s_wave[w];
+#pragma unroll
+        for (int k = 0; k < PER; ++k)
+            if (t0 + k < T)
+            {
+                offset[t0 + k] = run;
+                run += v[k];
+            }
+        __syncthreads();
+        if (tid == 1023) s_carry = run;  // the last thread ends at the chunk total
+        __syncthreads();
+    }
+    if (tid == 0) offset[T] = s_carry;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -237,18 +292,26 @@ void launch_bin(int pass, const CloudArg& pc, const ViewConst* views, const Leve
                 const BinArg& bin, adop_stats* stats, hipStream_t st)
 {
     if (pc.n < 1) return;
-    constexpr int PPT = 4;
     if (pass == 0)
+    {
         hipLaunchKernelGGL(bin_count_kernel, dim3((pc.n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, pc, views, lv, rp,
                            bin, stats);
+        return;
+    }
+    static const int ppt = getenv("ADOP_SCATTER_PPT") ? atoi(getenv("ADOP_SCATTER_PPT")) : 4;
+    if (ppt == 1)
+        hipLaunchKernelGGL((bin_scatter_kernel<1>), dim3((pc.n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, pc, lv, rp, bin);
+    else if (ppt == 2)
+        hipLaunchKernelGGL((bin_scatter_kernel<2>), dim3((pc.n + kBlock * 2 - 1) / (kBlock * 2)), dim3(kBlock), 0, st, pc,
+                           lv, rp, bin);
     else
-        hipLaunchKernelGGL((bin_scatter_kernel<PPT>), dim3((pc.n + kBlock * PPT - 1) / (kBlock * PPT)), dim3(kBlock), 0,
-                           st, pc, lv, rp, bin);
+        hipLaunchKernelGGL((bin_scatter_kernel<4>), dim3((pc.n + kBlock * 4 - 1) / (kBlock * 4)), dim3(kBlock), 0, st, pc,
+                           lv, rp, bin);
 }
 
 void launch_tile_scan(const BinArg& bin, int num_tiles, hipStream_t st)
 {
-    hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, st, bin.count, bin.offset, bin.cursor, num_tiles);
+    hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, st, bin.count, bin.offset, num_tiles);
 }
 
 }  // namespace adop

@@ -118,7 +118,8 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
             bool ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P[k].w, rp.check_normal != 0, rp.dist_cutoff,
                                              lv.l[0].w, &ip, &z, &radius_pixels, &view_p);
             // the blend (and the backward pass, if the caller keeps the buffer) read this instead of projecting again
-            if (valid) pc.cache[(size_t)b * pc.n + i] = ok ? make_float4(ip.x, ip.y, z, radius_pixels) : make_float4(0, 0, 0, 0);
+            if (valid && pc.cache)
+                pc.cache[(size_t)b * pc.n + i] = ok ? make_float4(ip.x, ip.y, z, radius_pixels) : make_float4(0, 0, 0, 0);
             zz[k]      = z;
             inmask[k]  = 0;
             bool alive = ok;
@@ -226,16 +227,37 @@ __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewCo
     bool tex_ok   = (unsigned)tex_index < (unsigned)pc.num_texels;  // device assert :362
     const float accept = rp.depth_accept + 1;
     bool staged = false;
+    float4 P    = make_float4(0, 0, 0, 0);
+    V3 nrm      = {0, 0, 0};
+    if (!pc.cache)  // kernel-uniform: no point cache, project again
+    {
+        if (valid) P = pc.position[i];
+        if (valid && pc.normal) nrm = unpack_normal10(pc.normal[i]);
+    }
 
     for (int b = 0; b < lv.B; ++b)
     {
         bool dropped = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;  // :314-315
-        // projected by the depth prepass of this call
-        const float4 R = valid ? pc.cache[(size_t)b * pc.n + i] : make_float4(0, 0, 0, 0);
-        V2 ip          = {R.x, R.y};
-        const float z  = R.z;
-        float radius_pixels = R.w;
-        bool ok = valid && !dropped && z != 0;
+        V2 ip = {0.f, 0.f};
+        float z = 0.f, radius_pixels = 0.f;
+        bool ok;
+        if (pc.cache)
+        {
+            // projected by the depth prepass of this call
+            const float4 R = valid ? pc.cache[(size_t)b * pc.n + i] : make_float4(0, 0, 0, 0);
+            ip             = {R.x, R.y};
+            z              = R.z;
+            radius_pixels  = R.w;
+            ok             = valid && !dropped && z != 0;
+        }
+        else
+        {
+            V3 pos = {P.x, P.y, P.z};
+            V3 view_p;
+            ok = valid && !dropped &&
+                 project_point(views[b], pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff, lv.l[0].w, &ip,
+                               &z, &radius_pixels, &view_p);
+        }
         if (STATS) stat_add(&stats->bad_index, ok && !tex_ok);
         ok = ok && tex_ok;
         if (!__ballot(ok) && !STATS) continue;  // wavefront-uniform

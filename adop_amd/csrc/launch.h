@@ -22,17 +22,21 @@ void launch_blend(const CloudArg& pc, const ViewConst* views, const Levels& lv, 
 void launch_resolve(const Levels& lv, int first_level, int grid, const float* accum, int S, const float* background,
                     int write_mask, float mask_value, hipStream_t st);
 
-// Forward pass through screen-space tile bins (binned_kernels.hip).
-constexpr int kBinStride = 16;  // uint32 per tile counter
+// Forward pass through screen-space tile bins (binned_kernels.hip, tile_kernels.hip).  A tile has kBlock level-0 pixels,
+// one per thread of a workgroup: 16 x 16 (32 x 8, with 128-byte rows in the output tensors, measured 5 % slower: more
+// points have their level-1 pixel in another tile).
+constexpr int kTileShiftX = 4;
+constexpr int kTileShiftY = 4;
 struct BinArg
 {
-    uint32_t* count;   // [T * kBinStride] entries per tile; one counter per 64-byte line: atomics that share a
-                       // line are serialised at the memory side (~25 ns each)
+    uint32_t* count;   // [T] entries per tile after the first pass; the second pass counts it down to zero to hand
+                       // out the slots of a bin
     uint32_t* offset;  // [T + 1] exclusive prefix sum
-    uint32_t* cursor;  // [T * kBinStride] next free slot while the bins are filled
     float4* entries;   // (ip.x, ip.y, +-depth, point id | flags), at most lt per point and view
+    uint32_t* info;    // [B * N] written by the first pass for the second: tile of the primary entry (bits 0..23),
+                       // levels before the LOD break (24..26), second entry one tile to the right / below (27, 28),
+                       // point has entries (31)
     int32_t tiles_x, tiles_y;  // tiles of one view
-    int32_t ts;                // log2 of the tile width in level-0 pixels
     int32_t lt;                // levels rendered in the tile's LDS (1 or 2); the others go through global atomics
 };
 constexpr uint32_t kEntryIdMask  = 0x0FFFFFFFu;  // entry word: point id; bits 28..30: levels before the LOD break;

@@ -23,55 +23,49 @@
 
 namespace adop
 {
-// Local layout of the pixels a tile touches: levels < lt are the tile's own 2^(ts-l) squares; a coarser level is
-// the window of ((2^ts - 1) >> l) + 2 pixels per axis that rint(ip * 0.5^l) can reach from the tile.
+// Local layout of the pixels a tile touches: levels < lt are the tile's own (32 >> l) x (8 >> l) rectangles; a coarser
+// level is the window of ((extent - 1) >> l) + 2 pixels per axis that rint(ip * 0.5^l) can reach from the tile.
 struct TileLayout
 {
-    int ox[ADOP_MAX_LAYERS], oy[ADOP_MAX_LAYERS], w[ADOP_MAX_LAYERS], base[ADOP_MAX_LAYERS + 1];
+    int ox[ADOP_MAX_LAYERS], oy[ADOP_MAX_LAYERS], wx[ADOP_MAX_LAYERS], wy[ADOP_MAX_LAYERS], base[ADOP_MAX_LAYERS + 1];
 };
 
-__device__ __forceinline__ TileLayout tile_layout(int tx, int ty, int ts, int lt, int num)
+__host__ __device__ inline int tile_extent(int shift, int l, int lt)
+{
+    return l < lt ? 1 << (shift - l) : (((1 << shift) - 1) >> l) + 2;
+}
+
+__device__ __forceinline__ TileLayout tile_layout(int tx, int ty, int lt, int num)
 {
     TileLayout t;
     int base = 0;
 #pragma unroll
     for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
     {
-        t.ox[l] = t.oy[l] = t.w[l] = 0;
-        t.base[l]                  = base;
+        t.ox[l] = t.oy[l] = t.wx[l] = t.wy[l] = 0;
+        t.base[l]                             = base;
         if (l < num)
         {
-            if (l < lt)
-            {
-                t.ox[l] = tx << (ts - l);
-                t.oy[l] = ty << (ts - l);
-                t.w[l]  = 1 << (ts - l);
-            }
-            else
-            {
-                t.ox[l] = (tx << ts) >> l;
-                t.oy[l] = (ty << ts) >> l;
-                t.w[l]  = (((1 << ts) - 1) >> l) + 2;
-            }
-            base += t.w[l] * t.w[l];
+            t.ox[l] = l < lt ? tx << (kTileShiftX - l) : (tx << kTileShiftX) >> l;
+            t.oy[l] = l < lt ? ty << (kTileShiftY - l) : (ty << kTileShiftY) >> l;
+            t.wx[l] = tile_extent(kTileShiftX, l, lt);
+            t.wy[l] = tile_extent(kTileShiftY, l, lt);
+            base += t.wx[l] * t.wy[l];
         }
     }
     t.base[ADOP_MAX_LAYERS] = base;
     return t;
 }
 
-__host__ __device__ inline int tile_pixels(int ts, int lt, int num)
+// number of local pixels of the levels [0, upto)
+__host__ __device__ inline int tile_pixels(int lt, int upto)
 {
     int n = 0;
-    for (int l = 0; l < num; ++l)
-    {
-        int w = l < lt ? 1 << (ts - l) : (((1 << ts) - 1) >> l) + 2;
-        n += w * w;
-    }
+    for (int l = 0; l < upto; ++l) n += tile_extent(kTileShiftX, l, lt) * tile_extent(kTileShiftY, l, lt);
     return n;
 }
 
-constexpr int kTileMaxPixels = 1408;  // ts = 5, lt = 2, five levels: 1024 + 256 + 81 + 25 + 9
+constexpr int kTileMaxPixels = 512;  // 256 + 64 own pixels and the coarse windows (9x3 + 5x2 + 3x2)
 
 __global__ __launch_bounds__(kBlock) void tile_depth_kernel(Levels lv, BinArg bin)
 {
@@ -84,7 +78,7 @@ __global__ __launch_bounds__(kBlock) void tile_depth_kernel(Levels lv, BinArg bi
     const int tx             = tr - ty * bin.tiles_x;
     const uint32_t start     = bin.offset[tile];
     const uint32_t end       = bin.offset[tile + 1];
-    const TileLayout T       = tile_layout(tx, ty, bin.ts, bin.lt, lv.num);
+    const TileLayout T       = tile_layout(tx, ty, bin.lt, lv.num);
     const int npix           = T.base[ADOP_MAX_LAYERS];
 
     for (int p = threadIdx.x; p < npix; p += kBlock) s_depth[p] = kClearPacked;
@@ -110,9 +104,9 @@ __global__ __launch_bounds__(kBlock) void tile_depth_kernel(Levels lv, BinArg bi
                 bool in = l < nlev && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h &&
                           (l < bin.lt || primary);
                 int cx = px - T.ox[l], cy = py - T.oy[l];
-                bool local = (unsigned)cx < (unsigned)T.w[l] && (unsigned)cy < (unsigned)T.w[l];
+                bool local = (unsigned)cx < (unsigned)T.wx[l] && (unsigned)cy < (unsigned)T.wy[l];
                 if (in && local)
-                    atomicMin(&s_depth[T.base[l] + cy * T.w[l] + cx], (unsigned long long)pk);
+                    atomicMin(&s_depth[T.base[l] + cy * T.wx[l] + cx], (unsigned long long)pk);
                 else if (in && l >= bin.lt)  // outside the window (does not happen for in-image points): straight to memory
                     atomicMin((unsigned long long*)(L.depth_index + (size_t)b * L.w * L.h + (size_t)py * L.w + px),
                               (unsigned long long)pk);
@@ -129,8 +123,8 @@ __global__ __launch_bounds__(kBlock) void tile_depth_kernel(Levels lv, BinArg bi
         if (l < lv.num)
         {
             const LevelArg& L = lv.l[l];
-            const int W       = T.w[l];
-            for (int q = threadIdx.x; q < W * W; q += kBlock)
+            const int W       = T.wx[l];
+            for (int q = threadIdx.x; q < W * T.wy[l]; q += kBlock)
             {
                 const int cy = q / W, cx = q - cy * W;
                 const int px = T.ox[l] + cx, py = T.oy[l] + cy;
@@ -148,13 +142,12 @@ __global__ __launch_bounds__(kBlock) void tile_depth_kernel(Levels lv, BinArg bi
     }
 }
 
-// Buckets of the gather (tile of 16 x 16 level-0 pixels = kBlock threads): bucket p < 256 is level-0 pixel p; the
-// level-1 pixels and the pixels of the coarse windows collect many more entries each, so their lists are split
-// in 2 and 3 parts (an entry picks the part by its batch slot): buckets 256 + 2*q + part and 384 + 3*c + part.
-constexpr int kTileShift    = 4;
-constexpr int kL1Parts      = 2;
-constexpr int kCoarseParts  = 3;
-constexpr int kL1Bucket0    = 256;
+// Buckets of the gather (a tile has kBlock level-0 pixels): bucket p < 256 is level-0 pixel p; the level-1 pixels and
+// the pixels of the coarse windows collect many more entries each, so their lists are split in 2 and up to 3 parts
+// (an entry picks the part by its batch slot): buckets 256 + 2*q + part and 384 + parts*c + part.
+constexpr int kL1Parts       = 2;
+constexpr int kMaxCoarseParts = 3;
+constexpr int kL1Bucket0     = 256;
 constexpr int kCoarseBucket0 = 384;
 constexpr uint32_t kListEnd = 0xFFFFu;
 
@@ -187,11 +180,12 @@ template <int CT, bool HALF, int K>
 __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels lv, ParamArg rp, BinArg bin,
                                                             float* __restrict__ accum, int S,
                                                             const float* __restrict__ background, int write_mask,
-                                                            float mask_value, int identity_index, adop_stats* stats, int dbg)
+                                                            float mask_value, int identity_index, adop_stats* stats)
 {
     constexpr int CMAX  = CT ? CT : kMaxChannels;
     constexpr int BATCH = K * kBlock;
-    constexpr int T0    = 1 << kTileShift;
+    constexpr int TX    = 1 << kTileShiftX;  // level-0 extent of the tile; TX * TY = kBlock
+    constexpr int TY    = 1 << kTileShiftY;
     extern __shared__ __align__(16) unsigned char smem[];
     const bool STATS = stats != nullptr;
     const int C      = CT ? CT : lv.C;
@@ -206,10 +200,12 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
     const uint32_t start     = bin.offset[tile];
     const uint32_t end       = bin.offset[tile + 1];
     const int lt             = bin.lt;
-    const TileLayout T       = tile_layout(tx, ty, kTileShift, lt, lv.num);
+    const TileLayout T       = tile_layout(tx, ty, lt, lv.num);
     const int npix           = T.base[ADOP_MAX_LAYERS];
-    const int first_coarse   = lt > 1 ? T0 * T0 + T0 * T0 / 4 : T0 * T0;  // local pixel index of the first coarse pixel
+    const int first_coarse   = lt > 1 ? TX * TY + TX * TY / 4 : TX * TY;  // local pixel index of the first coarse pixel
     const int ncoarse        = npix - first_coarse;
+    // parts per coarse pixel: the coarse buckets are the second buckets of the threads kBlock/2 .. kBlock-1
+    const int cparts = ncoarse * kMaxCoarseParts <= kBlock / 2 ? kMaxCoarseParts : (ncoarse * 2 <= kBlock / 2 ? 2 : 1);
 
     float* s_stage   = (float*)smem;                     // [BATCH * C]
     float* s_depth   = s_stage + BATCH * C;              // [npix] f32 depth of the local pixels
@@ -220,8 +216,7 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
 #pragma unroll
     for (int c = 0; c <= CMAX; ++c) acc0[c] = acc1[c] = 0.f;
 
-    if (dbg & 32) return;
-    if (end > start && !(dbg & 64))  // workgroup-uniform
+    if (end > start)  // workgroup-uniform
     {
         // entries of the first batch: requested together with the depth values below
         float4 Enext[K];
@@ -238,8 +233,8 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
             if (l < lv.num)
             {
                 const LevelArg& L = lv.l[l];
-                const int W       = T.w[l];
-                for (int q = tid; q < W * W; q += kBlock)
+                const int W       = T.wx[l];
+                for (int q = tid; q < W * T.wy[l]; q += kBlock)
                 {
                     const int cy = q / W, cx = q - cy * W;
                     const int px = T.ox[l] + cx, py = T.oy[l] + cy;
@@ -256,7 +251,7 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
         __syncthreads();
 
         const float accept = rp.depth_accept + 1;
-        for (uint32_t b0 = start; b0 < end && !(dbg & 8); b0 += BATCH)  // workgroup-uniform
+        for (uint32_t b0 = start; b0 < end; b0 += BATCH)  // workgroup-uniform
         {
             // -- entries of this thread, their descriptors, and the entries of the next batch (all requested before
             //    anything waits: a batch is a chain of dependent memory round trips) --------------------------------
@@ -275,7 +270,7 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
                 ok[k] = ok[k] && (unsigned)tex_index < (unsigned)pc.num_texels;  // device assert :362
 #pragma unroll
                 for (int c = 0; c < CMAX; ++c) t[k][c] = 0.f;
-                if (ok[k] && !(dbg & 4))
+                if (ok[k])
                 {
 #pragma unroll
                     for (int c = 0; c < CMAX; ++c)
@@ -308,13 +303,13 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
                         bool in = ok[k] && l < nlev && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h &&
                                   (l < lt || primary);
                         int cx = px - T.ox[l], cy = py - T.oy[l];
-                        bool local = (unsigned)cx < (unsigned)T.w[l] && (unsigned)cy < (unsigned)T.w[l];
+                        bool local = (unsigned)cx < (unsigned)T.wx[l] && (unsigned)cy < (unsigned)T.wy[l];
                         bool accepted = false;
                         if (in && local)
                         {
-                            const int q = cy * T.w[l] + cx;
+                            const int q = cy * T.wx[l] + cx;
                             accepted    = !(z > s_depth[T.base[l] + q] * accept);
-                            if (accepted && !(dbg & 2))
+                            if (accepted)
                             {
                                 int bucket;
                                 if (l == 0)
@@ -322,7 +317,7 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
                                 else if (l < lt)
                                     bucket = kL1Bucket0 + q * kL1Parts + (slot & (kL1Parts - 1));
                                 else
-                                    bucket = kCoarseBucket0 + (T.base[l] - first_coarse + q) * kCoarseParts + slot % kCoarseParts;
+                                    bucket = kCoarseBucket0 + (T.base[l] - first_coarse + q) * cparts + slot % cparts;
                                 const uint32_t node = (uint32_t)(l * BATCH + slot);
                                 uint32_t old = atomicExch(s_head + bucket, node);
                                 s_next[node] = (uint16_t)old;
@@ -375,7 +370,7 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
             __syncthreads();
             // -- gather: every thread walks the lists of its two buckets and empties them ------------------------------
             {
-                uint32_t node = (dbg & 1) ? kListEnd : s_head[tid];
+                uint32_t node = s_head[tid];
                 float n       = 0.f;
                 while (node != kListEnd)
                 {
@@ -385,7 +380,7 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
                 }
                 acc0[CMAX] += n;
                 s_head[tid] = kListEnd;
-                node        = (dbg & 1) ? kListEnd : s_head[kBlock + tid];
+                node        = s_head[kBlock + tid];
                 n           = 0.f;
                 while (node != kListEnd)
                 {
@@ -402,10 +397,9 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
 
     // -- resolve (CombineAndFill :726-754, CreateMask :828-847) ----------------------------------------------------
     // level 0: bucket tid is pixel tid of the tile
-    if (dbg & 16) return;
     {
         const LevelArg& L = lv.l[0];
-        const int px = T.ox[0] + (tid & (T0 - 1)), py = T.oy[0] + (tid >> kTileShift);
+        const int px = T.ox[0] + (tid & (TX - 1)), py = T.oy[0] + (tid >> kTileShiftX);
         if (px < L.w && py < L.h)
         {
             const float cou  = acc0[CMAX];
@@ -428,7 +422,7 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
         for (int c = 0; c <= CMAX; ++c) acc1[c] += (tid < kCoarseBucket0 - kL1Bucket0) ? __shfl_xor(acc1[c], 1, 64) : 0.f;
         if (tid < kCoarseBucket0 - kL1Bucket0 && (tid & 1) == 0)
         {
-            constexpr int T1  = T0 / 2;
+            constexpr int T1  = TX / 2;
             const LevelArg& L = lv.l[1];
             const int q       = tid >> 1;
             const int px = T.ox[1] + (q & (T1 - 1)), py = T.oy[1] + q / T1;
@@ -439,7 +433,7 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
                 const size_t pix = (size_t)py * L.w + px;
                 const size_t o   = (size_t)b * hw + pix;
                 L.weight[o]      = cou;
-                L.depth[o]       = end > start ? s_depth[T0 * T0 + q] : 100000.f;
+                L.depth[o]       = end > start ? s_depth[TX * TY + q] : 100000.f;
                 float* out       = L.out + (size_t)b * C * hw + pix;
 #pragma unroll
                 for (int c = 0; c < CMAX; ++c)
@@ -452,9 +446,9 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
     // weight of one pixel to the global accumulators with ONE cache-line atomic
     if (lt < lv.num && end > start)
     {
-        float* s_flush = (float*)smem;  // [ncoarse * kCoarseParts * S], reuses the stage: all threads are past the gather
+        float* s_flush = (float*)smem;  // [ncoarse * cparts * S], reuses the stage: all threads are past the gather
         const int u    = tid - (kCoarseBucket0 - kL1Bucket0);
-        if (u >= 0 && u < ncoarse * kCoarseParts)
+        if (u >= 0 && u < ncoarse * cparts)
         {
             float* f = s_flush + u * S;
 #pragma unroll
@@ -468,11 +462,15 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
             const int cp = i / S, j = i - cp * S;
             if (j <= C)
             {
-                const float* f = s_flush + cp * kCoarseParts * S;
-                const float cou = (f[C] + f[S + C]) + f[2 * S + C];
+                const float* f = s_flush + cp * cparts * S;
+                float cou = f[C], v = f[j];
+                for (int part = 1; part < cparts; ++part)
+                {
+                    cou += f[part * S + C];
+                    v += f[part * S + j];
+                }
                 if (cou != 0.f)
                 {
-                    const float v = (f[j] + f[S + j]) + f[2 * S + j];
                     // level and pixel of coarse pixel cp
                     int l = lt, r = cp;
 #pragma unroll
@@ -487,7 +485,7 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
                     for (int k = 1; k < ADOP_MAX_LAYERS; ++k)
                         if (k == l)
                         {
-                            W  = T.w[k];
+                            W  = T.wx[k];
                             ox = T.ox[k];
                             oy = T.oy[k];
                             Lw = lv.l[k].w;
@@ -512,10 +510,11 @@ void launch_tile_depth(const Levels& lv, const BinArg& bin, int num_tiles, hipSt
 template <int K>
 static size_t tile_blend_lds(const Levels& lv, const BinArg& bin, int S)
 {
-    size_t npix   = (size_t)tile_pixels(bin.ts, bin.lt, lv.num);
-    size_t stage  = (size_t)K * kBlock * lv.C * 4;
-    size_t rest   = npix * 4 + 2 * kBlock * 4 + (size_t)K * kBlock * lv.num * 2 + 16;
-    size_t flush  = npix * kCoarseParts * (size_t)S * 4;  // upper bound of the flush area (reuses the LDS from its start)
+    size_t npix    = (size_t)tile_pixels(bin.lt, lv.num);
+    size_t ncoarse = npix - (size_t)tile_pixels(bin.lt, bin.lt < lv.num ? bin.lt : lv.num);
+    size_t stage   = (size_t)K * kBlock * lv.C * 4;
+    size_t rest    = npix * 4 + 2 * kBlock * 4 + (size_t)K * kBlock * lv.num * 2 + 16;
+    size_t flush   = ncoarse * kMaxCoarseParts * (size_t)S * 4;  // the flush area reuses the LDS from its start
     return stage + rest > flush ? stage + rest : flush;
 }
 
@@ -524,9 +523,8 @@ static hipError_t launch_tile_blend_k(const CloudArg& pc, const Levels& lv, cons
                                       int num_tiles, float* accum, int S, const float* background, int write_mask,
                                       float mask_value, int identity_index, adop_stats* stats, hipStream_t st)
 {
-    if (bin.ts != kTileShift || bin.lt > 2) return hipErrorInvalidValue;
+    if (bin.lt > 2 || tile_pixels(bin.lt, lv.num) > kTileMaxPixels) return hipErrorInvalidValue;
     size_t lds = tile_blend_lds<K>(lv, bin, S);
-    static const int dbg = getenv("ADOP_TILE_DBG") ? atoi(getenv("ADOP_TILE_DBG")) : 0;
     static size_t allowed = 0;  // largest dynamic LDS size this instantiation has been enabled for
     if (lds > 65536 && lds > allowed)
     {
@@ -536,7 +534,7 @@ static hipError_t launch_tile_blend_k(const CloudArg& pc, const Levels& lv, cons
         allowed = lds;
     }
     hipLaunchKernelGGL((tile_blend_kernel<CT, HALF, K>), dim3(num_tiles), dim3(kBlock), lds, st, pc, lv, rp, bin,
-                       accum, S, background, write_mask, mask_value, identity_index, stats, dbg);
+                       accum, S, background, write_mask, mask_value, identity_index, stats);
     return hipSuccess;
 }
 
@@ -545,7 +543,7 @@ static hipError_t launch_tile_blend_t(const CloudArg& pc, const Levels& lv, cons
                                       int num_tiles, float* accum, int S, const float* background, int write_mask,
                                       float mask_value, int identity_index, adop_stats* stats, hipStream_t st)
 {
-    static const int k = getenv("ADOP_TILE_K") ? atoi(getenv("ADOP_TILE_K")) : 2;
+    static const int k = getenv("ADOP_TILE_K") ? atoi(getenv("ADOP_TILE_K")) : 1;
     if (k == 1)
         return launch_tile_blend_k<CT, HALF, 1>(pc, lv, rp, bin, num_tiles, accum, S, background, write_mask, mask_value,
                                                 identity_index, stats, st);
