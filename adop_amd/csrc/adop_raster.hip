@@ -99,6 +99,7 @@ struct WorkspaceLayout
     size_t pt_partial;  // double[B * kPartialBlocks * kPartialStride]
     size_t scratch;     // double[num_poses*7 + num_cameras*(cols+1)]
     size_t pixels;      // float[B * P * max(S, 2C)]: blend accumulators (forward) / [I|G] array (backward)
+    size_t dw;          // float2[B * P]: (depth, weight) per pixel for the backward descriptor pass
     size_t q_counts;    // uint32[kNumQueues]
     size_t q_prefix;    // uint32[kNumQueues + 1]
     size_t q_items;     // uint64[kNumQueues * q_cap]
@@ -165,6 +166,8 @@ WorkspaceLayout layout(const adop_scene* s, int B, int L, int w0, int h0)
     w.pixels = o;
     int per  = accum_stride(s->num_channels) > 2 * s->num_channels ? accum_stride(s->num_channels) : 2 * s->num_channels;
     o        = align_up(o + sizeof(float) * (size_t)B * pyramid_pixels(L, w0, h0) * (size_t)per, 256);
+    w.dw = o;
+    o    = align_up(o + sizeof(float2) * (size_t)B * pyramid_pixels(L, w0, h0), 256);
     // backward work queue: workgroup k of backward_tex_kernel appends to sub-queue k % kNumQueues
     size_t blocks = ((size_t)(s->num_points > 0 ? s->num_points : 0) + kBlock - 1) / kBlock;
     w.q_cap       = (uint32_t)(((blocks + kNumQueues - 1) / kNumQueues) * kBlock);
@@ -528,10 +531,11 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     }
 
     float* ig     = (float*)((char*)workspace + wl.pixels);
+    float2* dw    = (float2*)((char*)workspace + wl.dw);
     int bg_blocks = pixel_grid(lv) < kBgBlocks ? pixel_grid(lv) : kBgBlocks;
     {
         StageScope sc("CombineAndFillBackward", stream);
-        launch_interleave(lv, bg_blocks, ig, bg_partial, stream);
+        launch_interleave(lv, bg_blocks, ig, dw, bg_partial, stream);
     }
     int want_pose = grads->grad_pose != nullptr;
     int want_intr = grads->grad_intrinsics != nullptr;
@@ -555,7 +559,7 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     {
         {
             StageScope sc("RenderBackward/descriptor", stream);
-            launch_backward_tex(pc, dviews, lv, rp, half, ig, grads, scene->index_is_identity, b, b == 0, q, stats,
+            launch_backward_tex(pc, dviews, lv, rp, half, ig, dw, grads, scene->index_is_identity, b, b == 0, q, stats,
                                 stream);
         }
         StageScope sc("RenderBackward/spatial", stream);

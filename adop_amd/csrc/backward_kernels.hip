@@ -22,7 +22,7 @@ __global__ void fill_zero_u32_kernel(uint32_t* __restrict__ p, int n)
 // partial row per block.
 template <int CT>
 __global__ __launch_bounds__(kBlock) void interleave_kernel(Levels lv, float* __restrict__ ig,
-                                                            double* __restrict__ partial)
+                                                            float2* __restrict__ dw, double* __restrict__ partial)
 {
     constexpr int CMAX = CT ? CT : kMaxChannels;
     const int C        = CT ? CT : lv.C;
@@ -42,7 +42,10 @@ __global__ __launch_bounds__(kBlock) void interleave_kernel(Levels lv, float* __
         const LevelArg& L = lv.l[l];
         int p             = r - lv.pix_prefix[l];
         size_t hw         = (size_t)L.w * L.h;
-        bool empty        = L.weight[(size_t)b * hw + p] == 0;
+        const float wgt   = L.weight[(size_t)b * hw + p];
+        bool empty        = wgt == 0;
+        // (depth, weight) of the pixel side by side: the descriptor pass fetches both with one 8-byte load
+        dw[ws_pixel(lv, l, b, (uint32_t)p)] = make_float2(L.depth[(size_t)b * hw + p], wgt);
         const float* g    = L.gin + (size_t)b * C * hw + p;
         const float* im   = L.out + (size_t)b * C * hw + p;
         float* dst        = ig + (size_t)ws_pixel(lv, l, b, (uint32_t)p) * (2 * C);
@@ -149,6 +152,7 @@ __device__ __forceinline__ void load_channels(const float* __restrict__ src, flo
 template <int CT, bool HALF>
 __global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const ViewConst* __restrict__ views,
                                                                Levels lv, ParamArg rp, const float* __restrict__ ig,
+                                                               const float2* __restrict__ dw,
                                                                float* __restrict__ gtex, int identity_index,
                                                                int view_b, int first_view,
                                                                uint32_t* __restrict__ q_counts,
@@ -216,8 +220,9 @@ __global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const
             if (in[l])
             {
                 pix[l]     = (uint32_t)py * (uint32_t)L.w + (uint32_t)px;
-                dep[l]     = L.depth[(size_t)b * L.w * L.h + pix[l]];
-                wgt[l]     = L.weight[(size_t)b * L.w * L.h + pix[l]];  // same round trip as the depth
+                const float2 d_w = dw[ws_pixel(lv, l, b, pix[l])];  // (depth, weight) left by interleave_kernel
+                dep[l]           = d_w.x;
+                wgt[l]           = d_w.y;
                 int ex     = min(px, L.w - 1 - px);
                 int ey     = min(py, L.h - 1 - py);
                 edge_ok[l] = min(ex, ey) > 2;  // distanceFromEdge > 2, :489
@@ -575,9 +580,11 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
     }
 }
 
+constexpr int kFinalizeBlock = 1024;  // one workgroup; the partial rows are read with 16 loads in flight per thread
+
 // Reduces the per-block partial rows and runs NormalizeGradient (:1534-1547, launches :1611-1636) for the
 // background / pose / intrinsics outputs.  One block.
-__global__ __launch_bounds__(kBlock) void finalize_kernel(const ViewConst* __restrict__ views, int B, int C,
+__global__ __launch_bounds__(kFinalizeBlock) void finalize_kernel(const ViewConst* __restrict__ views, int B, int C,
                                                           const double* __restrict__ bg_partial, int bg_blocks,
                                                           const double* __restrict__ pt_partial, int pt_blocks,
                                                           float* __restrict__ gbg, double* __restrict__ gpose,
@@ -586,11 +593,11 @@ __global__ __launch_bounds__(kBlock) void finalize_kernel(const ViewConst* __res
                                                           int num_cameras, int cols, int normalize_mode,
                                                           double* __restrict__ scratch)
 {
-    __shared__ double sh[kBlock];
+    __shared__ double sh[kFinalizeBlock];
     // background: thread t sums channel t%16 over the partial rows t/16, t/16+16, ...
     {
         const int c = threadIdx.x % kMaxChannels, k0 = threadIdx.x / kMaxChannels;
-        constexpr int GR = kBlock / kMaxChannels;
+        constexpr int GR = kFinalizeBlock / kMaxChannels;
         double v = 0;
 #pragma unroll 16
         for (int k = k0; k < bg_blocks; k += GR) v += bg_partial[(size_t)k * kMaxChannels + c];
@@ -609,13 +616,13 @@ __global__ __launch_bounds__(kBlock) void finalize_kernel(const ViewConst* __res
     // scratch: [num_poses*7] pose sums + count, then [num_cameras*(cols+1)] intrinsics sums + count
     double* sp = scratch;
     double* si = scratch + (size_t)num_poses * 7;
-    for (int k = threadIdx.x; k < num_poses * 7 + num_cameras * (cols + 1); k += kBlock) scratch[k] = 0;
+    for (int k = threadIdx.x; k < num_poses * 7 + num_cameras * (cols + 1); k += kFinalizeBlock) scratch[k] = 0;
     __syncthreads();
     for (int b = 0; b < B; ++b)
     {
         // thread t sums value t%32 (21 used) over the partial rows t/32, t/32+8, ...
         const int q = threadIdx.x % 32, k0 = threadIdx.x / 32;
-        constexpr int GR = kBlock / 32;
+        constexpr int GR = kFinalizeBlock / 32;
         double v = 0;
         if (q < kAcc)
 #pragma unroll 16
@@ -642,7 +649,7 @@ __global__ __launch_bounds__(kBlock) void finalize_kernel(const ViewConst* __res
     }
     if (gpose)
     {
-        for (int f = threadIdx.x; f < num_poses; f += kBlock)
+        for (int f = threadIdx.x; f < num_poses; f += kFinalizeBlock)
         {
             float c        = (float)sp[(size_t)f * 7 + 6];
             gpose_count[f] = c;
@@ -655,9 +662,9 @@ __global__ __launch_bounds__(kBlock) void finalize_kernel(const ViewConst* __res
     }
     if (gintr)
     {
-        for (int k = threadIdx.x; k < num_cameras * cols; k += kBlock)
+        for (int k = threadIdx.x; k < num_cameras * cols; k += kFinalizeBlock)
             gintr[k] = (float)si[(size_t)(k / cols) * (cols + 1) + (k % cols)];
-        for (int k = threadIdx.x; k < num_cameras; k += kBlock) gintr_count[k] = (float)si[(size_t)k * (cols + 1) + cols];
+        for (int k = threadIdx.x; k < num_cameras; k += kFinalizeBlock) gintr_count[k] = (float)si[(size_t)k * (cols + 1) + cols];
         __syncthreads();
         if (threadIdx.x == 0)
         {
@@ -705,24 +712,24 @@ __global__ __launch_bounds__(kBlock) void normalize_points_kernel(float* __restr
 // ------------------------------------------------------------------------------------------------
 // launchers
 // ------------------------------------------------------------------------------------------------
-void launch_interleave(const Levels& lv, int blocks, float* ig, double* partial, hipStream_t st)
+void launch_interleave(const Levels& lv, int blocks, float* ig, float2* dw, double* partial, hipStream_t st)
 {
     if (lv.C == 8)
-        hipLaunchKernelGGL((interleave_kernel<8>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, partial);
+        hipLaunchKernelGGL((interleave_kernel<8>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, dw, partial);
     else if (lv.C == 4)
-        hipLaunchKernelGGL((interleave_kernel<4>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, partial);
+        hipLaunchKernelGGL((interleave_kernel<4>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, dw, partial);
     else
-        hipLaunchKernelGGL((interleave_kernel<0>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, partial);
+        hipLaunchKernelGGL((interleave_kernel<0>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, dw, partial);
 }
 
 template <int CT, bool HALF>
 static void launch_bwd_tex_t(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp,
-                             const float* ig, const adop_backward_buffers* g, int identity_index, int b,
+                             const float* ig, const float2* dw, const adop_backward_buffers* g, int identity_index, int b,
                              int first_view, const QueueArg& q, adop_stats* stats, hipStream_t st)
 {
     int grid = (pc.n + kBlock - 1) / kBlock;
     hipLaunchKernelGGL(fill_zero_u32_kernel, dim3(kNumQueues / kBlock), dim3(kBlock), 0, st, q.counts, kNumQueues);
-    hipLaunchKernelGGL((backward_tex_kernel<CT, HALF>), dim3(grid), dim3(kBlock), 0, st, pc, views, lv, rp, ig,
+    hipLaunchKernelGGL((backward_tex_kernel<CT, HALF>), dim3(grid), dim3(kBlock), 0, st, pc, views, lv, rp, ig, dw,
                        g->grad_texture, identity_index, b, first_view, q.counts, q.items, q.cap, stats);
 }
 
@@ -751,11 +758,11 @@ static void launch_bwd_ghost_t(const CloudArg& pc, const ViewConst* views, const
 
 // descriptor gradient of one view + the work queue of its ghost / spatial gradients
 void launch_backward_tex(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
-                         const float* ig, const adop_backward_buffers* g, int identity_index, int b, int first_view,
+                         const float* ig, const float2* dw, const adop_backward_buffers* g, int identity_index, int b, int first_view,
                          const QueueArg& q, adop_stats* stats, hipStream_t st)
 {
     if (pc.n < 1) return;
-    ADOP_DISPATCH_C_HALF(launch_bwd_tex_t, pc, views, lv, rp, ig, g, identity_index, b, first_view, q, stats, st);
+    ADOP_DISPATCH_C_HALF(launch_bwd_tex_t, pc, views, lv, rp, ig, dw, g, identity_index, b, first_view, q, stats, st);
 }
 
 // ghost / spatial gradients of the queued points of one view
@@ -774,7 +781,7 @@ void launch_finalize(const ViewConst* views, int B, int C, const double* bg_part
                      const double* pt_partial, int pt_blocks, const adop_backward_buffers* g, int num_poses,
                      int num_cameras, int cols, int normalize_mode, double* scratch, hipStream_t st)
 {
-    hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kBlock), 0, st, views, B, C, bg_partial, bg_blocks, pt_partial,
+    hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kFinalizeBlock), 0, st, views, B, C, bg_partial, bg_blocks, pt_partial,
                        pt_blocks, g->grad_background, g->grad_pose, g->grad_pose_count, num_poses, g->grad_intrinsics,
                        g->grad_intrinsics_count, num_cameras, cols, normalize_mode, scratch);
 }

@@ -49,7 +49,7 @@ hipError_t launch_tile_blend(const CloudArg& pc, const Levels& lv, const ParamAr
                              bool half, float* accum, int S, const float* background, int write_mask,
                              float mask_value, int identity_index, adop_stats* stats, hipStream_t st);
 
-void launch_interleave(const Levels& lv, int blocks, float* ig, double* partial, hipStream_t st);
+void launch_interleave(const Levels& lv, int blocks, float* ig, float2* dw, double* partial, hipStream_t st);
 // Work queue of the backward pass (points that receive a ghost / spatial gradient), split in kNumQueues sub-queues
 // of `cap` items each.
 struct QueueArg
@@ -60,7 +60,7 @@ struct QueueArg
     uint32_t cap;
 };
 void launch_backward_tex(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
-                         const float* ig, const adop_backward_buffers* g, int identity_index, int b, int first_view,
+                         const float* ig, const float2* dw, const adop_backward_buffers* g, int identity_index, int b, int first_view,
                          const QueueArg& q, adop_stats* stats, hipStream_t st);
 void launch_backward_ghost(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
                            const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr,
