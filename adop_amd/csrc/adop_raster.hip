@@ -405,20 +405,12 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
         const int T = bin.tiles_x * bin.tiles_y * num_views;
         {
             StageScope sc("Initialize", stream);
-            if ((st = fill_async(bin.count, sizeof(uint32_t) * (size_t)T, 0, stream)) != ADOP_OK) return st;
-            if (bin.lt < lv.num)
-            {
-                // coarse levels: packed depth and global accumulators as in the direct path
-                size_t first  = (size_t)lv.pix_prefix[bin.lt] * lv.B * S;
-                size_t accum_n = (size_t)lv.pix_prefix[lv.num] * lv.B * S - first;
-                if (S % 4 == 0)
-                    launch_clear(lv, bin.lt, pixel_grid(lv, bin.lt), accum + first, accum_n, stream);
-                else
-                {
-                    launch_clear(lv, bin.lt, pixel_grid(lv, bin.lt), accum, 0, stream);
-                    if ((st = fill_async(accum + first, accum_n * sizeof(float), 0, stream)) != ADOP_OK) return st;
-                }
-            }
+            // tile counters, and for the coarse levels the packed depth and the global accumulators of the direct path
+            size_t first   = (size_t)lv.pix_prefix[bin.lt] * lv.B * S;
+            size_t accum_n = (size_t)lv.pix_prefix[lv.num] * lv.B * S - first;
+            int grid       = pixel_grid(lv, bin.lt) > 32 ? pixel_grid(lv, bin.lt) : 32;
+            launch_clear(lv, bin.lt, grid, accum + first, S % 4 == 0 ? accum_n : 0, bin.count, T, stream);
+            if (S % 4 != 0 && (st = fill_async(accum + first, accum_n * sizeof(float), 0, stream)) != ADOP_OK) return st;
         }
         {
             StageScope sc("BinCount", stream);
@@ -453,10 +445,10 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
     {
         StageScope sc("Initialize", stream);
         if (S % 4 == 0)
-            launch_clear(lv, 0, pixel_grid(lv), accum, accum_n, stream);
+            launch_clear(lv, 0, pixel_grid(lv), accum, accum_n, nullptr, 0, stream);
         else
         {
-            launch_clear(lv, 0, pixel_grid(lv), accum, 0, stream);
+            launch_clear(lv, 0, pixel_grid(lv), accum, 0, nullptr, 0, stream);
             if ((st = fill_async(accum, accum_n * sizeof(float), 0, stream)) != ADOP_OK) return st;
         }
     }
@@ -535,7 +527,7 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     int bg_blocks = pixel_grid(lv) < kBgBlocks ? pixel_grid(lv) : kBgBlocks;
     {
         StageScope sc("CombineAndFillBackward", stream);
-        launch_interleave(lv, bg_blocks, ig, dw, bg_partial, stream);
+        launch_interleave(lv, bg_blocks, ig, dw, bg_partial, (uint32_t*)((char*)workspace + wl.q_counts), stream);
     }
     int want_pose = grads->grad_pose != nullptr;
     int want_intr = grads->grad_intrinsics != nullptr;

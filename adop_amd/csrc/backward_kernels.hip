@@ -11,19 +11,18 @@
 
 namespace adop
 {
-__global__ void fill_zero_u32_kernel(uint32_t* __restrict__ p, int n)
-{
-    int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) p[i] = 0u;
-}
 
 // CombineAndFillBackward (:851-900) fused with the I/G interleave.  One thread per pixel of every level/image.
 // Background gradient: per-thread fp32 partial over a handful of pixels, wave/block reduction in f64, one f64
 // partial row per block.
 template <int CT>
 __global__ __launch_bounds__(kBlock) void interleave_kernel(Levels lv, float* __restrict__ ig,
-                                                            float2* __restrict__ dw, double* __restrict__ partial)
+                                                            float2* __restrict__ dw, double* __restrict__ partial,
+                                                            uint32_t* __restrict__ q_counts)
 {
+    // counters of the backward work queue: empty before the first view (queue_scan_kernel empties them again)
+    if (blockIdx.x == 0)
+        for (int k = threadIdx.x; k < kNumQueues; k += kBlock) q_counts[k] = 0;
     constexpr int CMAX = CT ? CT : kMaxChannels;
     const int C        = CT ? CT : lv.C;
     __shared__ double red[kBlock / 64][kMaxChannels];
@@ -333,8 +332,9 @@ __global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const
             (unsigned long long)(uint32_t)i | ((unsigned long long)mask << 32);
 }
 
-// exclusive prefix over the sub-queue counters: prefix[0..kNumQueues], prefix[kNumQueues] = number of items
-__global__ __launch_bounds__(kBlock) void queue_scan_kernel(const uint32_t* __restrict__ counts,
+// exclusive prefix over the sub-queue counters: prefix[0..kNumQueues], prefix[kNumQueues] = number of items; the
+// counters are left at zero for the next view
+__global__ __launch_bounds__(kBlock) void queue_scan_kernel(uint32_t* __restrict__ counts,
                                                             uint32_t* __restrict__ prefix)
 {
     constexpr int PER = kNumQueues / kBlock;
@@ -347,6 +347,8 @@ __global__ __launch_bounds__(kBlock) void queue_scan_kernel(const uint32_t* __re
         local[k] = acc;
         acc += counts[threadIdx.x * PER + k];
     }
+#pragma unroll
+    for (int k = 0; k < PER; ++k) counts[threadIdx.x * PER + k] = 0;
     s_sum[threadIdx.x] = acc;
     __syncthreads();
     uint32_t base = 0;
@@ -712,14 +714,15 @@ __global__ __launch_bounds__(kBlock) void normalize_points_kernel(float* __restr
 // ------------------------------------------------------------------------------------------------
 // launchers
 // ------------------------------------------------------------------------------------------------
-void launch_interleave(const Levels& lv, int blocks, float* ig, float2* dw, double* partial, hipStream_t st)
+void launch_interleave(const Levels& lv, int blocks, float* ig, float2* dw, double* partial, uint32_t* q_counts,
+                       hipStream_t st)
 {
     if (lv.C == 8)
-        hipLaunchKernelGGL((interleave_kernel<8>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, dw, partial);
+        hipLaunchKernelGGL((interleave_kernel<8>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, dw, partial, q_counts);
     else if (lv.C == 4)
-        hipLaunchKernelGGL((interleave_kernel<4>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, dw, partial);
+        hipLaunchKernelGGL((interleave_kernel<4>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, dw, partial, q_counts);
     else
-        hipLaunchKernelGGL((interleave_kernel<0>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, dw, partial);
+        hipLaunchKernelGGL((interleave_kernel<0>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, dw, partial, q_counts);
 }
 
 template <int CT, bool HALF>
@@ -728,7 +731,6 @@ static void launch_bwd_tex_t(const CloudArg& pc, const ViewConst* views, const L
                              int first_view, const QueueArg& q, adop_stats* stats, hipStream_t st)
 {
     int grid = (pc.n + kBlock - 1) / kBlock;
-    hipLaunchKernelGGL(fill_zero_u32_kernel, dim3(kNumQueues / kBlock), dim3(kBlock), 0, st, q.counts, kNumQueues);
     hipLaunchKernelGGL((backward_tex_kernel<CT, HALF>), dim3(grid), dim3(kBlock), 0, st, pc, views, lv, rp, ig, dw,
                        g->grad_texture, identity_index, b, first_view, q.counts, q.items, q.cap, stats);
 }

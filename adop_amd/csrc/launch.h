@@ -14,7 +14,8 @@ struct EnvLevels
 void launch_prepare_views(const ViewChunk& ch, int first, int count, const double* poses, const float* intrinsics,
                           int cols, ViewConst* out, hipStream_t st);
 void launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t st);
-void launch_clear(const Levels& lv, int first_level, int grid, float* accum, size_t accum_floats, hipStream_t st);
+void launch_clear(const Levels& lv, int first_level, int grid, float* accum, size_t accum_floats, uint32_t* zero_u32,
+                  int zero_n, hipStream_t st);
 void launch_prepass(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, adop_stats* stats,
                     hipStream_t st);
 void launch_blend(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
@@ -49,7 +50,8 @@ hipError_t launch_tile_blend(const CloudArg& pc, const Levels& lv, const ParamAr
                              bool half, float* accum, int S, const float* background, int write_mask,
                              float mask_value, int identity_index, adop_stats* stats, hipStream_t st);
 
-void launch_interleave(const Levels& lv, int blocks, float* ig, float2* dw, double* partial, hipStream_t st);
+void launch_interleave(const Levels& lv, int blocks, float* ig, float2* dw, double* partial, uint32_t* q_counts,
+                       hipStream_t st);
 // Work queue of the backward pass (points that receive a ghost / spatial gradient), split in kNumQueues sub-queues
 // of `cap` items each.
 struct QueueArg
