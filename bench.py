@@ -207,12 +207,15 @@ def main():
     # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
     # FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 after calibration with a plain 1 GiB copy); measured for the default
     # workload only
-    measured_traffic = {("config3", "RenderForward"): 691.9e6} if not args.points and args.point_order == "morton" else {}
-    if os.environ.get("ADOP_FORWARD_PATH"):
-        measured_traffic = {}
+    measured_traffic = {}
+    if args.workload == "config3" and not args.points and args.point_order == "morton" and not args.no_point_cache:
+        # profiles/config3_tile_path_fwd_bwd_kernels_traffic_instructions.md, profiles/config3_fwd_bwd_kernels_traffic_atomics.md
+        measured_traffic = {"RenderBackward/descriptor": 763.5e6, "RenderBackward/spatial": 627.7e6, "TileBlend": 438.6e6,
+                            "BinCount": 412.9e6, "BinScatter": 222.9e6, "TileDepth": 101.0e6,
+                            "CombineAndFillBackward": 397.1e6, "RenderForward": 691.9e6}
     roofline = {"bound": "hbm", "kernel": KERNEL_OF_STAGE.get(dom, dom), "stage": dom, "achieved": round(dom_gbs, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
-                "traffic": measured_traffic.get((args.workload, dom)),
+                "traffic": measured_traffic.get(dom),
                 "kernel_ms": round(stages[dom], 4), "algorithmic_bytes": int(model[dom])}
     step_gbs = total_bytes / (ms_per_step * 1e-3) / 1e9
 

@@ -207,7 +207,8 @@ adop_status adop_apply_tangent(double* tangent, double* poses_se3, int32_t num_p
  * caller's stream around each stage while profiling is enabled on the calling thread.  Stage names are the
  * reference's: "Initialize", "DepthPrepass", "RenderForward", "CombineAndFill", "Prepare Backward",
  * "CombineAndFillBackward", "RenderBackward/descriptor" and "RenderBackward/spatial" (the two kernels RenderBackward is
- * split into), "Post Process Gradient". */
+ * split into), "Post Process Gradient".  When the forward runs through the tile bins (forward_path 2), "DepthPrepass"
+ * and "RenderForward" are replaced by "BinCount", "BinScatter", "TileDepth" and "TileBlend". */
 typedef struct adop_stage_time
 {
     char name[32];
