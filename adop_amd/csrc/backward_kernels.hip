@@ -371,7 +371,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
                                                                  uint32_t q_cap, double* __restrict__ partial)
 {
     constexpr int CMAX = CT ? CT : 1;
-    __shared__ double red[kBlock / 64][kPartialStride];
+    __shared__ float s_red[kAcc * kBlock];
     __shared__ uint32_t s_prefix[kNumQueues + 1];
     const int b         = view_b;
     const ViewConst& vc = views[b];
@@ -565,20 +565,19 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
 
     if (want_pose || want_intr)
     {
-        int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+        // block sums in f64 through LDS: 8 threads per value, 32 columns each (21 f64 wavefront reductions with
+        // cross-lane permutes took 7 us per workgroup)
 #pragma unroll
-        for (int k = 0; k < kAcc; ++k)
-        {
-            double v = wave_sum<double>((double)acc[k]);
-            if (lane == 0) red[wave][k] = v;
-        }
+        for (int k = 0; k < kAcc; ++k) s_red[k * kBlock + threadIdx.x] = acc[k];
         __syncthreads();
-        if (threadIdx.x < kAcc)
-        {
-            double v = 0;
-            for (int w = 0; w < kBlock / 64; ++w) v += red[w][threadIdx.x];
-            partial[((size_t)b * gridDim.x + blockIdx.x) * kPartialStride + threadIdx.x] = v;
-        }
+        const int k = threadIdx.x >> 3, part = threadIdx.x & 7;
+        double v    = 0;
+        if (k < kAcc)
+            for (int c = part; c < kBlock; c += 8) v += (double)s_red[k * kBlock + c];
+        v += __shfl_xor(v, 1, 64);
+        v += __shfl_xor(v, 2, 64);
+        v += __shfl_xor(v, 4, 64);
+        if (k < kAcc && part == 0) partial[((size_t)b * gridDim.x + blockIdx.x) * kPartialStride + k] = v;
     }
 }
 
