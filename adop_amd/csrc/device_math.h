@@ -43,13 +43,15 @@ __device__ __forceinline__ uint32_t f2u(float f)
 }
 
 // __float2int_rn semantics (PointRenderer.cu:266): nearest-even, saturating, NaN -> 0.
+// v_rndne_f32 + v_cvt_i32_f32: the conversion instruction itself saturates out-of-range values and turns NaN into 0
+// (a C++ cast would be undefined there, and spelling the three cases out costs six more instructions per pixel
+// coordinate in kernels that are bound by instruction issue).
 __device__ __forceinline__ int f2i_rn(float f)
 {
-    if (f != f) return 0;
-    float r = rintf(f);
-    if (r >= 2147483648.f) return 2147483647;
-    if (r <= -2147483648.f) return (-2147483647 - 1);
-    return (int)r;
+    const float r = rintf(f);
+    int i;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(i) : "v"(r));
+    return i;
 }
 
 // Fixed-polynomial arctangent family (Cephes single precision), + - * / sqrt only.
