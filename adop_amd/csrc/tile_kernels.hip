@@ -28,6 +28,7 @@ namespace adop
 struct TileLayout
 {
     int ox[ADOP_MAX_LAYERS], oy[ADOP_MAX_LAYERS], wx[ADOP_MAX_LAYERS], wy[ADOP_MAX_LAYERS], base[ADOP_MAX_LAYERS + 1];
+    int cwx[ADOP_MAX_LAYERS], cwy[ADOP_MAX_LAYERS];  // extents clipped to the image: a local pixel inside them is in the image
 };
 
 __host__ __device__ inline int tile_extent(int shift, int l, int lt)
@@ -35,14 +36,14 @@ __host__ __device__ inline int tile_extent(int shift, int l, int lt)
     return l < lt ? 1 << (shift - l) : (((1 << shift) - 1) >> l) + 2;
 }
 
-__device__ __forceinline__ TileLayout tile_layout(int tx, int ty, int lt, int num)
+__device__ __forceinline__ TileLayout tile_layout(const Levels& lv, int tx, int ty, int lt, int num)
 {
     TileLayout t;
     int base = 0;
 #pragma unroll
     for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
     {
-        t.ox[l] = t.oy[l] = t.wx[l] = t.wy[l] = 0;
+        t.ox[l] = t.oy[l] = t.wx[l] = t.wy[l] = t.cwx[l] = t.cwy[l] = 0;
         t.base[l]                             = base;
         if (l < num)
         {
@@ -50,6 +51,9 @@ __device__ __forceinline__ TileLayout tile_layout(int tx, int ty, int lt, int nu
             t.oy[l] = l < lt ? ty << (kTileShiftY - l) : (ty << kTileShiftY) >> l;
             t.wx[l] = tile_extent(kTileShiftX, l, lt);
             t.wy[l] = tile_extent(kTileShiftY, l, lt);
+            int rx = lv.l[l].w - t.ox[l], ry = lv.l[l].h - t.oy[l];
+            t.cwx[l] = rx < 0 ? 0 : (rx < t.wx[l] ? rx : t.wx[l]);
+            t.cwy[l] = ry < 0 ? 0 : (ry < t.wy[l] ? ry : t.wy[l]);
             base += t.wx[l] * t.wy[l];
         }
     }
@@ -78,7 +82,7 @@ __global__ __launch_bounds__(kBlock) void tile_depth_kernel(Levels lv, BinArg bi
     const int tx             = tr - ty * bin.tiles_x;
     const uint32_t start     = bin.offset[tile];
     const uint32_t end       = bin.offset[tile + 1];
-    const TileLayout T       = tile_layout(tx, ty, bin.lt, lv.num);
+    const TileLayout T       = tile_layout(lv, tx, ty, bin.lt, lv.num);
     const int npix           = T.base[ADOP_MAX_LAYERS];
 
     for (int p = threadIdx.x; p < npix; p += kBlock) s_depth[p] = kClearPacked;
@@ -94,20 +98,31 @@ __global__ __launch_bounds__(kBlock) void tile_depth_kernel(Levels lv, BinArg bi
         const uint32_t zbits = f2u(E.z) & 0x7FFFFFFFu;  // the sign carries the dropout flag
         const uint64_t pk    = ((uint64_t)zbits << 32) | id;
         float x = E.x, y = E.y;
+        uint32_t miss = 0;  // coarse levels whose pixel is not in the tile's window (does not happen for in-image points)
 #pragma unroll
         for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
         {
             if (l < lv.num)
             {
+                const int px = f2i_rn(x), py = f2i_rn(y);
+                const int cx = px - T.ox[l], cy = py - T.oy[l];
+                const bool live = l < nlev && (l < bin.lt || primary);
+                const bool hit  = live && (unsigned)cx < (unsigned)T.cwx[l] && (unsigned)cy < (unsigned)T.cwy[l];
+                if (hit) atomicMin(&s_depth[T.base[l] + cy * T.wx[l] + cx], (unsigned long long)pk);
+                if (l >= bin.lt && live && !hit) miss |= 1u << l;
+                x *= 0.5f;
+                y *= 0.5f;
+            }
+        }
+        if (miss)  // straight to memory
+        {
+            x = E.x;
+            y = E.y;
+            for (int l = 0; l < lv.num; ++l)
+            {
                 const LevelArg& L = lv.l[l];
-                int px = f2i_rn(x), py = f2i_rn(y);
-                bool in = l < nlev && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h &&
-                          (l < bin.lt || primary);
-                int cx = px - T.ox[l], cy = py - T.oy[l];
-                bool local = (unsigned)cx < (unsigned)T.wx[l] && (unsigned)cy < (unsigned)T.wy[l];
-                if (in && local)
-                    atomicMin(&s_depth[T.base[l] + cy * T.wx[l] + cx], (unsigned long long)pk);
-                else if (in && l >= bin.lt)  // outside the window (does not happen for in-image points): straight to memory
+                const int px = f2i_rn(x), py = f2i_rn(y);
+                if ((miss >> l & 1u) && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h)
                     atomicMin((unsigned long long*)(L.depth_index + (size_t)b * L.w * L.h + (size_t)py * L.w + px),
                               (unsigned long long)pk);
                 x *= 0.5f;
@@ -200,7 +215,7 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
     const uint32_t start     = bin.offset[tile];
     const uint32_t end       = bin.offset[tile + 1];
     const int lt             = bin.lt;
-    const TileLayout T       = tile_layout(tx, ty, lt, lv.num);
+    const TileLayout T       = tile_layout(lv, tx, ty, lt, lv.num);
     const int npix           = T.base[ADOP_MAX_LAYERS];
     const int first_coarse   = lt > 1 ? TX * TY + TX * TY / 4 : TX * TY;  // local pixel index of the first coarse pixel
     const int ncoarse        = npix - first_coarse;
@@ -293,55 +308,69 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
                 const bool primary  = (word & kEntryPrimary) != 0;
                 const float z       = E[k].z;
                 float x = E[k].x, y = E[k].y;
+                uint32_t miss = 0, accepted_mask = 0;
 #pragma unroll
                 for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
                 {
                     if (l < lv.num)
                     {
-                        const LevelArg& L = lv.l[l];
-                        int px = f2i_rn(x), py = f2i_rn(y);
-                        bool in = ok[k] && l < nlev && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h &&
-                                  (l < lt || primary);
-                        int cx = px - T.ox[l], cy = py - T.oy[l];
-                        bool local = (unsigned)cx < (unsigned)T.wx[l] && (unsigned)cy < (unsigned)T.wy[l];
-                        bool accepted = false;
-                        if (in && local)
+                        const int px = f2i_rn(x), py = f2i_rn(y);
+                        const int cx = px - T.ox[l], cy = py - T.oy[l];
+                        const bool live = ok[k] && l < nlev && (l < lt || primary);
+                        const bool hit  = live && (unsigned)cx < (unsigned)T.cwx[l] && (unsigned)cy < (unsigned)T.cwy[l];
+                        const int q     = hit ? cy * T.wx[l] + cx : 0;
+                        const bool accepted = hit && !(z > s_depth[T.base[l] + q] * accept);
+                        if (accepted)
                         {
-                            const int q = cy * T.wx[l] + cx;
-                            accepted    = !(z > s_depth[T.base[l] + q] * accept);
-                            if (accepted)
-                            {
-                                int bucket;
-                                if (l == 0)
-                                    bucket = q;
-                                else if (l < lt)
-                                    bucket = kL1Bucket0 + q * kL1Parts + (slot & (kL1Parts - 1));
-                                else
-                                    bucket = kCoarseBucket0 + (T.base[l] - first_coarse + q) * cparts + slot % cparts;
-                                const uint32_t node = (uint32_t)(l * BATCH + slot);
-                                uint32_t old = atomicExch(s_head + bucket, node);
-                                s_next[node] = (uint16_t)old;
-                            }
+                            int bucket;
+                            if (l == 0)
+                                bucket = q;
+                            else if (l < lt)
+                                bucket = kL1Bucket0 + q * kL1Parts + (slot & (kL1Parts - 1));
+                            else
+                                bucket = kCoarseBucket0 + (T.base[l] - first_coarse + q) * cparts + slot % cparts;
+                            const uint32_t node = (uint32_t)(l * BATCH + slot);
+                            uint32_t old = atomicExch(s_head + bucket, node);
+                            s_next[node] = (uint16_t)old;
+                            accepted_mask |= 1u << l;
                         }
-                        else if (in && l >= lt)
+                        if (l >= lt && live && !hit) miss |= 1u << l;
+                        x *= 0.5f;
+                        y *= 0.5f;
+                    }
+                }
+                if (miss)
+                {
+                    // coarse pixel outside the tile's window (does not happen for in-image points): blend straight to memory
+                    x = E[k].x;
+                    y = E[k].y;
+                    for (int l = 0; l < lv.num; ++l)
+                    {
+                        const LevelArg& L = lv.l[l];
+                        const int px = f2i_rn(x), py = f2i_rn(y);
+                        if ((miss >> l & 1u) && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h)
                         {
-                            // outside the window (does not happen for in-image points): blend straight to memory
                             size_t pix = (size_t)py * L.w + px;
                             float d    = __uint_as_float(((const uint32_t*)(L.depth_index + (size_t)b * L.w * L.h + pix))[1]);
-                            accepted   = !(z > d * accept);
-                            if (accepted)
+                            if (!(z > d * accept))
                             {
                                 float* a = accum + (size_t)ws_pixel(lv, l, b, (uint32_t)pix) * S;
 #pragma unroll
                                 for (int c = 0; c < CMAX; ++c)
                                     if (c < C) unsafeAtomicAdd(a + c, t[k][c]);
                                 unsafeAtomicAdd(a + C, 1.f);
+                                accepted_mask |= 1u << l;
                             }
                         }
-                        if (STATS) stat_add(&stats->accepted[l], accepted);
                         x *= 0.5f;
                         y *= 0.5f;
                     }
+                }
+                if (STATS)
+                {
+#pragma unroll
+                    for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+                        if (l < lv.num) stat_add(&stats->accepted[l], (accepted_mask >> l & 1u) != 0);
                 }
             }
             // -- descriptors staged by batch slot ----------------------------------------------------------------
