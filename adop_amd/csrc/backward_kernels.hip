@@ -171,20 +171,23 @@ __global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const
 
     const int i  = blockIdx.x * kBlock + threadIdx.x;
     bool valid   = i < pc.n;
-    bool drop_out = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;
+    bool drop_out;
     V2 ip = {0.f, 0.f};
     float z = 0.f, radius_pixels = 0.f;
     bool ok;
     if (pc.cache)  // kernel-uniform: the forward pass left the projected points with the caller
     {
+        // depth 0: culled; negative depth: dropped for this image (:314-315)
         const float4 R = valid ? pc.cache[(size_t)b * pc.n + i] : make_float4(0, 0, 0, 0);
         ip             = {R.x, R.y};
-        z              = R.z;
+        drop_out       = R.z < 0;
+        z              = fabsf(R.z);
         radius_pixels  = R.w;
         ok             = valid && z != 0;
     }
     else
     {
+        drop_out = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;
         float4 P = valid ? pc.position[i] : make_float4(0, 0, 0, 0);
         V3 pos   = {P.x, P.y, P.z};
         V3 nrm   = {0, 0, 0};

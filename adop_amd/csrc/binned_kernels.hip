@@ -98,18 +98,20 @@ __global__ __launch_bounds__(kBlock) void bin_count_kernel(CloudArg pc, const Vi
     for (int b = 0; b < lv.B; ++b)
     {
         const ViewConst& vc = views[b];
+        // requested before the projection: the kernel is bound by instruction issue, the load hides behind it
+        const float drop_flag = (valid && pc.dropout) ? pc.dropout[(size_t)b * pc.n + i] : 0.f;
         V2 ip = {0.f, 0.f};
         V3 view_p;
         float z = 0.f, radius_pixels = 0.f;
         bool ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff,
                                          lv.l[0].w, &ip, &z, &radius_pixels, &view_p);
         // the second pass (and the backward pass, if the caller keeps the buffer) read this instead of projecting
-        if (valid) pc.cache[(size_t)b * pc.n + i] = ok ? make_float4(ip.x, ip.y, z, radius_pixels) : make_float4(0, 0, 0, 0);
-        if (STATS)
-        {
-            bool dropped = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;
-            stat_add(&stats->bad_index, ok && !dropped && !tex_ok);
-        }
+        // (the sign of the depth carries the dropout flag: the readers need no second array)
+        const bool dropped = drop_flag == 1.f;  // :314-315
+        if (valid)
+            pc.cache[(size_t)b * pc.n + i] =
+                ok ? make_float4(ip.x, ip.y, dropped ? -z : z, radius_pixels) : make_float4(0, 0, 0, 0);
+        if (STATS) stat_add(&stats->bad_index, ok && !dropped && !tex_ok);
         if (!__ballot(ok) && !STATS)  // wavefront-uniform
         {
             if (valid) bin.info[(size_t)b * pc.n + i] = 0;
@@ -174,18 +176,12 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels
             info[k]     = i < pc.n ? bin.info[(size_t)b * pc.n + i] : 0u;
         }
         float4 R[PPT];
-        float drop[PPT];
 #pragma unroll
         for (int k = 0; k < PPT; ++k)
         {
             const int i = base + k * kBlock;
             R[k]        = make_float4(0, 0, 0, 0);
-            drop[k]     = 0.f;
-            if (info[k] & kInfoValid)
-            {
-                R[k] = pc.cache[(size_t)b * pc.n + i];
-                if (pc.dropout) drop[k] = pc.dropout[(size_t)b * pc.n + i];
-            }
+            if (info[k] & kInfoValid) R[k] = pc.cache[(size_t)b * pc.n + i];
         }
         bool any_in[PPT];
         uint32_t nlev[PPT], ptile[PPT], xtile[PPT], gslot[PPT], xslot[PPT];
@@ -224,8 +220,7 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels
         for (int k = 0; k < PPT; ++k)
         {
             const int i         = base + k * kBlock;
-            const float z       = R[k].z;
-            const float zs      = drop[k] == 1.f ? -z : z;  // z > 0: the sign carries the dropout flag (:314-315)
+            const float zs      = R[k].z;  // the sign carries the dropout flag (:314-315)
             const uint32_t word = (uint32_t)i | (nlev[k] << 28);
             if (any_in[k])
             {

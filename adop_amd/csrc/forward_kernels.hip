@@ -121,7 +121,12 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
                                              lv.l[0].w, &ip, &z, &radius_pixels, &view_p);
             // the blend (and the backward pass, if the caller keeps the buffer) read this instead of projecting again
             if (valid && pc.cache)
-                pc.cache[(size_t)b * pc.n + i] = ok ? make_float4(ip.x, ip.y, z, radius_pixels) : make_float4(0, 0, 0, 0);
+            {
+                // (the sign of the depth carries the dropout flag: the readers need no second array)
+                const bool dropped = pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;
+                pc.cache[(size_t)b * pc.n + i] =
+                    ok ? make_float4(ip.x, ip.y, dropped ? -z : z, radius_pixels) : make_float4(0, 0, 0, 0);
+            }
             zz[k]      = z;
             inmask[k]  = 0;
             bool alive = ok;
@@ -239,21 +244,21 @@ __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewCo
 
     for (int b = 0; b < lv.B; ++b)
     {
-        bool dropped = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;  // :314-315
         V2 ip = {0.f, 0.f};
         float z = 0.f, radius_pixels = 0.f;
         bool ok;
         if (pc.cache)
         {
-            // projected by the depth prepass of this call
+            // projected by the depth prepass of this call; dropped points (:314-315) carry a negative depth
             const float4 R = valid ? pc.cache[(size_t)b * pc.n + i] : make_float4(0, 0, 0, 0);
             ip             = {R.x, R.y};
             z              = R.z;
             radius_pixels  = R.w;
-            ok             = valid && !dropped && z != 0;
+            ok             = valid && z > 0;
         }
         else
         {
+            bool dropped = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;  // :314-315
             V3 pos = {P.x, P.y, P.z};
             V3 view_p;
             ok = valid && !dropped &&

@@ -134,7 +134,8 @@ typedef struct adop_forward_buffers
      * that both sides of a parity test see the same mask. */
     const float* dropout_points;
     /* Optional [B,N,4] f32 (no counterpart in the reference, which projects every point again in each of its
-     * three kernels): per view and point the level-0 image point (x,y), the depth (0 = culled) and the LOD
+     * three kernels): per view and point the level-0 image point (x,y), the depth (0 = culled; negative = the point is
+     * dropped for that image, dropout_points) and the LOD
      * radius in pixels.  adop_forward writes it; adop_backward reads it instead of projecting when the same
      * buffer is passed back in `fwd`.  NULL: adop_forward keeps the records in the workspace, adop_backward
      * projects again. */
