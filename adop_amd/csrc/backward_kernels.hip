@@ -15,6 +15,8 @@ namespace adop
 // CombineAndFillBackward (:851-900) fused with the I/G interleave.  One thread per pixel of every level/image.
 // Background gradient: per-thread fp32 partial over a handful of pixels, wave/block reduction in f64, one f64
 // partial row per block.
+typedef float v4f __attribute__((ext_vector_type(4)));
+
 template <int CT>
 __global__ __launch_bounds__(kBlock) void interleave_kernel(Levels lv, float* __restrict__ ig,
                                                             float2* __restrict__ dw, double* __restrict__ partial,
@@ -53,8 +55,8 @@ __global__ __launch_bounds__(kBlock) void interleave_kernel(Levels lv, float* __
         for (int c = 0; c < CMAX; ++c)
             if (c < C)
             {
-                I[c] = im[(size_t)c * hw];
-                G[c] = g[(size_t)c * hw];
+                I[c] = __builtin_nontemporal_load(im + (size_t)c * hw);
+                G[c] = __builtin_nontemporal_load(g + (size_t)c * hw);
                 if (empty) acc[c] += G[c];
             }
         if (CT == 8 || CT == 4)
@@ -82,7 +84,8 @@ __global__ __launch_bounds__(kBlock) void interleave_kernel(Levels lv, float* __
                 wave_lds_sync();
                 float4* d4 = (float4*)(dst - (size_t)lane * (2 * CT));  // record of the wavefront's first pixel
 #pragma unroll
-                for (int k = 0; k < V; ++k) d4[k * 64 + lane] = sw[k * 64 + lane];
+                for (int k = 0; k < V; ++k)
+                    __builtin_nontemporal_store(((const v4f*)sw)[k * 64 + lane], (v4f*)d4 + k * 64 + lane);
             }
             else
             {
@@ -178,7 +181,12 @@ __global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const
     if (pc.cache)  // kernel-uniform: the forward pass left the projected points with the caller
     {
         // depth 0: culled; negative depth: dropped for this image (:314-315)
-        const float4 R = valid ? pc.cache[(size_t)b * pc.n + i] : make_float4(0, 0, 0, 0);
+        float4 R = make_float4(0, 0, 0, 0);
+        if (valid)
+        {
+            const v4f r = __builtin_nontemporal_load((const v4f*)pc.cache + (size_t)b * pc.n + i);
+            R           = make_float4(r.x, r.y, r.z, r.w);
+        }
         ip             = {R.x, R.y};
         drop_out       = R.z < 0;
         z              = fabsf(R.z);
@@ -301,8 +309,9 @@ __global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const
 #pragma unroll
                 for (int c = 0; c < CMAX; ++c)
                 {
+                    // streamed once: kept out of the caches the gathers of this kernel live in
                     float* dst = gtex + (size_t)c * pc.num_texels + i;
-                    *dst       = first_view ? gt[c] : (*dst + gt[c]);
+                    __builtin_nontemporal_store(first_view ? gt[c] : (*dst + gt[c]), dst);
                 }
             }
         }
