@@ -15,8 +15,6 @@ namespace adop
 // CombineAndFillBackward (:851-900) fused with the I/G interleave.  One thread per pixel of every level/image.
 // Background gradient: per-thread fp32 partial over a handful of pixels, wave/block reduction in f64, one f64
 // partial row per block.
-typedef float v4f __attribute__((ext_vector_type(4)));
-
 template <int CT>
 __global__ __launch_bounds__(kBlock) void interleave_kernel(Levels lv, float* __restrict__ ig,
                                                             float2* __restrict__ dw, double* __restrict__ partial,
@@ -713,7 +711,7 @@ __global__ __launch_bounds__(kBlock) void normalize_points_kernel(float* __restr
 {
     int t = blockIdx.x * kBlock + threadIdx.x;
     if (t >= n) return;
-    float c = count[t];
+    float c = __builtin_nontemporal_load(count + t);
     if (!(c > 0)) return;
     size_t o = (mode == 0) ? 3 * (size_t)t : 4 * (size_t)t;
     g[o + 0] = g[o + 0] / c;

@@ -84,8 +84,8 @@ __global__ __launch_bounds__(kBlock) void bin_count_kernel(CloudArg pc, const Vi
 
     const int i      = blockIdx.x * kBlock + threadIdx.x;
     const bool valid = i < pc.n;
-    float4 P         = valid ? pc.position[i] : make_float4(0, 0, 0, 0);
-    int32_t nenc     = (valid && pc.normal) ? pc.normal[i] : 0;
+    float4 P         = valid ? nt_load4(pc.position + i) : make_float4(0, 0, 0, 0);
+    int32_t nenc     = (valid && pc.normal) ? __builtin_nontemporal_load(pc.normal + i) : 0;
     V3 pos           = {P.x, P.y, P.z};
     V3 nrm           = unpack_normal10(nenc);
     bool tex_ok      = true;
@@ -99,7 +99,7 @@ __global__ __launch_bounds__(kBlock) void bin_count_kernel(CloudArg pc, const Vi
     {
         const ViewConst& vc = views[b];
         // requested before the projection: the kernel is bound by instruction issue, the load hides behind it
-        const float drop_flag = (valid && pc.dropout) ? pc.dropout[(size_t)b * pc.n + i] : 0.f;
+        const float drop_flag = (valid && pc.dropout) ? __builtin_nontemporal_load(pc.dropout + (size_t)b * pc.n + i) : 0.f;
         V2 ip = {0.f, 0.f};
         V3 view_p;
         float z = 0.f, radius_pixels = 0.f;
@@ -109,12 +109,12 @@ __global__ __launch_bounds__(kBlock) void bin_count_kernel(CloudArg pc, const Vi
         // (the sign of the depth carries the dropout flag: the readers need no second array)
         const bool dropped = drop_flag == 1.f;  // :314-315
         if (valid)
-            pc.cache[(size_t)b * pc.n + i] =
-                ok ? make_float4(ip.x, ip.y, dropped ? -z : z, radius_pixels) : make_float4(0, 0, 0, 0);
+            nt_store4(pc.cache + (size_t)b * pc.n + i,
+                      ok ? make_float4(ip.x, ip.y, dropped ? -z : z, radius_pixels) : make_float4(0, 0, 0, 0));
         if (STATS) stat_add(&stats->bad_index, ok && !dropped && !tex_ok);
         if (!__ballot(ok) && !STATS)  // wavefront-uniform
         {
-            if (valid) bin.info[(size_t)b * pc.n + i] = 0;
+            if (valid) __builtin_nontemporal_store(0u, bin.info + (size_t)b * pc.n + i);
             continue;
         }
 
@@ -136,7 +136,7 @@ __global__ __launch_bounds__(kBlock) void bin_count_kernel(CloudArg pc, const Vi
                     if (d - (below ? (uint32_t)bin.tiles_x : 0u) == 1u) word |= kInfoRight;
                 }
             }
-            bin.info[(size_t)b * pc.n + i] = word;
+            __builtin_nontemporal_store(word, bin.info + (size_t)b * pc.n + i);
         }
         if (STATS)
         {
@@ -173,7 +173,7 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels
         for (int k = 0; k < PPT; ++k)
         {
             const int i = base + k * kBlock;
-            info[k]     = i < pc.n ? bin.info[(size_t)b * pc.n + i] : 0u;
+            info[k]     = i < pc.n ? __builtin_nontemporal_load(bin.info + (size_t)b * pc.n + i) : 0u;
         }
         float4 R[PPT];
 #pragma unroll
@@ -181,7 +181,7 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels
         {
             const int i = base + k * kBlock;
             R[k]        = make_float4(0, 0, 0, 0);
-            if (info[k] & kInfoValid) R[k] = pc.cache[(size_t)b * pc.n + i];
+            if (info[k] & kInfoValid) R[k] = nt_load4(pc.cache + (size_t)b * pc.n + i);
         }
         bool any_in[PPT];
         uint32_t nlev[PPT], ptile[PPT], xtile[PPT], gslot[PPT], xslot[PPT];

@@ -79,6 +79,20 @@ __device__ __forceinline__ uint32_t ws_pixel(const Levels& lv, int l, int b, uin
     return (uint32_t)lv.pix_prefix[l] * (uint32_t)lv.B + (uint32_t)b * (uint32_t)(lv.l[l].w * lv.l[l].h) + p;
 }
 
+// Streamed data (read or written once per kernel) goes past the caches with the nontemporal hint, so that the lines
+// the gathers of the same kernel reuse stay resident.
+typedef float v4f __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 nt_load4(const float4* p)
+{
+    const v4f r = __builtin_nontemporal_load((const v4f*)p);
+    return make_float4(r.x, r.y, r.z, r.w);
+}
+__device__ __forceinline__ void nt_store4(float4* p, float4 v)
+{
+    v4f r = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(r, (v4f*)p);
+}
+
 template <typename T>
 __device__ __forceinline__ T wave_sum(T v)
 {

@@ -31,7 +31,7 @@ __global__ void fill_u32_kernel(uint32_t* __restrict__ p, size_t n, uint32_t v)
 {
     size_t i      = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (; i < n; i += stride) p[i] = v;
+    for (; i < n; i += stride) __builtin_nontemporal_store(v, p + i);
 }
 
 // InitializeData (PointRenderer.cu:1039-1090): packed depth|index of every level, and the blend accumulators.

@@ -239,7 +239,7 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
         for (int k = 0; k < K; ++k)
         {
             const uint32_t e = start + k * kBlock + tid;
-            Enext[k]         = e < end ? bin.entries[e] : make_float4(0, 0, -1.f, 0);
+            Enext[k]         = e < end ? nt_load4(bin.entries + e) : make_float4(0, 0, -1.f, 0);  // last use of the entry
         }
         // final depth of the local pixels (tile_depth_kernel has completed)
 #pragma unroll
@@ -296,7 +296,7 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
             for (int k = 0; k < K; ++k)
             {
                 const uint32_t e = b0 + BATCH + k * kBlock + tid;
-                Enext[k]         = e < end ? bin.entries[e] : make_float4(0, 0, -1.f, 0);
+                Enext[k]         = e < end ? nt_load4(bin.entries + e) : make_float4(0, 0, -1.f, 0);  // last use of the entry
             }
             // -- fuzzy depth test per level (:380); an accepted (entry, level) is pushed on the list of its bucket ----
 #pragma unroll
@@ -435,13 +435,14 @@ __global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels 
             const size_t hw  = (size_t)L.w * L.h;
             const size_t pix = (size_t)py * L.w + px;
             const size_t o   = (size_t)b * hw + pix;
-            L.weight[o]      = cou;
-            L.depth[o]       = end > start ? s_depth[tid] : 100000.f;  // high word of the packed pixel
-            float* out       = L.out + (size_t)b * C * hw + pix;
+            // the outputs are not read again by this pass: stored past the caches
+            __builtin_nontemporal_store(cou, L.weight + o);
+            __builtin_nontemporal_store(end > start ? s_depth[tid] : 100000.f, L.depth + o);  // high word of the packed pixel
+            float* out = L.out + (size_t)b * C * hw + pix;
 #pragma unroll
             for (int c = 0; c < CMAX; ++c)
-                if (c < C) out[(size_t)c * hw] = (cou == 0) ? background[c] : acc0[c] / cou;
-            if (write_mask && L.mask) L.mask[o] = (cou == 0) ? mask_value : 1.f;
+                if (c < C) __builtin_nontemporal_store((cou == 0) ? background[c] : acc0[c] / cou, out + (size_t)c * hw);
+            if (write_mask && L.mask) __builtin_nontemporal_store((cou == 0) ? mask_value : 1.f, L.mask + o);
         }
     }
     // level 1: buckets kBlock + 2*q and kBlock + 2*q + 1 (adjacent lanes) are the two parts of pixel q
