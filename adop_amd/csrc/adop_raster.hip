@@ -508,12 +508,8 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
         if (!tex_self_clearing &&
             (st = fill_async(grads->grad_texture, sizeof(float) * (size_t)C * scene->num_texels, 0, stream)) != ADOP_OK)
             return st;
-        if (grads->grad_points)
-        {
-            if ((st = fill_async(grads->grad_points, sizeof(float) * 4 * (size_t)N, 0, stream)) != ADOP_OK) return st;
-            if ((st = fill_async(grads->grad_points_count, sizeof(float) * (size_t)N, 0, stream)) != ADOP_OK)
-                return st;
-        }
+        // grad_points / grad_points_count: every row is written by the kernels of the first view
+        // (backward_tex_kernel clears the rows without a spatial gradient, backward_ghost_kernel writes the others)
         if (stats)
         {
             // keep the forward counters, clear only the backward ones

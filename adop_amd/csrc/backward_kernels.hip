@@ -153,7 +153,9 @@ template <int CT, bool HALF>
 __global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const ViewConst* __restrict__ views,
                                                                Levels lv, ParamArg rp, const float* __restrict__ ig,
                                                                const float2* __restrict__ dw,
-                                                               float* __restrict__ gtex, int identity_index,
+                                                               float* __restrict__ gtex,
+                                                               float* __restrict__ gpoints,
+                                                               float* __restrict__ gpoints_count, int identity_index,
                                                                int view_b, int first_view,
                                                                uint32_t* __restrict__ q_counts,
                                                                unsigned long long* __restrict__ q_items,
@@ -320,6 +322,14 @@ __global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const
         }
     }
 
+    // Point gradients of the first view: points without a spatial gradient are cleared here (Build(info,false),
+    // :922-949), the others are written by backward_ghost_kernel; no separate zero-fill of the two buffers.
+    if (first_view && gpoints && valid && mask == 0)
+    {
+        nt_store4((float4*)gpoints + i, make_float4(0, 0, 0, 0));
+        __builtin_nontemporal_store(0.f, gpoints_count + i);
+    }
+
     // queue push: rank inside the workgroup, one returning atomic per workgroup on the sub-queue counter
     bool has               = mask != 0;
     unsigned long long bal = __ballot(has);
@@ -376,6 +386,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
                                                                  float* __restrict__ gpoints,
                                                                  float* __restrict__ gpoints_count, int want_pose,
                                                                  int want_intr, int identity_index, int view_b,
+                                                                 int first_view,
                                                                  const uint32_t* __restrict__ q_prefix,
                                                                  const unsigned long long* __restrict__ q_items,
                                                                  uint32_t q_cap, double* __restrict__ partial)
@@ -434,7 +445,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
         // view, level after level); this thread owns point i for this view
         float gp[3] = {0, 0, 0};
         float gp_n  = 0;
-        if (gpoints)
+        if (gpoints && !first_view)
         {
             const float* g = gpoints + 4 * (size_t)i;
             gp[0]          = g[0];
@@ -565,10 +576,15 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
         }
         if (gpoints)
         {
-            float* g         = gpoints + 4 * (size_t)i;
-            g[0]             = gp[0];
-            g[1]             = gp[1];
-            g[2]             = gp[2];
+            float* g = gpoints + 4 * (size_t)i;
+            if (first_view)
+                *(float4*)g = make_float4(gp[0], gp[1], gp[2], 0.f);  // nothing has cleared the row
+            else
+            {
+                g[0] = gp[0];
+                g[1] = gp[1];
+                g[2] = gp[2];
+            }
             gpoints_count[i] = gp_n;
         }
     }
@@ -741,7 +757,7 @@ static void launch_bwd_tex_t(const CloudArg& pc, const ViewConst* views, const L
 {
     int grid = (pc.n + kBlock - 1) / kBlock;
     hipLaunchKernelGGL((backward_tex_kernel<CT, HALF>), dim3(grid), dim3(kBlock), 0, st, pc, views, lv, rp, ig, dw,
-                       g->grad_texture, identity_index, b, first_view, q.counts, q.items, q.cap, stats);
+                       g->grad_texture, g->grad_points, g->grad_points_count, identity_index, b, first_view, q.counts, q.items, q.cap, stats);
 }
 
 template <int CT, bool HALF>
@@ -752,7 +768,7 @@ static void launch_bwd_ghost_t(const CloudArg& pc, const ViewConst* views, const
 {
     hipLaunchKernelGGL(queue_scan_kernel, dim3(1), dim3(kBlock), 0, st, q.counts, q.prefix);
     hipLaunchKernelGGL((backward_ghost_kernel<CT, HALF>), dim3(ghost_blocks), dim3(kBlock), 0, st, pc, views, lv, rp,
-                       ig, g->grad_points, g->grad_points_count, want_pose, want_intr, identity_index, b, q.prefix,
+                       ig, g->grad_points, g->grad_points_count, want_pose, want_intr, identity_index, b, b == 0, q.prefix,
                        q.items, q.cap, partial);
 }
 
