@@ -421,14 +421,15 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
             else
                 hi = mid;
         }
-        unsigned long long item = q_items[(size_t)lo * q_cap + (t - s_prefix[lo])];
+        // (the item and the point record are read once by this kernel: past the caches, which hold the [I|G] lines)
+        unsigned long long item = __builtin_nontemporal_load(q_items + (size_t)lo * q_cap + (t - s_prefix[lo]));
         const int i             = (int)(uint32_t)item;
         const uint32_t mask     = (uint32_t)(item >> 32);
 
-        float4 P = pc.position[i];
+        float4 P = nt_load4(pc.position + i);
         V3 pos   = {P.x, P.y, P.z};
         V3 nrm   = {0, 0, 0};
-        if (pc.normal) nrm = unpack_normal10(pc.normal[i]);
+        if (pc.normal) nrm = unpack_normal10(__builtin_nontemporal_load(pc.normal + i));
         V2 ip;
         V3 view_p;
         float z, radius_pixels;
