@@ -440,7 +440,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
         if (CT != 0)
         {
 #pragma unroll
-            for (int c = 0; c < CMAX; ++c) T[c] = tex_fetch<HALF>(pc.texture, (size_t)c * pc.num_texels + tex_index);
+            for (int c = 0; c < CMAX; ++c) T[c] = tex_fetch_stream<HALF>(pc.texture, (size_t)c * pc.num_texels + tex_index);
         }
         // running value of grad_points[i] / count[i]: the additions happen in the reference's order (view after
         // view, level after level); this thread owns point i for this view

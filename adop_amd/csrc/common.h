@@ -116,6 +116,18 @@ __device__ __forceinline__ float tex_fetch(const void* tex, size_t o)
     return ((const float*)tex)[o];
 }
 
+// the same with the nontemporal hint
+template <bool HALF>
+__device__ __forceinline__ float tex_fetch_stream(const void* tex, size_t o)
+{
+    if (HALF)
+    {
+        const unsigned short h = __builtin_nontemporal_load((const unsigned short*)tex + o);
+        return __half2float(__ushort_as_half(h));
+    }
+    return __builtin_nontemporal_load((const float*)tex + o);
+}
+
 // LDS written by some lanes of a wavefront is read by other lanes of the same wavefront: DS operations of one
 // wavefront execute in order, so only the compiler has to be kept from moving accesses across this point.
 __device__ __forceinline__ void wave_lds_sync()
