@@ -98,10 +98,10 @@ struct WorkspaceLayout
     size_t bg_partial;  // double[kBgBlocks * kMaxChannels]
     size_t pt_partial;  // double[B * kPartialBlocks * kPartialStride]
     size_t scratch;     // double[num_poses*7 + num_cameras*(cols+1)]
+    size_t fin_mini;    // double[kFinalizeParts * (kMaxChannels + B * kPartialStride)]: first-stage rows of finalize
     size_t pixels;      // float[B * P * max(S, 2C)]: blend accumulators (forward) / [I|G] array (backward)
     size_t dw;          // float2[B * P]: (depth, weight) per pixel for the backward descriptor pass
-    size_t q_counts;    // uint32[kNumQueues]
-    size_t q_prefix;    // uint32[kNumQueues + 1]
+    size_t q_counts;    // uint32[2][kNumQueues]: the views alternate between the two sets; + the finalize ticket
     size_t q_items;     // uint64[kNumQueues * q_cap]
     uint32_t q_cap;
     size_t proj;        // float4[B * N]: projected points of the forward pass when the caller keeps no point_cache
@@ -163,6 +163,8 @@ WorkspaceLayout layout(const adop_scene* s, int B, int L, int w0, int h0)
     w.scratch    = o;
     o = align_up(o + sizeof(double) * ((size_t)s->num_poses * 7 + (size_t)s->num_cameras * (s->intrinsics_cols + 1)),
                  256);
+    w.fin_mini = o;
+    o = align_up(o + sizeof(double) * kFinalizeParts * (kMaxChannels + (size_t)B * kPartialStride), 256);
     w.pixels = o;
     int per  = accum_stride(s->num_channels) > 2 * s->num_channels ? accum_stride(s->num_channels) : 2 * s->num_channels;
     o        = align_up(o + sizeof(float) * (size_t)B * pyramid_pixels(L, w0, h0) * (size_t)per, 256);
@@ -173,9 +175,7 @@ WorkspaceLayout layout(const adop_scene* s, int B, int L, int w0, int h0)
     w.q_cap       = (uint32_t)(((blocks + kNumQueues - 1) / kNumQueues) * kBlock);
     if (w.q_cap == 0) w.q_cap = kBlock;
     w.q_counts = o;
-    o          = align_up(o + sizeof(uint32_t) * kNumQueues, 256);
-    w.q_prefix = o;
-    o          = align_up(o + sizeof(uint32_t) * (kNumQueues + 1), 256);
+    o          = align_up(o + sizeof(uint32_t) * (2 * kNumQueues + 1), 256);
     w.q_items  = o;
     o          = align_up(o + sizeof(unsigned long long) * (size_t)kNumQueues * w.q_cap, 256);
     w.proj       = o;
@@ -307,8 +307,25 @@ ParamArg make_params(const adop_render_params* rp)
     return p;
 }
 
-adop_status upload_views(const adop_scene* s, const adop_view* views, int B, ViewConst* dst, hipStream_t st)
+// The per-view constants: up to 32 views go into *fused, for the first kernel of the call to compute; more views
+// (or no fused kernel) take prepare_views launches.
+adop_status upload_views(const adop_scene* s, const adop_view* views, int B, ViewConst* dst, hipStream_t st,
+                         ViewPrep* fused = nullptr)
 {
+    if (fused)
+    {
+        memset(fused, 0, sizeof(*fused));
+        if (B <= 32)
+        {
+            for (int k = 0; k < B; ++k) fused->chunk.v[k] = views[k];
+            fused->count      = B;
+            fused->cols       = s->intrinsics_cols;
+            fused->poses      = s->poses_se3;
+            fused->intrinsics = s->intrinsics;
+            fused->out        = dst;
+            return ADOP_OK;
+        }
+    }
     for (int first = 0; first < B; first += 32)
     {
         ViewChunk ch;
@@ -360,7 +377,8 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
     hipStream_t stream = (hipStream_t)hip_stream;
     ViewConst* dviews  = (ViewConst*)((char*)workspace + wl.views);
 
-    st = upload_views(scene, views, num_views, dviews, stream);
+    ViewPrep vp;
+    st = upload_views(scene, views, num_views, dviews, stream, &vp);
     if (st != ADOP_OK) return st;
     Levels lv   = make_levels(scene, num_views, buffers, nullptr);
     CloudArg pc = make_cloud(scene, buffers);
@@ -409,7 +427,7 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
             size_t first   = (size_t)lv.pix_prefix[bin.lt] * lv.B * S;
             size_t accum_n = (size_t)lv.pix_prefix[lv.num] * lv.B * S - first;
             int grid       = pixel_grid(lv, bin.lt) > 32 ? pixel_grid(lv, bin.lt) : 32;
-            launch_clear(lv, bin.lt, grid, accum + first, S % 4 == 0 ? accum_n : 0, bin.count, T, stream);
+            launch_clear(lv, bin.lt, grid, accum + first, S % 4 == 0 ? accum_n : 0, bin.count, T, vp, stream);
             if (S % 4 != 0 && (st = fill_async(accum + first, accum_n * sizeof(float), 0, stream)) != ADOP_OK) return st;
         }
         {
@@ -445,10 +463,10 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
     {
         StageScope sc("Initialize", stream);
         if (S % 4 == 0)
-            launch_clear(lv, 0, pixel_grid(lv), accum, accum_n, nullptr, 0, stream);
+            launch_clear(lv, 0, pixel_grid(lv), accum, accum_n, nullptr, 0, vp, stream);
         else
         {
-            launch_clear(lv, 0, pixel_grid(lv), accum, 0, nullptr, 0, stream);
+            launch_clear(lv, 0, pixel_grid(lv), accum, 0, nullptr, 0, vp, stream);
             if ((st = fill_async(accum, accum_n * sizeof(float), 0, stream)) != ADOP_OK) return st;
         }
     }
@@ -492,7 +510,8 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     double* pt_partial = (double*)((char*)workspace + wl.pt_partial);
     double* scratch    = (double*)((char*)workspace + wl.scratch);
 
-    st = upload_views(scene, views, num_views, dviews, stream);
+    ViewPrep vp;
+    st = upload_views(scene, views, num_views, dviews, stream, &vp);
     if (st != ADOP_OK) return st;
     Levels lv   = make_levels(scene, num_views, fwd, grads);
     CloudArg pc = make_cloud(scene, fwd);
@@ -523,7 +542,7 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     int bg_blocks = pixel_grid(lv) < kBgBlocks ? pixel_grid(lv) : kBgBlocks;
     {
         StageScope sc("CombineAndFillBackward", stream);
-        launch_interleave(lv, bg_blocks, ig, dw, bg_partial, (uint32_t*)((char*)workspace + wl.q_counts), stream);
+        launch_interleave(lv, bg_blocks, ig, dw, bg_partial, (uint32_t*)((char*)workspace + wl.q_counts), vp, stream);
     }
     int want_pose = grads->grad_pose != nullptr;
     int want_intr = grads->grad_intrinsics != nullptr;
@@ -533,7 +552,6 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     bool half = scene->texture_dtype == ADOP_TEXTURE_F16;
     QueueArg q;
     q.counts = (uint32_t*)((char*)workspace + wl.q_counts);
-    q.prefix = (uint32_t*)((char*)workspace + wl.q_prefix);
     q.items  = (unsigned long long*)((char*)workspace + wl.q_items);
     q.cap    = wl.q_cap;
     if (N < 1)
@@ -556,9 +574,8 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     }
     StageScope post("Post Process Gradient", stream);
     launch_finalize(dviews, num_views, C, bg_partial, bg_blocks, pt_partial, pt_blocks, grads, scene->num_poses,
-                    scene->num_cameras, scene->intrinsics_cols, params->normalize_mode, scratch, stream);
-    if (grads->grad_points)
-        launch_normalize_points(grads->grad_points, grads->grad_points_count, N, params->normalize_mode, stream);
+                    scene->num_cameras, scene->intrinsics_cols, params->normalize_mode, scratch,
+                    (double*)((char*)workspace + wl.fin_mini), q.counts + 2 * kNumQueues, N, stream);
     ADOP_HIP_CHECK(hipGetLastError());
     return ADOP_OK;
 }

@@ -18,11 +18,16 @@ namespace adop
 template <int CT>
 __global__ __launch_bounds__(kBlock) void interleave_kernel(Levels lv, float* __restrict__ ig,
                                                             float2* __restrict__ dw, double* __restrict__ partial,
-                                                            uint32_t* __restrict__ q_counts)
+                                                            uint32_t* __restrict__ q_counts, ViewPrep vp)
 {
-    // counters of the backward work queue: empty before the first view (queue_scan_kernel empties them again)
+    prepare_views_inline(vp);
+    // counters of the backward work queue: the set of the first view is empty before it (backward_ghost_kernel
+    // empties the set of the next view)
     if (blockIdx.x == 0)
+    {
         for (int k = threadIdx.x; k < kNumQueues; k += kBlock) q_counts[k] = 0;
+        if (threadIdx.x == 0) q_counts[2 * kNumQueues] = 0;  // ticket counter of finalize_kernel
+    }
     constexpr int CMAX = CT ? CT : kMaxChannels;
     const int C        = CT ? CT : lv.C;
     __shared__ double red[kBlock / 64][kMaxChannels];
@@ -352,32 +357,6 @@ __global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const
             (unsigned long long)(uint32_t)i | ((unsigned long long)mask << 32);
 }
 
-// exclusive prefix over the sub-queue counters: prefix[0..kNumQueues], prefix[kNumQueues] = number of items; the
-// counters are left at zero for the next view
-__global__ __launch_bounds__(kBlock) void queue_scan_kernel(uint32_t* __restrict__ counts,
-                                                            uint32_t* __restrict__ prefix)
-{
-    constexpr int PER = kNumQueues / kBlock;
-    __shared__ uint32_t s_sum[kBlock];
-    uint32_t local[PER];
-    uint32_t acc = 0;
-#pragma unroll
-    for (int k = 0; k < PER; ++k)
-    {
-        local[k] = acc;
-        acc += counts[threadIdx.x * PER + k];
-    }
-#pragma unroll
-    for (int k = 0; k < PER; ++k) counts[threadIdx.x * PER + k] = 0;
-    s_sum[threadIdx.x] = acc;
-    __syncthreads();
-    uint32_t base = 0;
-    for (int t = 0; t < (int)threadIdx.x; ++t) base += s_sum[t];
-#pragma unroll
-    for (int k = 0; k < PER; ++k) prefix[threadIdx.x * PER + k] = base + local[k];
-    if (threadIdx.x == kBlock - 1) prefix[kNumQueues] = base + acc;
-}
-
 // 4 waves per SIMD (<= 128 VGPRs): the grid of kPartialBlocks = 4 workgroups x 256 CUs is then resident at once; with
 // the 151 VGPRs the compiler takes by itself only 3 fit and a quarter of the grid runs as a second, mostly idle round.
 template <int CT, bool HALF>
@@ -387,7 +366,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
                                                                  float* __restrict__ gpoints_count, int want_pose,
                                                                  int want_intr, int identity_index, int view_b,
                                                                  int first_view,
-                                                                 const uint32_t* __restrict__ q_prefix,
+                                                                 const uint32_t* __restrict__ q_counts,
+                                                                 uint32_t* __restrict__ q_counts_next,
                                                                  const unsigned long long* __restrict__ q_items,
                                                                  uint32_t q_cap, double* __restrict__ partial)
 {
@@ -399,8 +379,41 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
     const float accept  = rp.depth_accept + 1;
     const int C         = CT ? CT : lv.C;
 
-    for (int k = threadIdx.x; k <= kNumQueues; k += kBlock) s_prefix[k] = q_prefix[k];
-    __syncthreads();
+    // Exclusive prefix over the sub-queue counters, by every workgroup for itself (8 KB from the L2; a kernel of its
+    // own for it cost more than all these prologues): s_prefix[0..kNumQueues], s_prefix[kNumQueues] = number of items.
+    {
+        constexpr int PER = kNumQueues / kBlock;
+        static_assert(PER == 8, "two 16-byte loads per thread");
+        __shared__ uint32_t s_wave[kBlock / 64];
+        const uint4 c0 = *(const uint4*)(q_counts + threadIdx.x * PER);
+        const uint4 c1 = *(const uint4*)(q_counts + threadIdx.x * PER + 4);
+        const uint32_t v[PER] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+        uint32_t sum = 0;
+#pragma unroll
+        for (int k = 0; k < PER; ++k) sum += v[k];
+        uint32_t inc = sum;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1)
+        {
+            uint32_t u = __shfl_up(inc, off, 64);
+            if ((int)(threadIdx.x & 63) >= off) inc += u;
+        }
+        if ((threadIdx.x & 63) == 63) s_wave[threadIdx.x >> 6] = inc;
+        __syncthreads();
+        uint32_t run = inc - sum;
+        for (int w = 0; w < (int)(threadIdx.x >> 6); ++w) run += s_wave[w];
+#pragma unroll
+        for (int k = 0; k < PER; ++k)
+        {
+            s_prefix[threadIdx.x * PER + k] = run;
+            run += v[k];
+        }
+        if (threadIdx.x == kBlock - 1) s_prefix[kNumQueues] = run;
+        // the other set of counters is the next view's: nothing reads it before this kernel has ended
+        if (blockIdx.x == 0)
+            for (int k = threadIdx.x; k < kNumQueues; k += kBlock) q_counts_next[k] = 0;
+        __syncthreads();
+    }
     const uint32_t total = s_prefix[kNumQueues];
 
     // per-thread sums of the pose / intrinsics gradients: a thread sees a few dozen contributions at most, so fp32
@@ -608,26 +621,53 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
     }
 }
 
-constexpr int kFinalizeBlock = 1024;  // one workgroup; the partial rows are read with 16 loads in flight per thread
+constexpr int kFinalizeBlock = 1024;  // the reduction as a kernel of its own: one workgroup, 16 loads in flight per thread
 
 // Reduces the per-block partial rows and runs NormalizeGradient (:1534-1547, launches :1611-1636) for the
-// background / pose / intrinsics outputs.  One block.
-__global__ __launch_bounds__(kFinalizeBlock) void finalize_kernel(const ViewConst* __restrict__ views, int B, int C,
-                                                          const double* __restrict__ bg_partial, int bg_blocks,
-                                                          const double* __restrict__ pt_partial, int pt_blocks,
-                                                          float* __restrict__ gbg, double* __restrict__ gpose,
-                                                          float* __restrict__ gpose_count, int num_poses,
-                                                          float* __restrict__ gintr, float* __restrict__ gintr_count,
-                                                          int num_cameras, int cols, int normalize_mode,
-                                                          double* __restrict__ scratch)
+// background / pose / intrinsics outputs.  One block of NT threads; sh holds NT values.
+struct FinalizeArg
 {
-    __shared__ double sh[kFinalizeBlock];
+    const ViewConst* views;
+    int B, C;
+    const double* bg_partial;
+    int bg_blocks;
+    const double* pt_partial;
+    int pt_blocks;
+    float* gbg;
+    double* gpose;
+    float* gpose_count;
+    int num_poses;
+    float* gintr;
+    float* gintr_count;
+    int num_cameras, cols, normalize_mode;
+    double* scratch;
+    double* mini;      // [kFinalizeParts * kMaxChannels] + [B * kFinalizeParts * kPartialStride]: rows of the first stage
+    uint32_t* ticket;  // zero at the start of the kernel
+};
+
+constexpr int kFinalizeSmall = 1024;  // pose / intrinsics sums of up to this many f64 stay in LDS
+
+template <int NT>
+__device__ static void finalize_block(const FinalizeArg& a, double* sh, double* s_small)
+{
+    const ViewConst* __restrict__ views = a.views;
+    const int B = a.B, C = a.C, bg_blocks = a.bg_blocks, pt_blocks = a.pt_blocks, num_poses = a.num_poses,
+              num_cameras = a.num_cameras, cols = a.cols, normalize_mode = a.normalize_mode;
+    const double* __restrict__ bg_partial = a.bg_partial;
+    const double* __restrict__ pt_partial = a.pt_partial;
+    float* __restrict__ gbg               = a.gbg;
+    double* __restrict__ gpose            = a.gpose;
+    float* __restrict__ gpose_count       = a.gpose_count;
+    float* __restrict__ gintr             = a.gintr;
+    float* __restrict__ gintr_count       = a.gintr_count;
+    // flat pointer: LDS when the sums fit (every round trip to memory is on this block's critical path)
+    double* scratch = (num_poses * 7 + num_cameras * (cols + 1) <= kFinalizeSmall) ? s_small : a.scratch;
     // background: thread t sums channel t%16 over the partial rows t/16, t/16+16, ...
     {
         const int c = threadIdx.x % kMaxChannels, k0 = threadIdx.x / kMaxChannels;
-        constexpr int GR = kFinalizeBlock / kMaxChannels;
+        constexpr int GR = NT / kMaxChannels;
         double v = 0;
-#pragma unroll 16
+#pragma unroll(NT >= 1024 ? 16 : 8)
         for (int k = k0; k < bg_blocks; k += GR) v += bg_partial[(size_t)k * kMaxChannels + c];
         sh[threadIdx.x] = v;
         __syncthreads();
@@ -644,16 +684,16 @@ __global__ __launch_bounds__(kFinalizeBlock) void finalize_kernel(const ViewCons
     // scratch: [num_poses*7] pose sums + count, then [num_cameras*(cols+1)] intrinsics sums + count
     double* sp = scratch;
     double* si = scratch + (size_t)num_poses * 7;
-    for (int k = threadIdx.x; k < num_poses * 7 + num_cameras * (cols + 1); k += kFinalizeBlock) scratch[k] = 0;
+    for (int k = threadIdx.x; k < num_poses * 7 + num_cameras * (cols + 1); k += NT) scratch[k] = 0;
     __syncthreads();
     for (int b = 0; b < B; ++b)
     {
         // thread t sums value t%32 (21 used) over the partial rows t/32, t/32+8, ...
         const int q = threadIdx.x % 32, k0 = threadIdx.x / 32;
-        constexpr int GR = kFinalizeBlock / 32;
+        constexpr int GR = NT / 32;
         double v = 0;
         if (q < kAcc)
-#pragma unroll 16
+#pragma unroll(NT >= 1024 ? 16 : 8)
             for (int k = k0; k < pt_blocks; k += GR) v += pt_partial[((size_t)b * pt_blocks + k) * kPartialStride + q];
         sh[threadIdx.x] = v;
         __syncthreads();
@@ -677,7 +717,7 @@ __global__ __launch_bounds__(kFinalizeBlock) void finalize_kernel(const ViewCons
     }
     if (gpose)
     {
-        for (int f = threadIdx.x; f < num_poses; f += kFinalizeBlock)
+        for (int f = threadIdx.x; f < num_poses; f += NT)
         {
             float c        = (float)sp[(size_t)f * 7 + 6];
             gpose_count[f] = c;
@@ -690,43 +730,101 @@ __global__ __launch_bounds__(kFinalizeBlock) void finalize_kernel(const ViewCons
     }
     if (gintr)
     {
-        for (int k = threadIdx.x; k < num_cameras * cols; k += kFinalizeBlock)
-            gintr[k] = (float)si[(size_t)(k / cols) * (cols + 1) + (k % cols)];
-        for (int k = threadIdx.x; k < num_cameras; k += kFinalizeBlock) gintr_count[k] = (float)si[(size_t)k * (cols + 1) + cols];
-        __syncthreads();
-        if (threadIdx.x == 0)
+        // NormalizeGradient<float,13> on the flat buffer whatever the row width (:1633) in mode 0: element t = floats
+        // 13t..13t+12 divided by count[t]; mode 1 normalises row t
+        const int total = num_cameras * cols;
+        for (int k = threadIdx.x; k < total; k += NT)
         {
-            int total = num_cameras * cols;
-            if (normalize_mode == 0)
+            float v     = (float)si[(size_t)(k / cols) * (cols + 1) + (k % cols)];
+            const int t = normalize_mode == 0 ? k / 13 : k / cols;
+            if (t < num_cameras)
             {
-                // NormalizeGradient<float,13> whatever the row width (:1633)
-                for (int t = 0; t < num_cameras; ++t)
-                {
-                    float c = gintr_count[t];
-                    if (c > 0)
-                        for (int k = 0; k < 13; ++k)
-                            if (13 * t + k < total) gintr[13 * t + k] = gintr[13 * t + k] / c;
-                }
+                const float c = (float)si[(size_t)t * (cols + 1) + cols];
+                if (c > 0) v = v / c;
             }
-            else
-            {
-                for (int t = 0; t < num_cameras; ++t)
-                {
-                    float c = gintr_count[t];
-                    if (c > 0)
-                        for (int k = 0; k < cols; ++k) gintr[cols * t + k] = gintr[cols * t + k] / c;
-                }
-            }
+            gintr[k] = v;
         }
+        for (int k = threadIdx.x; k < num_cameras; k += NT) gintr_count[k] = (float)si[(size_t)k * (cols + 1) + cols];
     }
 }
 
 // NormalizeGradient<float,3> on the [N,4] point-gradient buffer (:1620-1627).  mode 0 reproduces the reference's
 // vec3 view (element t = floats 3t..3t+2 divided by count[t]); mode 1 normalises row t by count[t].
-__global__ __launch_bounds__(kBlock) void normalize_points_kernel(float* __restrict__ g, const float* __restrict__ count,
-                                                                  int n, int mode)
+// Fused with the reduction of the partial rows, which then costs no launch of its own and hides behind the
+// normalisation.  One workgroup reads the ~400 KB of partial rows in 16 us when nothing else runs and in ~50 us next
+// to the normalisation's traffic, so with point gradients the reduction has two stages: workgroups 0..kFinalizeParts-1
+// each reduce a slice of the rows to one row, and the one that finishes last (ticket counter) reduces those rows, in
+// their fixed order, and writes the outputs.  The other workgroups normalise.  Without point gradients (n = 0) a
+// single workgroup of NT = kFinalizeBlock threads does the whole reduction.
+template <int NT>
+__device__ __forceinline__ void finalize_body(FinalizeArg a, float* __restrict__ g, const float* __restrict__ count, int n,
+                                              int mode)
 {
-    int t = blockIdx.x * kBlock + threadIdx.x;
+    const int first_stage = n > 0 ? kFinalizeParts : 0;
+    if ((int)blockIdx.x < (first_stage ? first_stage : 1))
+    {
+        __shared__ double sh[NT];
+        __shared__ double s_small[kFinalizeSmall];
+        __shared__ int s_last;
+        if (first_stage)
+        {
+            const int r  = blockIdx.x;
+            double* bg_m = a.mini;
+            double* pt_m = a.mini + kFinalizeParts * kMaxChannels;
+            {
+                const int c = threadIdx.x % kMaxChannels, k0 = threadIdx.x / kMaxChannels;
+                constexpr int GR = NT / kMaxChannels;
+                const int lo = (int)((long long)a.bg_blocks * r / kFinalizeParts);
+                const int hi = (int)((long long)a.bg_blocks * (r + 1) / kFinalizeParts);
+                double v     = 0;
+#pragma unroll 8
+                for (int k = lo + k0; k < hi; k += GR) v += a.bg_partial[(size_t)k * kMaxChannels + c];
+                sh[threadIdx.x] = v;
+                __syncthreads();
+                if (threadIdx.x < kMaxChannels)
+                {
+                    double t = 0;
+                    for (int q = 0; q < GR; ++q) t += sh[q * kMaxChannels + threadIdx.x];
+                    bg_m[r * kMaxChannels + threadIdx.x] = t;
+                }
+                __syncthreads();
+            }
+            for (int b = 0; b < a.B; ++b)
+            {
+                const int q = threadIdx.x % 32, k0 = threadIdx.x / 32;
+                constexpr int GR = NT / 32;
+                const int lo = (int)((long long)a.pt_blocks * r / kFinalizeParts);
+                const int hi = (int)((long long)a.pt_blocks * (r + 1) / kFinalizeParts);
+                double v     = 0;
+                if (q < kAcc)
+#pragma unroll 8
+                    for (int k = lo + k0; k < hi; k += GR)
+                        v += a.pt_partial[((size_t)b * a.pt_blocks + k) * kPartialStride + q];
+                sh[threadIdx.x] = v;
+                __syncthreads();
+                if (threadIdx.x < kAcc)
+                {
+                    double t = 0;
+                    for (int w = 0; w < GR; ++w) t += sh[w * 32 + threadIdx.x];
+                    pt_m[((size_t)b * kFinalizeParts + r) * kPartialStride + threadIdx.x] = t;
+                }
+                __syncthreads();
+            }
+            __threadfence();  // the rows of this workgroup are visible before its ticket is
+            __syncthreads();
+            if (threadIdx.x == 0) s_last = atomicAdd(a.ticket, 1u) == (uint32_t)(kFinalizeParts - 1);
+            __syncthreads();
+            if (!s_last) return;
+            __threadfence();
+            a.bg_partial = bg_m;
+            a.bg_blocks  = kFinalizeParts;
+            a.pt_partial = pt_m;
+            a.pt_blocks  = kFinalizeParts;
+        }
+        finalize_block<NT>(a, sh, s_small);
+        return;
+    }
+    int t = (blockIdx.x - first_stage) * NT + threadIdx.x;
     if (t >= n) return;
     float c = __builtin_nontemporal_load(count + t);
     if (!(c > 0)) return;
@@ -736,19 +834,31 @@ __global__ __launch_bounds__(kBlock) void normalize_points_kernel(float* __restr
     g[o + 2] = g[o + 2] / c;
 }
 
+__global__ __launch_bounds__(kFinalizeBlock) void finalize_kernel(FinalizeArg a)
+{
+    finalize_body<kFinalizeBlock>(a, nullptr, nullptr, 0, 0);
+}
+
+// 8 waves per SIMD (<= 64 VGPRs): the normalisation lives on memory latency; the registers the reduction would like
+// to take (104) halve its occupancy and cost it 40%.
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) void finalize_normalize_kernel(
+    FinalizeArg a, float* __restrict__ g, const float* __restrict__ count, int n, int mode)
+{
+    finalize_body<kBlock>(a, g, count, n, mode);
+}
 
 // ------------------------------------------------------------------------------------------------
 // launchers
 // ------------------------------------------------------------------------------------------------
 void launch_interleave(const Levels& lv, int blocks, float* ig, float2* dw, double* partial, uint32_t* q_counts,
-                       hipStream_t st)
+                       const ViewPrep& vp, hipStream_t st)
 {
     if (lv.C == 8)
-        hipLaunchKernelGGL((interleave_kernel<8>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, dw, partial, q_counts);
+        hipLaunchKernelGGL((interleave_kernel<8>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, dw, partial, q_counts, vp);
     else if (lv.C == 4)
-        hipLaunchKernelGGL((interleave_kernel<4>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, dw, partial, q_counts);
+        hipLaunchKernelGGL((interleave_kernel<4>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, dw, partial, q_counts, vp);
     else
-        hipLaunchKernelGGL((interleave_kernel<0>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, dw, partial, q_counts);
+        hipLaunchKernelGGL((interleave_kernel<0>), dim3(blocks), dim3(kBlock), 0, st, lv, ig, dw, partial, q_counts, vp);
 }
 
 template <int CT, bool HALF>
@@ -758,7 +868,8 @@ static void launch_bwd_tex_t(const CloudArg& pc, const ViewConst* views, const L
 {
     int grid = (pc.n + kBlock - 1) / kBlock;
     hipLaunchKernelGGL((backward_tex_kernel<CT, HALF>), dim3(grid), dim3(kBlock), 0, st, pc, views, lv, rp, ig, dw,
-                       g->grad_texture, g->grad_points, g->grad_points_count, identity_index, b, first_view, q.counts, q.items, q.cap, stats);
+                       g->grad_texture, g->grad_points, g->grad_points_count, identity_index, b, first_view,
+                       q.counts + (b & 1) * kNumQueues, q.items, q.cap, stats);
 }
 
 template <int CT, bool HALF>
@@ -767,10 +878,10 @@ static void launch_bwd_ghost_t(const CloudArg& pc, const ViewConst* views, const
                                int identity_index, int b, const QueueArg& q, int ghost_blocks, double* partial,
                                hipStream_t st)
 {
-    hipLaunchKernelGGL(queue_scan_kernel, dim3(1), dim3(kBlock), 0, st, q.counts, q.prefix);
     hipLaunchKernelGGL((backward_ghost_kernel<CT, HALF>), dim3(ghost_blocks), dim3(kBlock), 0, st, pc, views, lv, rp,
-                       ig, g->grad_points, g->grad_points_count, want_pose, want_intr, identity_index, b, b == 0, q.prefix,
-                       q.items, q.cap, partial);
+                       ig, g->grad_points, g->grad_points_count, want_pose, want_intr, identity_index, b, b == 0,
+                       q.counts + (b & 1) * kNumQueues, q.counts + ((b + 1) & 1) * kNumQueues, q.items, q.cap,
+                       partial);
 }
 
 #define ADOP_DISPATCH_C_HALF(FN, ...)                                   \
@@ -807,17 +918,18 @@ void launch_backward_ghost(const CloudArg& pc, const ViewConst* views, const Lev
 
 void launch_finalize(const ViewConst* views, int B, int C, const double* bg_partial, int bg_blocks,
                      const double* pt_partial, int pt_blocks, const adop_backward_buffers* g, int num_poses,
-                     int num_cameras, int cols, int normalize_mode, double* scratch, hipStream_t st)
+                     int num_cameras, int cols, int normalize_mode, double* scratch, double* mini, uint32_t* ticket, int n,
+                     hipStream_t st)
 {
-    hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kFinalizeBlock), 0, st, views, B, C, bg_partial, bg_blocks, pt_partial,
-                       pt_blocks, g->grad_background, g->grad_pose, g->grad_pose_count, num_poses, g->grad_intrinsics,
-                       g->grad_intrinsics_count, num_cameras, cols, normalize_mode, scratch);
-}
-
-void launch_normalize_points(float* g, const float* count, int n, int mode, hipStream_t st)
-{
-    if (n < 1) return;
-    hipLaunchKernelGGL(normalize_points_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, g, count, n, mode);
+    FinalizeArg a{views, B, C, bg_partial, bg_blocks, pt_partial, pt_blocks, g->grad_background, g->grad_pose,
+                  g->grad_pose_count, num_poses, g->grad_intrinsics, g->grad_intrinsics_count, num_cameras, cols,
+                  normalize_mode, scratch, mini, ticket};
+    if (!g->grad_points || n < 1) n = 0;
+    if (n == 0)
+        hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kFinalizeBlock), 0, st, a);
+    else
+        hipLaunchKernelGGL(finalize_normalize_kernel, dim3(kFinalizeParts + (n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, a,
+                           g->grad_points, g->grad_points_count, n, normalize_mode);
 }
 
 }  // namespace adop

@@ -17,6 +17,7 @@ constexpr int kPartialBlocks = 1024;  // grid of backward_ghost_kernel: per-bloc
 constexpr int kBgBlocks      = 2048;  // grid of interleave_kernel: per-block partial sums of the background gradient
 constexpr int kPartialStride = 24;    // doubles per (block, view), 21 used: 6 pose, pose count, intr count, 13 intr
 constexpr int kAcc           = 21;
+constexpr int kFinalizeParts = 16;    // workgroups of the first stage of the final two-stage reduction
 constexpr int kNumQueues     = 2048;  // sub-queues of the backward work queue (multiple of kBlock)
 constexpr int kMaxIntrinsicsCols = 24;  // 13 pinhole / 5 affine + up to 19 polynomial coefficients
 constexpr uint64_t kClearPacked = (uint64_t(0x47C35000u) << 32) | 0xFFFFFFFFull;  // bits(100000.f), PointRenderer.cu:1045
@@ -70,6 +71,18 @@ struct ParamArg
 struct ViewChunk
 {
     adop_view v[32];
+};
+
+// Up to 32 views whose constants the first kernel of a call computes on the side (count = 0: nothing to do, the
+// constants were written by prepare_views launches).
+struct ViewPrep
+{
+    ViewChunk chunk;
+    int count;
+    int cols;
+    const double* poses;
+    const float* intrinsics;
+    ViewConst* out;
 };
 
 // Workspace pixel index of pixel p of level l of image b: all levels and images of a call form one array
@@ -204,6 +217,13 @@ __device__ __forceinline__ ViewConst make_view_const(const adop_view& v, const d
     c.npoly        = cols - 5;
     c.pad          = 0;
     return c;
+}
+
+// The per-view constants computed inside the first kernel of a call: one block spends its first lanes on it.
+__device__ __forceinline__ void prepare_views_inline(const ViewPrep& vp)
+{
+    if (blockIdx.x == gridDim.x - 1 && (int)threadIdx.x < vp.count)
+        vp.out[threadIdx.x] = make_view_const(vp.chunk.v[threadIdx.x], vp.poses, vp.intrinsics, vp.cols);
 }
 
 // level of flattened per-image pixel index r (pix_prefix is increasing)

@@ -37,8 +37,10 @@ __global__ void fill_u32_kernel(uint32_t* __restrict__ p, size_t n, uint32_t v)
 // InitializeData (PointRenderer.cu:1039-1090): packed depth|index of every level, and the blend accumulators.
 // Levels below first_level are left alone (the tile path writes them itself).
 __global__ __launch_bounds__(kBlock) void clear_kernel(Levels lv, int first_level, float4* __restrict__ accum,
-                                                       size_t accum_vec4, uint32_t* __restrict__ zero_u32, int zero_n)
+                                                       size_t accum_vec4, uint32_t* __restrict__ zero_u32, int zero_n,
+                                                       ViewPrep vp)
 {
+    prepare_views_inline(vp);
     // counters of the tile bins (tile path only)
     for (int k = blockIdx.x * blockDim.x + threadIdx.x; k < zero_n; k += gridDim.x * blockDim.x) zero_u32[k] = 0;
     int r0        = lv.pix_prefix[first_level];
@@ -454,10 +456,10 @@ void launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t st)
 }
 
 void launch_clear(const Levels& lv, int first_level, int grid, float* accum, size_t accum_floats, uint32_t* zero_u32,
-                  int zero_n, hipStream_t st)
+                  int zero_n, const ViewPrep& vp, hipStream_t st)
 {
     hipLaunchKernelGGL(clear_kernel, dim3(grid), dim3(kBlock), 0, st, lv, first_level, (float4*)accum, accum_floats / 4,
-                       zero_u32, zero_n);
+                       zero_u32, zero_n, vp);
 }
 
 void launch_prepass(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, adop_stats* stats,

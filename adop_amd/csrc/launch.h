@@ -15,7 +15,7 @@ void launch_prepare_views(const ViewChunk& ch, int first, int count, const doubl
                           int cols, ViewConst* out, hipStream_t st);
 void launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t st);
 void launch_clear(const Levels& lv, int first_level, int grid, float* accum, size_t accum_floats, uint32_t* zero_u32,
-                  int zero_n, hipStream_t st);
+                  int zero_n, const ViewPrep& vp, hipStream_t st);
 void launch_prepass(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, adop_stats* stats,
                     hipStream_t st);
 void launch_blend(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
@@ -51,13 +51,12 @@ hipError_t launch_tile_blend(const CloudArg& pc, const Levels& lv, const ParamAr
                              float mask_value, int identity_index, adop_stats* stats, hipStream_t st);
 
 void launch_interleave(const Levels& lv, int blocks, float* ig, float2* dw, double* partial, uint32_t* q_counts,
-                       hipStream_t st);
+                       const ViewPrep& vp, hipStream_t st);
 // Work queue of the backward pass (points that receive a ghost / spatial gradient), split in kNumQueues sub-queues
 // of `cap` items each.
 struct QueueArg
 {
-    uint32_t* counts;           // [kNumQueues]
-    uint32_t* prefix;           // [kNumQueues + 1]
+    uint32_t* counts;           // [2][kNumQueues]: view b appends through set b & 1
     unsigned long long* items;  // [kNumQueues * cap]
     uint32_t cap;
 };
@@ -70,8 +69,8 @@ void launch_backward_ghost(const CloudArg& pc, const ViewConst* views, const Lev
                            hipStream_t st);
 void launch_finalize(const ViewConst* views, int B, int C, const double* bg_partial, int bg_blocks,
                      const double* pt_partial, int pt_blocks, const adop_backward_buffers* g, int num_poses,
-                     int num_cameras, int cols, int normalize_mode, double* scratch, hipStream_t st);
-void launch_normalize_points(float* g, const float* count, int n, int mode, hipStream_t st);
+                     int num_cameras, int cols, int normalize_mode, double* scratch, double* mini, uint32_t* ticket, int n,
+                     hipStream_t st);
 
 void launch_env_sample(const ViewChunk& chunk, const double* poses, const float* intrinsics, const Levels& lv,
                        const EnvLevels& ev, const float* tex, int eh, int ew, int add_to_out, hipStream_t st);
