@@ -108,7 +108,14 @@ __global__ __launch_bounds__(kBlock) void tile_depth_kernel(Levels lv, BinArg bi
                 const int cx = px - T.ox[l], cy = py - T.oy[l];
                 const bool live = l < nlev && (l < bin.lt || primary);
                 const bool hit  = live && (unsigned)cx < (unsigned)T.cwx[l] && (unsigned)cy < (unsigned)T.cwy[l];
-                if (hit) atomicMin(&s_depth[T.base[l] + cy * T.wx[l] + cx], (unsigned long long)pk);
+                if (hit)
+                {
+                    // Early depth test on the LDS copy from level 1 on: the entries of a tile share few coarse pixels,
+                    // LDS atomics of one instruction on one address run one after the other, and after the first
+                    // batches most entries lose against the value already there (a plain read is a broadcast).
+                    unsigned long long* dst = &s_depth[T.base[l] + cy * T.wx[l] + cx];
+                    if (l == 0 || pk < *(volatile unsigned long long*)dst) atomicMin(dst, (unsigned long long)pk);
+                }
                 if (l >= bin.lt && live && !hit) miss |= 1u << l;
                 x *= 0.5f;
                 y *= 0.5f;
