@@ -205,14 +205,14 @@ def main():
     dom = max((k for k in model if k in stages), key=lambda k: stages[k])
     dom_gbs = model[dom] / (stages[dom] * 1e-3) / 1e9
     # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
-    # FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 after calibration with a plain 1 GiB copy); measured for the default
+    # FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 after calibration with plain device copies); measured for the default
     # workload only
     measured_traffic = {}
     if args.workload == "config3" and not args.points and args.point_order == "morton" and not args.no_point_cache:
         # profiles/config3_tile_path_fwd_bwd_kernels_traffic_instructions.md, profiles/config3_fwd_bwd_kernels_traffic_atomics.md
-        measured_traffic = {"RenderBackward/descriptor": 763.5e6, "RenderBackward/spatial": 627.7e6, "TileBlend": 438.6e6,
-                            "BinCount": 412.9e6, "BinScatter": 222.9e6, "TileDepth": 101.0e6,
-                            "CombineAndFillBackward": 397.1e6, "RenderForward": 691.9e6}
+        measured_traffic = {"RenderBackward/descriptor": 912.7e6, "RenderBackward/spatial": 552.5e6, "TileBlend": 432.3e6,
+                            "BinCount": 458.9e6, "BinScatter": 204.3e6, "TileDepth": 101.0e6,
+                            "CombineAndFillBackward": 397.3e6, "RenderForward": 691.9e6}
     roofline = {"bound": "hbm", "kernel": KERNEL_OF_STAGE.get(dom, dom), "stage": dom, "achieved": round(dom_gbs, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
                 "traffic": measured_traffic.get(dom),
