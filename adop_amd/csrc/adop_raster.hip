@@ -104,7 +104,10 @@ struct WorkspaceLayout
     size_t q_counts;    // uint32[2][kNumQueues]: the views alternate between the two sets; + the finalize ticket
     size_t q_items;     // uint64[kNumQueues * q_cap]
     uint32_t q_cap;
-    size_t proj;        // float4[B * N]: projected points of the forward pass when the caller keeps no point_cache
+    size_t proj;        // float4[B * list_stride]: projected points of the forward pass when the caller keeps no point_cache
+    size_t list_stride; // N rounded up to whole prepass workgroups
+    size_t list_ids;    // uint32[B * list_stride]: candidate lists of the direct forward path (records in proj)
+    size_t list_count;  // uint32[B * 4 * ceil(N / 256)]
     size_t bin_count;   // uint32[max tiles]           tile bins of the forward pass
     size_t bin_offset;  // uint32[max tiles + 1]
     size_t bin_info;    // uint32[B * N]
@@ -178,8 +181,15 @@ WorkspaceLayout layout(const adop_scene* s, int B, int L, int w0, int h0)
     o          = align_up(o + sizeof(uint32_t) * (2 * kNumQueues + 1), 256);
     w.q_items  = o;
     o          = align_up(o + sizeof(unsigned long long) * (size_t)kNumQueues * w.q_cap, 256);
+    // (a view's slots are rounded up to whole prepass workgroups of at most 4 * kBlock points: list mode)
+    const size_t n_pad = (((size_t)(s->num_points > 0 ? s->num_points : 0) + 4 * kBlock - 1) / (4 * kBlock)) * (4 * kBlock);
+    w.list_stride = n_pad;
     w.proj       = o;
-    o            = align_up(o + sizeof(float4) * (size_t)B * (size_t)(s->num_points > 0 ? s->num_points : 0), 256);
+    o            = align_up(o + sizeof(float4) * (size_t)B * n_pad, 256);
+    w.list_ids   = o;
+    o            = align_up(o + sizeof(uint32_t) * (size_t)B * n_pad, 256);
+    w.list_count = o;
+    o = align_up(o + 4 * sizeof(uint32_t) * (size_t)B * (((size_t)(s->num_points > 0 ? s->num_points : 0) + kBlock - 1) / kBlock), 256);
     size_t T     = max_tiles(B, w0, h0);
     w.bin_count  = o;
     o            = align_up(o + sizeof(uint32_t) * T, 256);
@@ -289,6 +299,10 @@ CloudArg make_cloud(const adop_scene* s, const adop_forward_buffers* fb)
     c.intrinsics = s->intrinsics;
     c.dropout    = fb->dropout_points;
     c.cache      = (float4*)fb->point_cache;
+    c.list_ids   = nullptr;
+    c.list_count = nullptr;
+    c.list_span  = 0;
+    c.list_stride = 0;
     return c;
 }
 
@@ -459,6 +473,17 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
         return ADOP_OK;
     }
 
+    // Without a caller's point cache (no backward pass follows) the prepass hands the blend compacted lists of the
+    // points that can still pass a depth test instead of a record per point.
+    static const int env_lists = getenv("ADOP_DIRECT_LISTS") ? atoi(getenv("ADOP_DIRECT_LISTS")) : 1;
+    if (!pc.cache && env_lists && scene->num_points > 0)
+    {
+        pc.cache      = (float4*)((char*)workspace + wl.proj);
+        pc.list_ids   = (uint32_t*)((char*)workspace + wl.list_ids);
+        pc.list_count = (uint32_t*)((char*)workspace + wl.list_count);
+        pc.list_span  = prepass_points_per_block();
+        pc.list_stride = wl.list_stride;
+    }
     size_t accum_n   = (size_t)lv.pix_prefix[lv.num] * lv.B * S;  // floats, multiple of 4 unless S < 4
     {
         StageScope sc("Initialize", stream);

@@ -53,6 +53,16 @@ struct CloudArg
     const float* intrinsics;
     const float* dropout;  // [B,N] or null
     float4* cache;         // [B,N] projected points (ip.x, ip.y, depth or 0, LOD radius in pixels) or null
+    // Direct forward path without a caller's point cache: the prepass compacts, per wavefront, the points that may
+    // still pass a depth test; `cache` then holds their records in the first list_count[b][g][w] slots of the own
+    // range of wavefront w of workgroup g (b * list_stride + g * list_span + w * list_span / 4 ...), list_ids the point ids.
+    // Null: no lists.
+    // The ranges of the last workgroup reach past n: a view's lists take list_stride >= n rounded up to whole
+    // workgroups, and in list mode `cache` has B * list_stride records.
+    uint32_t* list_ids;    // [B, list_stride]
+    uint32_t* list_count;  // [B, number of prepass workgroups, 4]
+    int32_t list_span;     // points per prepass workgroup
+    size_t list_stride;    // slots per view
 };
 
 struct ParamArg

@@ -109,6 +109,8 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
         uint32_t cur[PPT][ADOP_MAX_LAYERS];
         uint32_t inmask[PPT];
         float zz[PPT];
+        float4 rec[PPT];  // list mode: the record of a point that may still pass a depth test (depth 0: none)
+        bool okk[PPT];
 #pragma unroll
         for (int k = 0; k < PPT; ++k)
         {
@@ -122,7 +124,7 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
             bool ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P[k].w, rp.check_normal != 0, rp.dist_cutoff,
                                              lv.l[0].w, &ip, &z, &radius_pixels, &view_p);
             // the blend (and the backward pass, if the caller keeps the buffer) read this instead of projecting again
-            if (valid && pc.cache)
+            if (valid && pc.cache && !pc.list_ids)
             {
                 // (the sign of the depth carries the dropout flag: the readers need no second array)
                 const bool dropped = pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;
@@ -131,6 +133,8 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
             }
             zz[k]      = z;
             inmask[k]  = 0;
+            rec[k]     = make_float4(ip.x, ip.y, 0.f, radius_pixels);
+            okk[k]     = ok;
             bool alive = ok;
 #pragma unroll
             for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
@@ -156,6 +160,42 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
                     ip.y *= 0.5f;
                 }
             }
+        }
+        // List mode: the points of every wavefront that may still pass a depth test, compacted into the first slots of
+        // the wavefront's own range (no LDS, no barrier, no atomics).  In a dense cloud they are a few percent,
+        // scattered over all wavefronts; the blend packs the four lists of a workgroup and runs on full wavefronts of
+        // them instead of on every wavefront of the cloud.
+        if (pc.list_ids)  // kernel-uniform
+        {
+            const int wave     = threadIdx.x >> 6;
+            const size_t range = (size_t)b * pc.list_stride + (size_t)blockIdx.x * (kBlock * PPT) + (size_t)wave * (64 * PPT);
+            uint32_t before    = 0;
+#pragma unroll
+            for (int k = 0; k < PPT; ++k)
+            {
+                // (only here are the early-z words looked at: all their loads were issued before anything waits)
+                // The depth only decreases from the value read: a point behind its band is behind the band of the
+                // final depth (:380).  The counter pass keeps every projected point: the blend counts texel indices
+                // out of range for them.  Dropped points are not blended (:314-315).
+                const int i = base + k * kBlock;
+                bool cand   = false;
+#pragma unroll
+                for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+                    if (inmask[k] >> l & 1u) cand |= !(zz[k] > __uint_as_float(cur[k][l]) * (rp.depth_accept + 1));
+                if (STATS) cand = okk[k];
+                if (cand && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f) cand = false;
+                if (cand) rec[k].z = zz[k];
+                const unsigned long long m = __ballot(cand);
+                if (cand)
+                {
+                    const size_t slot = range + before + (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
+                    pc.cache[slot]    = rec[k];
+                    pc.list_ids[slot] = (uint32_t)i;
+                }
+                before += (uint32_t)__popcll(m);
+            }
+            if (lane == 0)
+                pc.list_count[((size_t)b * gridDim.x + blockIdx.x) * (kBlock / 64) + wave] = before;
         }
         // phase 2: per 64-point run and level, the surviving lanes are grouped by pixel; one atomicMin per group
 #pragma unroll
@@ -230,46 +270,15 @@ __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewCo
     const int j                 = lane - sub * LG;
     const int subs              = 64 / LG;
 
-    int i      = blockIdx.x * kBlock + threadIdx.x;
-    bool valid = i < pc.n;
-    int tex_index = valid ? pc.index[i] : 0;
-    bool tex_ok   = (unsigned)tex_index < (unsigned)pc.num_texels;  // device assert :362
     const float accept = rp.depth_accept + 1;
-    bool staged = false;
-    float4 P    = make_float4(0, 0, 0, 0);
-    V3 nrm      = {0, 0, 0};
-    if (!pc.cache)  // kernel-uniform: no point cache, project again
-    {
-        if (valid) P = pc.position[i];
-        if (valid && pc.normal) nrm = unpack_normal10(pc.normal[i]);
-    }
 
-    for (int b = 0; b < lv.B; ++b)
+    // phases 1-3 for one projected point of view b in every lane (ok: the lane has one)
+    auto blend_point = [&](int b, bool ok, V2 ip, float z, float radius_pixels, int tex_index, bool tex_ok,
+                           bool& staged)
     {
-        V2 ip = {0.f, 0.f};
-        float z = 0.f, radius_pixels = 0.f;
-        bool ok;
-        if (pc.cache)
-        {
-            // projected by the depth prepass of this call; dropped points (:314-315) carry a negative depth
-            const float4 R = valid ? pc.cache[(size_t)b * pc.n + i] : make_float4(0, 0, 0, 0);
-            ip             = {R.x, R.y};
-            z              = R.z;
-            radius_pixels  = R.w;
-            ok             = valid && z > 0;
-        }
-        else
-        {
-            bool dropped = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;  // :314-315
-            V3 pos = {P.x, P.y, P.z};
-            V3 view_p;
-            ok = valid && !dropped &&
-                 project_point(views[b], pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff, lv.l[0].w, &ip,
-                               &z, &radius_pixels, &view_p);
-        }
         if (STATS) stat_add(&stats->bad_index, ok && !tex_ok);
         ok = ok && tex_ok;
-        if (!__ballot(ok) && !STATS) continue;  // wavefront-uniform
+        if (!__ballot(ok) && !STATS) return;  // wavefront-uniform
 
         // The descriptors are requested together with the depth words (one memory round trip instead of two); points
         // that end up rejected at every level fetch them in vain, which costs less than the extra latency.
@@ -322,7 +331,7 @@ __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewCo
         bool any = false;
 #pragma unroll
         for (int l = 0; l < ADOP_MAX_LAYERS; ++l) any |= acc[l];
-        if (!__ballot(any)) continue;  // wavefront-uniform
+        if (!__ballot(any)) return;  // wavefront-uniform
 
         // phase 2: stage the descriptors of this point (the same for every level and view)
         if (want_t)
@@ -379,6 +388,74 @@ __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewCo
                 }
             }
         }
+    };
+
+    if (pc.list_ids)  // kernel-uniform: the points that survived the prepass, one list per prepass wavefront
+    {
+        static_assert(kBlock / 64 == 4, "four lists per prepass workgroup");
+        const uint32_t per_wave = (uint32_t)pc.list_span / 4;
+        for (int b = 0; b < lv.B; ++b)
+        {
+            const uint4 c = *(const uint4*)(pc.list_count + ((size_t)b * gridDim.x + blockIdx.x) * 4);
+            const uint32_t p1 = c.x, p2 = p1 + c.y, p3 = p2 + c.z, n = p3 + c.w;
+            const size_t range = (size_t)b * pc.list_stride + (size_t)blockIdx.x * pc.list_span;
+            for (uint32_t t0 = 0; t0 < n; t0 += blockDim.x)
+            {
+                const uint32_t t = t0 + threadIdx.x;
+                const bool valid = t < n;
+                // the four lists back to back: list w holds the items [p_w, p_{w+1})
+                const uint32_t w   = (t >= p1) + (t >= p2) + (t >= p3);
+                const uint32_t off = t - (w == 0 ? 0u : (w == 1 ? p1 : (w == 2 ? p2 : p3)));
+                const size_t slot  = range + (size_t)w * per_wave + off;
+                const float4 R     = valid ? pc.cache[slot] : make_float4(0, 0, 0, 0);
+                const int i        = valid ? (int)pc.list_ids[slot] : 0;
+                int tex_index      = valid ? pc.index[i] : 0;
+                bool tex_ok        = (unsigned)tex_index < (unsigned)pc.num_texels;  // device assert :362
+                bool staged        = false;
+                wave_lds_sync();  // the staged descriptors of the previous round are no longer read
+                blend_point(b, valid && R.z > 0, V2{R.x, R.y}, R.z, R.w, tex_index, tex_ok, staged);
+            }
+        }
+        return;
+    }
+
+    int i      = blockIdx.x * kBlock + threadIdx.x;
+    bool valid = i < pc.n;
+    int tex_index = valid ? pc.index[i] : 0;
+    bool tex_ok   = (unsigned)tex_index < (unsigned)pc.num_texels;  // device assert :362
+    bool staged = false;
+    float4 P    = make_float4(0, 0, 0, 0);
+    V3 nrm      = {0, 0, 0};
+    if (!pc.cache)  // kernel-uniform: no point cache, project again
+    {
+        if (valid) P = pc.position[i];
+        if (valid && pc.normal) nrm = unpack_normal10(pc.normal[i]);
+    }
+
+    for (int b = 0; b < lv.B; ++b)
+    {
+        V2 ip = {0.f, 0.f};
+        float z = 0.f, radius_pixels = 0.f;
+        bool ok;
+        if (pc.cache)
+        {
+            // projected by the depth prepass of this call; dropped points (:314-315) carry a negative depth
+            const float4 R = valid ? pc.cache[(size_t)b * pc.n + i] : make_float4(0, 0, 0, 0);
+            ip             = {R.x, R.y};
+            z              = R.z;
+            radius_pixels  = R.w;
+            ok             = valid && z > 0;
+        }
+        else
+        {
+            bool dropped = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;  // :314-315
+            V3 pos = {P.x, P.y, P.z};
+            V3 view_p;
+            ok = valid && !dropped &&
+                 project_point(views[b], pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff, lv.l[0].w, &ip,
+                               &z, &radius_pixels, &view_p);
+        }
+        blend_point(b, ok, ip, z, radius_pixels, tex_index, tex_ok, staged);
     }
 }
 
@@ -462,12 +539,20 @@ void launch_clear(const Levels& lv, int first_level, int grid, float* accum, siz
                        zero_u32, zero_n, vp);
 }
 
+static int prepass_ppt()
+{
+    static const int ppt = getenv("ADOP_PREPASS_PPT") ? atoi(getenv("ADOP_PREPASS_PPT")) : 2;
+    return ppt == 4 ? 4 : (ppt == 2 ? 2 : 1);
+}
+
+int prepass_points_per_block() { return kBlock * prepass_ppt(); }
+
 void launch_prepass(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, adop_stats* stats,
                     hipStream_t st)
 {
     if (pc.n < 1) return;
     static const int group_from = getenv("ADOP_PREPASS_GROUP_FROM") ? atoi(getenv("ADOP_PREPASS_GROUP_FROM")) : 1;
-    static const int ppt        = getenv("ADOP_PREPASS_PPT") ? atoi(getenv("ADOP_PREPASS_PPT")) : 2;
+    const int ppt               = prepass_ppt();
     if (ppt == 4)
         hipLaunchKernelGGL((prepass_kernel<4>), dim3((pc.n + kBlock * 4 - 1) / (kBlock * 4)), dim3(kBlock), 0, st, pc,
                            views, lv, rp, group_from, stats);
@@ -483,10 +568,14 @@ template <int CT, bool HALF>
 static void launch_blend_t(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp,
                            float* accum, int S, adop_stats* stats, hipStream_t st)
 {
-    int grid   = (pc.n + kBlock - 1) / kBlock;
-    size_t lds = sizeof(float) * (size_t)kBlock * (size_t)lv.C;
     static const int group_from = getenv("ADOP_BLEND_GROUP_FROM") ? atoi(getenv("ADOP_BLEND_GROUP_FROM")) : 0;  // 0: group at every level
-    hipLaunchKernelGGL((blend_kernel<CT, HALF>), dim3(grid), dim3(kBlock), lds, st, pc, views, lv, rp,
+    // list mode: one small workgroup per prepass workgroup (a few percent of the points survive in a dense cloud)
+    static const int list_block = getenv("ADOP_LIST_BLOCK") ? atoi(getenv("ADOP_LIST_BLOCK")) : 128;
+    const int block = pc.list_ids ? ((list_block >= 64 && list_block <= kBlock && list_block % 64 == 0) ? list_block : 128)
+                                  : kBlock;
+    const int grid  = pc.list_ids ? (pc.n + pc.list_span - 1) / pc.list_span : (pc.n + kBlock - 1) / kBlock;
+    size_t lds      = sizeof(float) * (size_t)block * (size_t)lv.C;
+    hipLaunchKernelGGL((blend_kernel<CT, HALF>), dim3(grid), dim3(block), lds, st, pc, views, lv, rp,
                        accum, S, stats, group_from);
 }
 

@@ -66,6 +66,22 @@ def test_config1_forward(oracle_mod):
     assert (di[empty & (ref.depth[0] == 100000.0)] == ((0x47C35000 << 32) | 0xFFFFFFFF)).all()
 
 
+@pytest.mark.parametrize("collect_stats", [True, False], ids=["counters", "plain"])
+def test_forward_without_point_cache_dense_cloud(oracle_mod, collect_stats):
+    """Inference (no backward pass follows, the caller keeps no point cache): the direct path hands the blend
+    compacted lists of the points that can still pass a depth test.  ~24 points per level-0 pixel, a dropout mask,
+    two views; without the counters only the candidates are listed, with them every projected point."""
+    from adop_amd import scenes
+
+    announce(f"400k pts B=2 128x128 L4 forward without point cache, dropout 0.3, counters={collect_stats}")
+    hs = scenes.config2(n=400_000, w=128, h=128, batch=2)
+    hs.dropout = scenes.bernoulli_mask(11, 2, 400_000, 0.3)
+    ref = oracle_mod.forward(hs)
+    scene, info, ctx, images, masks = run_hip_forward(hs, collect_stats=collect_stats, train=False)
+    assert info.cache.point_cache is None
+    check_forward(hs, ref, ctx, images, masks, info, stats=collect_stats)
+
+
 def test_config2_forward_backward(oracle_mod):
     from adop_amd import scenes
 
