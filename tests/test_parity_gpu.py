@@ -106,6 +106,26 @@ def test_config3_reduced_all_grads(oracle_mod):
     _fwd_bwd(hs, oracle_mod)
 
 
+def test_backward_without_point_gradients(oracle_mod):
+    """No point gradient is asked for: nothing normalises point rows, the reduction of the pose / intrinsics /
+    background partial sums runs as a kernel of its own."""
+    from adop_amd import scenes
+
+    announce("config3 reduced 150k pts 320x180 C=8, gradients: descriptors, pose, intrinsics (no points)")
+    hs = scenes.config3(n=150_000, w=320, h=180)
+    _fwd_bwd(hs, oracle_mod, needs=(False, True, True))
+
+
+def test_more_views_than_one_constant_chunk(oracle_mod):
+    """34 views: the per-view constants take the chunked path (32 per launch), the backward work queue alternates
+    its two counter sets 34 times, every view accumulates into the same point / pose / intrinsics gradients."""
+    from adop_amd import scenes
+
+    announce("config2 30k pts B=34 96x96 L3 fwd+bwd ghost")
+    hs = scenes.config2(n=30_000, w=96, h=96, levels=3, batch=34)
+    _fwd_bwd(hs, oracle_mod)
+
+
 @pytest.mark.parametrize("mode", [0, 1])
 def test_normalize_modes_and_backward_mode4(oracle_mod, mode):
     from adop_amd import scenes
