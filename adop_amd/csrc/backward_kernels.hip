@@ -16,7 +16,7 @@ namespace adop
 // Background gradient: per-thread fp32 partial over a handful of pixels, wave/block reduction in f64, one f64
 // partial row per block.
 template <int CT>
-__global__ __launch_bounds__(kBlock) void interleave_kernel(Levels lv, float* __restrict__ ig,
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) void interleave_kernel(Levels lv, float* __restrict__ ig,
                                                             float2* __restrict__ dw, double* __restrict__ partial,
                                                             uint32_t* __restrict__ q_counts, ViewPrep vp)
 {

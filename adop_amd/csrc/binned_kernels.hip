@@ -70,8 +70,10 @@ __device__ __forceinline__ void entry_tiles(const Levels& lv, const ParamArg& rp
     }
 }
 
-// First pass over the points: projection (kept in the point cache) and the number of entries per tile.
-__global__ __launch_bounds__(kBlock) void bin_count_kernel(CloudArg pc, const ViewConst* __restrict__ views, Levels lv,
+// First pass over the points: projection (kept in the point cache) and the number of entries per tile.  A thread
+// handles PPT points whose loads are all issued before anything waits.
+template <int PPT>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(PPT > 2 ? 5 : 8, PPT > 2 ? 5 : 8))) void bin_count_kernel(CloudArg pc, const ViewConst* __restrict__ views, Levels lv,
                                                            ParamArg rp, BinArg bin, adop_stats* stats)
 {
     __shared__ unsigned long long s_gmask[kBlock];
@@ -81,75 +83,95 @@ __global__ __launch_bounds__(kBlock) void bin_count_kernel(CloudArg pc, const Vi
     const int wbase  = threadIdx.x & ~63;
     unsigned long long* gmask_w = s_gmask + wbase;
     uint32_t* gkey_w            = s_gkey + wbase;
+    const int base              = blockIdx.x * (kBlock * PPT) + threadIdx.x;
 
-    const int i      = blockIdx.x * kBlock + threadIdx.x;
-    const bool valid = i < pc.n;
-    float4 P         = valid ? nt_load4(pc.position + i) : make_float4(0, 0, 0, 0);
-    int32_t nenc     = (valid && pc.normal) ? __builtin_nontemporal_load(pc.normal + i) : 0;
-    V3 pos           = {P.x, P.y, P.z};
-    V3 nrm           = unpack_normal10(nenc);
-    bool tex_ok      = true;
-    if (STATS)
+    float4 P[PPT];
+    int32_t nenc[PPT];
+    bool tex_ok[PPT];
+#pragma unroll
+    for (int k = 0; k < PPT; ++k)
     {
-        int tex_index = valid ? pc.index[i] : 0;
-        tex_ok        = (unsigned)tex_index < (unsigned)pc.num_texels;
+        const int i      = base + k * kBlock;
+        const bool valid = i < pc.n;
+        P[k]             = valid ? nt_load4(pc.position + i) : make_float4(0, 0, 0, 0);
+        nenc[k]          = (valid && pc.normal) ? __builtin_nontemporal_load(pc.normal + i) : 0;
+        tex_ok[k]        = true;
+        if (STATS)
+        {
+            int tex_index = valid ? pc.index[i] : 0;
+            tex_ok[k]     = (unsigned)tex_index < (unsigned)pc.num_texels;
+        }
     }
 
     for (int b = 0; b < lv.B; ++b)
     {
         const ViewConst& vc = views[b];
-        // requested before the projection: the kernel is bound by instruction issue, the load hides behind it
-        const float drop_flag = (valid && pc.dropout) ? __builtin_nontemporal_load(pc.dropout + (size_t)b * pc.n + i) : 0.f;
-        V2 ip = {0.f, 0.f};
-        V3 view_p;
-        float z = 0.f, radius_pixels = 0.f;
-        bool ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff,
-                                         lv.l[0].w, &ip, &z, &radius_pixels, &view_p);
-        // the second pass (and the backward pass, if the caller keeps the buffer) read this instead of projecting
-        // (the sign of the depth carries the dropout flag: the readers need no second array)
-        const bool dropped = drop_flag == 1.f;  // :314-315
-        if (valid)
-            nt_store4(pc.cache + (size_t)b * pc.n + i,
-                      ok ? make_float4(ip.x, ip.y, dropped ? -z : z, radius_pixels) : make_float4(0, 0, 0, 0));
-        if (STATS) stat_add(&stats->bad_index, ok && !dropped && !tex_ok);
-        if (!__ballot(ok) && !STATS)  // wavefront-uniform
-        {
-            if (valid) __builtin_nontemporal_store(0u, bin.info + (size_t)b * pc.n + i);
-            continue;
-        }
-
-        bool in[ADOP_MAX_LAYERS];
-        bool any_in;
-        uint32_t nlev, ptile, xtile;
-        entry_tiles(lv, rp, bin, b, ok, ip, radius_pixels, in, &any_in, &nlev, &ptile, &xtile);
-        if (valid)
-        {
-            uint32_t word = 0;
-            if (any_in)
-            {
-                word = kInfoValid | ptile | (nlev << 24);
-                if (xtile != kNoTile)
-                {
-                    const uint32_t d = xtile - ptile;  // 1, tiles_x or tiles_x + 1
-                    const bool below = d >= (uint32_t)bin.tiles_x;
-                    if (below) word |= kInfoBelow;
-                    if (d - (below ? (uint32_t)bin.tiles_x : 0u) == 1u) word |= kInfoRight;
-                }
-            }
-            __builtin_nontemporal_store(word, bin.info + (size_t)b * pc.n + i);
-        }
-        if (STATS)
-        {
+        // requested before the projection: the load hides behind it
+        float drop_flag[PPT];
 #pragma unroll
-            for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
-                if (l < lv.num) stat_add(&stats->visible[l], in[l]);
+        for (int k = 0; k < PPT; ++k)
+        {
+            const int i  = base + k * kBlock;
+            drop_flag[k] = (i < pc.n && pc.dropout) ? __builtin_nontemporal_load(pc.dropout + (size_t)b * pc.n + i) : 0.f;
         }
-        if (!__ballot(any_in)) continue;
-        wave_lds_sync();
-        int G = wave_group_by_key(any_in, ptile, gkey_w, gmask_w);
-        wave_lds_sync();
-        if (lane < G) atomicAdd(&bin.count[gkey_w[lane]], (uint32_t)__popcll(gmask_w[lane]));
-        if (xtile != kNoTile) atomicAdd(&bin.count[xtile], 1u);
+#pragma unroll
+        for (int k = 0; k < PPT; ++k)
+        {
+            const int i      = base + k * kBlock;
+            const bool valid = i < pc.n;
+            V3 pos           = {P[k].x, P[k].y, P[k].z};
+            V3 nrm           = unpack_normal10(nenc[k]);
+            V2 ip            = {0.f, 0.f};
+            V3 view_p;
+            float z = 0.f, radius_pixels = 0.f;
+            bool ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P[k].w, rp.check_normal != 0, rp.dist_cutoff,
+                                             lv.l[0].w, &ip, &z, &radius_pixels, &view_p);
+            // the second pass (and the backward pass, if the caller keeps the buffer) read this instead of projecting
+            // (the sign of the depth carries the dropout flag: the readers need no second array)
+            const bool dropped = drop_flag[k] == 1.f;  // :314-315
+            if (valid)
+                nt_store4(pc.cache + (size_t)b * pc.n + i,
+                          ok ? make_float4(ip.x, ip.y, dropped ? -z : z, radius_pixels) : make_float4(0, 0, 0, 0));
+            if (STATS) stat_add(&stats->bad_index, ok && !dropped && !tex_ok[k]);
+            if (!__ballot(ok) && !STATS)  // wavefront-uniform
+            {
+                if (valid) __builtin_nontemporal_store(0u, bin.info + (size_t)b * pc.n + i);
+                continue;
+            }
+
+            bool in[ADOP_MAX_LAYERS];
+            bool any_in;
+            uint32_t nlev, ptile, xtile;
+            entry_tiles(lv, rp, bin, b, ok, ip, radius_pixels, in, &any_in, &nlev, &ptile, &xtile);
+            if (valid)
+            {
+                uint32_t word = 0;
+                if (any_in)
+                {
+                    word = kInfoValid | ptile | (nlev << 24);
+                    if (xtile != kNoTile)
+                    {
+                        const uint32_t d = xtile - ptile;  // 1, tiles_x or tiles_x + 1
+                        const bool below = d >= (uint32_t)bin.tiles_x;
+                        if (below) word |= kInfoBelow;
+                        if (d - (below ? (uint32_t)bin.tiles_x : 0u) == 1u) word |= kInfoRight;
+                    }
+                }
+                __builtin_nontemporal_store(word, bin.info + (size_t)b * pc.n + i);
+            }
+            if (STATS)
+            {
+#pragma unroll
+                for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+                    if (l < lv.num) stat_add(&stats->visible[l], in[l]);
+            }
+            if (!__ballot(any_in)) continue;
+            wave_lds_sync();
+            int G = wave_group_by_key(any_in, ptile, gkey_w, gmask_w);
+            wave_lds_sync();
+            if (lane < G) atomicAdd(&bin.count[gkey_w[lane]], (uint32_t)__popcll(gmask_w[lane]));
+            if (xtile != kNoTile) atomicAdd(&bin.count[xtile], 1u);
+        }
     }
 }
 
@@ -289,8 +311,16 @@ void launch_bin(int pass, const CloudArg& pc, const ViewConst* views, const Leve
     if (pc.n < 1) return;
     if (pass == 0)
     {
-        hipLaunchKernelGGL(bin_count_kernel, dim3((pc.n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, pc, views, lv, rp,
-                           bin, stats);
+        static const int cppt = getenv("ADOP_COUNT_PPT") ? atoi(getenv("ADOP_COUNT_PPT")) : 2;
+        if (cppt == 2)
+            hipLaunchKernelGGL((bin_count_kernel<2>), dim3((pc.n + kBlock * 2 - 1) / (kBlock * 2)), dim3(kBlock), 0, st,
+                               pc, views, lv, rp, bin, stats);
+        else if (cppt == 4)
+            hipLaunchKernelGGL((bin_count_kernel<4>), dim3((pc.n + kBlock * 4 - 1) / (kBlock * 4)), dim3(kBlock), 0, st,
+                               pc, views, lv, rp, bin, stats);
+        else
+            hipLaunchKernelGGL((bin_count_kernel<1>), dim3((pc.n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, pc, views,
+                               lv, rp, bin, stats);
         return;
     }
     static const int ppt = getenv("ADOP_SCATTER_PPT") ? atoi(getenv("ADOP_SCATTER_PPT")) : 4;

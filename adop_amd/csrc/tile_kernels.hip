@@ -199,7 +199,7 @@ __device__ __forceinline__ void add_staged(float* acc, const float* s_stage, int
 
 // K entries per thread and batch (BATCH = K * kBlock, a power of two).
 template <int CT, bool HALF, int K>
-__global__ __launch_bounds__(kBlock) void tile_blend_kernel(CloudArg pc, Levels lv, ParamArg rp, BinArg bin,
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu((CT != 0 && K == 1) ? 8 : 4, 8))) void tile_blend_kernel(CloudArg pc, Levels lv, ParamArg rp, BinArg bin,
                                                             float* __restrict__ accum, int S,
                                                             const float* __restrict__ background, int write_mask,
                                                             float mask_value, int identity_index, adop_stats* stats)
