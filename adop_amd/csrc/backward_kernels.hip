@@ -418,9 +418,10 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
 
     // per-thread sums of the pose / intrinsics gradients: a thread sees a few dozen contributions at most, so fp32
     // here costs ~1e-7 relative; everything beyond the thread (wavefront, block, grid) is summed in f64
-    float acc[kAcc];
+    // (they live in LDS, one column per thread: 21 registers less in a kernel whose occupancy is set by registers)
+    float* acc = s_red + threadIdx.x;  // acc[k * kBlock]
 #pragma unroll
-    for (int k = 0; k < kAcc; ++k) acc[k] = 0;
+    for (int k = 0; k < kAcc; ++k) acc[k * kBlock] = 0;
 
     for (uint32_t t = blockIdx.x * kBlock + threadIdx.x; t < total; t += gridDim.x * kBlock)
     {
@@ -553,8 +554,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
                 if (want_pose)
                 {
 #pragma unroll
-                    for (int k = 0; k < 6; ++k) acc[k] += bo.g_pose[k];
-                    acc[6] += 1.0f;
+                    for (int k = 0; k < 6; ++k) acc[k * kBlock] += bo.g_pose[k];
+                    acc[6 * kBlock] += 1.0f;
                 }
                 if (want_intr)
                 {
@@ -564,7 +565,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
                         bo.g_k[4] *= 0.1f;
                         bo.g_k[4] *= 0;  // :653-654
 #pragma unroll
-                        for (int k = 0; k < 5; ++k) acc[8 + k] += kf * bo.g_k[k];
+                        for (int k = 0; k < 5; ++k) acc[(8 + k) * kBlock] += kf * bo.g_k[k];
                         float df = rp.distortion_gradient_factor;
                         bo.g_dis[2] *= 0.25f;
                         bo.g_dis[3] *= 0.1f;
@@ -573,14 +574,14 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
                         bo.g_dis[6] *= 0.1f;
                         bo.g_dis[7] *= 0.1f;
 #pragma unroll
-                        for (int k = 0; k < 8; ++k) acc[13 + k] += df * bo.g_dis[k];
-                        acc[7] += 1.0f / 1024.0f;  // :680-681
+                        for (int k = 0; k < 8; ++k) acc[(13 + k) * kBlock] += df * bo.g_dis[k];
+                        acc[7 * kBlock] += 1.0f / 1024.0f;  // :680-681
                     }
                     else
                     {
 #pragma unroll
-                        for (int k = 0; k < 5; ++k) acc[8 + k] += bo.g_k[k];
-                        acc[7] += 1.0f;  // :718
+                        for (int k = 0; k < 5; ++k) acc[(8 + k) * kBlock] += bo.g_k[k];
+                        acc[7 * kBlock] += 1.0f;  // :718
                     }
                 }
             }
@@ -607,8 +608,6 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
     {
         // block sums in f64 through LDS: 8 threads per value, 32 columns each (21 f64 wavefront reductions with
         // cross-lane permutes took 7 us per workgroup)
-#pragma unroll
-        for (int k = 0; k < kAcc; ++k) s_red[k * kBlock + threadIdx.x] = acc[k];
         __syncthreads();
         const int k = threadIdx.x >> 3, part = threadIdx.x & 7;
         double v    = 0;
