@@ -755,6 +755,8 @@ __device__ static void finalize_block(const FinalizeArg& a, double* sh, double* 
 // each reduce a slice of the rows to one row, and the one that finishes last (ticket counter) reduces those rows, in
 // their fixed order, and writes the outputs.  The other workgroups normalise.  Without point gradients (n = 0) a
 // single workgroup of NT = kFinalizeBlock threads does the whole reduction.
+constexpr int kNormPer = 4;  // point-gradient rows per thread of the normalisation
+
 template <int NT>
 __device__ __forceinline__ void finalize_body(FinalizeArg a, float* __restrict__ g, const float* __restrict__ count, int n,
                                               int mode)
@@ -823,14 +825,41 @@ __device__ __forceinline__ void finalize_body(FinalizeArg a, float* __restrict__
         finalize_block<NT>(a, sh, s_small);
         return;
     }
-    int t = (blockIdx.x - first_stage) * NT + threadIdx.x;
-    if (t >= n) return;
-    float c = __builtin_nontemporal_load(count + t);
-    if (!(c > 0)) return;
-    size_t o = (mode == 0) ? 3 * (size_t)t : 4 * (size_t)t;
-    g[o + 0] = g[o + 0] / c;
-    g[o + 1] = g[o + 1] / c;
-    g[o + 2] = g[o + 2] / c;
+    // kNormPer elements per thread, kNormPer wavefront-strided count loads in flight (the chain count -> row -> store is
+    // two dependent round trips and most counts are zero)
+    const int t0 = (blockIdx.x - first_stage) * (NT * kNormPer) + threadIdx.x;
+    float c[kNormPer];
+#pragma unroll
+    for (int k = 0; k < kNormPer; ++k)
+    {
+        const int t = t0 + k * NT;
+        c[k]        = t < n ? __builtin_nontemporal_load(count + t) : 0.f;
+    }
+    float v[kNormPer][3];
+#pragma unroll
+    for (int k = 0; k < kNormPer; ++k)
+    {
+        const int t    = t0 + k * NT;
+        const size_t o = (mode == 0) ? 3 * (size_t)t : 4 * (size_t)t;
+        if (c[k] > 0)
+        {
+            v[k][0] = g[o + 0];
+            v[k][1] = g[o + 1];
+            v[k][2] = g[o + 2];
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < kNormPer; ++k)
+    {
+        const int t    = t0 + k * NT;
+        const size_t o = (mode == 0) ? 3 * (size_t)t : 4 * (size_t)t;
+        if (c[k] > 0)
+        {
+            g[o + 0] = v[k][0] / c[k];
+            g[o + 1] = v[k][1] / c[k];
+            g[o + 2] = v[k][2] / c[k];
+        }
+    }
 }
 
 __global__ __launch_bounds__(kFinalizeBlock) void finalize_kernel(FinalizeArg a)
@@ -927,7 +956,7 @@ void launch_finalize(const ViewConst* views, int B, int C, const double* bg_part
     if (n == 0)
         hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kFinalizeBlock), 0, st, a);
     else
-        hipLaunchKernelGGL(finalize_normalize_kernel, dim3(kFinalizeParts + (n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, a,
+        hipLaunchKernelGGL(finalize_normalize_kernel, dim3(kFinalizeParts + (n + kBlock * kNormPer - 1) / (kBlock * kNormPer)), dim3(kBlock), 0, st, a,
                            g->grad_points, g->grad_points_count, n, normalize_mode);
 }
 
