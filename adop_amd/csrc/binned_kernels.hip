@@ -76,14 +76,9 @@ template <int PPT>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(PPT > 2 ? 5 : 8, PPT > 2 ? 5 : 8))) void bin_count_kernel(CloudArg pc, const ViewConst* __restrict__ views, Levels lv,
                                                            ParamArg rp, BinArg bin, adop_stats* stats)
 {
-    __shared__ unsigned long long s_gmask[kBlock];
-    __shared__ uint32_t s_gkey[kBlock];
     const bool STATS = stats != nullptr;  // counter pass (uniform branch)
     const int lane   = threadIdx.x & 63;
-    const int wbase  = threadIdx.x & ~63;
-    unsigned long long* gmask_w = s_gmask + wbase;
-    uint32_t* gkey_w            = s_gkey + wbase;
-    const int base              = blockIdx.x * (kBlock * PPT) + threadIdx.x;
+    const int base   = blockIdx.x * (kBlock * PPT) + threadIdx.x;
 
     float4 P[PPT];
     int32_t nenc[PPT];
@@ -166,27 +161,25 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(PPT > 2 
                     if (l < lv.num) stat_add(&stats->visible[l], in[l]);
             }
             if (!__ballot(any_in)) continue;
-            wave_lds_sync();
-            int G = wave_group_by_key(any_in, ptile, gkey_w, gmask_w);
-            wave_lds_sync();
-            if (lane < G) atomicAdd(&bin.count[gkey_w[lane]], (uint32_t)__popcll(gmask_w[lane]));
-            if (xtile != kNoTile) atomicAdd(&bin.count[xtile], 1u);
+            // one atomic per distinct tile of the wavefront, for the primary and for the second entries
+            const unsigned long long below = (1ull << lane) - 1ull;
+            const unsigned long long pm    = wave_group_mask(any_in, ptile);
+            const unsigned long long xm    = wave_group_mask(xtile != kNoTile, xtile);
+            if (any_in && (pm & below) == 0) atomicAdd(&bin.count[ptile], (uint32_t)__popcll(pm));
+            if (xtile != kNoTile && (xm & below) == 0) atomicAdd(&bin.count[xtile], (uint32_t)__popcll(xm));
         }
     }
 }
 
 // Second pass: PPT points per thread, so that the cache loads, the slot reservations (one returning atomic per
-// distinct tile of a wavefront) and the entry stores of PPT runs of 64 points are in flight together — the kernel
-// is a chain of three dependent memory round trips.
+// distinct tile of a wavefront, for the primary entries and for the second entries alike) and the entry stores of PPT
+// runs of 64 points are in flight together — the kernel is a chain of three dependent memory round trips.
 template <int PPT>
 __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels lv, ParamArg rp, BinArg bin)
 {
-    __shared__ unsigned long long s_gmask[PPT][kBlock];
-    __shared__ uint32_t s_gkey[PPT][kBlock];
-    __shared__ uint32_t s_gbase[PPT][kBlock];
-    const int lane  = threadIdx.x & 63;
-    const int wbase = threadIdx.x & ~63;
-    const int base  = blockIdx.x * (kBlock * PPT) + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int base = blockIdx.x * (kBlock * PPT) + threadIdx.x;
+    const unsigned long long below = (1ull << lane) - 1ull;
 
     for (int b = 0; b < lv.B; ++b)
     {
@@ -205,54 +198,48 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels
             R[k]        = make_float4(0, 0, 0, 0);
             if (info[k] & kInfoValid) R[k] = nt_load4(pc.cache + (size_t)b * pc.n + i);
         }
-        bool any_in[PPT];
-        uint32_t nlev[PPT], ptile[PPT], xtile[PPT], gslot[PPT], xslot[PPT];
-        int mine[PPT], G[PPT];
+        // groups of equal tile inside the wavefront: the lowest lane of a group reserves the slots of all its lanes
+        // (slots are handed out from the end of the bin: the tile's counter runs down from its count to zero)
+        unsigned long long pm[PPT], xm[PPT];
+        uint32_t pbase[PPT], xbase[PPT];
 #pragma unroll
         for (int k = 0; k < PPT; ++k)
         {
-            any_in[k] = (info[k] & kInfoValid) != 0;
-            nlev[k]   = info[k] >> 24 & 7u;
-            ptile[k]  = info[k] & kInfoTileMask;
-            xtile[k]  = kNoTile;
-            if (info[k] & (kInfoRight | kInfoBelow))
-                xtile[k] = ptile[k] + ((info[k] & kInfoRight) ? 1u : 0u) + ((info[k] & kInfoBelow) ? (uint32_t)bin.tiles_x : 0u);
-            G[k]     = wave_group_by_key(any_in[k], ptile[k], s_gkey[k] + wbase, s_gmask[k] + wbase, &mine[k]);
-            gslot[k] = 0;
-            xslot[k] = 0;
-        }
-        wave_lds_sync();
-#pragma unroll
-        for (int k = 0; k < PPT; ++k)
-        {
-            // slots are handed out from the end of the bin: the tile's counter runs down from its count to zero
-            if (lane < G[k])
+            const bool any_in    = (info[k] & kInfoValid) != 0;
+            const uint32_t ptile = info[k] & kInfoTileMask;
+            const bool has_x     = (info[k] & (kInfoRight | kInfoBelow)) != 0;
+            const uint32_t xtile = ptile + ((info[k] & kInfoRight) ? 1u : 0u) + ((info[k] & kInfoBelow) ? (uint32_t)bin.tiles_x : 0u);
+            pm[k]                = wave_group_mask(any_in, ptile);
+            xm[k]                = wave_group_mask(has_x, xtile);
+            pbase[k] = xbase[k] = 0;
+            if (any_in && (pm[k] & below) == 0)
             {
-                const uint32_t t = s_gkey[k][wbase + lane];
-                const uint32_t n = (uint32_t)__popcll(s_gmask[k][wbase + lane]);
-                gslot[k]         = bin.offset[t] + atomicSub(&bin.count[t], n) - n;
+                const uint32_t n = (uint32_t)__popcll(pm[k]);
+                pbase[k]         = bin.offset[ptile] + atomicSub(&bin.count[ptile], n) - n;
             }
-            if (xtile[k] != kNoTile) xslot[k] = bin.offset[xtile[k]] + atomicSub(&bin.count[xtile[k]], 1u) - 1u;
+            if (has_x && (xm[k] & below) == 0)
+            {
+                const uint32_t n = (uint32_t)__popcll(xm[k]);
+                xbase[k]         = bin.offset[xtile] + atomicSub(&bin.count[xtile], n) - n;
+            }
         }
-#pragma unroll
-        for (int k = 0; k < PPT; ++k)
-            if (lane < G[k]) s_gbase[k][wbase + lane] = gslot[k];
-        wave_lds_sync();
 #pragma unroll
         for (int k = 0; k < PPT; ++k)
         {
             const int i         = base + k * kBlock;
             const float zs      = R[k].z;  // the sign carries the dropout flag (:314-315)
-            const uint32_t word = (uint32_t)i | (nlev[k] << 28);
-            if (any_in[k])
-            {
-                const unsigned long long m = s_gmask[k][wbase + mine[k]];
-                const uint32_t slot        = s_gbase[k][wbase + mine[k]] + (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
-                bin.entries[slot] = make_float4(R[k].x, R[k].y, zs, __uint_as_float(word | kEntryPrimary));
-            }
-            if (xtile[k] != kNoTile) bin.entries[xslot[k]] = make_float4(R[k].x, R[k].y, zs, __uint_as_float(word));
+            const uint32_t word = (uint32_t)i | ((info[k] >> 24 & 7u) << 28);
+            // every lane asks its group's leader for the base (inactive lanes ask lane 0 for nothing)
+            const int pl      = pm[k] ? __ffsll((long long)pm[k]) - 1 : 0;
+            const int xl      = xm[k] ? __ffsll((long long)xm[k]) - 1 : 0;
+            const uint32_t pb = (uint32_t)__shfl((int)pbase[k], pl, 64);
+            const uint32_t xb = (uint32_t)__shfl((int)xbase[k], xl, 64);
+            if (pm[k])
+                bin.entries[pb + (uint32_t)__popcll(pm[k] & below)] =
+                    make_float4(R[k].x, R[k].y, zs, __uint_as_float(word | kEntryPrimary));
+            if (xm[k])
+                bin.entries[xb + (uint32_t)__popcll(xm[k] & below)] = make_float4(R[k].x, R[k].y, zs, __uint_as_float(word));
         }
-        wave_lds_sync();  // the group tables are reused by the next view
     }
 }
 
@@ -323,7 +310,7 @@ void launch_bin(int pass, const CloudArg& pc, const ViewConst* views, const Leve
                                lv, rp, bin, stats);
         return;
     }
-    static const int ppt = getenv("ADOP_SCATTER_PPT") ? atoi(getenv("ADOP_SCATTER_PPT")) : 4;
+    static const int ppt = getenv("ADOP_SCATTER_PPT") ? atoi(getenv("ADOP_SCATTER_PPT")) : 2;
     if (ppt == 1)
         hipLaunchKernelGGL((bin_scatter_kernel<1>), dim3((pc.n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, pc, lv, rp, bin);
     else if (ppt == 2)

@@ -190,6 +190,24 @@ __device__ __forceinline__ int wave_group_by_key(bool active, uint32_t key, uint
     return g;
 }
 
+// The same grouping without tables: every active lane gets the lane mask of its own group (0 for inactive lanes).
+// The lowest lane of a mask is the group's leader; the others fetch what it holds with a cross-lane read.
+__device__ __forceinline__ unsigned long long wave_group_mask(bool active, uint32_t key)
+{
+    unsigned long long remaining = __ballot(active);
+    unsigned long long mine      = 0;
+    while (remaining)
+    {
+        int leader           = __ffsll((long long)remaining) - 1;
+        uint32_t k           = (uint32_t)__builtin_amdgcn_readlane((int)key, leader);
+        bool hit             = active && key == k;
+        unsigned long long m = __ballot(hit);
+        if (hit) mine = m;
+        remaining &= ~m;
+    }
+    return mine;
+}
+
 // d_render_params.Pose() / PinholeIntrinsics() / OcamIntrinsics() (PointRenderer.cu:73-96) for one view.
 __device__ __forceinline__ ViewConst make_view_const(const adop_view& v, const double* __restrict__ poses,
                                                      const float* __restrict__ intrinsics, int cols)
