@@ -101,14 +101,6 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(PPT > 2 
     for (int b = 0; b < lv.B; ++b)
     {
         const ViewConst& vc = views[b];
-        // requested before the projection: the load hides behind it
-        float drop_flag[PPT];
-#pragma unroll
-        for (int k = 0; k < PPT; ++k)
-        {
-            const int i  = base + k * kBlock;
-            drop_flag[k] = (i < pc.n && pc.dropout) ? __builtin_nontemporal_load(pc.dropout + (size_t)b * pc.n + i) : 0.f;
-        }
 #pragma unroll
         for (int k = 0; k < PPT; ++k)
         {
@@ -123,7 +115,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(PPT > 2 
                                              lv.l[0].w, &ip, &z, &radius_pixels, &view_p);
             // the second pass (and the backward pass, if the caller keeps the buffer) read this instead of projecting
             // (the sign of the depth carries the dropout flag: the readers need no second array)
-            const bool dropped = drop_flag[k] == 1.f;  // :314-315
+            // (only the projected points' flags are read: the 55 % outside the image cost no dropout bytes)
+            const bool dropped = ok && pc.dropout && __builtin_nontemporal_load(pc.dropout + (size_t)b * pc.n + i) == 1.f;  // :314-315
             if (valid)
                 nt_store4(pc.cache + (size_t)b * pc.n + i,
                           ok ? make_float4(ip.x, ip.y, dropped ? -z : z, radius_pixels) : make_float4(0, 0, 0, 0));
