@@ -210,8 +210,8 @@ def main():
     measured_traffic = {}
     if args.workload == "config3" and not args.points and args.point_order == "morton" and not args.no_point_cache:
         # profiles/config3_tile_path_fwd_bwd_kernels_traffic_instructions.md, profiles/config3_fwd_bwd_kernels_traffic_atomics.md
-        measured_traffic = {"RenderBackward/descriptor": 912.7e6, "RenderBackward/spatial": 486.1e6, "TileBlend": 438.4e6,
-                            "BinCount": 459.2e6, "BinScatter": 204.3e6, "TileDepth": 101.0e6,
+        measured_traffic = {"RenderBackward/descriptor": 912.7e6, "RenderBackward/spatial": 486.2e6, "TileBlend": 438.1e6,
+                            "BinCount": 436.4e6, "BinScatter": 196.9e6, "TileDepth": 101.0e6,
                             "CombineAndFillBackward": 397.3e6, "RenderForward": 691.9e6}
     roofline = {"bound": "hbm", "kernel": KERNEL_OF_STAGE.get(dom, dom), "stage": dom, "achieved": round(dom_gbs, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
