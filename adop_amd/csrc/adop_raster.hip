@@ -1,18 +1,31 @@
 // adop_raster.hip — C-ABI of the one-pixel point rasterizer and the launch sequences (gfx950 / CDNA4).
 //
-// Pipeline of one forward call (reference: BlendPointCloudForward, PointRenderer.cu:1389-1531):
-//   prepare_views   poses_se3 (f64) / intrinsics rows -> per-view constants in the workspace
-//   clear           depth_index = (bits(100000.f)<<32)|~0, blend accumulators = 0          (InitializeData :1039-1090)
-//   prepass         per point/view/level: LDS pre-reduced 64-bit atomicMin of (depth bits | point id)  (:203-301)
-//   blend           per point: fuzzy depth test, LDS pre-reduced descriptor sums, one cache-line atomic per pixel (:303-393)
-//   resolve         per pixel: out = sum/weight or background, weight, mask, f32 depth      (:726-754,:828-847)
-// and of one backward call (BlendPointCloudBackward, :1549-1644):
-//   interleave      per pixel: background-gradient partial sums (CombineAndFillBackward :851-900) and the
-//                   pixel-major [image | upstream gradient] array the next kernel gathers from
-//   render_backward per point: descriptor gradient + ghost/spatial gradient (RenderBackward :396-724); the
-//                   per-image pose and per-camera intrinsics sums are kept per thread in f64, reduced per block
-//                   and written as per-block partials (no same-address atomics)
-//   finalize        partials -> grad_background / grad_pose / grad_intrinsics, NormalizeGradient (:1534-1547)
+// One forward call (reference: BlendPointCloudForward, PointRenderer.cu:1389-1531) runs one of two paths
+// (adop_render_params.forward_path; 0 lets the library choose).
+// Tile path (binned_kernels.hip, tile_kernels.hip):
+//   clear           depth_index / blend accumulators of the coarse levels, tile counters; one workgroup also turns
+//                   poses_se3 (f64) / intrinsics rows into the per-view constants          (InitializeData :1039-1090)
+//   bin_count       per point: projection (kept as the point cache), entries per 16x16-pixel screen tile
+//   tile_scan       prefix sum of the tile counts
+//   bin_scatter     per point: 16-byte entry into the bin of its tile (and of the tile of its level-1 pixel)
+//   tile_depth      per tile: 64-bit min of (depth bits | point id) in LDS, levels 0-1 owned, coarser ones merged
+//                   with global atomics                                                     (DepthPrepassMulti :203-301)
+//   tile_blend      per tile: fuzzy depth test, per-pixel lists in LDS, gather; levels 0-1 resolved to the outputs,
+//                   coarser levels added to the accumulators                                (RenderForwardMulti :303-393)
+//   resolve         coarse levels: out = sum/weight or background, weight, mask, f32 depth (:726-754,:828-847)
+// Direct path (forward_kernels.hip): clear, prepass (per point/view/level: pre-reduced 64-bit atomicMin), blend (per
+// point: fuzzy depth test, pre-reduced descriptor sums, one cache-line atomic per pixel), resolve.
+// One backward call (BlendPointCloudBackward, :1549-1644; backward_kernels.hip):
+//   interleave      per pixel: background-gradient partial sums (CombineAndFillBackward :851-900), the pixel-major
+//                   [image | upstream gradient] array and (depth, weight) pairs the next kernels gather from; one
+//                   workgroup computes the per-view constants
+//   per view:
+//   backward_tex    per point: depth tests, descriptor gradient, which levels get a ghost / spatial gradient
+//                   (RenderBackward :396-489); appends those points to a work queue
+//   backward_ghost  per queue item: four-neighbour gather, image-space gradient, ProjectPoint*Backward (:491-724);
+//                   pose / intrinsics sums per thread in fp32, per workgroup in f64, one partial row per workgroup
+//   finalize_normalize  partial rows -> grad_background / grad_pose / grad_intrinsics, NormalizeGradient
+//                   (:1534-1547) of all outputs
 //
 // No MFMA anywhere: the path is scan + scatter/gather + atomics, bounded by HBM and atomic transaction rate.
 #include <hip/hip_runtime.h>
