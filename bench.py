@@ -213,6 +213,9 @@ def main():
         measured_traffic = {"RenderBackward/descriptor": 912.7e6, "RenderBackward/spatial": 486.2e6, "TileBlend": 438.1e6,
                             "BinCount": 436.4e6, "BinScatter": 196.9e6, "TileDepth": 101.0e6,
                             "CombineAndFillBackward": 397.3e6, "RenderForward": 691.9e6}
+    if args.workload == "config4" and not args.points and args.point_order == "morton":
+        # profiles/config4_direct_path_forward_kernels_traffic_instructions.md
+        measured_traffic = {"DepthPrepass": 5053.5e6, "RenderForward": 1548.3e6}
     roofline = {"bound": "hbm", "kernel": KERNEL_OF_STAGE.get(dom, dom), "stage": dom, "achieved": round(dom_gbs, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
                 "traffic": measured_traffic.get(dom),
