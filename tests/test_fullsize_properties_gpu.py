@@ -38,6 +38,30 @@ def test_both_forward_paths_agree(full_scene):
     assert list(sa.visible) == list(sb.visible) and list(sa.accepted) == list(sb.accepted)
 
 
+def test_inference_forward_agrees_with_training_forward(full_scene):
+    """Without a point cache (no backward pass follows) the direct path blends from compacted candidate lists and the
+    tile path keeps its records in the workspace: same packed depth|index, depth and weight, images within 1e-5 of
+    the forward that keeps the cache, with and without the counters (the lists hold every projected point with them,
+    only the candidates without)."""
+    import torch
+
+    ref = run_hip_forward(full_scene, forward_path=2)
+    for path in (1, 2):
+        for counters in (True, False):
+            announce(f"config3 full size: inference forward, forward_path={path}, counters={counters}")
+            got = run_hip_forward(full_scene, collect_stats=counters, forward_path=path, train=False)
+            assert got[1].cache.point_cache is None
+            for l, (La, Lb) in enumerate(zip(ref[1].cache.layers_cuda, got[1].cache.layers_cuda)):
+                assert bool((La.depth_index_tensor == Lb.depth_index_tensor).all()), (path, counters, l)
+                assert bool((La.depth.view(torch.int32) == Lb.depth.view(torch.int32)).all()), (path, counters, l)
+                assert bool((La.weight == Lb.weight).all()), (path, counters, l)
+                ia, ib = ref[3][l], got[3][l]
+                assert float((ia - ib).abs().max()) <= 1e-5 * float(ia.abs().max()), (path, counters, l)
+            if counters:
+                sa, sb = ref[1].cache.read_stats(), got[1].cache.read_stats()
+                assert list(sa.visible) == list(sb.visible) and list(sa.accepted) == list(sb.accepted)
+
+
 def test_counts_and_depth_invariants(full):
     import torch
 
