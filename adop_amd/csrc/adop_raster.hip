@@ -114,8 +114,8 @@ struct WorkspaceLayout
     size_t fin_mini;    // double[kFinalizeParts * (kMaxChannels + B * kPartialStride)]: first-stage rows of finalize
     size_t pixels;      // float[B * P * max(S, 2C)]: blend accumulators (forward) / [I|G] array (backward)
     size_t dw;          // float2[B * P]: (depth, weight) per pixel for the backward descriptor pass
-    size_t q_counts;    // uint32[2][kNumQueues]: the views alternate between the two sets; + the finalize ticket
-    size_t q_items;     // uint64[kNumQueues * q_cap]
+    size_t q_counts;    // uint32[B][kNumQueues]: one set of sub-queue counters per view; + the finalize ticket
+    size_t q_items;     // uint64[B][kNumQueues * q_cap]
     uint32_t q_cap;
     size_t proj;        // float4[B * list_stride]: projected points of the forward pass when the caller keeps no point_cache
     size_t list_stride; // N rounded up to whole prepass workgroups
@@ -191,9 +191,9 @@ WorkspaceLayout layout(const adop_scene* s, int B, int L, int w0, int h0)
     w.q_cap       = (uint32_t)(((blocks + kNumQueues - 1) / kNumQueues) * kBlock);
     if (w.q_cap == 0) w.q_cap = kBlock;
     w.q_counts = o;
-    o          = align_up(o + sizeof(uint32_t) * (2 * kNumQueues + 1), 256);
+    o          = align_up(o + sizeof(uint32_t) * ((size_t)B * kNumQueues + 1), 256);
     w.q_items  = o;
-    o          = align_up(o + sizeof(unsigned long long) * (size_t)kNumQueues * w.q_cap, 256);
+    o          = align_up(o + sizeof(unsigned long long) * (size_t)B * kNumQueues * w.q_cap, 256);
     // (a view's slots are rounded up to whole prepass workgroups of at most 4 * kBlock points: list mode)
     const size_t n_pad = (((size_t)(s->num_points > 0 ? s->num_points : 0) + 4 * kBlock - 1) / (4 * kBlock)) * (4 * kBlock);
     w.list_stride = n_pad;
@@ -599,13 +599,13 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
                              stream)) != ADOP_OK)
             return st;
     }
+    {
+        // one pass over the points for all views: the descriptor gradient is summed in registers and written once
+        StageScope sc("RenderBackward/descriptor", stream);
+        launch_backward_tex(pc, dviews, lv, rp, half, ig, dw, grads, scene->index_is_identity, q, stats, stream);
+    }
     for (int b = 0; b < num_views; ++b)
     {
-        {
-            StageScope sc("RenderBackward/descriptor", stream);
-            launch_backward_tex(pc, dviews, lv, rp, half, ig, dw, grads, scene->index_is_identity, b, b == 0, q, stats,
-                                stream);
-        }
         StageScope sc("RenderBackward/spatial", stream);
         launch_backward_ghost(pc, dviews, lv, rp, half, ig, grads, want_pose, want_intr, scene->index_is_identity, b,
                               q, pt_blocks, pt_partial, stream);
@@ -613,7 +613,7 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     StageScope post("Post Process Gradient", stream);
     launch_finalize(dviews, num_views, C, bg_partial, bg_blocks, pt_partial, pt_blocks, grads, scene->num_poses,
                     scene->num_cameras, scene->intrinsics_cols, params->normalize_mode, scratch,
-                    (double*)((char*)workspace + wl.fin_mini), q.counts + 2 * kNumQueues, N, stream);
+                    (double*)((char*)workspace + wl.fin_mini), q.counts + (size_t)num_views * kNumQueues, N, stream);
     ADOP_HIP_CHECK(hipGetLastError());
     return ADOP_OK;
 }

@@ -21,13 +21,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
                                                             uint32_t* __restrict__ q_counts, ViewPrep vp)
 {
     prepare_views_inline(vp);
-    // counters of the backward work queue: the set of the first view is empty before it (backward_ghost_kernel
-    // empties the set of the next view)
-    if (blockIdx.x == 0)
-    {
-        for (int k = threadIdx.x; k < kNumQueues; k += kBlock) q_counts[k] = 0;
-        if (threadIdx.x == 0) q_counts[2 * kNumQueues] = 0;  // ticket counter of finalize_kernel
-    }
+    // counters of the backward work queues (one set per view): empty before backward_tex_kernel
+    for (int k = blockIdx.x * kBlock + threadIdx.x; k <= lv.B * kNumQueues; k += gridDim.x * kBlock)
+        q_counts[k] = 0;  // (the last word is the ticket counter of finalize_normalize_kernel)
     constexpr int CMAX = CT ? CT : kMaxChannels;
     const int C        = CT ? CT : lv.C;
     __shared__ double red[kBlock / 64][kMaxChannels];
@@ -154,14 +150,13 @@ __device__ __forceinline__ void load_channels(const float* __restrict__ src, flo
 //
 // backward_ghost_kernel — one thread per queue item, all lanes busy: the four-neighbour gather from the
 // pixel-major [I|G] array, the approximate image-space gradient (:491-611) and ProjectPoint*Backward.
-template <int CT, bool HALF>
-__global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const ViewConst* __restrict__ views,
+template <int CT, bool HALF, bool MULTI>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(CT != 0 ? 8 : 4, 8))) void backward_tex_kernel(CloudArg pc, const ViewConst* __restrict__ views,
                                                                Levels lv, ParamArg rp, const float* __restrict__ ig,
                                                                const float2* __restrict__ dw,
                                                                float* __restrict__ gtex,
                                                                float* __restrict__ gpoints,
                                                                float* __restrict__ gpoints_count, int identity_index,
-                                                               int view_b, int first_view,
                                                                uint32_t* __restrict__ q_counts,
                                                                unsigned long long* __restrict__ q_items,
                                                                uint32_t q_cap, adop_stats* stats)
@@ -170,145 +165,182 @@ __global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const
     __shared__ uint32_t s_wave_count[kBlock / 64];
     __shared__ uint32_t s_base;
     const bool STATS    = stats != nullptr;  // counter pass (uniform branch)
-    const int b         = view_b;
-    const ViewConst& vc = views[b];
     const float accept  = rp.depth_accept + 1;
     const int C         = CT ? CT : lv.C;
     const int lane      = threadIdx.x & 63;
     const int wave      = threadIdx.x >> 6;
 
-    const int i  = blockIdx.x * kBlock + threadIdx.x;
-    bool valid   = i < pc.n;
-    bool drop_out;
-    V2 ip = {0.f, 0.f};
-    float z = 0.f, radius_pixels = 0.f;
-    bool ok;
-    if (pc.cache)  // kernel-uniform: the forward pass left the projected points with the caller
-    {
-        // depth 0: culled; negative depth: dropped for this image (:314-315)
-        float4 R = make_float4(0, 0, 0, 0);
-        if (valid)
-        {
-            const v4f r = __builtin_nontemporal_load((const v4f*)pc.cache + (size_t)b * pc.n + i);
-            R           = make_float4(r.x, r.y, r.z, r.w);
-        }
-        ip             = {R.x, R.y};
-        drop_out       = R.z < 0;
-        z              = fabsf(R.z);
-        radius_pixels  = R.w;
-        ok             = valid && z != 0;
-    }
-    else
-    {
-        drop_out = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;
-        float4 P = valid ? pc.position[i] : make_float4(0, 0, 0, 0);
-        V3 pos   = {P.x, P.y, P.z};
-        V3 nrm   = {0, 0, 0};
-        if (valid && pc.normal) nrm = unpack_normal10(pc.normal[i]);
-        V3 view_p;
-        ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff, lv.l[0].w,
-                                    &ip, &z, &radius_pixels, &view_p);
-    }
-    int tex_index = identity_index ? i : (valid ? pc.index[i] : 0);
-    ok            = ok && (unsigned)tex_index < (unsigned)pc.num_texels;
-
-    // phase 1: pixel of every level, depth loads (independent)
-    uint32_t pix[ADOP_MAX_LAYERS];
-    bool in[ADOP_MAX_LAYERS];
-    bool edge_ok[ADOP_MAX_LAYERS];
-    float dep[ADOP_MAX_LAYERS];
-    float wgt[ADOP_MAX_LAYERS];
-#pragma unroll
-    for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
-    {
-        in[l]      = false;
-        edge_ok[l] = false;
-        pix[l]     = 0;
-        dep[l]     = 0.f;
-        wgt[l]     = 0.f;
-        if (l < lv.num)
-        {
-            const LevelArg& L = lv.l[l];
-            int px = f2i_rn(ip.x), py = f2i_rn(ip.y);
-            bool lod_skip = rp.drop_by_radius && radius_pixels < rp.drop_threshold;  // continue, :451-454
-            in[l]         = ok && !lod_skip && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h;
-            if (in[l])
-            {
-                pix[l]     = (uint32_t)py * (uint32_t)L.w + (uint32_t)px;
-                const float2 d_w = dw[ws_pixel(lv, l, b, pix[l])];  // (depth, weight) left by interleave_kernel
-                dep[l]           = d_w.x;
-                wgt[l]           = d_w.y;
-                int ex     = min(px, L.w - 1 - px);
-                int ey     = min(py, L.h - 1 - py);
-                edge_ok[l] = min(ex, ey) > 2;  // distanceFromEdge > 2, :489
-            }
-            radius_pixels *= 0.5f;
-            ip.x *= 0.5f;
-            ip.y *= 0.5f;
-        }
-    }
-    // phase 2: depth test in level order, `break` at the first failure (:462)
-    bool pass[ADOP_MAX_LAYERS];
-    {
-        bool alive = true;
-#pragma unroll
-        for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
-        {
-            pass[l] = false;
-            if (in[l] && alive)
-            {
-                if (z > dep[l] * accept)
-                    alive = false;
-                else
-                    pass[l] = true;
-            }
-        }
-    }
-    // phase 3: descriptor gradient of the rendered (not dropped) points; spatial-gradient eligibility
-    const bool point_grad = (rp.ghost_gradients && drop_out) | (!rp.ghost_gradients && !drop_out);
-    uint32_t mask         = 0;
+    const int i     = blockIdx.x * kBlock + threadIdx.x;
+    const bool valid = i < pc.n;
+    const int tex_index    = identity_index ? i : (valid ? pc.index[i] : 0);
+    const bool tex_in_range = (unsigned)tex_index < (unsigned)pc.num_texels;
+    // the descriptor gradient of the point, summed over the views and levels in registers and written once
     float gt[CMAX];
 #pragma unroll
     for (int c = 0; c < CMAX; ++c) gt[c] = 0.f;
     bool gt_live = false;
-#pragma unroll
-    for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+
+    // the views one after the other: view b appends to work queue b (MULTI = false: one view, no loop)
+    const int num_views = MULTI ? lv.B : 1;
+    for (int b = 0; b < num_views; ++b)
     {
-        bool go = pass[l];
-        if (pass[l] && !drop_out)
+        const ViewConst& vc = views[b];
+        bool drop_out;
+        V2 ip = {0.f, 0.f};
+        float z = 0.f, radius_pixels = 0.f;
+        bool ok;
+        if (pc.cache)  // kernel-uniform: the forward pass left the projected points with the caller
         {
-            if (wgt[l] == 0)
-                go = false;  // continue, :473
-            else
+            // depth 0: culled; negative depth: dropped for this image (:314-315)
+            float4 R = make_float4(0, 0, 0, 0);
+            if (valid)
             {
-                float iw        = 1.f / wgt[l];
-                const float* pg = ig + (size_t)ws_pixel(lv, l, b, pix[l]) * (2 * C) + C;  // G of the pixel
-                if (CT == 0)
-                {
-                    // any channel count: one atomic per channel and level (:478-484)
-#pragma unroll 1
-                    for (int c = 0; c < C; ++c)
-                        unsafeAtomicAdd(gtex + (size_t)c * pc.num_texels + tex_index, iw * pg[c]);
-                }
-                else
-                {
-                    float G[CMAX];
-                    load_channels<CT ? CT : 4>(pg, G);
+                const v4f r = __builtin_nontemporal_load((const v4f*)pc.cache + (size_t)b * pc.n + i);
+                R           = make_float4(r.x, r.y, r.z, r.w);
+            }
+            ip             = {R.x, R.y};
+            drop_out       = R.z < 0;
+            z              = fabsf(R.z);
+            radius_pixels  = R.w;
+            ok             = valid && z != 0;
+        }
+        else
+        {
+            drop_out = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;
+            float4 P = valid ? pc.position[i] : make_float4(0, 0, 0, 0);
+            V3 pos   = {P.x, P.y, P.z};
+            V3 nrm   = {0, 0, 0};
+            if (valid && pc.normal) nrm = unpack_normal10(pc.normal[i]);
+            V3 view_p;
+            ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff, lv.l[0].w,
+                                        &ip, &z, &radius_pixels, &view_p);
+        }
+        ok = ok && tex_in_range;
+
+        // phase 1: pixel of every level, depth loads (independent)
+        uint32_t pix[ADOP_MAX_LAYERS];
+        bool in[ADOP_MAX_LAYERS];
+        bool edge_ok[ADOP_MAX_LAYERS];
+        float dep[ADOP_MAX_LAYERS];
+        float wgt[ADOP_MAX_LAYERS];
 #pragma unroll
-                    for (int c = 0; c < CMAX; ++c) gt[c] += iw * G[c];
-                    gt_live = true;
+        for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+        {
+            in[l]      = false;
+            edge_ok[l] = false;
+            pix[l]     = 0;
+            dep[l]     = 0.f;
+            wgt[l]     = 0.f;
+            if (l < lv.num)
+            {
+                const LevelArg& L = lv.l[l];
+                int px = f2i_rn(ip.x), py = f2i_rn(ip.y);
+                bool lod_skip = rp.drop_by_radius && radius_pixels < rp.drop_threshold;  // continue, :451-454
+                in[l]         = ok && !lod_skip && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h;
+                if (in[l])
+                {
+                    pix[l]     = (uint32_t)py * (uint32_t)L.w + (uint32_t)px;
+                    const float2 d_w = dw[ws_pixel(lv, l, b, pix[l])];  // (depth, weight) left by interleave_kernel
+                    dep[l]           = d_w.x;
+                    wgt[l]           = d_w.y;
+                    int ex     = min(px, L.w - 1 - px);
+                    int ey     = min(py, L.h - 1 - py);
+                    edge_ok[l] = min(ex, ey) > 2;  // distanceFromEdge > 2, :489
+                }
+                radius_pixels *= 0.5f;
+                ip.x *= 0.5f;
+                ip.y *= 0.5f;
+            }
+        }
+        // phase 2: depth test in level order, `break` at the first failure (:462)
+        bool pass[ADOP_MAX_LAYERS];
+        {
+            bool alive = true;
+#pragma unroll
+            for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+            {
+                pass[l] = false;
+                if (in[l] && alive)
+                {
+                    if (z > dep[l] * accept)
+                        alive = false;
+                    else
+                        pass[l] = true;
                 }
             }
         }
-        bool spatial = go && point_grad && edge_ok[l];
-        if (spatial) mask |= 1u << l;
-        if (STATS && l < lv.num) stat_add(&stats->spatial[l], spatial);
-    }
+        // phase 3: descriptor gradient of the rendered (not dropped) points; spatial-gradient eligibility
+        const bool point_grad = (rp.ghost_gradients && drop_out) | (!rp.ghost_gradients && !drop_out);
+        uint32_t mask         = 0;
+#pragma unroll
+        for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+        {
+            bool go = pass[l];
+            if (pass[l] && !drop_out)
+            {
+                if (wgt[l] == 0)
+                    go = false;  // continue, :473
+                else
+                {
+                    float iw        = 1.f / wgt[l];
+                    const float* pg = ig + (size_t)ws_pixel(lv, l, b, pix[l]) * (2 * C) + C;  // G of the pixel
+                    if (CT == 0)
+                    {
+                        // any channel count: one atomic per channel and level (:478-484)
+#pragma unroll 1
+                        for (int c = 0; c < C; ++c)
+                            unsafeAtomicAdd(gtex + (size_t)c * pc.num_texels + tex_index, iw * pg[c]);
+                    }
+                    else
+                    {
+                        float G[CMAX];
+                        load_channels<CT ? CT : 4>(pg, G);
+#pragma unroll
+                        for (int c = 0; c < CMAX; ++c) gt[c] += iw * G[c];
+                        gt_live = true;
+                    }
+                }
+            }
+            bool spatial = go && point_grad && edge_ok[l];
+            if (spatial) mask |= 1u << l;
+            if (STATS && l < lv.num) stat_add(&stats->spatial[l], spatial);
+        }
+        // Point gradients of the first view: points without a spatial gradient are cleared here (Build(info,false),
+        // :922-949), the others are written by backward_ghost_kernel; no separate zero-fill of the two buffers.
+        if (b == 0 && gpoints && valid && mask == 0)
+        {
+            nt_store4((float4*)gpoints + i, make_float4(0, 0, 0, 0));
+            __builtin_nontemporal_store(0.f, gpoints_count + i);
+        }
+
+        // queue push: rank inside the workgroup, one returning atomic per workgroup on the sub-queue counter
+        bool has               = mask != 0;
+        unsigned long long bal = __ballot(has);
+        uint32_t rank_in_wave  = (uint32_t)__popcll(bal & ((1ull << lane) - 1ull));
+        if (lane == 0) s_wave_count[wave] = (uint32_t)__popcll(bal);
+        __syncthreads();
+        uint32_t before = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < kBlock / 64; ++w)
+        {
+            uint32_t c = s_wave_count[w];
+            if (w < wave) before += c;
+            total += c;
+        }
+        const uint32_t q = blockIdx.x % kNumQueues;
+        if (threadIdx.x == 0) s_base = total ? atomicAdd(&q_counts[(size_t)b * kNumQueues + q], total) : 0u;
+        __syncthreads();
+        if (has)
+            q_items[((size_t)b * kNumQueues + q) * q_cap + s_base + before + rank_in_wave] =
+                (unsigned long long)(uint32_t)i | ((unsigned long long)mask << 32);
+        __syncthreads();  // s_wave_count and s_base are reused by the next view
+    }  // views
+
     if (CT != 0)
     {
         if (identity_index)
         {
-            // texel i belongs to this thread alone: plain coalesced stores, which also clear the buffer on the first view
+            // texel i belongs to this thread alone: plain coalesced stores, which also clear the buffer
             if (valid)
             {
 #pragma unroll
@@ -316,7 +348,7 @@ __global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const
                 {
                     // streamed once: kept out of the caches the gathers of this kernel live in
                     float* dst = gtex + (size_t)c * pc.num_texels + i;
-                    __builtin_nontemporal_store(first_view ? gt[c] : (*dst + gt[c]), dst);
+                    __builtin_nontemporal_store(gt[c], dst);
                 }
             }
         }
@@ -326,35 +358,6 @@ __global__ __launch_bounds__(kBlock) void backward_tex_kernel(CloudArg pc, const
             for (int c = 0; c < CMAX; ++c) unsafeAtomicAdd(gtex + (size_t)c * pc.num_texels + tex_index, gt[c]);
         }
     }
-
-    // Point gradients of the first view: points without a spatial gradient are cleared here (Build(info,false),
-    // :922-949), the others are written by backward_ghost_kernel; no separate zero-fill of the two buffers.
-    if (first_view && gpoints && valid && mask == 0)
-    {
-        nt_store4((float4*)gpoints + i, make_float4(0, 0, 0, 0));
-        __builtin_nontemporal_store(0.f, gpoints_count + i);
-    }
-
-    // queue push: rank inside the workgroup, one returning atomic per workgroup on the sub-queue counter
-    bool has               = mask != 0;
-    unsigned long long bal = __ballot(has);
-    uint32_t rank_in_wave  = (uint32_t)__popcll(bal & ((1ull << lane) - 1ull));
-    if (lane == 0) s_wave_count[wave] = (uint32_t)__popcll(bal);
-    __syncthreads();
-    uint32_t before = 0, total = 0;
-#pragma unroll
-    for (int w = 0; w < kBlock / 64; ++w)
-    {
-        uint32_t c = s_wave_count[w];
-        if (w < wave) before += c;
-        total += c;
-    }
-    const uint32_t q = blockIdx.x % kNumQueues;
-    if (threadIdx.x == 0) s_base = total ? atomicAdd(&q_counts[q], total) : 0u;
-    __syncthreads();
-    if (has)
-        q_items[(size_t)q * q_cap + s_base + before + rank_in_wave] =
-            (unsigned long long)(uint32_t)i | ((unsigned long long)mask << 32);
 }
 
 // 4 waves per SIMD (<= 128 VGPRs): the grid of kPartialBlocks = 4 workgroups x 256 CUs is then resident at once; with
@@ -367,7 +370,6 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
                                                                  int want_intr, int identity_index, int view_b,
                                                                  int first_view,
                                                                  const uint32_t* __restrict__ q_counts,
-                                                                 uint32_t* __restrict__ q_counts_next,
                                                                  const unsigned long long* __restrict__ q_items,
                                                                  uint32_t q_cap, double* __restrict__ partial)
 {
@@ -409,9 +411,6 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
             run += v[k];
         }
         if (threadIdx.x == kBlock - 1) s_prefix[kNumQueues] = run;
-        // the other set of counters is the next view's: nothing reads it before this kernel has ended
-        if (blockIdx.x == 0)
-            for (int k = threadIdx.x; k < kNumQueues; k += kBlock) q_counts_next[k] = 0;
         __syncthreads();
     }
     const uint32_t total = s_prefix[kNumQueues];
@@ -891,13 +890,18 @@ void launch_interleave(const Levels& lv, int blocks, float* ig, float2* dw, doub
 
 template <int CT, bool HALF>
 static void launch_bwd_tex_t(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp,
-                             const float* ig, const float2* dw, const adop_backward_buffers* g, int identity_index, int b,
-                             int first_view, const QueueArg& q, adop_stats* stats, hipStream_t st)
+                             const float* ig, const float2* dw, const adop_backward_buffers* g, int identity_index,
+                             const QueueArg& q, adop_stats* stats, hipStream_t st)
 {
     int grid = (pc.n + kBlock - 1) / kBlock;
-    hipLaunchKernelGGL((backward_tex_kernel<CT, HALF>), dim3(grid), dim3(kBlock), 0, st, pc, views, lv, rp, ig, dw,
-                       g->grad_texture, g->grad_points, g->grad_points_count, identity_index, b, first_view,
-                       q.counts + (b & 1) * kNumQueues, q.items, q.cap, stats);
+    if (lv.B > 1)
+        hipLaunchKernelGGL((backward_tex_kernel<CT, HALF, true>), dim3(grid), dim3(kBlock), 0, st, pc, views, lv, rp, ig,
+                           dw, g->grad_texture, g->grad_points, g->grad_points_count, identity_index, q.counts, q.items,
+                           q.cap, stats);
+    else
+        hipLaunchKernelGGL((backward_tex_kernel<CT, HALF, false>), dim3(grid), dim3(kBlock), 0, st, pc, views, lv, rp, ig,
+                           dw, g->grad_texture, g->grad_points, g->grad_points_count, identity_index, q.counts, q.items,
+                           q.cap, stats);
 }
 
 template <int CT, bool HALF>
@@ -908,8 +912,7 @@ static void launch_bwd_ghost_t(const CloudArg& pc, const ViewConst* views, const
 {
     hipLaunchKernelGGL((backward_ghost_kernel<CT, HALF>), dim3(ghost_blocks), dim3(kBlock), 0, st, pc, views, lv, rp,
                        ig, g->grad_points, g->grad_points_count, want_pose, want_intr, identity_index, b, b == 0,
-                       q.counts + (b & 1) * kNumQueues, q.counts + ((b + 1) & 1) * kNumQueues, q.items, q.cap,
-                       partial);
+                       q.counts + (size_t)b * kNumQueues, q.items + (size_t)b * kNumQueues * q.cap, q.cap, partial);
 }
 
 #define ADOP_DISPATCH_C_HALF(FN, ...)                                   \
@@ -925,11 +928,11 @@ static void launch_bwd_ghost_t(const CloudArg& pc, const ViewConst* views, const
 
 // descriptor gradient of one view + the work queue of its ghost / spatial gradients
 void launch_backward_tex(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
-                         const float* ig, const float2* dw, const adop_backward_buffers* g, int identity_index, int b, int first_view,
+                         const float* ig, const float2* dw, const adop_backward_buffers* g, int identity_index,
                          const QueueArg& q, adop_stats* stats, hipStream_t st)
 {
     if (pc.n < 1) return;
-    ADOP_DISPATCH_C_HALF(launch_bwd_tex_t, pc, views, lv, rp, ig, dw, g, identity_index, b, first_view, q, stats, st);
+    ADOP_DISPATCH_C_HALF(launch_bwd_tex_t, pc, views, lv, rp, ig, dw, g, identity_index, q, stats, st);
 }
 
 // ghost / spatial gradients of the queued points of one view

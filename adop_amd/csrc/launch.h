@@ -57,12 +57,12 @@ void launch_interleave(const Levels& lv, int blocks, float* ig, float2* dw, doub
 // of `cap` items each.
 struct QueueArg
 {
-    uint32_t* counts;           // [2][kNumQueues]: view b appends through set b & 1
-    unsigned long long* items;  // [kNumQueues * cap]
+    uint32_t* counts;           // [B][kNumQueues]: one set per view
+    unsigned long long* items;  // [B][kNumQueues * cap]
     uint32_t cap;
 };
 void launch_backward_tex(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
-                         const float* ig, const float2* dw, const adop_backward_buffers* g, int identity_index, int b, int first_view,
+                         const float* ig, const float2* dw, const adop_backward_buffers* g, int identity_index,
                          const QueueArg& q, adop_stats* stats, hipStream_t st);
 void launch_backward_ghost(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
                            const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr,
