@@ -117,8 +117,8 @@ def test_backward_without_point_gradients(oracle_mod):
 
 
 def test_more_views_than_one_constant_chunk(oracle_mod):
-    """34 views: the per-view constants take the chunked path (32 per launch), the backward work queue alternates
-    its two counter sets 34 times, every view accumulates into the same point / pose / intrinsics gradients."""
+    """34 views: the per-view constants take the chunked path (32 per launch), the descriptor pass fills 34 work
+    queues, every view accumulates into the same point / pose / intrinsics gradients."""
     from adop_amd import scenes
 
     announce("config2 30k pts B=34 96x96 L3 fwd+bwd ghost")
