@@ -147,6 +147,16 @@ ENTRY_POINTS = {
          C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p],
     ),
     "adop_apply_tangent": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "adop_knn_workspace_size": (C.c_size_t, [C.c_int32]),
+    "adop_knn_distance": (
+        C.c_int,
+        [C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_void_p, C.c_void_p,
+         C.c_size_t, C.c_void_p],
+    ),
+    "adop_morton_codes": (
+        C.c_int,
+        [C.c_void_p, C.c_int32, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_void_p, C.c_void_p],
+    ),
     "adop_profile_enable": (C.c_int, [C.c_int32]),
     "adop_profile_read": (C.c_int32, [C.POINTER(StageTime), C.c_int32]),
     "adop_last_error_string": (C.c_char_p, []),

@@ -703,6 +703,90 @@ adop_status adop_apply_tangent(double* tangent, double* poses_se3, int32_t num_p
     return ADOP_OK;
 }
 
+// Grid of the nearest-neighbour search: ~8 points per cell for a volume-filling cloud, at most kKnnMaxDim cells per
+// axis (a surface-like cloud puts more points into fewer cells; the search stays exact, only slower).
+static constexpr int kKnnMaxDim = 160;
+
+static size_t knn_cells_max() { return (size_t)kKnnMaxDim * kKnnMaxDim * kKnnMaxDim; }
+
+size_t adop_knn_workspace_size(int32_t num_points)
+{
+    if (num_points < 0) return 0;
+    size_t o = 0;
+    o        = align_up(o + sizeof(uint32_t) * knn_cells_max(), 256);        // count
+    o        = align_up(o + sizeof(uint32_t) * (knn_cells_max() + 1), 256);  // offset
+    o        = align_up(o + sizeof(float4) * (size_t)num_points, 256);      // points in cell order
+    return o;
+}
+
+adop_status adop_knn_distance(const float* position, int32_t num_points, int32_t rank, const float* bbox_min,
+                              const float* bbox_max, float* out_distance, void* workspace, size_t workspace_bytes,
+                              void* hip_stream)
+{
+    if (!position || !bbox_min || !bbox_max || !out_distance) return fail(ADOP_INVALID_ARG, "null argument");
+    if (rank < 1 || rank > 8) return fail(ADOP_INVALID_ARG, "rank must be 1..8");
+    if (num_points <= rank) return fail(ADOP_INVALID_ARG, "the cloud needs more than `rank` points");
+    if (!workspace || workspace_bytes < adop_knn_workspace_size(num_points))
+        return fail(ADOP_WORKSPACE_TOO_SMALL, "workspace too small");
+    float ext[3];
+    for (int k = 0; k < 3; ++k)
+    {
+        ext[k] = bbox_max[k] - bbox_min[k];
+        if (!(ext[k] >= 0) || !(ext[k] < 1.0e30f)) return fail(ADOP_INVALID_ARG, "bounding box is not finite");
+    }
+    KnnGrid g;
+    const float longest = ext[0] > ext[1] ? (ext[0] > ext[2] ? ext[0] : ext[2]) : (ext[1] > ext[2] ? ext[1] : ext[2]);
+    double volume       = 1.0;
+    for (int k = 0; k < 3; ++k) volume *= ext[k] > 1e-6f * longest ? ext[k] : (longest > 0 ? 1e-6 * longest : 1.0);
+    float cell = (float)cbrt(volume * 8.0 / (double)num_points);
+    if (!(cell > longest / kKnnMaxDim)) cell = longest / kKnnMaxDim;
+    if (!(cell > 0)) cell = 1.f;  // all points coincide
+    g.cell     = cell;
+    g.inv_cell = 1.0f / cell;
+    for (int k = 0; k < 3; ++k)
+    {
+        g.min[k] = bbox_min[k];
+        int d    = (int)(ext[k] / cell) + 1;
+        g.dim[k] = d < 1 ? 1 : (d > kKnnMaxDim ? kKnnMaxDim : d);
+    }
+    const size_t cells = (size_t)g.dim[0] * g.dim[1] * g.dim[2];
+    hipStream_t stream = (hipStream_t)hip_stream;
+    uint32_t* count    = (uint32_t*)workspace;
+    uint32_t* offset   = (uint32_t*)((char*)workspace + align_up(sizeof(uint32_t) * knn_cells_max(), 256));
+    float4* sorted     = (float4*)((char*)offset + align_up(sizeof(uint32_t) * (knn_cells_max() + 1), 256));
+    adop_status st     = fill_async(count, sizeof(uint32_t) * cells, 0, stream);
+    if (st != ADOP_OK) return st;
+    launch_knn_bin(0, (const float4*)position, num_points, g, count, offset, sorted, stream);
+    BinArg scan;
+    memset(&scan, 0, sizeof(scan));
+    scan.count  = count;
+    scan.offset = offset;
+    launch_tile_scan(scan, (int)cells, stream);
+    launch_knn_bin(1, (const float4*)position, num_points, g, count, offset, sorted, stream);
+    if (!launch_knn_search(rank, sorted, num_points, g, offset, out_distance, stream))
+        return fail(ADOP_INVALID_ARG, "rank must be 1..8");
+    ADOP_HIP_CHECK(hipGetLastError());
+    return ADOP_OK;
+}
+
+adop_status adop_morton_codes(const float* position, int32_t num_points, const float* bbox_min, const float* bbox_max,
+                              uint64_t* out_codes, void* hip_stream)
+{
+    if (!position || !bbox_min || !bbox_max || !out_codes || num_points < 0) return fail(ADOP_INVALID_ARG, "null argument");
+    if (num_points == 0) return ADOP_OK;
+    float scale[3];
+    for (int k = 0; k < 3; ++k)
+    {
+        const float ext = bbox_max[k] - bbox_min[k];
+        if (!(ext >= 0) || !(ext < 1.0e30f)) return fail(ADOP_INVALID_ARG, "bounding box is not finite");
+        scale[k] = ext > 0 ? 2097151.f / ext : 0.f;
+    }
+    launch_morton((const float4*)position, num_points, bbox_min, scale, (unsigned long long*)out_codes,
+                  (hipStream_t)hip_stream);
+    ADOP_HIP_CHECK(hipGetLastError());
+    return ADOP_OK;
+}
+
 adop_status adop_profile_enable(int32_t enable)
 {
     g_profile = enable != 0;

@@ -78,6 +78,14 @@ struct ParamArg
     float K_gradient_factor;
 };
 
+// Uniform grid of the nearest-neighbour search: cubic cells of edge `cell` from `min`, dim cells per axis.
+struct KnnGrid
+{
+    float min[3];
+    float cell, inv_cell;
+    int32_t dim[3];
+};
+
 struct ViewChunk
 {
     adop_view v[32];

@@ -16,6 +16,12 @@ void launch_prepare_views(const ViewChunk& ch, int first, int count, const doubl
 void launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t st);
 void launch_clear(const Levels& lv, int first_level, int grid, float* accum, size_t accum_floats, uint32_t* zero_u32,
                   int zero_n, const ViewPrep& vp, hipStream_t st);
+void launch_knn_bin(int pass, const float4* position, int n, const KnnGrid& g, uint32_t* count, const uint32_t* offset,
+                    float4* sorted, hipStream_t st);
+bool launch_knn_search(int rank, const float4* sorted, int n, const KnnGrid& g, const uint32_t* offset, float* out,
+                       hipStream_t st);
+void launch_morton(const float4* position, int n, const float* mn, const float* scale, unsigned long long* code,
+                   hipStream_t st);
 int prepass_points_per_block();  // points per workgroup of prepass_kernel (the unit of its candidate lists)
 void launch_prepass(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, adop_stats* stats,
                     hipStream_t st);

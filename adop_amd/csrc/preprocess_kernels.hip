@@ -1,0 +1,170 @@
+// preprocess_kernels.hip — point-cloud preprocessing that decides how well the rasterizer runs (gfx950):
+// the distance of every point to its n-th nearest neighbour (SceneData::ComputeRadius, SceneData.cpp:441-484: a
+// kd-tree k-nearest-neighbour search per point on the host) and the Morton code of every point (the key of
+// ReorderMorton64, SceneData.cpp:101).
+//
+// Nearest neighbours: the points are binned into a uniform grid (count, prefix sum, scatter: the structure of the
+// rasterizer's tile bins), stored cell after cell, and every point then walks the shells of cells around its own
+// until the n-th best distance cannot be beaten from outside the cube searched so far.  The distances are formed as
+// sqrt((dx*dx + dy*dy) + dz*dz) in fp32; the result is the n-th smallest of them over all other points, whatever the
+// search order, so a brute-force search over the same arithmetic gives the same bits.
+#include "common.h"
+#include "launch.h"
+
+#pragma clang fp contract(off)
+
+namespace adop
+{
+__device__ __forceinline__ int3 grid_cell(const KnnGrid& g, float x, float y, float z)
+{
+    int cx = (int)((x - g.min[0]) * g.inv_cell);
+    int cy = (int)((y - g.min[1]) * g.inv_cell);
+    int cz = (int)((z - g.min[2]) * g.inv_cell);
+    cx     = cx < 0 ? 0 : (cx >= g.dim[0] ? g.dim[0] - 1 : cx);
+    cy     = cy < 0 ? 0 : (cy >= g.dim[1] ? g.dim[1] - 1 : cy);
+    cz     = cz < 0 ? 0 : (cz >= g.dim[2] ? g.dim[2] - 1 : cz);
+    return make_int3(cx, cy, cz);
+}
+
+__device__ __forceinline__ uint32_t grid_index(const KnnGrid& g, int cx, int cy, int cz)
+{
+    return ((uint32_t)cz * (uint32_t)g.dim[1] + (uint32_t)cy) * (uint32_t)g.dim[0] + (uint32_t)cx;
+}
+
+// pass 0: points per cell; pass 1: the points cell after cell, (x, y, z, bits of the point id)
+__global__ __launch_bounds__(kBlock) void knn_bin_kernel(int pass, const float4* __restrict__ position, int n, KnnGrid g,
+                                                         uint32_t* __restrict__ count, const uint32_t* __restrict__ offset,
+                                                         float4* __restrict__ sorted)
+{
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const float4 p    = nt_load4(position + i);
+    const int3 c      = grid_cell(g, p.x, p.y, p.z);
+    const uint32_t ci = grid_index(g, c.x, c.y, c.z);
+    if (pass == 0)
+        atomicAdd(&count[ci], 1u);
+    else  // the counter runs down to zero: slots are handed out from the end of the cell's range
+        sorted[offset[ci] + atomicSub(&count[ci], 1u) - 1u] = make_float4(p.x, p.y, p.z, __uint_as_float((uint32_t)i));
+}
+
+// One thread per point, in cell order (the lanes of a wavefront search nearly the same cells).  The cube of cells
+// around the point's cell grows until the K-th best distance cannot be beaten from outside it; a row of cells along x
+// is one contiguous run of the cell-ordered array, so a cube of (2r+1)^3 cells is (2r+1)^2 runs.  A larger cube is
+// searched from scratch (with ~8 points per cell the first cube, r = 1, settles nearly every point).
+template <int K>  // K = n + 1 best squared distances are kept (the point itself is one of them)
+__global__ __launch_bounds__(kBlock) void knn_search_kernel(const float4* __restrict__ sorted, int n, KnnGrid g,
+                                                            const uint32_t* __restrict__ offset, float* __restrict__ out)
+{
+    const int t = blockIdx.x * kBlock + threadIdx.x;
+    if (t >= n) return;
+    const float4 p = sorted[t];
+    const int3 c   = grid_cell(g, p.x, p.y, p.z);
+    float best[K];
+    for (int r = 1;; ++r)
+    {
+#pragma unroll
+        for (int k = 0; k < K; ++k) best[k] = 3.0e38f;
+        const int z0 = max(c.z - r, 0), z1 = min(c.z + r, g.dim[2] - 1);
+        const int y0 = max(c.y - r, 0), y1 = min(c.y + r, g.dim[1] - 1);
+        const int x0 = max(c.x - r, 0), x1 = min(c.x + r, g.dim[0] - 1);
+        for (int cz = z0; cz <= z1; ++cz)
+            for (int cy = y0; cy <= y1; ++cy)
+            {
+                const uint32_t row = grid_index(g, 0, cy, cz);
+                const uint32_t e   = offset[row + x1 + 1];
+                for (uint32_t q = offset[row + x0]; q < e; ++q)
+                {
+                    const float4 o = sorted[q];
+                    const float dx = p.x - o.x, dy = p.y - o.y, dz = p.z - o.z;
+                    float d2 = (dx * dx + dy * dy) + dz * dz;
+                    if (d2 < best[K - 1])
+                    {
+#pragma unroll
+                        for (int k = 0; k < K; ++k)  // insertion into the ascending list
+                        {
+                            const float b = best[k];
+                            const bool lt = d2 < b;
+                            best[k]       = lt ? d2 : b;
+                            d2            = lt ? b : d2;
+                        }
+                    }
+                }
+            }
+        // Nothing outside the cube is closer than the nearest face of the cube that has cells behind it (slightly
+        // shrunk: the cell of a point and the faces are computed in fp32).  No such face: the cube is the whole grid.
+        float bound = 3.0e38f;
+        if (c.x - r > 0) bound = fminf(bound, p.x - (g.min[0] + (float)(c.x - r) * g.cell));
+        if (c.y - r > 0) bound = fminf(bound, p.y - (g.min[1] + (float)(c.y - r) * g.cell));
+        if (c.z - r > 0) bound = fminf(bound, p.z - (g.min[2] + (float)(c.z - r) * g.cell));
+        if (c.x + r < g.dim[0] - 1) bound = fminf(bound, (g.min[0] + (float)(c.x + r + 1) * g.cell) - p.x);
+        if (c.y + r < g.dim[1] - 1) bound = fminf(bound, (g.min[1] + (float)(c.y + r + 1) * g.cell) - p.y);
+        if (c.z + r < g.dim[2] - 1) bound = fminf(bound, (g.min[2] + (float)(c.z + r + 1) * g.cell) - p.z);
+        if (bound == 3.0e38f) break;
+        bound = fmaxf(bound, 0.f) * 0.999f;
+        if (best[K - 1] <= bound * bound) break;
+    }
+    out[__float_as_uint(p.w)] = sqrtf(best[K - 1]);
+}
+
+// Morton code of every point: 21 bits per axis of the position inside the bounding box, x in the lowest bit.
+__device__ __forceinline__ unsigned long long spread21(unsigned long long v)
+{
+    v &= 0x1FFFFFull;
+    v = (v | v << 32) & 0x1F00000000FFFFull;
+    v = (v | v << 16) & 0x1F0000FF0000FFull;
+    v = (v | v << 8) & 0x100F00F00F00F00Full;
+    v = (v | v << 4) & 0x10C30C30C30C30C3ull;
+    v = (v | v << 2) & 0x1249249249249249ull;
+    return v;
+}
+
+__global__ __launch_bounds__(kBlock) void morton_kernel(const float4* __restrict__ position, int n, float min_x,
+                                                        float min_y, float min_z, float scale_x, float scale_y,
+                                                        float scale_z, unsigned long long* __restrict__ code)
+{
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const float4 p = nt_load4(position + i);
+    const float m  = 2097151.f;  // 2^21 - 1
+    const float fx = fminf(fmaxf((p.x - min_x) * scale_x, 0.f), m);
+    const float fy = fminf(fmaxf((p.y - min_y) * scale_y, 0.f), m);
+    const float fz = fminf(fmaxf((p.z - min_z) * scale_z, 0.f), m);
+    code[i] = spread21((unsigned long long)fx) | spread21((unsigned long long)fy) << 1 | spread21((unsigned long long)fz) << 2;
+}
+
+// ------------------------------------------------------------------------------------------------
+// launchers
+// ------------------------------------------------------------------------------------------------
+void launch_knn_bin(int pass, const float4* position, int n, const KnnGrid& g, uint32_t* count, const uint32_t* offset,
+                    float4* sorted, hipStream_t st)
+{
+    hipLaunchKernelGGL(knn_bin_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, pass, position, n, g, count,
+                       offset, sorted);
+}
+
+bool launch_knn_search(int rank, const float4* sorted, int n, const KnnGrid& g, const uint32_t* offset, float* out,
+                       hipStream_t st)
+{
+    const dim3 grid((n + kBlock - 1) / kBlock), block(kBlock);
+    switch (rank)
+    {
+        case 1: hipLaunchKernelGGL(knn_search_kernel<2>, grid, block, 0, st, sorted, n, g, offset, out); return true;
+        case 2: hipLaunchKernelGGL(knn_search_kernel<3>, grid, block, 0, st, sorted, n, g, offset, out); return true;
+        case 3: hipLaunchKernelGGL(knn_search_kernel<4>, grid, block, 0, st, sorted, n, g, offset, out); return true;
+        case 4: hipLaunchKernelGGL(knn_search_kernel<5>, grid, block, 0, st, sorted, n, g, offset, out); return true;
+        case 5: hipLaunchKernelGGL(knn_search_kernel<6>, grid, block, 0, st, sorted, n, g, offset, out); return true;
+        case 6: hipLaunchKernelGGL(knn_search_kernel<7>, grid, block, 0, st, sorted, n, g, offset, out); return true;
+        case 7: hipLaunchKernelGGL(knn_search_kernel<8>, grid, block, 0, st, sorted, n, g, offset, out); return true;
+        case 8: hipLaunchKernelGGL(knn_search_kernel<9>, grid, block, 0, st, sorted, n, g, offset, out); return true;
+    }
+    return false;
+}
+
+void launch_morton(const float4* position, int n, const float* mn, const float* scale, unsigned long long* code,
+                   hipStream_t st)
+{
+    hipLaunchKernelGGL(morton_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, position, n, mn[0], mn[1],
+                       mn[2], scale[0], scale[1], scale[2], code);
+}
+
+}  // namespace adop

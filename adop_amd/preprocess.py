@@ -1,0 +1,105 @@
+"""Point-cloud preprocessing of SceneData (data/SceneData.cpp:96-118) on the device: Morton order, shuffled
+256-point blocks, the radius of every point from its 4th nearest neighbour, blocks sorted by radius.
+
+The order of the cloud and the radii decide how the rasterizer runs (coherent wavefronts, the LOD early exit), so the
+steps sit next to it.  The distance search and the Morton codes are HIP kernels behind the C-ABI
+(``adop_knn_distance``, ``adop_morton_codes``); sorting and permuting go through torch.
+"""
+import ctypes as C
+
+import torch
+
+from . import _capi
+from .render import _check, _stream_ptr
+
+
+def _bbox(position):
+    lo, hi = torch.aminmax(position, dim=0)  # one pass over the contiguous [N,4] array
+    both = torch.stack([lo[:3], hi[:3]]).cpu()
+    return (C.c_float * 3)(*both[0].tolist()), (C.c_float * 3)(*both[1].tolist())
+
+
+def KNearestNeighbourDistance(position, rank=4):
+    """Distance of every point to its ``rank``-th nearest other point: ``data[i](0)`` of ComputeRadius
+    (SceneData.cpp:441-463).  position: [N,4] f32 on the device."""
+    assert position.is_cuda and position.dtype == torch.float32 and position.dim() == 2 and position.shape[1] == 4
+    position = position.contiguous()
+    n = int(position.shape[0])
+    lib = _capi.load_library()
+    out = torch.empty(n, dtype=torch.float32, device=position.device)
+    ws = torch.empty(int(lib.adop_knn_workspace_size(n)), dtype=torch.uint8, device=position.device)
+    mn, mx = _bbox(position)
+    rc = lib.adop_knn_distance(C.c_void_p(position.data_ptr()), n, int(rank), mn, mx, C.c_void_p(out.data_ptr()),
+                               C.c_void_p(ws.data_ptr()), int(ws.numel()), _stream_ptr())
+    _check(rc, lib)
+    return out
+
+
+def MortonCodes(position):
+    """63-bit Morton code of every point inside the cloud's bounding box (the key of ReorderMorton64)."""
+    assert position.is_cuda and position.dtype == torch.float32 and position.dim() == 2 and position.shape[1] == 4
+    position = position.contiguous()
+    n = int(position.shape[0])
+    lib = _capi.load_library()
+    codes = torch.empty(n, dtype=torch.int64, device=position.device)
+    mn, mx = _bbox(position)
+    rc = lib.adop_morton_codes(C.c_void_p(position.data_ptr()), n, mn, mx, C.c_void_p(codes.data_ptr()), _stream_ptr())
+    _check(rc, lib)
+    return codes
+
+
+def ReorderMorton64(position):
+    """Permutation that sorts the cloud along the Morton curve (stable: equal codes keep their order)."""
+    return torch.sort(MortonCodes(position), stable=True).indices
+
+
+def RandomBlockShuffle(num_points, block_size=256, generator=None):
+    """Permutation that shuffles whole blocks of ``block_size`` consecutive points (a last, shorter block stays
+    last)."""
+    nb = num_points // block_size
+    dev = "cuda"
+    perm = torch.randperm(nb, generator=generator, device="cpu").to(dev)
+    idx = (perm[:, None] * block_size + torch.arange(block_size, device=dev)[None, :]).reshape(-1)
+    tail = torch.arange(nb * block_size, num_points, device=dev)
+    return torch.cat([idx, tail])
+
+
+def ComputeRadius(position, rank=4, generator=None):
+    """SceneData::ComputeRadius (SceneData.cpp:441-484): returns ``data`` [N,4] with data[:,0] = distance to the
+    rank-th neighbour, data[:,2] = sqrt(1 / u), u ~ U(0,1), data[:,3] = data[:,0] * data[:,2] (the drop-out radius the
+    rasterizer reads as position.w, NeuralPointCloudCuda.cpp:21-35)."""
+    n = int(position.shape[0])
+    data = torch.zeros(n, 4, dtype=torch.float32, device=position.device)
+    data[:, 0] = KNearestNeighbourDistance(position, rank)
+    u = torch.rand(n, generator=generator, dtype=torch.float64, device="cpu").clamp_min_(1e-300).to(position.device)
+    data[:, 2] = torch.sqrt(1.0 / u).to(torch.float32)
+    data[:, 3] = data[:, 0] * data[:, 2]
+    return data
+
+
+def SortBlocksByRadius(radius, block_size=256):
+    """Permutation that sorts every full block of ``block_size`` points by ascending radius
+    (SceneData.cpp:671-684; the last, shorter block keeps its order)."""
+    n = int(radius.shape[0])
+    nb = n // block_size
+    head = radius[: nb * block_size].reshape(nb, block_size)
+    order = torch.sort(head, dim=1, stable=True).indices + (torch.arange(nb, device=radius.device) * block_size)[:, None]
+    return torch.cat([order.reshape(-1), torch.arange(nb * block_size, n, device=radius.device)])
+
+
+def PreprocessPointCloud(position, normal=None, rank=4, block_size=256, seed=0):
+    """The initial processing of a new scene in the reference's order (SceneData.cpp:101-104): ReorderMorton64,
+    RandomBlockShuffle(256), ComputeRadius, SortBlocksByRadius(256).  Returns (position [N,4] with the drop-out radius in
+    w, normal, data [N,4], order) where ``order`` maps new to original point ids."""
+    gen = torch.Generator(device="cpu").manual_seed(int(seed))
+    position = position.contiguous()
+    order = ReorderMorton64(position)
+    order = order[RandomBlockShuffle(int(position.shape[0]), block_size, gen)]
+    position = position[order].contiguous()
+    data = ComputeRadius(position, rank, gen)
+    by_radius = SortBlocksByRadius(data[:, 3], block_size)
+    order = order[by_radius]
+    position = position[by_radius].clone()
+    data = data[by_radius].contiguous()
+    position[:, 3] = data[:, 3]
+    return position, (None if normal is None else normal[order].contiguous()), data, order

@@ -63,12 +63,73 @@ def tile_path_model(k, N, B, C_, P_levels, V, has_dropout, lt=2):
     return k
 
 
+def bench_preprocess(args):
+    """Point-cloud preprocessing (the caller side of the path): 4th-nearest-neighbour distance and Morton codes of the
+    config-3 cloud in random order.  One step = both kernels' chains on all points."""
+    import numpy as np
+    import torch
+    from adop_amd import preprocess, scenes
+
+    t0 = time.time()
+    hs = scenes.config3(point_order="random", **({"n": args.points} if args.points else {}))
+    gen_s = time.time() - t0
+    N = hs.num_points
+    pos = torch.from_numpy(hs.position).cuda()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    for _ in range(max(args.warmup, 1)):
+        preprocess.KNearestNeighbourDistance(pos, 4)
+        preprocess.MortonCodes(pos)
+    torch.cuda.synchronize()
+    t_knn = t_mor = 0.0
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        ev[0].record()
+        preprocess.KNearestNeighbourDistance(pos, 4)
+        ev[1].record()
+        preprocess.MortonCodes(pos)
+        ev[2].record()
+        torch.cuda.synchronize()
+        t_knn += ev[0].elapsed_time(ev[1])
+        t_mor += ev[1].elapsed_time(ev[2])
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    t_knn /= args.steps
+    t_mor /= args.steps
+    # algorithmic bytes of the neighbour search: the cloud is read twice and written once in cell order (binning),
+    # read once more by the search, 4 bytes per point out; neighbours are read through the caches
+    knn_bytes = N * (16 + 16 + 16 + 16 + 4)
+    cpu = None
+    if not args.no_cpu_baseline:
+        import oracle.preprocess as op
+        m = args.cpu_points or 20000
+        tc0 = time.perf_counter()
+        op.knn_distance(hs.position[:m], 4)
+        op.morton_codes(hs.position[:m])
+        sec = time.perf_counter() - tc0
+        cpu = {"value": m / sec, "unit": "points/s", "cores": 1, "kind": "port",
+               "sample": f"brute-force neighbour search among the first {m} of {N} points + their Morton codes",
+               "seconds": round(sec, 3)}
+    print(json.dumps({
+        "metric": "preprocess points/s", "value": N / (ms_per_step * 1e-3), "unit": "points/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"preprocess: 4th-nearest-neighbour distance + Morton codes, {N} points of config3 in "
+                               "random order"},
+        "roofline": {"bound": "hbm", "kernel": "knn_search_kernel", "stage": "knn_distance",
+                     "achieved": round(knn_bytes / (t_knn * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(knn_bytes / (t_knn * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel_ms": round(t_knn, 4), "algorithmic_bytes": int(knn_bytes)},
+        "cpu_baseline": cpu,
+        "step": {"stage_ms": {"knn_distance": round(t_knn, 4), "morton_codes": round(t_mor, 4)},
+                 "scene_gen_s": round(gen_s, 1)},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="config3", choices=["config2", "config3", "config4", "config5"])
+    ap.add_argument("--workload", default="config3", choices=["config2", "config3", "config4", "config5", "preprocess"])
     ap.add_argument("--points", type=int, default=0, help="override the point count (0 = the configuration's)")
     ap.add_argument("--point-order", default="morton", choices=["morton", "random"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -93,6 +154,9 @@ def main():
     lib = _capi.load_library()
     dev = "cuda:0"
     torch.cuda.set_device(0)
+    if args.workload == "preprocess":
+        bench_preprocess(args)
+        return
 
     t0 = time.time()
     kw = {"n": args.points} if args.points else {}

@@ -203,6 +203,22 @@ adop_status adop_env_sample_backward(const adop_scene* scene, const adop_view* v
  * tangent = 0; f64. tangent [F,6], poses_se3 [F,8]. */
 adop_status adop_apply_tangent(double* tangent, double* poses_se3, int32_t num_poses, void* hip_stream);
 
+/* Point-cloud preprocessing (the rasterizer's speed depends on it: the LOD radius of every point and the order of
+ * the cloud).  Replaces the host-side kd-tree search of SceneData::ComputeRadius (SceneData.cpp:441-484):
+ * out_distance[i] = distance from point i to its `rank`-th nearest other point (the reference asks its tree for the
+ * rank + 1 nearest, which include the point itself, and takes the last; rank = 4 there, 1..8 here), computed as
+ * sqrt((dx*dx + dy*dy) + dz*dz) in fp32.  position [N,4] f32 (xyz used), N > rank; bbox_min / bbox_max: host
+ * float[3], the bounding box of the cloud. */
+size_t adop_knn_workspace_size(int32_t num_points);
+adop_status adop_knn_distance(const float* position, int32_t num_points, int32_t rank, const float* bbox_min,
+                              const float* bbox_max, float* out_distance, void* workspace, size_t workspace_bytes,
+                              void* hip_stream);
+
+/* The sort key of PointCloud::ReorderMorton64 (SceneData.cpp:101): out_codes[i] = 63-bit Morton code of point i, 21
+ * bits per axis of its position inside the bounding box (x in the lowest bit).  position [N,4] f32, out_codes [N] u64. */
+adop_status adop_morton_codes(const float* position, int32_t num_points, const float* bbox_min, const float* bbox_max,
+                              uint64_t* out_codes, void* hip_stream);
+
 /* Stage timers.  The reference wraps each stage in SAIGA_OPTIONAL_TIME_MEASURE(name, info->timer_system)
  * (PointRenderer.cu:906,913,919,1095,1414,1430,1447,1565,1594,1602,1610); here HIP events are recorded on the
  * caller's stream around each stage while profiling is enabled on the calling thread.  Stage names are the
