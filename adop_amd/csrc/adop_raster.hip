@@ -225,6 +225,7 @@ adop_status validate(const adop_scene* s, const adop_view* views, int B, const a
     if (fb->num_layers < 1 || fb->num_layers > ADOP_MAX_LAYERS)
         return fail(ADOP_UNSUPPORTED_LAYERS, "invalid number of layers");  // :1199
     if (s->num_points < 0 || !s->position || !s->index) return fail(ADOP_INVALID_ARG, "point cloud missing");
+    if (s->num_points > (1 << 30)) return fail(ADOP_INVALID_ARG, "at most 2^30 points per call");
     if (rp->check_normal && !s->normal)
         return fail(ADOP_INVALID_ARG, "check_normal requires normals");  // NeuralScene.cpp:28
     if (s->num_channels < 1 || s->num_channels > kMaxChannels)
@@ -425,7 +426,9 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
     static const int env_path = getenv("ADOP_FORWARD_PATH") ? atoi(getenv("ADOP_FORWARD_PATH")) : 0;
     int path = params->forward_path ? params->forward_path : env_path;
     if (path < 0 || path > 2) return fail(ADOP_INVALID_ARG, "forward_path must be 0, 1 or 2");
+    // (bin offsets are 32-bit: a point has at most kTileLevels entries per view)
     const bool can_bin = scene->num_points > 0 && scene->num_points < (1 << 28) &&
+                         (size_t)kTileLevels * num_views * scene->num_points < ((size_t)1 << 32) &&
                          max_tiles(num_views, views[0].w, views[0].h) < ((size_t)1 << 24);
     // The tile path bins every projected point; a cloud with very many points per pixel is faster through the direct
     // path, whose early depth test drops most of them before they cost anything.

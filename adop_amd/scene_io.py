@@ -395,3 +395,85 @@ class SceneData:
             background=np.zeros(texture.shape[0], np.float32) if background is None else background,
             poses_se3=self.poses_se3(), intrinsics=self.intrinsics(), views=[self.view(f, scale) for f in frames],
             params=params, num_layers=num_layers, name=os.path.basename(self.scene_path))
+
+
+# ---------------------------------------------------------------------------------------------------
+# training crops
+# ---------------------------------------------------------------------------------------------------
+def RandomImageCrop(n, tries_per_crop, image_size_input, image_size_crop, prefer_border, random_translation,
+                    min_max_zoom=(1.0, 1.0), generator=None):
+    """Crop transforms for ``n`` training crops of one image -> [n,5] f32 rows (fx fy cx cy s) with fx = fy = zoom,
+    s = 0: crop pixel = zoom * image pixel + (cx, cy), the matrix the rasterizer applies after the camera intrinsics
+    (Dataset.cpp:140-160).  The arguments are those of saiga's RandomImageCrop, whose source is not part of the
+    reference; the sampling law is this module's own:
+
+      * zoom uniform in ``min_max_zoom``;
+      * the crop window lies inside the zoomed image where that is larger than the crop (otherwise it is centred);
+        without ``random_translation`` it is centred; with ``prefer_border`` the offset is drawn from a range a
+        quarter crop wider on either side and clamped, which puts more windows against the image border;
+      * of ``tries_per_crop`` candidates the one whose centre is farthest from the crops already chosen is kept.
+    """
+    g = generator if generator is not None else np.random.default_rng()
+    size_in = np.asarray(image_size_input, np.float64)
+    size_crop = np.asarray(image_size_crop, np.float64)
+    chosen, centres = [], []
+    for _ in range(n):
+        best, best_centre, best_dis = None, None, -1.0
+        for _ in range(max(1, tries_per_crop)):
+            zoom = float(g.uniform(min_max_zoom[0], min_max_zoom[1]))
+            room = size_in * zoom - size_crop  # free play of the window inside the zoomed image
+            if random_translation:
+                margin = 0.25 * size_crop if prefer_border else 0.0
+                t = g.uniform(np.minimum(0.0, room) - margin, np.maximum(0.0, room) + margin)
+                t = np.where(room > 0, np.clip(t, 0.0, np.maximum(room, 0.0)), 0.5 * room)
+            else:
+                t = 0.5 * room
+            centre = (t + 0.5 * size_crop) / zoom  # in pixels of the input image
+            dis = min((float(np.linalg.norm(centre - c)) for c in centres), default=0.0)
+            if dis > best_dis:
+                best, best_centre, best_dis = (zoom, zoom, -t[0], -t[1], 0.0), centre, dis
+        chosen.append(best)
+        centres.append(best_centre)
+    return np.array(chosen, np.float32).reshape(n, 5)
+
+
+class SceneDataTrainSampler:
+    """The geometry side of SceneDataTrainSampler (Dataset.cpp:37-227): for a frame, ``inner_batch_size`` views of
+    ``crop_size`` with random crop transforms (``down_scale``) or the full image.  Target images, uv images and
+    masks belong to the loss and are not produced here."""
+
+    def __init__(self, scene, indices, down_scale, crop_size, inner_batch_size, seed=0):
+        self.scene, self.indices, self.down_scale = scene, list(indices), bool(down_scale)
+        self.inner_batch_size = int(inner_batch_size)
+        self.image_size_input = [(c.w, c.h) for c in scene.scene_cameras]
+        if down_scale:
+            assert crop_size[0] > 0
+        self.image_size_crop = [tuple(crop_size) if down_scale else (c.w, c.h) for c in scene.scene_cameras]
+        # Dataset.h:54-60
+        self.random_translation, self.prefere_border, self.inner_sample_size = True, True, 1
+        self.min_max_zoom = (0.75, 1.5)
+        self.generator = np.random.default_rng(seed)
+
+    def __len__(self):
+        return len(self.indices)
+
+    def Get(self, index):
+        """-> (views, zoom): ``inner_batch_size`` adop views of frame ``indices[index]`` and the zoom of each."""
+        actual = self.indices[index]
+        fd = self.scene.frames[actual]
+        cam = fd.camera_index
+        w, h = self.image_size_crop[cam]
+        rows = np.tile(np.float32([1, 1, 0, 0, 0]), (self.inner_batch_size, 1))
+        if self.down_scale:
+            rows = RandomImageCrop(self.inner_batch_size, self.inner_sample_size, self.image_size_input[cam],
+                                   self.image_size_crop[cam], self.prefere_border, self.random_translation,
+                                   self.min_max_zoom, self.generator)
+        views = []
+        for r in rows:
+            v = _capi.View()
+            v.w, v.h = int(w), int(h)
+            v.image_index, v.camera_index = actual, cam
+            v.camera_model_type = int(self.scene.dataset_params.camera_model)
+            v.crop_fx, v.crop_fy, v.crop_cx, v.crop_cy, v.crop_s = [float(x) for x in r]
+            views.append(v)
+        return views, rows[:, 0].copy()

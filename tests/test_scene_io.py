@@ -149,3 +149,66 @@ def test_inconsistent_scenes_are_rejected(tmp_path):
     os.remove(tmp_path / "camera1.ini")
     with pytest.raises(AssertionError, match="camera1.ini"):
         scene_io.SceneData.load(str(tmp_path))
+
+
+def window_in_image(row, crop):
+    """corners of the crop window in pixels of the input image: (crop pixel - c) / zoom"""
+    z = row[0]
+    lo = np.array([-row[2], -row[3]]) / z
+    return lo, lo + np.asarray(crop) / z
+
+
+@pytest.mark.parametrize("prefer_border", [False, True])
+def test_random_crops_stay_inside_the_image(prefer_border):
+    g = np.random.default_rng(3)
+    size_in, crop = (1920, 1080), (512, 512)
+    rows = scene_io.RandomImageCrop(400, 1, size_in, crop, prefer_border, True, (0.75, 1.5), g)
+    assert rows.shape == (400, 5) and rows.dtype == np.float32
+    np.testing.assert_array_equal(rows[:, 0], rows[:, 1])
+    assert np.all(rows[:, 4] == 0) and rows[:, 0].min() >= 0.75 and rows[:, 0].max() <= 1.5
+    assert rows[:, 0].max() - rows[:, 0].min() > 0.6  # the zoom range is used
+    touching = 0
+    for r in rows:
+        lo, hi = window_in_image(r, crop)
+        assert np.all(lo >= -1e-3) and np.all(hi <= np.array(size_in) + 1e-3), (r, lo, hi)
+        touching += bool(np.any(lo < 1e-3) or np.any(hi > np.array(size_in) - 1e-3))
+    # clamping a wider range puts many windows against the border; a plain uniform offset almost none
+    assert (touching > 100) if prefer_border else (touching < 20)
+
+
+def test_crops_without_translation_and_small_images_are_centred():
+    rows = scene_io.RandomImageCrop(5, 1, (640, 480), (256, 128), True, False, (1.0, 1.0), np.random.default_rng(0))
+    np.testing.assert_array_equal(rows, np.tile(np.float32([1, 1, -192, -176, 0]), (5, 1)))
+    # the zoomed image (160 x 120) is smaller than the crop: centred, cx > 0
+    rows = scene_io.RandomImageCrop(3, 2, (640, 480), (256, 128), True, True, (0.25, 0.25), np.random.default_rng(0))
+    np.testing.assert_array_equal(rows, np.tile(np.float32([0.25, 0.25, 48, 4, 0]), (3, 1)))
+
+
+def test_more_tries_spread_the_crops():
+    def mean_nearest(tries):
+        out = []
+        for seed in range(20):
+            rows = scene_io.RandomImageCrop(8, tries, (1920, 1080), (256, 256), False, True, (1, 1),
+                                            np.random.default_rng(seed))
+            c = (-rows[:, 2:4] + 128) / rows[:, :1]
+            d = np.linalg.norm(c[:, None] - c[None], axis=2) + 1e9 * np.eye(8)
+            out.append(d.min(1).mean())
+        return np.mean(out)
+
+    assert mean_nearest(8) > 1.3 * mean_nearest(1)
+
+
+def test_train_sampler_views(tmp_path):
+    hand_written_scene(tmp_path)
+    sd = scene_io.SceneData.load(str(tmp_path))
+    sampler = scene_io.SceneDataTrainSampler(sd, [2, 1], True, (256, 192), 4, seed=1)
+    assert len(sampler) == 2
+    views, zoom = sampler.Get(1)
+    assert len(views) == 4 and zoom.shape == (4,)
+    for v, z in zip(views, zoom):
+        assert (v.w, v.h, v.image_index, v.camera_index, v.crop_s) == (256, 192, 1, 1, 0.0)
+        assert v.crop_fx == v.crop_fy == z and 0.75 <= z <= 1.5
+    full = scene_io.SceneDataTrainSampler(sd, [0], False, (0, 0), 2)
+    views, zoom = full.Get(0)
+    assert [(v.w, v.h, v.crop_fx, v.crop_cx, v.crop_cy) for v in views] == [(640, 480, 1.0, 0.0, 0.0)] * 2
+    assert list(zoom) == [1.0, 1.0]

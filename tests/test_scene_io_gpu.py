@@ -38,3 +38,35 @@ def test_scene_from_disk_renders_like_its_source(oracle_mod, tmp_path):
     want = download_forward(src, info, images, masks)
     for a, b in zip(got.out, want.out):  # poses differ by a double rounding: all but a stray pixel agree
         assert np.mean(a != b) < 1e-3
+
+
+@pytest.mark.parametrize("forward_path", [1, 2], ids=["direct", "tiles"])
+def test_crop_view_is_a_window_of_the_full_render(forward_path):
+    """A crop transform with zoom 1 and an offset that is a multiple of 2^(levels-1) pixels shifts every level by whole
+    pixels (the subtraction is exact in fp32 for the points inside the window), so the crop renders exactly the
+    window of the full image: packed depth and depth bit for bit, weights equal, descriptors to summation order."""
+    from adop_amd import scenes
+
+    n, w, h, levels = 80000, 256, 192, 4
+    ox, oy, cw, ch = 64, 40, 128, 96
+    full = scenes.config2(n=n, w=w, h=h, levels=levels, batch=1, seed=2, ghost=False)
+    full.params.forward_path = forward_path
+    crop = scenes.config2(n=n, w=w, h=h, levels=levels, batch=1, seed=2, ghost=False)
+    crop.params.forward_path = forward_path
+    crop.views = [scenes.make_view(cw, ch, crop=(1.0, 1.0, -float(ox), -float(oy), 0.0))]
+    announce(f"crop window {cw}x{ch}+{ox}+{oy} of {w}x{h}, N={n} L={levels} forward_path={forward_path}")
+    scene, info, ctx, images, masks = run_hip_forward(full)
+    F = download_forward(full, info, images, masks)
+    scene, info, ctx, images, masks = run_hip_forward(crop)
+    G = download_forward(crop, info, images, masks)
+    ids = (1 << 32) - 1
+    for l in range(levels):
+        x0, y0 = ox >> l, oy >> l
+        win = (slice(None), slice(None), slice(y0, y0 + (ch >> l)), slice(x0, x0 + (cw >> l)))
+        # the same depth wins; where two points tie in depth the id breaks the tie the same way
+        assert np.array_equal(G.depth_index[l], F.depth_index[l][win]), l
+        assert np.array_equal(G.depth[l].view(np.uint32), F.depth[l][win].view(np.uint32)), l
+        assert np.array_equal(G.weight[l], F.weight[l][win]), l
+        assert (G.depth_index[l] & ids != ids).mean() > 0.3  # the window is not empty
+        a, b = G.out[l], F.out[l][win]
+        assert np.abs(a - b).max() <= 1e-5 * max(1.0, np.abs(b).max()), l
