@@ -157,6 +157,16 @@ ENTRY_POINTS = {
         C.c_int,
         [C.c_void_p, C.c_int32, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_void_p, C.c_void_p],
     ),
+    "adop_frames_workspace_size": (C.c_size_t, [C.c_int32]),
+    "adop_point_distance_to_camera": (
+        C.c_int,
+        [C.POINTER(Scene), C.POINTER(View), C.c_int32, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p],
+    ),
+    "adop_close_points": (
+        C.c_int,
+        [C.c_void_p, C.c_int32, C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_void_p, C.c_void_p,
+         C.c_int32, C.c_int32, C.c_void_p, C.c_size_t, C.c_void_p],
+    ),
     "adop_profile_enable": (C.c_int, [C.c_int32]),
     "adop_profile_read": (C.c_int32, [C.POINTER(StageTime), C.c_int32]),
     "adop_last_error_string": (C.c_char_p, []),

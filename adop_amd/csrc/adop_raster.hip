@@ -722,13 +722,18 @@ size_t adop_knn_workspace_size(int32_t num_points)
     return o;
 }
 
-adop_status adop_knn_distance(const float* position, int32_t num_points, int32_t rank, const float* bbox_min,
-                              const float* bbox_max, float* out_distance, void* workspace, size_t workspace_bytes,
-                              void* hip_stream)
+// The grid of a cloud (a function of the bounding box and the number of points only) and, with `bin`, the points in
+// cell order in the workspace: count [cells], offset [cells + 1], sorted [N].
+struct KnnWorkspace
 {
-    if (!position || !bbox_min || !bbox_max || !out_distance) return fail(ADOP_INVALID_ARG, "null argument");
-    if (rank < 1 || rank > 8) return fail(ADOP_INVALID_ARG, "rank must be 1..8");
-    if (num_points <= rank) return fail(ADOP_INVALID_ARG, "the cloud needs more than `rank` points");
+    KnnGrid g;
+    uint32_t *count, *offset;
+    float4* sorted;
+};
+
+static adop_status knn_prepare(const float* position, int32_t num_points, const float* bbox_min, const float* bbox_max,
+                               void* workspace, size_t workspace_bytes, bool bin, hipStream_t stream, KnnWorkspace* out)
+{
     if (!workspace || workspace_bytes < adop_knn_workspace_size(num_points))
         return fail(ADOP_WORKSPACE_TOO_SMALL, "workspace too small");
     float ext[3];
@@ -737,7 +742,7 @@ adop_status adop_knn_distance(const float* position, int32_t num_points, int32_t
         ext[k] = bbox_max[k] - bbox_min[k];
         if (!(ext[k] >= 0) || !(ext[k] < 1.0e30f)) return fail(ADOP_INVALID_ARG, "bounding box is not finite");
     }
-    KnnGrid g;
+    KnnGrid& g          = out->g;
     const float longest = ext[0] > ext[1] ? (ext[0] > ext[2] ? ext[0] : ext[2]) : (ext[1] > ext[2] ? ext[1] : ext[2]);
     double volume       = 1.0;
     for (int k = 0; k < 3; ++k) volume *= ext[k] > 1e-6f * longest ? ext[k] : (longest > 0 ? 1e-6 * longest : 1.0);
@@ -753,21 +758,93 @@ adop_status adop_knn_distance(const float* position, int32_t num_points, int32_t
         g.dim[k] = d < 1 ? 1 : (d > kKnnMaxDim ? kKnnMaxDim : d);
     }
     const size_t cells = (size_t)g.dim[0] * g.dim[1] * g.dim[2];
-    hipStream_t stream = (hipStream_t)hip_stream;
-    uint32_t* count    = (uint32_t*)workspace;
-    uint32_t* offset   = (uint32_t*)((char*)workspace + align_up(sizeof(uint32_t) * knn_cells_max(), 256));
-    float4* sorted     = (float4*)((char*)offset + align_up(sizeof(uint32_t) * (knn_cells_max() + 1), 256));
-    adop_status st     = fill_async(count, sizeof(uint32_t) * cells, 0, stream);
+    out->count         = (uint32_t*)workspace;
+    out->offset        = (uint32_t*)((char*)workspace + align_up(sizeof(uint32_t) * knn_cells_max(), 256));
+    out->sorted        = (float4*)((char*)out->offset + align_up(sizeof(uint32_t) * (knn_cells_max() + 1), 256));
+    if (!bin) return ADOP_OK;
+    adop_status st = fill_async(out->count, sizeof(uint32_t) * cells, 0, stream);
     if (st != ADOP_OK) return st;
-    launch_knn_bin(0, (const float4*)position, num_points, g, count, offset, sorted, stream);
+    launch_knn_bin(0, (const float4*)position, num_points, g, out->count, out->offset, out->sorted, stream);
     BinArg scan;
     memset(&scan, 0, sizeof(scan));
-    scan.count  = count;
-    scan.offset = offset;
+    scan.count  = out->count;
+    scan.offset = out->offset;
     launch_tile_scan(scan, (int)cells, stream);
-    launch_knn_bin(1, (const float4*)position, num_points, g, count, offset, sorted, stream);
-    if (!launch_knn_search(rank, sorted, num_points, g, offset, out_distance, stream))
+    launch_knn_bin(1, (const float4*)position, num_points, g, out->count, out->offset, out->sorted, stream);
+    return ADOP_OK;
+}
+
+adop_status adop_knn_distance(const float* position, int32_t num_points, int32_t rank, const float* bbox_min,
+                              const float* bbox_max, float* out_distance, void* workspace, size_t workspace_bytes,
+                              void* hip_stream)
+{
+    if (!position || !bbox_min || !bbox_max || !out_distance) return fail(ADOP_INVALID_ARG, "null argument");
+    if (rank < 1 || rank > 8) return fail(ADOP_INVALID_ARG, "rank must be 1..8");
+    if (num_points <= rank) return fail(ADOP_INVALID_ARG, "the cloud needs more than `rank` points");
+    hipStream_t stream = (hipStream_t)hip_stream;
+    KnnWorkspace w;
+    adop_status st = knn_prepare(position, num_points, bbox_min, bbox_max, workspace, workspace_bytes, true, stream, &w);
+    if (st != ADOP_OK) return st;
+    if (!launch_knn_search(rank, w.sorted, num_points, w.g, w.offset, out_distance, stream))
         return fail(ADOP_INVALID_ARG, "rank must be 1..8");
+    ADOP_HIP_CHECK(hipGetLastError());
+    return ADOP_OK;
+}
+
+adop_status adop_close_points(const float* position, int32_t num_points, const float* radius, const float* bbox_min,
+                              const float* bbox_max, int32_t* state, uint32_t* round_undecided, int32_t num_rounds,
+                              int32_t resume, void* workspace, size_t workspace_bytes, void* hip_stream)
+{
+    if (!position || !radius || !bbox_min || !bbox_max || !state || !round_undecided)
+        return fail(ADOP_INVALID_ARG, "null argument");
+    if (num_points < 1) return fail(ADOP_INVALID_ARG, "empty cloud");
+    if (num_rounds < 1 || num_rounds > 1024) return fail(ADOP_INVALID_ARG, "num_rounds must be 1..1024");
+    hipStream_t stream = (hipStream_t)hip_stream;
+    KnnWorkspace w;
+    adop_status st =
+        knn_prepare(position, num_points, bbox_min, bbox_max, workspace, workspace_bytes, !resume, stream, &w);
+    if (st != ADOP_OK) return st;
+    if (!resume && (st = fill_async(state, sizeof(int32_t) * (size_t)num_points, 0, stream)) != ADOP_OK) return st;
+    if ((st = fill_async(round_undecided, sizeof(uint32_t) * (size_t)num_rounds, 0, stream)) != ADOP_OK) return st;
+    for (int r = 0; r < num_rounds; ++r)
+        launch_close_points(w.sorted, num_points, w.g, w.offset, radius, state, round_undecided, r, stream);
+    ADOP_HIP_CHECK(hipGetLastError());
+    return ADOP_OK;
+}
+
+size_t adop_frames_workspace_size(int32_t num_frames)
+{
+    return num_frames < 1 ? 0 : align_up(sizeof(ViewConst) * (size_t)num_frames, 256);
+}
+
+adop_status adop_point_distance_to_camera(const adop_scene* scene, const adop_view* frames, int32_t num_frames,
+                                          float* out_distance, void* workspace, size_t workspace_bytes,
+                                          void* hip_stream)
+{
+    if (!scene || !frames || !out_distance) return fail(ADOP_INVALID_ARG, "null argument");
+    if (num_frames < 1) return fail(ADOP_INVALID_ARG, "num_frames must be >= 1");
+    if (scene->num_points < 0 || !scene->position) return fail(ADOP_INVALID_ARG, "point cloud missing");
+    if (!scene->poses_se3 || !scene->intrinsics || scene->num_poses < 1 || scene->num_cameras < 1)
+        return fail(ADOP_INVALID_ARG, "poses / intrinsics missing");
+    if (scene->intrinsics_cols != 13) return fail(ADOP_INVALID_ARG, "pinhole intrinsics need 13 columns");
+    for (int f = 0; f < num_frames; ++f)
+    {
+        const adop_view& v = frames[f];
+        // FrameData::Project3 (SceneData.cpp:26-34) is the pinhole + distortion model
+        if (v.camera_model_type != ADOP_CAMERA_PINHOLE_DISTORTION)
+            return fail(ADOP_INVALID_ARG, "the camera distance needs the pinhole model");
+        if (v.image_index < 0 || v.image_index >= scene->num_poses || v.camera_index < 0 ||
+            v.camera_index >= scene->num_cameras || v.w < 1 || v.h < 1)
+            return fail(ADOP_INVALID_ARG, "frame out of range");
+    }
+    if (!workspace || workspace_bytes < adop_frames_workspace_size(num_frames))
+        return fail(ADOP_WORKSPACE_TOO_SMALL, "workspace too small");
+    if (scene->num_points == 0) return ADOP_OK;
+    hipStream_t stream = (hipStream_t)hip_stream;
+    ViewConst* dviews  = (ViewConst*)workspace;
+    adop_status st     = upload_views(scene, frames, num_frames, dviews, stream);
+    if (st != ADOP_OK) return st;
+    launch_camera_distance((const float4*)scene->position, scene->num_points, dviews, num_frames, out_distance, stream);
     ADOP_HIP_CHECK(hipGetLastError());
     return ADOP_OK;
 }

@@ -20,6 +20,10 @@ void launch_knn_bin(int pass, const float4* position, int n, const KnnGrid& g, u
                     float4* sorted, hipStream_t st);
 bool launch_knn_search(int rank, const float4* sorted, int n, const KnnGrid& g, const uint32_t* offset, float* out,
                        hipStream_t st);
+void launch_camera_distance(const float4* position, int n, const ViewConst* views, int num_frames, float* out,
+                            hipStream_t st);
+void launch_close_points(const float4* sorted, int n, const KnnGrid& g, const uint32_t* offset, const float* radius,
+                         int32_t* state, uint32_t* round_count, int round, hipStream_t st);
 void launch_morton(const float4* position, int n, const float* mn, const float* scale, unsigned long long* code,
                    hipStream_t st);
 int prepass_points_per_block();  // points per workgroup of prepass_kernel (the unit of its candidate lists)

@@ -106,6 +106,97 @@ __global__ __launch_bounds__(kBlock) void knn_search_kernel(const float4* __rest
     out[__float_as_uint(p.w)] = sqrtf(best[K - 1]);
 }
 
+// SceneData::PointDistanceToCamera (SceneData.cpp:645-669): distance from every point to the nearest camera that sees
+// it (in front of the camera, projected inside the image with the frame's pinhole + distortion model), 10258.4 (the
+// root of the reference's start value 105235545) where no frame does.  The distance is taken in camera space
+// (|V p| = |p - c| for the camera centre c).  The frames are read through uniform loads.
+__global__ __launch_bounds__(kBlock) void camera_distance_kernel(const float4* __restrict__ position, int n,
+                                                                 const ViewConst* __restrict__ views, int num_frames,
+                                                                 float* __restrict__ out)
+{
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const float4 P = nt_load4(position + i);
+    const V3 pos   = {P.x, P.y, P.z};
+    float best     = 105235545.f;
+    for (int f = 0; f < num_frames; ++f)
+    {
+        const ViewConst& vc = views[f];
+        const V3 r          = quat_rotate(vc.qx, vc.qy, vc.qz, vc.qw, pos);
+        const V3 v          = {r.x + vc.tx, r.y + vc.ty, r.z + vc.tz};
+        if (!(v.z > 0.f)) continue;
+        const V2 np   = {v.x / v.z, v.y / v.z};
+        const V2 dp   = distort<false>(np, vc.d, 3.0e38f, nullptr, nullptr);
+        const V2 ip   = k_apply(vc.k, dp);
+        const bool in = ip.x >= 0.f && ip.y >= 0.f && ip.x < (float)vc.w && ip.y < (float)vc.h;
+        const float d = (v.x * v.x + v.y * v.y) + v.z * v.z;
+        if (in && d < best) best = d;
+    }
+    out[i] = sqrtf(best);
+}
+
+// SceneData::RemoveClosePoints (SceneData.cpp:598-642) walks the points in order and erases point i when a point it
+// has kept before lies within radius[i] of it: state[i] = kept unless a kept j < i is that close.  Here the points
+// are decided in rounds: a point whose earlier neighbours are all decided is decided; states only ever go from
+// undecided to kept / erased, so reading a neighbour's state of this round instead of the last one is as good.
+// One thread per point in cell order; count[round] receives the points still undecided after this round, and a round
+// that finds count[round - 1] == 0 has nothing to do.
+constexpr int kStateUndecided = 0, kStateKept = 1, kStateErased = 2;
+
+__global__ __launch_bounds__(kBlock) void close_points_kernel(const float4* __restrict__ sorted, int n, KnnGrid g,
+                                                              const uint32_t* __restrict__ offset,
+                                                              const float* __restrict__ radius, int32_t* state,
+                                                              uint32_t* round_count, int round)
+{
+    if (round > 0 && *(volatile uint32_t*)(round_count + round - 1) == 0) return;
+    const int t = blockIdx.x * kBlock + threadIdx.x;
+    bool pending = false;
+    if (t < n)
+    {
+        const float4 p   = sorted[t];
+        const uint32_t i = __float_as_uint(p.w);
+        if (__atomic_load_n(&state[i], __ATOMIC_RELAXED) == kStateUndecided)
+        {
+            const float rad = radius[i];
+            const float r2  = rad * rad;
+            const int3 c    = grid_cell(g, p.x, p.y, p.z);
+            // cells the ball can reach (the cell of a point is computed in fp32: one cell of slack)
+            const float reach = fminf(fmaxf(rad, 0.f) * g.inv_cell, 1.0e6f);
+            const int rc      = (int)reach + 1;
+            const int z0 = max(c.z - rc, 0), z1 = min(c.z + rc, g.dim[2] - 1);
+            const int y0 = max(c.y - rc, 0), y1 = min(c.y + rc, g.dim[1] - 1);
+            const int x0 = max(c.x - rc, 0), x1 = min(c.x + rc, g.dim[0] - 1);
+            int result = kStateKept;
+            for (int cz = z0; cz <= z1 && result != kStateErased; ++cz)
+                for (int cy = y0; cy <= y1 && result != kStateErased; ++cy)
+                {
+                    const uint32_t row = grid_index(g, 0, cy, cz);
+                    const uint32_t e   = offset[row + x1 + 1];
+                    for (uint32_t q = offset[row + x0]; q < e; ++q)
+                    {
+                        const float4 o   = sorted[q];
+                        const uint32_t j = __float_as_uint(o.w);
+                        if (j >= i) continue;
+                        const float dx = p.x - o.x, dy = p.y - o.y, dz = p.z - o.z;
+                        const float d2 = (dx * dx + dy * dy) + dz * dz;
+                        if (!(d2 < r2)) continue;
+                        const int sj = __atomic_load_n(&state[j], __ATOMIC_RELAXED);
+                        if (sj == kStateKept)
+                        {
+                            result = kStateErased;
+                            break;
+                        }
+                        if (sj == kStateUndecided) result = kStateUndecided;
+                    }
+                }
+            if (result != kStateUndecided) __atomic_store_n(&state[i], result, __ATOMIC_RELAXED);
+            pending = result == kStateUndecided;
+        }
+    }
+    const unsigned long long m = __ballot(pending);
+    if (m && (threadIdx.x & 63) == (__ffsll((long long)m) - 1)) atomicAdd(round_count + round, (uint32_t)__popcll(m));
+}
+
 // Morton code of every point: 21 bits per axis of the position inside the bounding box, x in the lowest bit.
 __device__ __forceinline__ unsigned long long spread21(unsigned long long v)
 {
@@ -158,6 +249,20 @@ bool launch_knn_search(int rank, const float4* sorted, int n, const KnnGrid& g, 
         case 8: hipLaunchKernelGGL(knn_search_kernel<9>, grid, block, 0, st, sorted, n, g, offset, out); return true;
     }
     return false;
+}
+
+void launch_camera_distance(const float4* position, int n, const ViewConst* views, int num_frames, float* out,
+                            hipStream_t st)
+{
+    hipLaunchKernelGGL(camera_distance_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, position, n, views,
+                       num_frames, out);
+}
+
+void launch_close_points(const float4* sorted, int n, const KnnGrid& g, const uint32_t* offset, const float* radius,
+                         int32_t* state, uint32_t* round_count, int round, hipStream_t st)
+{
+    hipLaunchKernelGGL(close_points_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, sorted, n, g, offset,
+                       radius, state, round_count, round);
 }
 
 void launch_morton(const float4* position, int n, const float* mn, const float* scale, unsigned long long* code,

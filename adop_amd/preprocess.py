@@ -1,9 +1,10 @@
-"""Point-cloud preprocessing of SceneData (data/SceneData.cpp:96-118) on the device: Morton order, shuffled
-256-point blocks, the radius of every point from its 4th nearest neighbour, blocks sorted by radius.
+"""Point-cloud preprocessing of SceneData (data/SceneData.cpp:96-118) on the device: the filters for lonely and
+close points, Morton order, shuffled 256-point blocks, the radius of every point from its 4th nearest neighbour,
+blocks sorted by radius.
 
 The order of the cloud and the radii decide how the rasterizer runs (coherent wavefronts, the LOD early exit), so the
 steps sit next to it.  The distance search and the Morton codes are HIP kernels behind the C-ABI
-(``adop_knn_distance``, ``adop_morton_codes``); sorting and permuting go through torch.
+(``adop_knn_distance``, ``adop_morton_codes``, ``adop_point_distance_to_camera``, ``adop_close_points``); sorting and permuting go through torch.
 """
 import ctypes as C
 
@@ -46,6 +47,69 @@ def MortonCodes(position):
     rc = lib.adop_morton_codes(C.c_void_p(position.data_ptr()), n, mn, mx, C.c_void_p(codes.data_ptr()), _stream_ptr())
     _check(rc, lib)
     return codes
+
+
+def PointDistanceToCamera(position, poses_se3, intrinsics, frames):
+    """SceneData::PointDistanceToCamera (SceneData.cpp:645-669): distance of every point to the nearest camera that
+    sees it.  position [N,4] f32, poses_se3 [F,8] f64 (view transforms), intrinsics [K,13] f32 on the device;
+    ``frames``: one adop view per frame (w, h, image_index, camera_index)."""
+    assert position.is_cuda and position.dtype == torch.float32 and position.dim() == 2 and position.shape[1] == 4
+    assert poses_se3.is_cuda and poses_se3.dtype == torch.float64 and poses_se3.shape[1] == 8
+    assert intrinsics.is_cuda and intrinsics.dtype == torch.float32 and intrinsics.shape[1] == 13
+    position, poses_se3, intrinsics = position.contiguous(), poses_se3.contiguous(), intrinsics.contiguous()
+    lib = _capi.load_library()
+    s = _capi.Scene()
+    s.position, s.num_points = position.data_ptr(), int(position.shape[0])
+    s.poses_se3, s.num_poses = poses_se3.data_ptr(), int(poses_se3.shape[0])
+    s.intrinsics, s.num_cameras, s.intrinsics_cols = intrinsics.data_ptr(), int(intrinsics.shape[0]), 13
+    views = (_capi.View * len(frames))(*frames)
+    out = torch.empty(s.num_points, dtype=torch.float32, device=position.device)
+    ws = torch.empty(int(lib.adop_frames_workspace_size(len(frames))), dtype=torch.uint8, device=position.device)
+    rc = lib.adop_point_distance_to_camera(C.byref(s), views, len(frames), C.c_void_p(out.data_ptr()),
+                                           C.c_void_p(ws.data_ptr()), int(ws.numel()), _stream_ptr())
+    _check(rc, lib)
+    return out
+
+
+def RemoveLonelyPoints(position, camera_distance, n=5, dis_th=0.02):
+    """Keep mask of SceneData::RemoveLonelyPoints (SceneData.cpp:550-595): a point goes when the distance to its
+    n-th nearest neighbour, relative to its camera distance, exceeds ``dis_th``."""
+    d = KNearestNeighbourDistance(position, n)
+    return ~(d / camera_distance > dis_th)
+
+
+def RemoveClosePoints(position, camera_distance, dis_th=0.00005, rounds_per_call=8):
+    """Keep mask of SceneData::RemoveClosePoints (SceneData.cpp:598-642): in index order, a point goes when a point
+    kept before it lies within dis_th / camera_distance of it."""
+    assert position.is_cuda and position.dtype == torch.float32 and position.dim() == 2 and position.shape[1] == 4
+    position = position.contiguous()
+    n = int(position.shape[0])
+    radius = (dis_th / camera_distance).to(torch.float32).contiguous()
+    lib = _capi.load_library()
+    state = torch.empty(n, dtype=torch.int32, device=position.device)
+    undecided = torch.empty(rounds_per_call, dtype=torch.int32, device=position.device)
+    ws = torch.empty(int(lib.adop_knn_workspace_size(n)), dtype=torch.uint8, device=position.device)
+    mn, mx = _bbox(position)
+    resume = 0
+    while True:
+        rc = lib.adop_close_points(C.c_void_p(position.data_ptr()), n, C.c_void_p(radius.data_ptr()), mn, mx,
+                                   C.c_void_p(state.data_ptr()), C.c_void_p(undecided.data_ptr()), rounds_per_call,
+                                   resume, C.c_void_p(ws.data_ptr()), int(ws.numel()), _stream_ptr())
+        _check(rc, lib)
+        if int(undecided[-1].item()) == 0:
+            return state == 1
+        resume = 1
+
+
+def FilterPointCloud(position, poses_se3, intrinsics, frames, lonely=(5, 0.02), close=0.00005):
+    """The two filters of a new scene in the reference's order (SceneData.cpp:98-99): RemoveLonelyPoints(5, 0.02), then
+    RemoveClosePoints(0.00005) on what is left.  Returns the ids of the surviving points, ascending."""
+    ids = torch.arange(int(position.shape[0]), device=position.device)
+    cam = PointDistanceToCamera(position, poses_se3, intrinsics, frames)  # per point: erasing others does not change it
+    keep = RemoveLonelyPoints(position, cam, *lonely)
+    position, cam, ids = position[keep].contiguous(), cam[keep], ids[keep]
+    keep = RemoveClosePoints(position, cam, close)
+    return ids[keep]
 
 
 def ReorderMorton64(position):

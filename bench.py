@@ -94,6 +94,26 @@ def bench_preprocess(args):
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     t_knn /= args.steps
     t_mor /= args.steps
+    # The point filters of a new scene (outside the timed steps): camera distance over 100 frames on an orbit, lonely
+    # points (5th neighbour), close points (0.00005 / camera distance).
+    frames = 100
+    poses = torch.from_numpy(np.stack([scenes.orbit_pose(f, radius=3.0, deg_per_frame=3.6) for f in range(frames)])).cuda()
+    intr = torch.from_numpy(hs.intrinsics).cuda()
+    fviews = [scenes.make_view(hs.views[0].w, hs.views[0].h, image_index=f) for f in range(frames)]
+    filt = {}
+    for name, fn in (("camera_distance_100_frames", lambda: preprocess.PointDistanceToCamera(pos, poses, intr, fviews)),
+                     ("lonely_points", lambda: preprocess.RemoveLonelyPoints(pos, cam, 5, 0.02)),
+                     ("close_points", lambda: preprocess.RemoveClosePoints(pos, cam, 0.00005))):
+        ts = []
+        for _ in range(3):
+            torch.cuda.synchronize()
+            tf = time.perf_counter()
+            r = fn()
+            torch.cuda.synchronize()
+            ts.append((time.perf_counter() - tf) * 1e3)
+        if name == "camera_distance_100_frames":
+            cam = r
+        filt[name] = round(sorted(ts)[1], 3)
     # algorithmic bytes of the neighbour search: the cloud is read twice and written once in cell order (binning),
     # read once more by the search, 4 bytes per point out; neighbours are read through the caches
     knn_bytes = N * (16 + 16 + 16 + 16 + 4)
@@ -120,6 +140,7 @@ def bench_preprocess(args):
                      "kernel_ms": round(t_knn, 4), "algorithmic_bytes": int(knn_bytes)},
         "cpu_baseline": cpu,
         "step": {"stage_ms": {"knn_distance": round(t_knn, 4), "morton_codes": round(t_mor, 4)},
+                 "filters_ms": filt,
                  "scene_gen_s": round(gen_s, 1)},
     }))
 

@@ -214,6 +214,26 @@ adop_status adop_knn_distance(const float* position, int32_t num_points, int32_t
                               const float* bbox_max, float* out_distance, void* workspace, size_t workspace_bytes,
                               void* hip_stream);
 
+/* Replaces SceneData::PointDistanceToCamera (SceneData.cpp:645-669): out_distance[i] = distance from point i to
+ * the nearest camera that sees it (z > 0 and the projection through the frame's pinhole + distortion model,
+ * FrameData::Project3 :26-34, inside [0,w) x [0,h)); sqrt(105235545) where no frame does.  `frames`: one adop_view
+ * per frame (w, h, image_index, camera_index; the crop transform is not used); scene: position, poses_se3,
+ * intrinsics [K,13].  Workspace: adop_frames_workspace_size(num_frames) bytes. */
+size_t adop_frames_workspace_size(int32_t num_frames);
+adop_status adop_point_distance_to_camera(const adop_scene* scene, const adop_view* frames, int32_t num_frames,
+                                          float* out_distance, void* workspace, size_t workspace_bytes,
+                                          void* hip_stream);
+
+/* Replaces the sequential sweep of SceneData::RemoveClosePoints (SceneData.cpp:598-642): state[i] = 2 (erased) when a
+ * point j < i with state[j] = 1 (kept) lies closer than radius[i] (d2 < radius^2 in fp32), else 1; the result equals
+ * the sweep in index order.  The points are decided in rounds (a point waits for its earlier neighbours):
+ * round_undecided [num_rounds] (device) receives the number of points still 0 (undecided) after every round; when
+ * the last entry is not 0 call again with resume = 1 and the workspace untouched.  state [N] int32 (device),
+ * radius [N] f32, workspace: adop_knn_workspace_size(num_points) bytes. */
+adop_status adop_close_points(const float* position, int32_t num_points, const float* radius, const float* bbox_min,
+                              const float* bbox_max, int32_t* state, uint32_t* round_undecided, int32_t num_rounds,
+                              int32_t resume, void* workspace, size_t workspace_bytes, void* hip_stream);
+
 /* The sort key of PointCloud::ReorderMorton64 (SceneData.cpp:101): out_codes[i] = 63-bit Morton code of point i, 21
  * bits per axis of its position inside the bounding box (x in the lowest bit).  position [N,4] f32, out_codes [N] u64. */
 adop_status adop_morton_codes(const float* position, int32_t num_points, const float* bbox_min, const float* bbox_max,

@@ -112,3 +112,112 @@ def test_knn_distance_two_million_points_against_kdtree_sample():
     sample = g.integers(0, n, 3000)
     want = tree.query(xyz[sample].astype(np.float64), k=5)[0][:, 4]
     assert np.allclose(got[sample], want, rtol=2e-6, atol=1e-9)
+
+
+def _orbit_scene(n, frames, seed):
+    """A Gaussian cloud and `frames` cameras on a sphere looking at it, two camera models (one with distortion)."""
+    from adop_amd import scene_io, scenes
+
+    g = np.random.default_rng(seed)
+    p = np.zeros((n, 4), np.float32)
+    p[:, :3] = g.standard_normal((n, 3)) * 0.7
+    views = np.stack([scenes.look_at_view(g.uniform(1.5, 3.0) * d / np.linalg.norm(d)) for d in g.standard_normal((frames, 3))])
+    poses = np.stack([scene_io.invert_pose(v[:7]) for v in views])  # camera -> world, as in poses.txt
+    K = np.stack([scenes.pinhole_row(300, 300, 160, 120), scenes.pinhole_row(250, 260, 150, 110, 0.5,
+                 [0.1, -0.05, 0.01, 0.02, 0.0, 0.0, 0.002, -0.001])])
+    fr = [(320, 240, f, f % 2) for f in range(frames)]
+    return p, views, poses, K, fr
+
+
+def test_point_distance_to_camera():
+    import torch
+    import oracle.preprocess as op
+    from adop_amd import preprocess, scenes
+
+    p, views, poses, K, fr = _orbit_scene(20000, 37, 1)  # more frames than one chunk of view constants
+    announce("camera distance: N=20000, 37 frames, 2 cameras")
+    want = op.point_distance_to_camera(p, poses, K, fr)
+    got = preprocess.PointDistanceToCamera(torch.from_numpy(p).cuda(), torch.from_numpy(views).cuda(),
+                                           torch.from_numpy(K).cuda(),
+                                           [scenes.make_view(w, h, image_index=f, camera_index=c) for w, h, f, c in fr])
+    got = got.cpu().numpy()
+    seen = want < 1.0e4
+    assert seen.mean() > 0.5 and np.array_equal(seen, got < 1.0e4)
+    # the reference measures |p - c| in world space, the kernel |V p| in camera space: equal to fp32 rounding
+    np.testing.assert_allclose(got, want, rtol=1e-5)
+    one = preprocess.PointDistanceToCamera(torch.from_numpy(p).cuda(), torch.from_numpy(views).cuda(),
+                                           torch.from_numpy(K).cuda(), [scenes.make_view(320, 240, image_index=3)])
+    want1 = op.point_distance_to_camera(p, poses, K, [(320, 240, 3, 0)])
+    assert 0.05 < (want1 < 1.0e4).mean() < 0.95  # one camera leaves points unseen: they keep the start value
+    np.testing.assert_allclose(one.cpu().numpy(), want1, rtol=1e-5)
+    with pytest.raises(RuntimeError):
+        preprocess.PointDistanceToCamera(torch.from_numpy(p).cuda(), torch.from_numpy(views).cuda(),
+                                         torch.from_numpy(K).cuda(), [scenes.make_view(320, 240, image_index=37)])
+
+
+@pytest.mark.parametrize("name", ["uniform", "plane", "duplicates", "coincident", "line"])
+def test_remove_close_points_equals_the_sequential_sweep(name):
+    import torch
+    import oracle.preprocess as op
+    from adop_amd import preprocess
+
+    g = np.random.default_rng(21)
+    if name == "line":
+        # every point within reach of its predecessor: one chain of dependencies through the whole cloud
+        p = np.zeros((700, 4), np.float32)
+        p[:, 0] = np.arange(700) * 0.01
+        radius = np.full(700, 0.015, np.float32)
+    else:
+        p = _clouds()[name][:6000]
+        radius = g.uniform(0.0, 0.06, len(p)).astype(np.float32)
+    announce(f"close points, cloud={name} N={len(p)}")
+    want = op.remove_close_points(p, radius)
+    # RemoveClosePoints takes dis_th / camera distance as the radius: camera distance 1 / radius, dis_th 1
+    cam = torch.from_numpy(1.0 / np.maximum(radius, 1e-30)).cuda()
+    got = preprocess.RemoveClosePoints(torch.from_numpy(p).cuda(), cam, dis_th=1.0).cpu().numpy()
+    radius_used = (1.0 / cam).float().cpu().numpy()
+    if not np.array_equal(radius_used, radius):
+        want = op.remove_close_points(p, radius_used)
+    assert np.array_equal(got, want), (name, int((got != want).sum()))
+    if name == "line":
+        assert np.array_equal(want, np.arange(700) % 2 == 0)
+    if name == "coincident":
+        assert want.sum() == 1
+
+
+def test_remove_lonely_points():
+    import torch
+    import oracle.preprocess as op
+    from adop_amd import preprocess
+
+    g = np.random.default_rng(4)
+    p = np.zeros((9000, 4), np.float32)
+    p[:8900, :3] = g.random((8900, 3)) * 0.5
+    p[8900:, :3] = g.random((100, 3)) * 4 + 1  # stragglers
+    cam = g.uniform(1.0, 3.0, 9000).astype(np.float32)
+    announce("lonely points: N=9000")
+    keep = preprocess.RemoveLonelyPoints(torch.from_numpy(p).cuda(), torch.from_numpy(cam).cuda(), 5, 0.02).cpu().numpy()
+    want = ~(op.knn_distance(p, 5) / cam > np.float32(0.02))
+    assert np.array_equal(keep, want) and keep[:8900].mean() > 0.5 and keep[8900:].mean() < 0.1
+
+
+def test_filter_point_cloud_composes_the_filters():
+    import torch
+    import oracle.preprocess as op
+    from adop_amd import preprocess, scenes
+
+    p, views, poses, K, fr = _orbit_scene(6000, 5, 8)
+    p[3000:3300] = p[:300] + np.float32(1e-6)  # near-duplicates for the close-point filter
+    announce("FilterPointCloud: N=6000, 5 frames")
+    got = preprocess.FilterPointCloud(torch.from_numpy(p).cuda(), torch.from_numpy(views).cuda(), torch.from_numpy(K).cuda(),
+                                      [scenes.make_view(w, h, image_index=f, camera_index=c) for w, h, f, c in fr],
+                                      lonely=(5, 0.1)).cpu().numpy()
+    cam = preprocess.PointDistanceToCamera(torch.from_numpy(p).cuda(), torch.from_numpy(views).cuda(),
+                                           torch.from_numpy(K).cuda(),
+                                           [scenes.make_view(w, h, image_index=f, camera_index=c) for w, h, f, c in fr]).cpu().numpy()
+    ids = np.arange(6000)
+    keep = ~(op.knn_distance(p, 5) / cam > np.float32(0.1))
+    q, cam2, ids = p[keep], cam[keep], ids[keep]
+    keep2 = op.remove_close_points(q, (np.float32(0.00005) / cam2).astype(np.float32))
+    assert np.array_equal(got, ids[keep2])
+    assert 0 < (~keep).sum() < 3000 and 200 < (~keep2).sum() <= 320

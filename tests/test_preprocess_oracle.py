@@ -84,3 +84,55 @@ def test_sort_blocks():
         assert np.all((blk >= b * 256) & (blk < (b + 1) * 256))
         assert blk.tolist() == sorted(range(b * 256, (b + 1) * 256), key=lambda i: (r[i], i))
     assert order[768:].tolist() == list(range(768, 1000))  # the last, shorter block is left alone
+
+
+SENTINEL = np.sqrt(np.float32(105235545.0))
+
+
+def test_camera_distance_hand_computed_cases():
+    identity = [0, 0, 0, 1, 0, 0, 0]
+    K = np.zeros((2, 13), np.float32)
+    K[0, :5] = [100, 100, 50, 40, 0]  # 100 x 80 image, centre (50, 40)
+    K[1, :5] = [100, 100, 50, 40, 0]
+    K[1, 5] = 5.0  # k1: x' = x (1 + 5 r^2)
+    pts = np.float32([[0, 0, 5, 0],        # on the axis: 5
+                      [0, 0, -5, 0],       # behind the camera
+                      [3, 0, 5, 0],        # x/z = 0.6 -> pixel 110: outside
+                      [2.4, 0, 5, 0],      # x/z = 0.48 -> pixel 98: inside, distance sqrt(2.4^2 + 25)
+                      [1.5, 0, 5, 0],      # x/z = 0.3 -> 80 undistorted; 0.3 (1 + 0.45) = 0.435 -> 93.5 with k1
+                      [2.0, 0, 5, 0]])     # x/z = 0.4 -> 90 undistorted; 0.4 (1 + 0.8) = 0.72 -> 122 with k1: outside
+    d0 = op.point_distance_to_camera(pts, [identity], K, [(100, 80, 0, 0)])
+    want0 = np.float32([5, SENTINEL, SENTINEL, np.sqrt(2.4 ** 2 + 25), np.sqrt(1.5 ** 2 + 25), np.sqrt(29.0)])
+    np.testing.assert_allclose(d0, want0, rtol=1e-6)
+    d1 = op.point_distance_to_camera(pts, [identity], K, [(100, 80, 0, 1)])
+    assert d1[4] == d0[4] and d1[5] == SENTINEL and d1[3] == SENTINEL
+    # a second camera at (10, 0, 5) looking down -x sees the points from the side: the nearer camera wins
+    s = np.sqrt(0.5)
+    side = [0, -s, 0, s, 10, 0, 5]  # camera -> world: the camera's +z is the world's -x
+    both = op.point_distance_to_camera(pts, [identity, side], K, [(100, 80, 0, 0), (100, 80, 1, 0)])
+    alone = op.point_distance_to_camera(pts, [identity, side], K, [(100, 80, 1, 0)])
+    np.testing.assert_allclose(alone[0], 10, rtol=1e-6)  # (0,0,5) is 10 away on the axis
+    assert alone[1] == SENTINEL  # (0,0,-5): 10 in front, 10 to the side: tangent 1 -> 100 pixels off the centre
+    np.testing.assert_allclose(both[0], 5, rtol=1e-6)
+    np.testing.assert_allclose(both[2], min(7.0, SENTINEL), rtol=1e-6)  # (3,0,5): unseen by the first, 7 from the second
+
+
+@pytest.mark.parametrize("name", ["uniform", "plane", "duplicates"])
+def test_close_point_sweep_has_the_defining_properties(name):
+    from scipy.spatial import cKDTree
+
+    g = np.random.default_rng(2)
+    p = _clouds()[name]
+    radius = g.uniform(0.0, 0.08, len(p)).astype(np.float32)
+    keep = op.remove_close_points(p, radius)
+    assert 0.2 < keep.mean() < 0.95
+    xyz = p[:, :3].astype(np.float64)
+    tree = cKDTree(xyz)
+    for i in range(len(p)):
+        near = [j for j in tree.query_ball_point(xyz[i], float(radius[i]) * (1 + 1e-6) + 1e-12) if j < i and keep[j]]
+        # leave pairs at the radius to within rounding to the fp32 sweep
+        sure = [j for j in near if np.linalg.norm(xyz[i] - xyz[j]) < float(radius[i]) * (1 - 1e-6)]
+        if keep[i]:
+            assert not sure, i  # no kept point has an earlier kept point within its radius
+        else:
+            assert near, i  # every erased point has one
