@@ -1,5 +1,6 @@
-"""BASELINE configuration 3 at full size (10 M points, 1920x1080, 4 levels, 8 channels): too big for the CPU
-checker inside a test, so the HIP path is held to size-independent properties of the rasterizer."""
+"""The BASELINE configurations 3, 4 and 5 at full size (10 M points at 1920x1080 with 8 channels; 100 M points forward
+only with fp16 descriptors; 20 M points through the OCam model at 2200x1500 in 8 views): too big for the CPU checker
+inside a test, so the HIP path is held to size-independent properties of the rasterizer."""
 import numpy as np
 import pytest
 
@@ -8,17 +9,17 @@ from helpers import announce, run_hip_forward
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module")
-def full_scene():
+@pytest.fixture(scope="module", params=["config3", "config5", "config4"])
+def full_scene(request):
     from adop_amd import scenes
 
-    announce("config3 full size: generate")
-    return scenes.config3()
+    announce(f"{request.param} full size: generate")
+    return getattr(scenes, request.param)()
 
 
 @pytest.fixture(scope="module", params=[1, 2], ids=["direct", "tiles"])
 def full(request, full_scene):
-    announce(f"config3 full size: forward, forward_path={request.param}")
+    announce(f"{full_scene.name} full size: forward, forward_path={request.param}")
     return full_scene, run_hip_forward(full_scene, forward_path=request.param)
 
 
@@ -48,7 +49,7 @@ def test_inference_forward_agrees_with_training_forward(full_scene):
     ref = run_hip_forward(full_scene, forward_path=2)
     for path in (1, 2):
         for counters in (True, False):
-            announce(f"config3 full size: inference forward, forward_path={path}, counters={counters}")
+            announce(f"{full_scene.name} full size: inference forward, forward_path={path}, counters={counters}")
             got = run_hip_forward(full_scene, collect_stats=counters, forward_path=path, train=False)
             assert got[1].cache.point_cache is None
             for l, (La, Lb) in enumerate(zip(ref[1].cache.layers_cuda, got[1].cache.layers_cuda)):
@@ -73,7 +74,7 @@ def test_counts_and_depth_invariants(full):
         # sum of the weights = number of blended point-levels; weights are whole numbers
         assert int(w.sum(dtype=torch.float64).item()) == st.accepted[l]
         assert bool((w == w.round()).all())
-        assert st.accepted[l] <= st.visible[l] <= N
+        assert st.accepted[l] <= st.visible[l] <= N * hs.batch
         di = L.depth_index_tensor
         hi = (di >> 32).to(torch.int32).view(torch.float32)
         assert bool((hi == L.depth).all())                       # f32 depth = high word, bit for bit
@@ -98,20 +99,22 @@ def test_index_word_points_at_a_point_with_that_depth(full):
 
     hs, (scene, info, ctx, images, masks) = full
     L = info.cache.layers_cuda[0]
-    di = L.depth_index_tensor.view(-1)
+    di = L.depth_index_tensor[0].reshape(-1)  # the image of the first view
     lo = (di & 0xFFFFFFFF)
-    sel = torch.nonzero(lo != 0xFFFFFFFF).view(-1)[::997][:20000]
+    sel = torch.nonzero(lo != 0xFFFFFFFF).view(-1)[::97][:20000]
     ids = lo[sel].long()
     p = scene.point_cloud_cuda.t_position[ids, :3].double()
-    q = scene.poses_se3[0, :4]
-    t = scene.poses_se3[0, 4:7]
-    x, y, z, w = q.tolist()
+    pose = scene.poses_se3[hs.views[0].image_index]
+    x, y, z, w = pose[:4].tolist()
+    t = pose[4:7]
     R = torch.tensor([[1 - 2 * (y * y + z * z), 2 * (x * y - z * w), 2 * (x * z + y * w)],
                       [2 * (x * y + z * w), 1 - 2 * (x * x + z * z), 2 * (y * z - x * w)],
                       [2 * (x * z - y * w), 2 * (y * z + x * w), 1 - 2 * (x * x + y * y)]], dtype=torch.float64,
                      device=p.device)
-    vz = (p @ R.T + t)[:, 2]
-    assert bool(((L.depth.view(-1)[sel].double() - vz).abs() <= 1e-5 * vz.abs()).all())
+    v = p @ R.T + t
+    vz = v.norm(dim=1) if hs.views[0].camera_model_type == 1 else v[:, 2]  # the OCam depth is the distance
+    assert len(sel) > 1000
+    assert bool(((L.depth[0].reshape(-1)[sel].double() - vz).abs() <= 1e-5 * vz.abs()).all())
 
 
 def test_forward_is_deterministic_in_depth_and_linear_in_the_texture(full):
@@ -123,13 +126,14 @@ def test_forward_is_deterministic_in_depth_and_linear_in_the_texture(full):
     out1 = [im.clone() for im in images]
     # second run with the texture scaled by 2 and shifted: out must scale the same way where something was blended
     tex = scene.texture.clone()
-    scene.texture = (2.0 * tex + 0.25).contiguous()
+    exact = tex.dtype == torch.float32  # fp16 descriptors: 2 t + 0.25 rounds, so the texture is only doubled
+    scene.texture = (2.0 * tex + 0.25).contiguous() if exact else (2.0 * tex).contiguous()
     images2, _ = render.BlendPointCloudForward(None, info)
     torch.cuda.synchronize()
     for l, L in enumerate(info.cache.layers_cuda):
         assert bool((first[l] == L.depth_index_tensor).all())   # bit-identical packed buffers
         covered = (L.weight > 0).expand_as(images2[l])
-        a, b = images2[l][covered], (2.0 * out1[l] + 0.25)[covered]
+        a, b = images2[l][covered], (2.0 * out1[l] + (0.25 if exact else 0.0))[covered]
         assert float((a - b).abs().max()) <= 1e-5 * float(b.abs().max())
     scene.texture = tex
 
@@ -141,6 +145,8 @@ def test_backward_sums(full):
     from adop_amd import render
 
     hs, (scene, info, ctx, images, masks) = full
+    if hs.name == "config4":
+        pytest.skip("configuration 4 is the viewer path: forward only")
     images, _ = render.BlendPointCloudForward(ctx, info)
     g = torch.Generator(device="cuda").manual_seed(1)
     gout = [torch.randn(im.shape, device="cuda", generator=g) for im in images]
@@ -151,11 +157,14 @@ def test_backward_sums(full):
     assert float((g_bg.double() - want_bg).abs().max()) <= 1e-5 * float(want_bg.abs().max())
     spatial = sum(st.spatial[: hs.num_layers])
     assert int(info.cache.output_gradient_point_count.sum(dtype=torch.float64).item()) == spatial
-    assert float(info.cache.output_gradient_pose_tangent_count[0]) == float(np.float32(spatial))
+    # every view's spatial gradients are counted on the pose of its image (fp32 counters, one per pose)
+    pose_count = float(info.cache.output_gradient_pose_tangent_count.double().sum())
+    assert abs(pose_count - spatial) <= 1e-6 * spatial
     assert all(bool(torch.isfinite(t).all()) for t in (g_tex, g_pts, g_pose, g_intr))
-    # dropped points get no descriptor gradient
-    dropped = info.cache.dropout_points[0] == 1
-    assert float(g_tex[:, dropped].abs().max()) == 0
+    # points dropped in every view get no descriptor gradient
+    if info.cache.dropout_points is not None:
+        dropped = (info.cache.dropout_points == 1).all(dim=0)
+        assert float(g_tex[:, dropped].abs().max()) == 0
     # linearity in the upstream gradient
     g_tex2 = render.BlendPointCloudBackward(ctx, info, [3.0 * x for x in gout])[0]
     torch.cuda.synchronize()
