@@ -135,8 +135,8 @@ constexpr int kTilePathMaxPointsPerPixel = 16;
 
 size_t max_tiles(int B, int w0, int h0)
 {
-    size_t tx = ((size_t)(w0 > 0 ? w0 : 1) - 1 >> kTileShiftX) + 1;
-    size_t ty = ((size_t)(h0 > 0 ? h0 : 1) - 1 >> kTileShiftY) + 1;
+    size_t tx = (((size_t)(w0 > 0 ? w0 : 1) - 1) >> kTileShiftX) + 1;
+    size_t ty = (((size_t)(h0 > 0 ? h0 : 1) - 1) >> kTileShiftY) + 1;
     return tx * ty * (size_t)B;
 }
 
@@ -706,71 +706,109 @@ adop_status adop_apply_tangent(double* tangent, double* poses_se3, int32_t num_p
     return ADOP_OK;
 }
 
-// Grid of the nearest-neighbour search: ~8 points per cell for a volume-filling cloud, at most kKnnMaxDim cells per
-// axis (a surface-like cloud puts more points into fewer cells; the search stays exact, only slower).
-static constexpr int kKnnMaxDim = 160;
+// Grids of the nearest-neighbour search.  The first one is sized on the host for ~8 points per cell of a volume-filling
+// cloud, at most kKnnCoarseDim cells per axis; the second one on the device from the neighbour distances of sample
+// points, within a budget of cells that grows with the cloud.
+static constexpr int kKnnCoarseDim = 160;
 
-static size_t knn_cells_max() { return (size_t)kKnnMaxDim * kKnnMaxDim * kKnnMaxDim; }
+static uint32_t knn_max_cells(int32_t num_points)
+{
+    size_t want = (size_t)(num_points > 0 ? num_points : 0) * 16;
+    if (want < ((size_t)1 << 22)) want = (size_t)1 << 22;  // > kKnnCoarseDim^3
+    if (want > ((size_t)1 << 27)) want = (size_t)1 << 27;
+    return (uint32_t)want;
+}
+
+struct KnnWorkspace
+{
+    KnnGrid* grid;  // device
+    float* sample;
+    uint32_t *count, *offset, *chunk;
+    float4* sorted;
+    size_t total;
+};
+
+static KnnWorkspace knn_layout(void* workspace, int32_t num_points)
+{
+    const uint32_t cells = knn_max_cells(num_points);
+    size_t o             = 0;
+    const size_t o_grid  = o;
+    o                    = align_up(o + sizeof(KnnGrid), 256);
+    const size_t o_sample = o;
+    o                    = align_up(o + sizeof(float) * 2048, 256);
+    const size_t o_count = o;
+    o                    = align_up(o + sizeof(uint32_t) * (size_t)cells, 256);
+    const size_t o_offset = o;
+    o                    = align_up(o + sizeof(uint32_t) * ((size_t)cells + 1), 256);
+    const size_t o_chunk = o;
+    o                    = align_up(o + sizeof(uint32_t) * knn_chunk_words(cells), 256);
+    const size_t o_sorted = o;
+    o                    = align_up(o + sizeof(float4) * (size_t)(num_points > 0 ? num_points : 0), 256);
+    KnnWorkspace w;
+    memset(&w, 0, sizeof(w));
+    w.total = o;
+    if (workspace)
+    {
+        char* base = (char*)workspace;
+        w.grid     = (KnnGrid*)(base + o_grid);
+        w.sample   = (float*)(base + o_sample);
+        w.count    = (uint32_t*)(base + o_count);
+        w.offset   = (uint32_t*)(base + o_offset);
+        w.chunk    = (uint32_t*)(base + o_chunk);
+        w.sorted   = (float4*)(base + o_sorted);
+    }
+    return w;
+}
 
 size_t adop_knn_workspace_size(int32_t num_points)
 {
     if (num_points < 0) return 0;
-    size_t o = 0;
-    o        = align_up(o + sizeof(uint32_t) * knn_cells_max(), 256);        // count
-    o        = align_up(o + sizeof(uint32_t) * (knn_cells_max() + 1), 256);  // offset
-    o        = align_up(o + sizeof(float4) * (size_t)num_points, 256);      // points in cell order
-    return o;
+    return knn_layout(nullptr, num_points).total;
 }
 
-// The grid of a cloud (a function of the bounding box and the number of points only) and, with `bin`, the points in
-// cell order in the workspace: count [cells], offset [cells + 1], sorted [N].
-struct KnnWorkspace
-{
-    KnnGrid g;
-    uint32_t *count, *offset;
-    float4* sorted;
-};
-
+// The points in cell order of the search grid (both in the workspace).  build = false: the workspace still holds them
+// from the last call.
 static adop_status knn_prepare(const float* position, int32_t num_points, const float* bbox_min, const float* bbox_max,
-                               void* workspace, size_t workspace_bytes, bool bin, hipStream_t stream, KnnWorkspace* out)
+                               int sample_rank, void* workspace, size_t workspace_bytes, bool build, hipStream_t stream,
+                               KnnWorkspace* out)
 {
     if (!workspace || workspace_bytes < adop_knn_workspace_size(num_points))
         return fail(ADOP_WORKSPACE_TOO_SMALL, "workspace too small");
-    float ext[3];
+    *out = knn_layout(workspace, num_points);
+    if (!build) return ADOP_OK;
+    KnnGrid g;
+    memset(&g, 0, sizeof(g));
     for (int k = 0; k < 3; ++k)
     {
-        ext[k] = bbox_max[k] - bbox_min[k];
-        if (!(ext[k] >= 0) || !(ext[k] < 1.0e30f)) return fail(ADOP_INVALID_ARG, "bounding box is not finite");
+        g.ext[k] = bbox_max[k] - bbox_min[k];
+        if (!(g.ext[k] >= 0) || !(g.ext[k] < 1.0e30f)) return fail(ADOP_INVALID_ARG, "bounding box is not finite");
     }
-    KnnGrid& g          = out->g;
+    const float* ext    = g.ext;
     const float longest = ext[0] > ext[1] ? (ext[0] > ext[2] ? ext[0] : ext[2]) : (ext[1] > ext[2] ? ext[1] : ext[2]);
     double volume       = 1.0;
     for (int k = 0; k < 3; ++k) volume *= ext[k] > 1e-6f * longest ? ext[k] : (longest > 0 ? 1e-6 * longest : 1.0);
     float cell = (float)cbrt(volume * 8.0 / (double)num_points);
-    if (!(cell > longest / kKnnMaxDim)) cell = longest / kKnnMaxDim;
+    if (!(cell > longest / kKnnCoarseDim)) cell = longest / kKnnCoarseDim;
     if (!(cell > 0)) cell = 1.f;  // all points coincide
     g.cell     = cell;
     g.inv_cell = 1.0f / cell;
+    g.cells    = 1;
     for (int k = 0; k < 3; ++k)
     {
         g.min[k] = bbox_min[k];
         int d    = (int)(ext[k] / cell) + 1;
-        g.dim[k] = d < 1 ? 1 : (d > kKnnMaxDim ? kKnnMaxDim : d);
+        g.dim[k] = d < 1 ? 1 : (d > kKnnCoarseDim ? kKnnCoarseDim : d);
+        g.cells *= (uint32_t)g.dim[k];
     }
-    const size_t cells = (size_t)g.dim[0] * g.dim[1] * g.dim[2];
-    out->count         = (uint32_t*)workspace;
-    out->offset        = (uint32_t*)((char*)workspace + align_up(sizeof(uint32_t) * knn_cells_max(), 256));
-    out->sorted        = (float4*)((char*)out->offset + align_up(sizeof(uint32_t) * (knn_cells_max() + 1), 256));
-    if (!bin) return ADOP_OK;
-    adop_status st = fill_async(out->count, sizeof(uint32_t) * cells, 0, stream);
-    if (st != ADOP_OK) return st;
-    launch_knn_bin(0, (const float4*)position, num_points, g, out->count, out->offset, out->sorted, stream);
-    BinArg scan;
-    memset(&scan, 0, sizeof(scan));
-    scan.count  = out->count;
-    scan.offset = out->offset;
-    launch_tile_scan(scan, (int)cells, stream);
-    launch_knn_bin(1, (const float4*)position, num_points, g, out->count, out->offset, out->sorted, stream);
+    const uint32_t max_cells = knn_max_cells(num_points);
+    const float4* pos        = (const float4*)position;
+    launch_knn_set_grid(g, out->grid, stream);
+    launch_knn_build(pos, num_points, out->grid, max_cells, out->count, out->offset, out->chunk, out->sorted, stream);
+    const int samples = knn_num_samples(num_points);
+    if (!launch_knn_search(sample_rank, out->sorted, num_points, out->grid, out->offset, out->sample, samples, stream))
+        return fail(ADOP_INVALID_ARG, "rank must be 1..8");
+    launch_knn_refine_grid(out->sample, samples, out->grid, max_cells, stream);
+    launch_knn_build(pos, num_points, out->grid, max_cells, out->count, out->offset, out->chunk, out->sorted, stream);
     return ADOP_OK;
 }
 
@@ -783,9 +821,10 @@ adop_status adop_knn_distance(const float* position, int32_t num_points, int32_t
     if (num_points <= rank) return fail(ADOP_INVALID_ARG, "the cloud needs more than `rank` points");
     hipStream_t stream = (hipStream_t)hip_stream;
     KnnWorkspace w;
-    adop_status st = knn_prepare(position, num_points, bbox_min, bbox_max, workspace, workspace_bytes, true, stream, &w);
+    adop_status st =
+        knn_prepare(position, num_points, bbox_min, bbox_max, rank, workspace, workspace_bytes, true, stream, &w);
     if (st != ADOP_OK) return st;
-    if (!launch_knn_search(rank, w.sorted, num_points, w.g, w.offset, out_distance, stream))
+    if (!launch_knn_search(rank, w.sorted, num_points, w.grid, w.offset, out_distance, 0, stream))
         return fail(ADOP_INVALID_ARG, "rank must be 1..8");
     ADOP_HIP_CHECK(hipGetLastError());
     return ADOP_OK;
@@ -801,13 +840,14 @@ adop_status adop_close_points(const float* position, int32_t num_points, const f
     if (num_rounds < 1 || num_rounds > 1024) return fail(ADOP_INVALID_ARG, "num_rounds must be 1..1024");
     hipStream_t stream = (hipStream_t)hip_stream;
     KnnWorkspace w;
+    // (the grid is sized for the 4th-neighbour distance, the one the cloud's radii come from)
     adop_status st =
-        knn_prepare(position, num_points, bbox_min, bbox_max, workspace, workspace_bytes, !resume, stream, &w);
+        knn_prepare(position, num_points, bbox_min, bbox_max, 4, workspace, workspace_bytes, !resume, stream, &w);
     if (st != ADOP_OK) return st;
     if (!resume && (st = fill_async(state, sizeof(int32_t) * (size_t)num_points, 0, stream)) != ADOP_OK) return st;
     if ((st = fill_async(round_undecided, sizeof(uint32_t) * (size_t)num_rounds, 0, stream)) != ADOP_OK) return st;
     for (int r = 0; r < num_rounds; ++r)
-        launch_close_points(w.sorted, num_points, w.g, w.offset, radius, state, round_undecided, r, stream);
+        launch_close_points(w.sorted, num_points, w.grid, w.offset, radius, state, round_undecided, r, stream);
     ADOP_HIP_CHECK(hipGetLastError());
     return ADOP_OK;
 }

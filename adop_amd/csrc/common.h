@@ -78,12 +78,15 @@ struct ParamArg
     float K_gradient_factor;
 };
 
-// Uniform grid of the nearest-neighbour search: cubic cells of edge `cell` from `min`, dim cells per axis.
+// Uniform grid of the nearest-neighbour search: cubic cells of edge `cell` from `min`, dim cells per axis.  The grid
+// lives in device memory: the second one of a search is sized on the device from sampled neighbour distances.
 struct KnnGrid
 {
     float min[3];
+    float ext[3];  // size of the bounding box
     float cell, inv_cell;
     int32_t dim[3];
+    uint32_t cells;  // dim[0] * dim[1] * dim[2]
 };
 
 struct ViewChunk

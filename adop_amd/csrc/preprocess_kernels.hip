@@ -7,7 +7,11 @@
 // rasterizer's tile bins), stored cell after cell, and every point then walks the shells of cells around its own
 // until the n-th best distance cannot be beaten from outside the cube searched so far.  The distances are formed as
 // sqrt((dx*dx + dy*dy) + dz*dz) in fp32; the result is the n-th smallest of them over all other points, whatever the
-// search order, so a brute-force search over the same arithmetic gives the same bits.
+// search order and whatever the grid, so a brute-force search over the same arithmetic gives the same bits.
+// The cost is the number of candidates, which the cell size decides, and the right cell size depends on how the cloud
+// fills space (scans are surfaces: a grid sized by volume puts hundreds of points into the few cells that have any).
+// So the search runs twice: on a coarse grid sized by volume for 2048 sample points only, then, with cells of twice
+// the median distance those found, for all points.  The second grid is computed on the device (no host round trip).
 #include "common.h"
 #include "launch.h"
 
@@ -32,12 +36,13 @@ __device__ __forceinline__ uint32_t grid_index(const KnnGrid& g, int cx, int cy,
 }
 
 // pass 0: points per cell; pass 1: the points cell after cell, (x, y, z, bits of the point id)
-__global__ __launch_bounds__(kBlock) void knn_bin_kernel(int pass, const float4* __restrict__ position, int n, KnnGrid g,
-                                                         uint32_t* __restrict__ count, const uint32_t* __restrict__ offset,
-                                                         float4* __restrict__ sorted)
+__global__ __launch_bounds__(kBlock) void knn_bin_kernel(int pass, const float4* __restrict__ position, int n,
+                                                         const KnnGrid* __restrict__ gp, uint32_t* __restrict__ count,
+                                                         const uint32_t* __restrict__ offset, float4* __restrict__ sorted)
 {
     const int i = blockIdx.x * kBlock + threadIdx.x;
     if (i >= n) return;
+    const KnnGrid g = *gp;
     const float4 p    = nt_load4(position + i);
     const int3 c      = grid_cell(g, p.x, p.y, p.z);
     const uint32_t ci = grid_index(g, c.x, c.y, c.z);
@@ -50,15 +55,17 @@ __global__ __launch_bounds__(kBlock) void knn_bin_kernel(int pass, const float4*
 // One thread per point, in cell order (the lanes of a wavefront search nearly the same cells).  The cube of cells
 // around the point's cell grows until the K-th best distance cannot be beaten from outside it; a row of cells along x
 // is one contiguous run of the cell-ordered array, so a cube of (2r+1)^3 cells is (2r+1)^2 runs.  A larger cube is
-// searched from scratch (with ~8 points per cell the first cube, r = 1, settles nearly every point).
+// searched from scratch (the first cube, r = 1, settles nearly every point).
 template <int K>  // K = n + 1 best squared distances are kept (the point itself is one of them)
-__global__ __launch_bounds__(kBlock) void knn_search_kernel(const float4* __restrict__ sorted, int n, KnnGrid g,
+__global__ __launch_bounds__(kBlock) void knn_search_kernel(const float4* __restrict__ sorted, int n,
+                                                            const KnnGrid* __restrict__ gp,
                                                             const uint32_t* __restrict__ offset, float* __restrict__ out)
 {
     const int t = blockIdx.x * kBlock + threadIdx.x;
     if (t >= n) return;
-    const float4 p = sorted[t];
-    const int3 c   = grid_cell(g, p.x, p.y, p.z);
+    const KnnGrid g = *gp;
+    const float4 p  = sorted[t];
+    const int3 c    = grid_cell(g, p.x, p.y, p.z);
     float best[K];
     for (int r = 1;; ++r)
     {
@@ -106,6 +113,260 @@ __global__ __launch_bounds__(kBlock) void knn_search_kernel(const float4* __rest
     out[__float_as_uint(p.w)] = sqrtf(best[K - 1]);
 }
 
+// The same search for `samples` points evenly spaced in cell order, one wavefront per point (on the first grid a
+// point has thousands of candidates: the lanes share them, every lane keeps the K best of its share, and the K-th
+// best of the wavefront is found by K rounds of taking the smallest head off the lanes' lists).  out[s] = distance
+// of sample s.  All branches on r, the bound and the result are uniform over the wavefront.
+template <int K>
+__global__ __launch_bounds__(kBlock) void knn_sample_kernel(const float4* __restrict__ sorted, int n,
+                                                            const KnnGrid* __restrict__ gp,
+                                                            const uint32_t* __restrict__ offset, float* __restrict__ out,
+                                                            int samples)
+{
+    const int slot = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (slot >= samples) return;
+    const int t     = (int)((long long)slot * n / samples);
+    const KnnGrid g = *gp;
+    const float4 p  = sorted[t];
+    const int3 c    = grid_cell(g, p.x, p.y, p.z);
+    float kth       = 3.0e38f;
+    for (int r = 1;; ++r)
+    {
+        float best[K];
+#pragma unroll
+        for (int k = 0; k < K; ++k) best[k] = 3.0e38f;
+        const int z0 = max(c.z - r, 0), z1 = min(c.z + r, g.dim[2] - 1);
+        const int y0 = max(c.y - r, 0), y1 = min(c.y + r, g.dim[1] - 1);
+        const int x0 = max(c.x - r, 0), x1 = min(c.x + r, g.dim[0] - 1);
+        for (int cz = z0; cz <= z1; ++cz)
+            for (int cy = y0; cy <= y1; ++cy)
+            {
+                const uint32_t row = grid_index(g, 0, cy, cz);
+                const uint32_t e   = offset[row + x1 + 1];
+                for (uint32_t q = offset[row + x0] + lane; q < e; q += 64)
+                {
+                    const float4 o = sorted[q];
+                    const float dx = p.x - o.x, dy = p.y - o.y, dz = p.z - o.z;
+                    float d2 = (dx * dx + dy * dy) + dz * dz;
+                    if (d2 < best[K - 1])
+                    {
+#pragma unroll
+                        for (int k = 0; k < K; ++k)
+                        {
+                            const float b = best[k];
+                            const bool lt = d2 < b;
+                            best[k]       = lt ? d2 : b;
+                            d2            = lt ? b : d2;
+                        }
+                    }
+                }
+            }
+        // K-th smallest over the lanes' ascending lists
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+        {
+            float m = best[0];
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) m = fminf(m, __shfl_xor(m, off, 64));
+            kth = m;
+            const unsigned long long holders = __ballot(best[0] == m);
+            if (lane == __ffsll((long long)holders) - 1)
+            {
+#pragma unroll
+                for (int j = 0; j + 1 < K; ++j) best[j] = best[j + 1];
+                best[K - 1] = 3.0e38f;
+            }
+        }
+        float bound = 3.0e38f;
+        if (c.x - r > 0) bound = fminf(bound, p.x - (g.min[0] + (float)(c.x - r) * g.cell));
+        if (c.y - r > 0) bound = fminf(bound, p.y - (g.min[1] + (float)(c.y - r) * g.cell));
+        if (c.z - r > 0) bound = fminf(bound, p.z - (g.min[2] + (float)(c.z - r) * g.cell));
+        if (c.x + r < g.dim[0] - 1) bound = fminf(bound, (g.min[0] + (float)(c.x + r + 1) * g.cell) - p.x);
+        if (c.y + r < g.dim[1] - 1) bound = fminf(bound, (g.min[1] + (float)(c.y + r + 1) * g.cell) - p.y);
+        if (c.z + r < g.dim[2] - 1) bound = fminf(bound, (g.min[2] + (float)(c.z + r + 1) * g.cell) - p.z);
+        if (bound == 3.0e38f) break;
+        bound = fmaxf(bound, 0.f) * 0.999f;
+        if (kth <= bound * bound) break;
+    }
+    if (lane == 0) out[slot] = sqrtf(kth);
+}
+
+// The grid a host-side choice starts from, placed in device memory.
+__global__ void knn_set_grid_kernel(KnnGrid g, KnnGrid* __restrict__ dst)
+{
+    if (blockIdx.x == 0 && threadIdx.x == 0) *dst = g;
+}
+
+// Second grid: cells of twice the median sampled neighbour distance (a cube of 3 cells then settles every point whose
+// own distance is below twice the median, with ~60 candidates on a surface, ~260 in a volume), never coarser than the
+// first grid, at most kKnnMaxDim cells per axis and `budget` cells in all.  One workgroup; the samples are sorted in
+// LDS (bitonic network).
+constexpr int kKnnSamples = 2048;
+constexpr int kKnnMaxDim  = 2048;
+
+__global__ __launch_bounds__(1024) void knn_refine_grid_kernel(const float* __restrict__ sample, int samples,
+                                                               KnnGrid* __restrict__ gp, uint32_t budget)
+{
+    __shared__ float s[kKnnSamples];
+    for (int i = threadIdx.x; i < kKnnSamples; i += 1024) s[i] = i < samples ? sample[i] : 3.0e38f;
+    __syncthreads();
+    for (int k = 2; k <= kKnnSamples; k <<= 1)
+        for (int j = k >> 1; j > 0; j >>= 1)
+        {
+            for (int i = threadIdx.x; i < kKnnSamples; i += 1024)
+            {
+                const int o = i ^ j;
+                if (o > i)
+                {
+                    const float a = s[i], b = s[o];
+                    const bool up = (i & k) == 0;
+                    if ((a > b) == up)
+                    {
+                        s[i] = b;
+                        s[o] = a;
+                    }
+                }
+            }
+            __syncthreads();
+        }
+    if (threadIdx.x != 0) return;
+    KnnGrid g          = *gp;
+    const float median = s[samples / 2];
+    const float longest = fmaxf(g.ext[0], fmaxf(g.ext[1], g.ext[2]));
+    float cell = 2.0f * median;
+    if (!(cell < g.cell)) cell = g.cell;  // also NaN / the 3e38 of a cloud with fewer points than neighbours asked for
+    if (!(cell > longest / (float)(kKnnMaxDim - 1))) cell = longest / (float)(kKnnMaxDim - 1);
+    if (!(cell > 0.f)) cell = g.cell;
+    for (;;)
+    {
+        unsigned long long cells = 1;
+        for (int k = 0; k < 3; ++k)
+        {
+            int d    = (int)(g.ext[k] / cell) + 1;
+            g.dim[k] = d < 1 ? 1 : (d > kKnnMaxDim ? kKnnMaxDim : d);
+            cells *= (unsigned long long)g.dim[k];
+        }
+        if (cells <= budget)
+        {
+            g.cells = (uint32_t)cells;
+            break;
+        }
+        cell *= 1.26f;
+    }
+    g.cell     = cell;
+    g.inv_cell = 1.0f / cell;
+    *gp        = g;
+}
+
+// Zeroes the cell counters of the grid.
+__global__ __launch_bounds__(kBlock) void knn_clear_kernel(uint32_t* __restrict__ count, const KnnGrid* __restrict__ gp)
+{
+    const uint32_t cells = gp->cells;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < cells; i += (size_t)gridDim.x * kBlock)
+        __builtin_nontemporal_store(0u, count + i);
+}
+
+// Exclusive prefix sum over the cell counters (offset[0..cells]) in three launches: sums of chunks of 8192 cells,
+// their prefix sum (one workgroup: at most 16384 chunks), the prefix sum inside every chunk.
+constexpr int kScanChunk = 8192;
+
+__device__ __forceinline__ uint32_t block_exclusive_scan_1024(uint32_t sum, uint32_t* s_wave, uint32_t* total)
+{
+    const int tid = threadIdx.x;
+    uint32_t inc  = sum;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1)
+    {
+        const uint32_t u = __shfl_up(inc, off, 64);
+        if ((tid & 63) >= off) inc += u;
+    }
+    __syncthreads();  // s_wave of the last call has been read
+    if ((tid & 63) == 63) s_wave[tid >> 6] = inc;
+    __syncthreads();
+    uint32_t run = inc - sum, all = 0;
+    for (int w = 0; w < 16; ++w)
+    {
+        if (w < (tid >> 6)) run += s_wave[w];
+        all += s_wave[w];
+    }
+    *total = all;
+    return run;
+}
+
+__global__ __launch_bounds__(1024) void knn_scan_reduce_kernel(const uint32_t* __restrict__ count,
+                                                               const KnnGrid* __restrict__ gp,
+                                                               uint32_t* __restrict__ chunk_sum)
+{
+    __shared__ uint32_t s_wave[16];
+    const uint32_t cells = gp->cells;
+    const uint32_t nb    = (cells + kScanChunk - 1) / kScanChunk;
+    for (uint32_t b = blockIdx.x; b < nb; b += gridDim.x)
+    {
+        const size_t t0 = (size_t)b * kScanChunk + (size_t)threadIdx.x * 8;
+        uint32_t sum    = 0;
+        if (t0 + 8 <= cells)
+        {
+            const uint4 a = ((const uint4*)(count + t0))[0], c = ((const uint4*)(count + t0))[1];
+            sum = a.x + a.y + a.z + a.w + c.x + c.y + c.z + c.w;
+        }
+        else
+            for (int k = 0; k < 8; ++k) sum += t0 + k < cells ? count[t0 + k] : 0u;
+        uint32_t total;
+        block_exclusive_scan_1024(sum, s_wave, &total);
+        if (threadIdx.x == 0) chunk_sum[b] = total;
+    }
+}
+
+__global__ __launch_bounds__(1024) void knn_scan_chunks_kernel(const uint32_t* __restrict__ chunk_sum,
+                                                               const KnnGrid* __restrict__ gp,
+                                                               uint32_t* __restrict__ chunk_offset)
+{
+    __shared__ uint32_t s_wave[16];
+    const uint32_t nb = (gp->cells + kScanChunk - 1) / kScanChunk;
+    uint32_t carry    = 0;
+    for (uint32_t c0 = 0; c0 < nb; c0 += 1024)
+    {
+        const uint32_t i = c0 + threadIdx.x;
+        const uint32_t v = i < nb ? chunk_sum[i] : 0u;
+        uint32_t total;
+        const uint32_t run = block_exclusive_scan_1024(v, s_wave, &total);
+        if (i < nb) chunk_offset[i] = carry + run;
+        carry += total;
+    }
+    if (threadIdx.x == 0) chunk_offset[nb] = carry;
+}
+
+__global__ __launch_bounds__(1024) void knn_scan_apply_kernel(const uint32_t* __restrict__ count,
+                                                              const KnnGrid* __restrict__ gp,
+                                                              const uint32_t* __restrict__ chunk_offset,
+                                                              uint32_t* __restrict__ offset)
+{
+    __shared__ uint32_t s_wave[16];
+    const uint32_t cells = gp->cells;
+    const uint32_t nb    = (cells + kScanChunk - 1) / kScanChunk;
+    for (uint32_t b = blockIdx.x; b < nb; b += gridDim.x)
+    {
+        const size_t t0 = (size_t)b * kScanChunk + (size_t)threadIdx.x * 8;
+        uint32_t v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] = t0 + k < cells ? count[t0 + k] : 0u;
+        uint32_t sum = 0;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) sum += v[k];
+        uint32_t total;
+        uint32_t run = chunk_offset[b] + block_exclusive_scan_1024(sum, s_wave, &total);
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            if (t0 + k < cells)
+            {
+                offset[t0 + k] = run;
+                run += v[k];
+            }
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0) offset[cells] = chunk_offset[nb];
+}
+
 // SceneData::PointDistanceToCamera (SceneData.cpp:645-669): distance from every point to the nearest camera that sees
 // it (in front of the camera, projected inside the image with the frame's pinhole + distortion model), 10258.4 (the
 // root of the reference's start value 105235545) where no frame does.  The distance is taken in camera space
@@ -143,7 +404,8 @@ __global__ __launch_bounds__(kBlock) void camera_distance_kernel(const float4* _
 // that finds count[round - 1] == 0 has nothing to do.
 constexpr int kStateUndecided = 0, kStateKept = 1, kStateErased = 2;
 
-__global__ __launch_bounds__(kBlock) void close_points_kernel(const float4* __restrict__ sorted, int n, KnnGrid g,
+__global__ __launch_bounds__(kBlock) void close_points_kernel(const float4* __restrict__ sorted, int n,
+                                                              const KnnGrid* __restrict__ gp,
                                                               const uint32_t* __restrict__ offset,
                                                               const float* __restrict__ radius, int32_t* state,
                                                               uint32_t* round_count, int round)
@@ -153,6 +415,7 @@ __global__ __launch_bounds__(kBlock) void close_points_kernel(const float4* __re
     bool pending = false;
     if (t < n)
     {
+        const KnnGrid g  = *gp;
         const float4 p   = sorted[t];
         const uint32_t i = __float_as_uint(p.w);
         if (__atomic_load_n(&state[i], __ATOMIC_RELAXED) == kStateUndecided)
@@ -226,28 +489,66 @@ __global__ __launch_bounds__(kBlock) void morton_kernel(const float4* __restrict
 // ------------------------------------------------------------------------------------------------
 // launchers
 // ------------------------------------------------------------------------------------------------
-void launch_knn_bin(int pass, const float4* position, int n, const KnnGrid& g, uint32_t* count, const uint32_t* offset,
-                    float4* sorted, hipStream_t st)
+void launch_knn_set_grid(const KnnGrid& g, KnnGrid* dst, hipStream_t st)
 {
-    hipLaunchKernelGGL(knn_bin_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, pass, position, n, g, count,
+    hipLaunchKernelGGL(knn_set_grid_kernel, dim3(1), dim3(64), 0, st, g, dst);
+}
+
+void launch_knn_refine_grid(const float* sample, int samples, KnnGrid* g, uint32_t budget, hipStream_t st)
+{
+    hipLaunchKernelGGL(knn_refine_grid_kernel, dim3(1), dim3(1024), 0, st, sample, samples, g, budget);
+}
+
+int knn_num_samples(int n) { return n < kKnnSamples ? n : kKnnSamples; }
+
+// count, prefix sum and scatter of the points into the cells of *g (device)
+void launch_knn_build(const float4* position, int n, const KnnGrid* g, uint32_t max_cells, uint32_t* count,
+                      uint32_t* offset, uint32_t* chunk_sum, float4* sorted, hipStream_t st)
+{
+    const int chunks = (int)((max_cells + kScanChunk - 1) / kScanChunk);
+    const int blocks = chunks < 1024 ? chunks : 1024;
+    const int clear  = (int)((max_cells / 4 + kBlock - 1) / kBlock);
+    hipLaunchKernelGGL(knn_clear_kernel, dim3(clear < 4096 ? (clear ? clear : 1) : 4096), dim3(kBlock), 0, st, count, g);
+    hipLaunchKernelGGL(knn_bin_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, 0, position, n, g, count,
+                       offset, sorted);
+    // chunk sums and their offsets share one array: [chunks] sums, [chunks + 1] offsets
+    hipLaunchKernelGGL(knn_scan_reduce_kernel, dim3(blocks), dim3(1024), 0, st, count, g, chunk_sum);
+    hipLaunchKernelGGL(knn_scan_chunks_kernel, dim3(1), dim3(1024), 0, st, chunk_sum, g, chunk_sum + chunks);
+    hipLaunchKernelGGL(knn_scan_apply_kernel, dim3(blocks), dim3(1024), 0, st, count, g, chunk_sum + chunks, offset);
+    hipLaunchKernelGGL(knn_bin_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, 1, position, n, g, count,
                        offset, sorted);
 }
 
-bool launch_knn_search(int rank, const float4* sorted, int n, const KnnGrid& g, const uint32_t* offset, float* out,
-                       hipStream_t st)
+size_t knn_chunk_words(uint32_t max_cells)
 {
-    const dim3 grid((n + kBlock - 1) / kBlock), block(kBlock);
+    const size_t chunks = (max_cells + kScanChunk - 1) / kScanChunk;
+    return 2 * chunks + 1;
+}
+
+bool launch_knn_search(int rank, const float4* sorted, int n, const KnnGrid* g, const uint32_t* offset, float* out,
+                       int samples, hipStream_t st)
+{
+    const dim3 block(kBlock);
+    const dim3 grid(samples > 0 ? (samples + kBlock / 64 - 1) / (kBlock / 64) : (n + kBlock - 1) / kBlock);
+#define ADOP_KNN_CASE(R)                                                                                         \
+    case R:                                                                                                      \
+        if (samples > 0)                                                                                         \
+            hipLaunchKernelGGL(knn_sample_kernel<R + 1>, grid, block, 0, st, sorted, n, g, offset, out, samples); \
+        else                                                                                                     \
+            hipLaunchKernelGGL(knn_search_kernel<R + 1>, grid, block, 0, st, sorted, n, g, offset, out);          \
+        return true;
     switch (rank)
     {
-        case 1: hipLaunchKernelGGL(knn_search_kernel<2>, grid, block, 0, st, sorted, n, g, offset, out); return true;
-        case 2: hipLaunchKernelGGL(knn_search_kernel<3>, grid, block, 0, st, sorted, n, g, offset, out); return true;
-        case 3: hipLaunchKernelGGL(knn_search_kernel<4>, grid, block, 0, st, sorted, n, g, offset, out); return true;
-        case 4: hipLaunchKernelGGL(knn_search_kernel<5>, grid, block, 0, st, sorted, n, g, offset, out); return true;
-        case 5: hipLaunchKernelGGL(knn_search_kernel<6>, grid, block, 0, st, sorted, n, g, offset, out); return true;
-        case 6: hipLaunchKernelGGL(knn_search_kernel<7>, grid, block, 0, st, sorted, n, g, offset, out); return true;
-        case 7: hipLaunchKernelGGL(knn_search_kernel<8>, grid, block, 0, st, sorted, n, g, offset, out); return true;
-        case 8: hipLaunchKernelGGL(knn_search_kernel<9>, grid, block, 0, st, sorted, n, g, offset, out); return true;
+        ADOP_KNN_CASE(1)
+        ADOP_KNN_CASE(2)
+        ADOP_KNN_CASE(3)
+        ADOP_KNN_CASE(4)
+        ADOP_KNN_CASE(5)
+        ADOP_KNN_CASE(6)
+        ADOP_KNN_CASE(7)
+        ADOP_KNN_CASE(8)
     }
+#undef ADOP_KNN_CASE
     return false;
 }
 
@@ -258,7 +559,7 @@ void launch_camera_distance(const float4* position, int n, const ViewConst* view
                        num_frames, out);
 }
 
-void launch_close_points(const float4* sorted, int n, const KnnGrid& g, const uint32_t* offset, const float* radius,
+void launch_close_points(const float4* sorted, int n, const KnnGrid* g, const uint32_t* offset, const float* radius,
                          int32_t* state, uint32_t* round_count, int round, hipStream_t st)
 {
     hipLaunchKernelGGL(close_points_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, sorted, n, g, offset,

@@ -115,7 +115,8 @@ def bench_preprocess(args):
             cam = r
         filt[name] = round(sorted(ts)[1], 3)
     # algorithmic bytes of the neighbour search: the cloud is read twice and written once in cell order (binning),
-    # read once more by the search, 4 bytes per point out; neighbours are read through the caches
+    # read once more by the search, 4 bytes per point out; neighbours are read through the caches (the library bins
+    # twice, for its first and second grid: its choice, not the algorithm's)
     knn_bytes = N * (16 + 16 + 16 + 16 + 4)
     cpu = None
     if not args.no_cpu_baseline:
