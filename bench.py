@@ -205,7 +205,7 @@ def main():
     B, N, Cn, L = hs.batch, hs.num_points, hs.num_channels, hs.num_layers
     ws = C.c_void_p(cache.workspace.data_ptr())
     ws_n = cache.workspace.numel()
-    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    stream_of = [C.c_void_p(torch.cuda.current_stream().cuda_stream)]
 
     gb = None
     keep = []
@@ -235,12 +235,12 @@ def main():
         if args.workload == "config4":
             views[0].image_index = frame[0] % scene.poses_se3.shape[0]  # orbit
             frame[0] += 1
-        rc = lib.adop_forward(C.byref(s), views, B, C.byref(hs.params), C.byref(fb), ws, ws_n, stats, stream)
+        rc = lib.adop_forward(C.byref(s), views, B, C.byref(hs.params), C.byref(fb), ws, ws_n, stats, stream_of[0])
         if rc != 0:
             raise RuntimeError(lib.adop_last_error_string().decode())
         if backward:
             rc = lib.adop_backward(C.byref(s), views, B, C.byref(hs.params), C.byref(fb), C.byref(gb), ws, ws_n,
-                                   stats, stream)
+                                   stats, stream_of[0])
             if rc != 0:
                 raise RuntimeError(lib.adop_last_error_string().decode())
 
@@ -278,6 +278,27 @@ def main():
     n = lib.adop_profile_read(arr, 16)
     lib.adop_profile_enable(0)
     stages = {arr[i].name.decode(): arr[i].total_ms / args.steps for i in range(n)}  # ms per step
+
+    # the same step recorded once into a HIP graph and replayed (outside the timed region above: what the host-side
+    # launches cost); configuration 4 changes a host-side argument every frame and is not recorded
+    graph_ms = None
+    if args.workload != "config4":
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        eager_stream = stream_of[0]
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                stream_of[0] = C.c_void_p(side.cuda_stream)
+                step()
+        stream_of[0] = eager_stream
+        for _ in range(max(args.warmup, 1)):
+            graph.replay()
+        torch.cuda.synchronize()
+        tg = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - tg) * 1e3 / args.steps
 
     P = sum(w * h for (w, h) in hs.level_sizes())
     S_d = 2 if hs.texture.dtype == np.float16 else 4
@@ -358,7 +379,8 @@ def main():
                  "hbm_frac": round(step_gbs / HBM_PEAK_GBS, 4),
                  "stage_ms": {k: round(v, 4) for k, v in stages.items()},
                  "stage_GBps": {k: round(model[k] / (stages[k] * 1e-3) / 1e9, 1) for k in model if k in stages},
-                 "visible": V, "accepted": A, "spatial": G, "scene_gen_s": round(gen_s, 1)},
+                 "visible": V, "accepted": A, "spatial": G, "scene_gen_s": round(gen_s, 1),
+                 "graph_replay_ms_per_step": None if graph_ms is None else round(graph_ms, 4)},
     }
     print(json.dumps(out))
 
