@@ -244,12 +244,20 @@ def main():
             if rc != 0:
                 raise RuntimeError(lib.adop_last_error_string().decode())
 
+    copy_gbs = None
     if args.calibrate_copy:
+        # plain device copy of 1 GiB (2 GiB of traffic): what the memory system delivers to the simplest kernel
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
         dst = torch.empty_like(src)
         for _ in range(3):
             dst.copy_(src)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            dst.copy_(src)
+        e1.record()
         torch.cuda.synchronize()
+        copy_gbs = 10 * 2 * src.numel() * 4 / (e0.elapsed_time(e1) * 1e-3) / 1e9
         del src, dst
 
     # untimed pass with counters: V_l, A_l, G_l of the byte model
@@ -380,7 +388,8 @@ def main():
                  "stage_ms": {k: round(v, 4) for k, v in stages.items()},
                  "stage_GBps": {k: round(model[k] / (stages[k] * 1e-3) / 1e9, 1) for k in model if k in stages},
                  "visible": V, "accepted": A, "spatial": G, "scene_gen_s": round(gen_s, 1),
-                 "graph_replay_ms_per_step": None if graph_ms is None else round(graph_ms, 4)},
+                 "graph_replay_ms_per_step": None if graph_ms is None else round(graph_ms, 4),
+                 "device_copy_GBps": None if copy_gbs is None else round(copy_gbs, 1)},
     }
     print(json.dumps(out))
 
