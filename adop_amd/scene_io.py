@@ -50,6 +50,31 @@ def _fmt(values):
     return " ".join(f"{float(v):.15e}" for v in values)  # setprecision(15) << scientific, SceneData.h:169
 
 
+def _bool(text):
+    return text.strip().lower() in ("1", "true", "yes", "on")
+
+
+def RenderParamsFromIni(path):
+    """The [RenderParams] section of one of the reference's experiment files (configs/train_*.ini; RenderParams,
+    Settings.h:22-52) -> (adop render params, dropout probability).  Keys the section does not hold keep the
+    reference's defaults."""
+    from . import scenes
+    sec = read_ini(path).get("RenderParams", {})
+    assert not _bool(sec.get("render_outliers", "false")), "the outlier cloud is a dead path in the reference"
+    p = scenes.default_params(check_normal=1, ghost_gradients=0, drop_out_points_by_radius=1, depth_accept=0.01,
+                              drop_out_radius_threshold=0.6, distortion_gradient_factor=0.005,
+                              K_gradient_factor=0.5)  # the defaults of Settings.h:22-47
+    for key in ("check_normal", "ghost_gradients", "drop_out_points_by_radius"):
+        if key in sec:
+            setattr(p, key, int(_bool(sec[key])))
+    for key in ("drop_out_radius_threshold", "depth_accept", "distortion_gradient_factor", "K_gradient_factor"):
+        if key in sec:
+            setattr(p, key, float(sec[key]))
+    if "test_backward_mode" in sec:
+        p.test_backward_mode = int(sec["test_backward_mode"])
+    return p, float(sec.get("dropout", 0.25))
+
+
 @dataclass
 class SceneCameraParams:
     """data/SceneData.h:153-290"""

@@ -212,3 +212,25 @@ def test_train_sampler_views(tmp_path):
     views, zoom = full.Get(0)
     assert [(v.w, v.h, v.crop_fx, v.crop_cx, v.crop_cy) for v in views] == [(640, 480, 1.0, 0.0, 0.0)] * 2
     assert list(zoom) == [1.0, 1.0]
+
+
+def test_render_params_from_an_experiment_file(tmp_path):
+    # the section as the reference's experiment files hold it (values of its boat experiment)
+    write(tmp_path / "train.ini", "[TrainParams]\nbatch_size = 4\n\n[RenderParams]\nrender_outliers = false\n"
+          "check_normal = true\nghost_gradients = true\ndrop_out_points_by_radius = true\noutlier_count = 1000000\n"
+          "drop_out_radius_threshold = 0.6000000238\ndropout = 0.2500000000\ndepth_accept = 0.0099999998\n"
+          "test_backward_mode = 0\ndistortion_gradient_factor = 0.0099999998\nK_gradient_factor = 0.5000000000\n\n"
+          "[PipelineParams]\ntrain = true\n")
+    p, dropout = scene_io.RenderParamsFromIni(str(tmp_path / "train.ini"))
+    assert (p.check_normal, p.ghost_gradients, p.drop_out_points_by_radius, p.test_backward_mode) == (1, 1, 1, 0)
+    assert dropout == 0.25
+    assert np.float32(p.depth_accept) == np.float32(0.01) and np.float32(p.drop_out_radius_threshold) == np.float32(0.6)
+    assert np.float32(p.distortion_gradient_factor) == np.float32(0.01) and p.K_gradient_factor == 0.5
+    # a file without the section: the defaults of the reference's struct
+    write(tmp_path / "empty.ini", "[TrainParams]\nbatch_size = 1\n")
+    p, dropout = scene_io.RenderParamsFromIni(str(tmp_path / "empty.ini"))
+    assert (p.check_normal, p.ghost_gradients, p.drop_out_points_by_radius, dropout) == (1, 0, 1, 0.25)
+    assert np.float32(p.distortion_gradient_factor) == np.float32(0.005)
+    write(tmp_path / "outliers.ini", "[RenderParams]\nrender_outliers = true\n")
+    with pytest.raises(AssertionError, match="outlier"):
+        scene_io.RenderParamsFromIni(str(tmp_path / "outliers.ini"))
