@@ -706,11 +706,8 @@ adop_status adop_apply_tangent(double* tangent, double* poses_se3, int32_t num_p
     return ADOP_OK;
 }
 
-// Grids of the nearest-neighbour search.  The first one is sized on the host for ~8 points per cell of a volume-filling
-// cloud, at most kKnnCoarseDim cells per axis; the second one on the device from the neighbour distances of sample
-// points, within a budget of cells that grows with the cloud.
-static constexpr int kKnnCoarseDim = 160;
-
+// Grids of the nearest-neighbour search: both are sized on the device (preprocess_kernels.hip), the second one within a
+// budget of cells that grows with the cloud.
 static uint32_t knn_max_cells(int32_t num_points)
 {
     size_t want = (size_t)(num_points > 0 ? num_points : 0) * 16;
@@ -719,31 +716,41 @@ static uint32_t knn_max_cells(int32_t num_points)
     return (uint32_t)want;
 }
 
+constexpr uint32_t kKnnFirstCells = 160u * 160u * 160u;  // the first grid has at most 160 cells per axis
+
 struct KnnWorkspace
 {
-    KnnGrid* grid;  // device
+    KnnGrid *grid, *grid0;  // second (search) grid and first grid, device
     float* sample;
-    uint32_t *count, *offset, *chunk;
-    float4* sorted;
+    uint32_t *count, *offset, *chunk;  // second grid
+    uint32_t *count0, *offset0;        // first grid
+    float4 *sorted, *sorted0;
+    uint32_t *list, *list2, *counts;
     size_t total;
 };
 
 static KnnWorkspace knn_layout(void* workspace, int32_t num_points)
 {
     const uint32_t cells = knn_max_cells(num_points);
+    const size_t n       = (size_t)(num_points > 0 ? num_points : 0);
     size_t o             = 0;
-    const size_t o_grid  = o;
-    o                    = align_up(o + sizeof(KnnGrid), 256);
-    const size_t o_sample = o;
-    o                    = align_up(o + sizeof(float) * 2048, 256);
-    const size_t o_count = o;
-    o                    = align_up(o + sizeof(uint32_t) * (size_t)cells, 256);
-    const size_t o_offset = o;
-    o                    = align_up(o + sizeof(uint32_t) * ((size_t)cells + 1), 256);
-    const size_t o_chunk = o;
-    o                    = align_up(o + sizeof(uint32_t) * knn_chunk_words(cells), 256);
-    const size_t o_sorted = o;
-    o                    = align_up(o + sizeof(float4) * (size_t)(num_points > 0 ? num_points : 0), 256);
+    auto take            = [&](size_t bytes) {
+        const size_t at = o;
+        o               = align_up(o + bytes, 256);
+        return at;
+    };
+    const size_t o_grid = take(sizeof(KnnGrid)), o_grid0 = take(sizeof(KnnGrid));
+    const size_t o_sample  = take(sizeof(float) * 2048);
+    const size_t o_counts  = take(sizeof(uint32_t) * 2);
+    const size_t o_count   = take(sizeof(uint32_t) * (size_t)cells);
+    const size_t o_offset  = take(sizeof(uint32_t) * ((size_t)cells + 1));
+    const size_t o_chunk   = take(sizeof(uint32_t) * knn_chunk_words(cells));
+    const size_t o_count0  = take(sizeof(uint32_t) * (size_t)kKnnFirstCells);
+    const size_t o_offset0 = take(sizeof(uint32_t) * ((size_t)kKnnFirstCells + 1));
+    const size_t o_sorted  = take(sizeof(float4) * n);
+    const size_t o_sorted0 = take(sizeof(float4) * n);
+    const size_t o_list    = take(sizeof(uint32_t) * n);
+    const size_t o_list2   = take(sizeof(uint32_t) * n);
     KnnWorkspace w;
     memset(&w, 0, sizeof(w));
     w.total = o;
@@ -751,11 +758,18 @@ static KnnWorkspace knn_layout(void* workspace, int32_t num_points)
     {
         char* base = (char*)workspace;
         w.grid     = (KnnGrid*)(base + o_grid);
+        w.grid0    = (KnnGrid*)(base + o_grid0);
         w.sample   = (float*)(base + o_sample);
+        w.counts   = (uint32_t*)(base + o_counts);
         w.count    = (uint32_t*)(base + o_count);
         w.offset   = (uint32_t*)(base + o_offset);
         w.chunk    = (uint32_t*)(base + o_chunk);
+        w.count0   = (uint32_t*)(base + o_count0);
+        w.offset0  = (uint32_t*)(base + o_offset0);
         w.sorted   = (float4*)(base + o_sorted);
+        w.sorted0  = (float4*)(base + o_sorted0);
+        w.list     = (uint32_t*)(base + o_list);
+        w.list2    = (uint32_t*)(base + o_list2);
     }
     return w;
 }
@@ -776,38 +790,25 @@ static adop_status knn_prepare(const float* position, int32_t num_points, const 
         return fail(ADOP_WORKSPACE_TOO_SMALL, "workspace too small");
     *out = knn_layout(workspace, num_points);
     if (!build) return ADOP_OK;
-    KnnGrid g;
-    memset(&g, 0, sizeof(g));
+    KnnGrid box;  // the caller's bounding box; the grids are sized on the device
+    memset(&box, 0, sizeof(box));
     for (int k = 0; k < 3; ++k)
     {
-        g.ext[k] = bbox_max[k] - bbox_min[k];
-        if (!(g.ext[k] >= 0) || !(g.ext[k] < 1.0e30f)) return fail(ADOP_INVALID_ARG, "bounding box is not finite");
-    }
-    const float* ext    = g.ext;
-    const float longest = ext[0] > ext[1] ? (ext[0] > ext[2] ? ext[0] : ext[2]) : (ext[1] > ext[2] ? ext[1] : ext[2]);
-    double volume       = 1.0;
-    for (int k = 0; k < 3; ++k) volume *= ext[k] > 1e-6f * longest ? ext[k] : (longest > 0 ? 1e-6 * longest : 1.0);
-    float cell = (float)cbrt(volume * 8.0 / (double)num_points);
-    if (!(cell > longest / kKnnCoarseDim)) cell = longest / kKnnCoarseDim;
-    if (!(cell > 0)) cell = 1.f;  // all points coincide
-    g.cell     = cell;
-    g.inv_cell = 1.0f / cell;
-    g.cells    = 1;
-    for (int k = 0; k < 3; ++k)
-    {
-        g.min[k] = bbox_min[k];
-        int d    = (int)(ext[k] / cell) + 1;
-        g.dim[k] = d < 1 ? 1 : (d > kKnnCoarseDim ? kKnnCoarseDim : d);
-        g.cells *= (uint32_t)g.dim[k];
+        box.min[k] = bbox_min[k];
+        box.ext[k] = bbox_max[k] - bbox_min[k];
+        if (!(box.ext[k] >= 0) || !(box.ext[k] < 1.0e30f)) return fail(ADOP_INVALID_ARG, "bounding box is not finite");
     }
     const uint32_t max_cells = knn_max_cells(num_points);
     const float4* pos        = (const float4*)position;
-    launch_knn_set_grid(g, out->grid, stream);
-    launch_knn_build(pos, num_points, out->grid, max_cells, out->count, out->offset, out->chunk, out->sorted, stream);
+    // first grid (kept: the search falls back on it for points in sparse parts of the cloud)
+    launch_knn_first_grid(pos, num_points, box, out->grid0, stream);
+    launch_knn_build(pos, num_points, out->grid0, kKnnFirstCells, out->count0, out->offset0, out->chunk, out->sorted0,
+                     stream);
     const int samples = knn_num_samples(num_points);
-    if (!launch_knn_search(sample_rank, out->sorted, num_points, out->grid, out->offset, out->sample, samples, stream))
+    if (!launch_knn_sample(sample_rank, out->sorted0, num_points, out->grid0, out->offset0, out->sample, samples, stream))
         return fail(ADOP_INVALID_ARG, "rank must be 1..8");
-    launch_knn_refine_grid(out->sample, samples, out->grid, max_cells, stream);
+    // second grid
+    launch_knn_refine_grid(out->sample, samples, out->grid0, out->grid, max_cells, stream);
     launch_knn_build(pos, num_points, out->grid, max_cells, out->count, out->offset, out->chunk, out->sorted, stream);
     return ADOP_OK;
 }
@@ -824,7 +825,9 @@ adop_status adop_knn_distance(const float* position, int32_t num_points, int32_t
     adop_status st =
         knn_prepare(position, num_points, bbox_min, bbox_max, rank, workspace, workspace_bytes, true, stream, &w);
     if (st != ADOP_OK) return st;
-    if (!launch_knn_search(rank, w.sorted, num_points, w.grid, w.offset, out_distance, 0, stream))
+    if ((st = fill_async(w.counts, 2 * sizeof(uint32_t), 0, stream)) != ADOP_OK) return st;
+    KnnSearchArg a{w.grid, w.grid0, w.sorted, w.sorted0, w.offset, w.offset0, w.list, w.list2, w.counts};
+    if (!launch_knn_search(rank, num_points, a, out_distance, stream))
         return fail(ADOP_INVALID_ARG, "rank must be 1..8");
     ADOP_HIP_CHECK(hipGetLastError());
     return ADOP_OK;

@@ -16,14 +16,24 @@ void launch_prepare_views(const ViewChunk& ch, int first, int count, const doubl
 void launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t st);
 void launch_clear(const Levels& lv, int first_level, int grid, float* accum, size_t accum_floats, uint32_t* zero_u32,
                   int zero_n, const ViewPrep& vp, hipStream_t st);
-void launch_knn_set_grid(const KnnGrid& g, KnnGrid* dst, hipStream_t st);
-void launch_knn_refine_grid(const float* sample, int samples, KnnGrid* g, uint32_t budget, hipStream_t st);
+void launch_knn_first_grid(const float4* position, int n, const KnnGrid& box, KnnGrid* dst, hipStream_t st);
+void launch_knn_refine_grid(const float* sample, int samples, const KnnGrid* first, KnnGrid* g, uint32_t budget,
+                            hipStream_t st);
 int knn_num_samples(int n);
 size_t knn_chunk_words(uint32_t max_cells);  // uint32 words of the scan's scratch array
 void launch_knn_build(const float4* position, int n, const KnnGrid* g, uint32_t max_cells, uint32_t* count,
                       uint32_t* offset, uint32_t* chunk_sum, float4* sorted, hipStream_t st);
-bool launch_knn_search(int rank, const float4* sorted, int n, const KnnGrid* g, const uint32_t* offset, float* out,
+bool launch_knn_sample(int rank, const float4* sorted, int n, const KnnGrid* g, const uint32_t* offset, float* out,
                        int samples, hipStream_t st);
+struct KnnSearchArg
+{
+    const KnnGrid *grid, *grid0;          // second / first grid (device)
+    const float4 *sorted, *sorted0;       // the points in cell order of either grid
+    const uint32_t *offset, *offset0;
+    uint32_t *list, *list2;               // [n] points left over by the first / second stage
+    uint32_t* counts;                     // [2] their numbers, zero at the start
+};
+bool launch_knn_search(int rank, int n, const KnnSearchArg& a, float* out, hipStream_t st);
 void launch_camera_distance(const float4* position, int n, const ViewConst* views, int num_frames, float* out,
                             hipStream_t st);
 void launch_close_points(const float4* sorted, int n, const KnnGrid* g, const uint32_t* offset, const float* radius,

@@ -10,8 +10,10 @@
 // search order and whatever the grid, so a brute-force search over the same arithmetic gives the same bits.
 // The cost is the number of candidates, which the cell size decides, and the right cell size depends on how the cloud
 // fills space (scans are surfaces: a grid sized by volume puts hundreds of points into the few cells that have any).
-// So the search runs twice: on a coarse grid sized by volume for 2048 sample points only, then, with cells of twice
-// the median distance those found, for all points.  The second grid is computed on the device (no host round trip).
+// So there are two grids, both sized on the device (no host round trip): a first one sized by volume, on which 2048
+// sample points are searched, and a second one with cells of twice the median distance those found.  All points are
+// searched on the second grid (2 shells at most), what that leaves on the first (4 shells), and the stray points
+// neither settles against all points.
 #include "common.h"
 #include "launch.h"
 
@@ -19,15 +21,14 @@
 
 namespace adop
 {
+// Cell of a point; points outside the grid's box (the box leaves the far tails of the cloud out) belong to the nearest
+// boundary cell.
 __device__ __forceinline__ int3 grid_cell(const KnnGrid& g, float x, float y, float z)
 {
-    int cx = (int)((x - g.min[0]) * g.inv_cell);
-    int cy = (int)((y - g.min[1]) * g.inv_cell);
-    int cz = (int)((z - g.min[2]) * g.inv_cell);
-    cx     = cx < 0 ? 0 : (cx >= g.dim[0] ? g.dim[0] - 1 : cx);
-    cy     = cy < 0 ? 0 : (cy >= g.dim[1] ? g.dim[1] - 1 : cy);
-    cz     = cz < 0 ? 0 : (cz >= g.dim[2] ? g.dim[2] - 1 : cz);
-    return make_int3(cx, cy, cz);
+    const float fx = fminf(fmaxf((x - g.min[0]) * g.inv_cell, 0.f), (float)(g.dim[0] - 1));
+    const float fy = fminf(fmaxf((y - g.min[1]) * g.inv_cell, 0.f), (float)(g.dim[1] - 1));
+    const float fz = fminf(fmaxf((z - g.min[2]) * g.inv_cell, 0.f), (float)(g.dim[2] - 1));
+    return make_int3((int)fx, (int)fy, (int)fz);
 }
 
 __device__ __forceinline__ uint32_t grid_index(const KnnGrid& g, int cx, int cy, int cz)
@@ -52,22 +53,17 @@ __global__ __launch_bounds__(kBlock) void knn_bin_kernel(int pass, const float4*
         sorted[offset[ci] + atomicSub(&count[ci], 1u) - 1u] = make_float4(p.x, p.y, p.z, __uint_as_float((uint32_t)i));
 }
 
-// One thread per point, in cell order (the lanes of a wavefront search nearly the same cells).  The cube of cells
-// around the point's cell grows until the K-th best distance cannot be beaten from outside it; a row of cells along x
-// is one contiguous run of the cell-ordered array, so a cube of (2r+1)^3 cells is (2r+1)^2 runs.  A larger cube is
-// searched from scratch (the first cube, r = 1, settles nearly every point).
+// The search of one point by one thread: the cube of cells around the point's cell grows until the K-th best distance
+// cannot be beaten from outside it; a row of cells along x is one contiguous run of the cell-ordered array, so a cube
+// of (2r+1)^3 cells is (2r+1)^2 runs.  A larger cube is searched from scratch (the first cube, r = 1, settles nearly
+// every point).  Gives up after rmax shells: false, and the caller hands the point to the next, coarser stage.
 template <int K>  // K = n + 1 best squared distances are kept (the point itself is one of them)
-__global__ __launch_bounds__(kBlock) void knn_search_kernel(const float4* __restrict__ sorted, int n,
-                                                            const KnnGrid* __restrict__ gp,
-                                                            const uint32_t* __restrict__ offset, float* __restrict__ out)
+__device__ __forceinline__ bool knn_cubes(const float4 p, const KnnGrid& g, const float4* __restrict__ sorted,
+                                          const uint32_t* __restrict__ offset, int rmax, float* kth)
 {
-    const int t = blockIdx.x * kBlock + threadIdx.x;
-    if (t >= n) return;
-    const KnnGrid g = *gp;
-    const float4 p  = sorted[t];
-    const int3 c    = grid_cell(g, p.x, p.y, p.z);
+    const int3 c = grid_cell(g, p.x, p.y, p.z);
     float best[K];
-    for (int r = 1;; ++r)
+    for (int r = 1; r <= rmax; ++r)
     {
 #pragma unroll
         for (int k = 0; k < K; ++k) best[k] = 3.0e38f;
@@ -106,17 +102,150 @@ __global__ __launch_bounds__(kBlock) void knn_search_kernel(const float4* __rest
         if (c.x + r < g.dim[0] - 1) bound = fminf(bound, (g.min[0] + (float)(c.x + r + 1) * g.cell) - p.x);
         if (c.y + r < g.dim[1] - 1) bound = fminf(bound, (g.min[1] + (float)(c.y + r + 1) * g.cell) - p.y);
         if (c.z + r < g.dim[2] - 1) bound = fminf(bound, (g.min[2] + (float)(c.z + r + 1) * g.cell) - p.z);
-        if (bound == 3.0e38f) break;
         bound = fmaxf(bound, 0.f) * 0.999f;
-        if (best[K - 1] <= bound * bound) break;
+        if (bound >= 1.0e38f || best[K - 1] <= bound * bound)
+        {
+            *kth = best[K - 1];
+            return true;
+        }
     }
-    out[__float_as_uint(p.w)] = sqrtf(best[K - 1]);
+    return false;
 }
 
-// The same search for `samples` points evenly spaced in cell order, one wavefront per point (on the first grid a
-// point has thousands of candidates: the lanes share them, every lane keeps the K best of its share, and the K-th
-// best of the wavefront is found by K rounds of taking the smallest head off the lanes' lists).  out[s] = distance
-// of sample s.  All branches on r, the bound and the result are uniform over the wavefront.
+// Appends `value` of the lanes with `push` to a list (one atomic per wavefront).  Called by all lanes of a wavefront.
+__device__ __forceinline__ void wave_push(bool push, uint32_t value, uint32_t* __restrict__ list, uint32_t* count)
+{
+    const unsigned long long m = __ballot(push);
+    if (!m) return;
+    const int lane   = threadIdx.x & 63;
+    const int leader = __ffsll((long long)m) - 1;
+    uint32_t base    = 0;
+    if (lane == leader) base = atomicAdd(count, (uint32_t)__popcll(m));
+    base = (uint32_t)__shfl((int)base, leader, 64);
+    if (push) list[base + (uint32_t)__popcll(m & ((1ull << lane) - 1ull))] = value;
+}
+
+// Stage 1: every point, one thread each in cell order of the second grid (the lanes of a wavefront search nearly the
+// same cells), at most 2 shells; what is left (points in sparse parts of the cloud) goes to list.
+template <int K>
+__global__ __launch_bounds__(kBlock) void knn_search_kernel(const float4* __restrict__ sorted, int n,
+                                                            const KnnGrid* __restrict__ gp,
+                                                            const uint32_t* __restrict__ offset, float* __restrict__ out,
+                                                            uint32_t* __restrict__ list, uint32_t* list_count)
+{
+    const int t = blockIdx.x * kBlock + threadIdx.x;
+    bool left   = false;
+    if (t < n)
+    {
+        const KnnGrid g = *gp;
+        const float4 p  = sorted[t];
+        float kth;
+        if (knn_cubes<K>(p, g, sorted, offset, 2, &kth))
+            out[__float_as_uint(p.w)] = sqrtf(kth);
+        else
+            left = true;
+    }
+    wave_push(left, (uint32_t)t, list, list_count);
+}
+
+// Stage 2: the points stage 1 left, on the first (coarser) grid, at most 4 shells; the rest goes to list2.
+template <int K>
+__global__ __launch_bounds__(kBlock) void knn_list_kernel(const float4* __restrict__ points,
+                                                          const uint32_t* __restrict__ list,
+                                                          const uint32_t* __restrict__ list_count,
+                                                          const float4* __restrict__ sorted0,
+                                                          const KnnGrid* __restrict__ gp0,
+                                                          const uint32_t* __restrict__ offset0, float* __restrict__ out,
+                                                          uint32_t* __restrict__ list2, uint32_t* list2_count)
+{
+    const uint32_t count = *list_count;
+    const KnnGrid g      = *gp0;
+    const uint32_t lane  = threadIdx.x & 63;
+    for (uint32_t e0 = blockIdx.x * kBlock + (threadIdx.x & ~63u); e0 < count; e0 += gridDim.x * kBlock)  // wavefront-uniform
+    {
+        const uint32_t e = e0 + lane;
+        bool left        = false;
+        uint32_t t       = 0;
+        if (e < count)
+        {
+            t              = list[e];
+            const float4 p = points[t];
+            float kth;
+            if (knn_cubes<K>(p, g, sorted0, offset0, 4, &kth))
+                out[__float_as_uint(p.w)] = sqrtf(kth);
+            else
+                left = true;
+        }
+        wave_push(left, t, list2, list2_count);
+    }
+}
+
+// K-th smallest of the union of the lanes' ascending lists (destroys them): K rounds of taking the smallest head.
+template <int K>
+__device__ __forceinline__ float wave_kth(float* best)
+{
+    const int lane = threadIdx.x & 63;
+    float kth      = 3.0e38f;
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+    {
+        float m = best[0];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) m = fminf(m, __shfl_xor(m, off, 64));
+        kth = m;
+        const unsigned long long holders = __ballot(best[0] == m);
+        if (lane == __ffsll((long long)holders) - 1)
+        {
+#pragma unroll
+            for (int j = 0; j + 1 < K; ++j) best[j] = best[j + 1];
+            best[K - 1] = 3.0e38f;
+        }
+    }
+    return kth;
+}
+
+// Stage 3: stray points far from everything (no cube of a few shells of either grid settles them): one wavefront
+// per point goes through all points.
+template <int K>
+__global__ __launch_bounds__(kBlock) void knn_brute_kernel(const float4* __restrict__ points, int n,
+                                                           const uint32_t* __restrict__ list,
+                                                           const uint32_t* __restrict__ list_count,
+                                                           float* __restrict__ out)
+{
+    const uint32_t count = *list_count;
+    const int lane       = threadIdx.x & 63;
+    for (uint32_t e = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6); e < count; e += gridDim.x * (kBlock / 64))
+    {
+        const float4 p = points[list[e]];
+        float best[K];
+#pragma unroll
+        for (int k = 0; k < K; ++k) best[k] = 3.0e38f;
+        for (int q = lane; q < n; q += 64)
+        {
+            const float4 o = points[q];
+            const float dx = p.x - o.x, dy = p.y - o.y, dz = p.z - o.z;
+            float d2 = (dx * dx + dy * dy) + dz * dz;
+            if (d2 < best[K - 1])
+            {
+#pragma unroll
+                for (int k = 0; k < K; ++k)
+                {
+                    const float b = best[k];
+                    const bool lt = d2 < b;
+                    best[k]       = lt ? d2 : b;
+                    d2            = lt ? b : d2;
+                }
+            }
+        }
+        const float kth = wave_kth<K>(best);
+        if (lane == 0) out[__float_as_uint(p.w)] = sqrtf(kth);
+    }
+}
+
+// The search of stage 1 for `samples` points evenly spaced in cell order, one wavefront per point (on the first grid a
+// point has thousands of candidates: the lanes share them, every lane keeps the K best of its share).  out[s] =
+// distance of sample s, 3e38 for a sample that 4 shells do not settle (a stray point: it shall not size the grid).
+// All branches on r, the bound and the result are uniform over the wavefront.
 template <int K>
 __global__ __launch_bounds__(kBlock) void knn_sample_kernel(const float4* __restrict__ sorted, int n,
                                                             const KnnGrid* __restrict__ gp,
@@ -130,8 +259,8 @@ __global__ __launch_bounds__(kBlock) void knn_sample_kernel(const float4* __rest
     const KnnGrid g = *gp;
     const float4 p  = sorted[t];
     const int3 c    = grid_cell(g, p.x, p.y, p.z);
-    float kth       = 3.0e38f;
-    for (int r = 1;; ++r)
+    float result    = 3.0e38f;
+    for (int r = 1; r <= 4; ++r)
     {
         float best[K];
 #pragma unroll
@@ -162,22 +291,7 @@ __global__ __launch_bounds__(kBlock) void knn_sample_kernel(const float4* __rest
                     }
                 }
             }
-        // K-th smallest over the lanes' ascending lists
-#pragma unroll
-        for (int k = 0; k < K; ++k)
-        {
-            float m = best[0];
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) m = fminf(m, __shfl_xor(m, off, 64));
-            kth = m;
-            const unsigned long long holders = __ballot(best[0] == m);
-            if (lane == __ffsll((long long)holders) - 1)
-            {
-#pragma unroll
-                for (int j = 0; j + 1 < K; ++j) best[j] = best[j + 1];
-                best[K - 1] = 3.0e38f;
-            }
-        }
+        const float kth = wave_kth<K>(best);
         float bound = 3.0e38f;
         if (c.x - r > 0) bound = fminf(bound, p.x - (g.min[0] + (float)(c.x - r) * g.cell));
         if (c.y - r > 0) bound = fminf(bound, p.y - (g.min[1] + (float)(c.y - r) * g.cell));
@@ -185,32 +299,23 @@ __global__ __launch_bounds__(kBlock) void knn_sample_kernel(const float4* __rest
         if (c.x + r < g.dim[0] - 1) bound = fminf(bound, (g.min[0] + (float)(c.x + r + 1) * g.cell) - p.x);
         if (c.y + r < g.dim[1] - 1) bound = fminf(bound, (g.min[1] + (float)(c.y + r + 1) * g.cell) - p.y);
         if (c.z + r < g.dim[2] - 1) bound = fminf(bound, (g.min[2] + (float)(c.z + r + 1) * g.cell) - p.z);
-        if (bound == 3.0e38f) break;
         bound = fmaxf(bound, 0.f) * 0.999f;
-        if (kth <= bound * bound) break;
+        if (bound >= 1.0e38f || kth <= bound * bound)
+        {
+            result = sqrtf(kth);
+            break;
+        }
     }
-    if (lane == 0) out[slot] = sqrtf(kth);
+    if (lane == 0) out[slot] = result;
 }
 
-// The grid a host-side choice starts from, placed in device memory.
-__global__ void knn_set_grid_kernel(KnnGrid g, KnnGrid* __restrict__ dst)
-{
-    if (blockIdx.x == 0 && threadIdx.x == 0) *dst = g;
-}
+constexpr int kKnnSamples   = 2048;
+constexpr int kKnnMaxDim    = 2048;
+constexpr int kKnnCoarseDim = 160;
 
-// Second grid: cells of twice the median sampled neighbour distance (a cube of 3 cells then settles every point whose
-// own distance is below twice the median, with ~60 candidates on a surface, ~260 in a volume), never coarser than the
-// first grid, at most kKnnMaxDim cells per axis and `budget` cells in all.  One workgroup; the samples are sorted in
-// LDS (bitonic network).
-constexpr int kKnnSamples = 2048;
-constexpr int kKnnMaxDim  = 2048;
-
-__global__ __launch_bounds__(1024) void knn_refine_grid_kernel(const float* __restrict__ sample, int samples,
-                                                               KnnGrid* __restrict__ gp, uint32_t budget)
+// ascending bitonic sort of kKnnSamples floats in LDS by a workgroup of 1024 threads
+__device__ __forceinline__ void sort_samples(float* s)
 {
-    __shared__ float s[kKnnSamples];
-    for (int i = threadIdx.x; i < kKnnSamples; i += 1024) s[i] = i < samples ? sample[i] : 3.0e38f;
-    __syncthreads();
     for (int k = 2; k <= kKnnSamples; k <<= 1)
         for (int j = k >> 1; j > 0; j >>= 1)
         {
@@ -230,8 +335,83 @@ __global__ __launch_bounds__(1024) void knn_refine_grid_kernel(const float* __re
             }
             __syncthreads();
         }
+}
+
+// First grid.  Its box is not the bounding box of the cloud (one far outlier would stretch that until all other points
+// share a cell) but, per axis, the 1st to 99th percentile of 2048 points taken at equal steps through the array,
+// widened by 5 % of that range on either side and cut to the caller's box; the points outside it go to the boundary
+// cells, which keeps the search exact (a cube of cells then stands for a region open to the outside).  Cells for ~8
+// points each if the cloud filled the box, at most kKnnCoarseDim per axis.  One workgroup.
+__global__ __launch_bounds__(1024) void knn_first_grid_kernel(const float4* __restrict__ position, int n, KnnGrid box,
+                                                              KnnGrid* __restrict__ dst)
+{
+    __shared__ float s[kKnnSamples];
+    const int samples = n < kKnnSamples ? n : kKnnSamples;
+    float lo[3], hi[3];
+#pragma unroll
+    for (int axis = 0; axis < 3; ++axis)
+    {
+        for (int i = threadIdx.x; i < kKnnSamples; i += 1024)
+        {
+            float v = 3.0e38f;
+            if (i < samples)
+            {
+                const float4 p = position[(size_t)((long long)i * n / samples)];
+                v              = axis == 0 ? p.x : (axis == 1 ? p.y : p.z);
+            }
+            s[i] = v;
+        }
+        __syncthreads();
+        sort_samples(s);
+        const float a = s[samples / 100], b = s[samples - 1 - samples / 100];
+        const float box_hi = box.min[axis] + box.ext[axis];
+        lo[axis] = fmaxf(a - 0.05f * (b - a), box.min[axis]);
+        hi[axis] = fminf(b + 0.05f * (b - a), box_hi);
+        if (!(hi[axis] >= lo[axis]))  // not a number among the samples
+        {
+            lo[axis] = box.min[axis];
+            hi[axis] = box_hi;
+        }
+        __syncthreads();
+    }
     if (threadIdx.x != 0) return;
-    KnnGrid g          = *gp;
+    KnnGrid g;
+    for (int k = 0; k < 3; ++k)
+    {
+        g.min[k] = lo[k];
+        g.ext[k] = hi[k] - lo[k];
+    }
+    const float longest = fmaxf(g.ext[0], fmaxf(g.ext[1], g.ext[2]));
+    float volume        = 1.f;  // thin axes count as a millionth of the longest one
+    for (int k = 0; k < 3; ++k) volume *= g.ext[k] > 1e-6f * longest ? g.ext[k] : (longest > 0.f ? 1e-6f * longest : 1.f);
+    float cell = cbrtf(volume * 8.0f / (float)n);
+    if (!(cell > longest / kKnnCoarseDim)) cell = longest / kKnnCoarseDim;
+    if (!(cell > 0.f)) cell = 1.f;  // all samples coincide
+    g.cell     = cell;
+    g.inv_cell = 1.0f / cell;
+    g.cells    = 1;
+    for (int k = 0; k < 3; ++k)
+    {
+        int d    = (int)(g.ext[k] / cell) + 1;
+        g.dim[k] = d < 1 ? 1 : (d > kKnnCoarseDim ? kKnnCoarseDim : d);
+        g.cells *= (uint32_t)g.dim[k];
+    }
+    *dst = g;
+}
+
+// Second grid: cells of twice the median sampled neighbour distance (a cube of 3 cells then settles every point whose
+// own distance is below twice the median, with ~60 candidates on a surface, ~260 in a volume), never coarser than the
+// first grid, at most kKnnMaxDim cells per axis and `budget` cells in all, over the same box.  One workgroup.
+__global__ __launch_bounds__(1024) void knn_refine_grid_kernel(const float* __restrict__ sample, int samples,
+                                                               const KnnGrid* __restrict__ first,
+                                                               KnnGrid* __restrict__ gp, uint32_t budget)
+{
+    __shared__ float s[kKnnSamples];
+    for (int i = threadIdx.x; i < kKnnSamples; i += 1024) s[i] = i < samples ? sample[i] : 3.0e38f;
+    __syncthreads();
+    sort_samples(s);
+    if (threadIdx.x != 0) return;
+    KnnGrid g          = *first;
     const float median = s[samples / 2];
     const float longest = fmaxf(g.ext[0], fmaxf(g.ext[1], g.ext[2]));
     float cell = 2.0f * median;
@@ -489,14 +669,15 @@ __global__ __launch_bounds__(kBlock) void morton_kernel(const float4* __restrict
 // ------------------------------------------------------------------------------------------------
 // launchers
 // ------------------------------------------------------------------------------------------------
-void launch_knn_set_grid(const KnnGrid& g, KnnGrid* dst, hipStream_t st)
+void launch_knn_first_grid(const float4* position, int n, const KnnGrid& box, KnnGrid* dst, hipStream_t st)
 {
-    hipLaunchKernelGGL(knn_set_grid_kernel, dim3(1), dim3(64), 0, st, g, dst);
+    hipLaunchKernelGGL(knn_first_grid_kernel, dim3(1), dim3(1024), 0, st, position, n, box, dst);
 }
 
-void launch_knn_refine_grid(const float* sample, int samples, KnnGrid* g, uint32_t budget, hipStream_t st)
+void launch_knn_refine_grid(const float* sample, int samples, const KnnGrid* first, KnnGrid* g, uint32_t budget,
+                            hipStream_t st)
 {
-    hipLaunchKernelGGL(knn_refine_grid_kernel, dim3(1), dim3(1024), 0, st, sample, samples, g, budget);
+    hipLaunchKernelGGL(knn_refine_grid_kernel, dim3(1), dim3(1024), 0, st, sample, samples, first, g, budget);
 }
 
 int knn_num_samples(int n) { return n < kKnnSamples ? n : kKnnSamples; }
@@ -525,28 +706,37 @@ size_t knn_chunk_words(uint32_t max_cells)
     return 2 * chunks + 1;
 }
 
-bool launch_knn_search(int rank, const float4* sorted, int n, const KnnGrid* g, const uint32_t* offset, float* out,
+bool launch_knn_sample(int rank, const float4* sorted, int n, const KnnGrid* g, const uint32_t* offset, float* out,
                        int samples, hipStream_t st)
 {
-    const dim3 block(kBlock);
-    const dim3 grid(samples > 0 ? (samples + kBlock / 64 - 1) / (kBlock / 64) : (n + kBlock - 1) / kBlock);
-#define ADOP_KNN_CASE(R)                                                                                         \
-    case R:                                                                                                      \
-        if (samples > 0)                                                                                         \
-            hipLaunchKernelGGL(knn_sample_kernel<R + 1>, grid, block, 0, st, sorted, n, g, offset, out, samples); \
-        else                                                                                                     \
-            hipLaunchKernelGGL(knn_search_kernel<R + 1>, grid, block, 0, st, sorted, n, g, offset, out);          \
+    const dim3 block(kBlock), grid((samples + kBlock / 64 - 1) / (kBlock / 64));
+#define ADOP_KNN_CASE(R) \
+    case R: hipLaunchKernelGGL(knn_sample_kernel<R + 1>, grid, block, 0, st, sorted, n, g, offset, out, samples); return true;
+    switch (rank)
+    {
+        ADOP_KNN_CASE(1) ADOP_KNN_CASE(2) ADOP_KNN_CASE(3) ADOP_KNN_CASE(4)
+        ADOP_KNN_CASE(5) ADOP_KNN_CASE(6) ADOP_KNN_CASE(7) ADOP_KNN_CASE(8)
+    }
+#undef ADOP_KNN_CASE
+    return false;
+}
+
+// The three stages of the search: second grid (all points), first grid (what that left), all points (strays).
+bool launch_knn_search(int rank, int n, const KnnSearchArg& a, float* out, hipStream_t st)
+{
+    const dim3 block(kBlock), grid((n + kBlock - 1) / kBlock), grid2(512), grid3(1024);
+#define ADOP_KNN_CASE(R)                                                                                              \
+    case R:                                                                                                           \
+        hipLaunchKernelGGL(knn_search_kernel<R + 1>, grid, block, 0, st, a.sorted, n, a.grid, a.offset, out, a.list,   \
+                           a.counts);                                                                                 \
+        hipLaunchKernelGGL(knn_list_kernel<R + 1>, grid2, block, 0, st, a.sorted, a.list, a.counts, a.sorted0, a.grid0, \
+                           a.offset0, out, a.list2, a.counts + 1);                                                    \
+        hipLaunchKernelGGL(knn_brute_kernel<R + 1>, grid3, block, 0, st, a.sorted, n, a.list2, a.counts + 1, out);     \
         return true;
     switch (rank)
     {
-        ADOP_KNN_CASE(1)
-        ADOP_KNN_CASE(2)
-        ADOP_KNN_CASE(3)
-        ADOP_KNN_CASE(4)
-        ADOP_KNN_CASE(5)
-        ADOP_KNN_CASE(6)
-        ADOP_KNN_CASE(7)
-        ADOP_KNN_CASE(8)
+        ADOP_KNN_CASE(1) ADOP_KNN_CASE(2) ADOP_KNN_CASE(3) ADOP_KNN_CASE(4)
+        ADOP_KNN_CASE(5) ADOP_KNN_CASE(6) ADOP_KNN_CASE(7) ADOP_KNN_CASE(8)
     }
 #undef ADOP_KNN_CASE
     return false;

@@ -208,7 +208,8 @@ adop_status adop_apply_tangent(double* tangent, double* poses_se3, int32_t num_p
  * out_distance[i] = distance from point i to its `rank`-th nearest other point (the reference asks its tree for the
  * rank + 1 nearest, which include the point itself, and takes the last; rank = 4 there, 1..8 here), computed as
  * sqrt((dx*dx + dy*dy) + dz*dz) in fp32.  position [N,4] f32 (xyz used), N > rank; bbox_min / bbox_max: host
- * float[3], the bounding box of the cloud. */
+ * float[3], a box that contains the cloud (the search lays its grids over the bulk of the cloud inside it; points
+ * far from the rest cost a scan of all points each). */
 size_t adop_knn_workspace_size(int32_t num_points);
 adop_status adop_knn_distance(const float* position, int32_t num_points, int32_t rank, const float* bbox_min,
                               const float* bbox_max, float* out_distance, void* workspace, size_t workspace_bytes,

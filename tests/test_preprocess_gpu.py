@@ -221,3 +221,31 @@ def test_filter_point_cloud_composes_the_filters():
     keep2 = op.remove_close_points(q, (np.float32(0.00005) / cam2).astype(np.float32))
     assert np.array_equal(got, ids[keep2])
     assert 0 < (~keep).sum() < 3000 and 200 < (~keep2).sum() <= 320
+
+
+def test_knn_distance_with_far_outliers():
+    """Reconstructed clouds carry stray points far outside the scene.  The search grid is laid over the bulk of the
+    cloud (percentiles of a sample), the strays go to its boundary cells, and the result stays exact."""
+    import time
+    import torch
+    from scipy.spatial import cKDTree
+    from adop_amd import preprocess
+
+    g = np.random.default_rng(31)
+    n = 1_000_000
+    p = np.zeros((n, 4), np.float32)
+    p[:, :3] = g.random((n, 3))
+    stray = g.choice(n, 40, replace=False)
+    p[stray, :3] = g.standard_normal((40, 3)) * [3000.0, 100.0, 1.0e4]
+    announce("knn distance, 1 M points in the unit cube + 40 strays up to 1e4 away")
+    dev = torch.from_numpy(p).cuda()
+    preprocess.KNearestNeighbourDistance(dev, 4)  # first call: library load
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    got = preprocess.KNearestNeighbourDistance(dev, 4).cpu().numpy()
+    seconds = time.perf_counter() - t0
+    tree = cKDTree(p[:, :3].astype(np.float64))
+    check = np.concatenate([stray, g.integers(0, n, 3000)])
+    want = tree.query(p[check, :3].astype(np.float64), k=5)[0][:, 4]
+    assert np.allclose(got[check], want, rtol=2e-6, atol=1e-9)
+    assert seconds < 0.5, seconds  # a grid over the bounding box would put the whole cube into one cell
