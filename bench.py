@@ -324,10 +324,10 @@ def main():
     # workload only
     measured_traffic = {}
     if args.workload == "config3" and not args.points and args.point_order == "morton" and not args.no_point_cache:
-        # profiles/config3_tile_path_fwd_bwd_kernels_traffic_instructions.md, profiles/config3_fwd_bwd_kernels_traffic_atomics.md
+        # profiles/config3_tile_path_fwd_bwd_kernels_traffic_instructions.md, profiles/config3_direct_path_fwd_bwd_kernels_traffic_instructions.md
         measured_traffic = {"RenderBackward/descriptor": 912.7e6, "RenderBackward/spatial": 486.2e6, "TileBlend": 438.1e6,
                             "BinCount": 436.4e6, "BinScatter": 196.9e6, "TileDepth": 101.0e6,
-                            "CombineAndFillBackward": 397.3e6, "RenderForward": 691.9e6}
+                            "CombineAndFillBackward": 397.3e6, "RenderForward": 611.0e6, "DepthPrepass": 578.9e6}
     if args.workload == "config4" and not args.points and args.point_order == "morton":
         # profiles/config4_direct_path_forward_kernels_traffic_instructions.md
         measured_traffic = {"DepthPrepass": 5053.5e6, "RenderForward": 1548.3e6}
