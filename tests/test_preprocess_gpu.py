@@ -225,7 +225,7 @@ def test_filter_point_cloud_composes_the_filters():
 
 def test_knn_distance_with_far_outliers():
     """Reconstructed clouds carry stray points far outside the scene.  The search grid is laid over the bulk of the
-    cloud (percentiles of a sample), the strays go to its boundary cells, and the result stays exact."""
+    cloud (percentiles of a sample), the strays go to its boundary cells, and the result stays exact (and fast)."""
     import time
     import torch
     from scipy.spatial import cKDTree
@@ -248,4 +248,5 @@ def test_knn_distance_with_far_outliers():
     check = np.concatenate([stray, g.integers(0, n, 3000)])
     want = tree.query(p[check, :3].astype(np.float64), k=5)[0][:, 4]
     assert np.allclose(got[check], want, rtol=2e-6, atol=1e-9)
-    assert seconds < 0.5, seconds  # a grid over the bounding box would put the whole cube into one cell
+    print("seconds", seconds)
+    assert seconds < 1.0, seconds  # (~0.01 s; with the grid over the bounding box, all in one cell: 2.6 s)
