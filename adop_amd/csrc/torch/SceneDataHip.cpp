@@ -1,0 +1,139 @@
+// SceneDataHip.cpp — see SceneDataHip.h.
+#include "SceneDataHip.h"
+
+#include <c10/hip/HIPStream.h>
+
+#include "../../../include/adop_raster.h"
+
+namespace
+{
+void* Stream()
+{
+    return (void*)c10::hip::getCurrentHIPStream().stream();
+}
+
+void Check(adop_status st)
+{
+    TORCH_CHECK(st == ADOP_OK, "adop_raster: ", adop_last_error_string());
+}
+
+torch::Tensor CheckedPosition(torch::Tensor position)
+{
+    TORCH_CHECK(position.is_cuda() && position.scalar_type() == torch::kFloat32 && position.dim() == 2 &&
+                    position.size(1) == 4,
+                "position must be a [N,4] float tensor on the device");
+    return position.contiguous();
+}
+
+// bounding box of the cloud as host floats (one reduction over the contiguous array)
+void BoundingBox(const torch::Tensor& position, float* mn, float* mx)
+{
+    auto [lo, hi] = torch::aminmax(position, 0);
+    auto both     = torch::stack({lo, hi}).cpu();
+    auto a        = both.accessor<float, 2>();
+    for (int k = 0; k < 3; ++k)
+    {
+        mn[k] = a[0][k];
+        mx[k] = a[1][k];
+    }
+}
+
+torch::Tensor Workspace(size_t bytes, const torch::Tensor& like)
+{
+    return torch::empty({(int64_t)(bytes > 0 ? bytes : 1)}, like.options().dtype(torch::kUInt8));
+}
+}  // namespace
+
+torch::Tensor KNearestNeighbourDistance(torch::Tensor position, int n)
+{
+    position = CheckedPosition(position);
+    const int N = (int)position.size(0);
+    auto out    = torch::empty({N}, position.options());
+    auto ws     = Workspace(adop_knn_workspace_size(N), position);
+    float mn[3], mx[3];
+    BoundingBox(position, mn, mx);
+    Check(adop_knn_distance(position.data_ptr<float>(), N, n, mn, mx, out.data_ptr<float>(), ws.data_ptr(),
+                            (size_t)ws.numel(), Stream()));
+    return out;
+}
+
+torch::Tensor MortonCodes(torch::Tensor position)
+{
+    position = CheckedPosition(position);
+    const int N = (int)position.size(0);
+    auto codes  = torch::empty({N}, position.options().dtype(torch::kInt64));
+    float mn[3], mx[3];
+    BoundingBox(position, mn, mx);
+    Check(adop_morton_codes(position.data_ptr<float>(), N, mn, mx, (uint64_t*)codes.data_ptr<int64_t>(), Stream()));
+    return codes;
+}
+
+torch::Tensor ReorderMorton64(torch::Tensor position)
+{
+    return std::get<1>(torch::sort(MortonCodes(position), /*stable=*/true, 0, false));
+}
+
+torch::Tensor PointDistanceToCamera(torch::Tensor position, torch::Tensor poses_se3, torch::Tensor intrinsics,
+                                    const std::vector<ReducedImageInfo>& frames)
+{
+    position   = CheckedPosition(position);
+    poses_se3  = poses_se3.contiguous();
+    intrinsics = intrinsics.contiguous();
+    TORCH_CHECK(poses_se3.is_cuda() && poses_se3.scalar_type() == torch::kFloat64 && poses_se3.size(1) == 8);
+    TORCH_CHECK(intrinsics.is_cuda() && intrinsics.scalar_type() == torch::kFloat32 && intrinsics.size(1) == 13);
+    adop_scene s{};
+    s.position        = position.data_ptr<float>();
+    s.num_points      = (int32_t)position.size(0);
+    s.poses_se3       = poses_se3.data_ptr<double>();
+    s.num_poses       = (int32_t)poses_se3.size(0);
+    s.intrinsics      = intrinsics.data_ptr<float>();
+    s.num_cameras     = (int32_t)intrinsics.size(0);
+    s.intrinsics_cols = 13;
+    std::vector<adop_view> views;
+    for (const auto& i : frames)
+        views.push_back(adop_view{i.w, i.h, i.image_index, i.camera_index, (int32_t)i.camera_model_type,
+                                  i.crop_transform.fx, i.crop_transform.fy, i.crop_transform.cx, i.crop_transform.cy,
+                                  i.crop_transform.s});
+    auto out = torch::empty({position.size(0)}, position.options());
+    auto ws  = Workspace(adop_frames_workspace_size((int32_t)views.size()), position);
+    Check(adop_point_distance_to_camera(&s, views.data(), (int32_t)views.size(), out.data_ptr<float>(), ws.data_ptr(),
+                                        (size_t)ws.numel(), Stream()));
+    return out;
+}
+
+torch::Tensor RemoveLonelyPoints(torch::Tensor position, torch::Tensor camera_distance, int n, float dis_th)
+{
+    // d / cam_dis > dis_th erases the point (SceneData.cpp:585-590)
+    return torch::logical_not(KNearestNeighbourDistance(position, n) / camera_distance > dis_th);
+}
+
+torch::Tensor RemoveClosePoints(torch::Tensor position, torch::Tensor camera_distance, float dis_th)
+{
+    position = CheckedPosition(position);
+    const int N = (int)position.size(0);
+    auto radius = (dis_th / camera_distance).to(torch::kFloat32).contiguous();  // :619
+    auto state  = torch::empty({N}, position.options().dtype(torch::kInt32));
+    const int rounds = 8;
+    auto undecided   = torch::empty({rounds}, position.options().dtype(torch::kInt32));
+    auto ws          = Workspace(adop_knn_workspace_size(N), position);
+    float mn[3], mx[3];
+    BoundingBox(position, mn, mx);
+    for (int resume = 0;; resume = 1)
+    {
+        Check(adop_close_points(position.data_ptr<float>(), N, radius.data_ptr<float>(), mn, mx,
+                                state.data_ptr<int32_t>(), (uint32_t*)undecided.data_ptr<int32_t>(), rounds, resume,
+                                ws.data_ptr(), (size_t)ws.numel(), Stream()));
+        if (undecided[rounds - 1].item<int32_t>() == 0) break;  // every point waits for its earlier neighbours only
+    }
+    return state == 1;
+}
+
+torch::Tensor SortBlocksByRadius(torch::Tensor radius, int block_size)
+{
+    const int64_t n = radius.size(0), nb = n / block_size;
+    auto head   = radius.slice(0, 0, nb * block_size).reshape({nb, block_size});
+    auto order  = std::get<1>(torch::sort(head, /*stable=*/true, 1, false)) +
+                 (torch::arange(nb, radius.options().dtype(torch::kInt64)) * block_size).unsqueeze(1);
+    auto tail = torch::arange(nb * block_size, n, radius.options().dtype(torch::kInt64));
+    return torch::cat({order.reshape({-1}), tail});
+}

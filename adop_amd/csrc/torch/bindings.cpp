@@ -3,6 +3,7 @@
 #include <torch/extension.h>
 
 #include "PointRendererHip.h"
+#include "SceneDataHip.h"
 
 namespace py = pybind11;
 
@@ -99,4 +100,29 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("render", &Render, py::arg("scene"), py::arg("views"), py::arg("params"), py::arg("num_layers"),
           py::arg("training") = true, py::arg("through_module") = false);
     m.def("apply_tangent_to_pose", &ApplyTangentToPose);
+    // point-cloud processing of a new scene (SceneDataHip.cpp)
+    m.def("knn_distance", &KNearestNeighbourDistance, py::arg("position"), py::arg("n") = 4);
+    m.def("morton_codes", &MortonCodes);
+    m.def("reorder_morton64", &ReorderMorton64);
+    m.def("point_distance_to_camera",
+          [](torch::Tensor position, torch::Tensor poses, torch::Tensor intrinsics, const std::vector<ViewTuple>& frames) {
+              std::vector<ReducedImageInfo> f;
+              for (auto& v : frames)
+              {
+                  ReducedImageInfo i;
+                  i.w                 = std::get<0>(v);
+                  i.h                 = std::get<1>(v);
+                  i.image_index       = std::get<2>(v);
+                  i.camera_index      = std::get<3>(v);
+                  i.camera_model_type = (CameraModel)std::get<4>(v);
+                  i.crop_transform    = {std::get<5>(v), std::get<6>(v), std::get<7>(v), std::get<8>(v), std::get<9>(v)};
+                  f.push_back(i);
+              }
+              return PointDistanceToCamera(position, poses, intrinsics, f);
+          });
+    m.def("remove_lonely_points", &RemoveLonelyPoints, py::arg("position"), py::arg("camera_distance"), py::arg("n") = 5,
+          py::arg("dis_th") = 0.02f);
+    m.def("remove_close_points", &RemoveClosePoints, py::arg("position"), py::arg("camera_distance"),
+          py::arg("dis_th") = 0.00005f);
+    m.def("sort_blocks_by_radius", &SortBlocksByRadius, py::arg("radius"), py::arg("block_size") = 256);
 }

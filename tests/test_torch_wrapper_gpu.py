@@ -162,3 +162,39 @@ def test_apply_tangent(oracle_mod):
     torch.cuda.synchronize()
     assert np.abs(t["poses_se3"].cpu().numpy() - want).max() < 1e-12
     assert float(t["tangent_poses"].detach().abs().sum()) == 0
+
+
+def test_scene_data_processing_in_cpp():
+    """SceneDataHip.cpp (the point-cloud processing of a new scene over libTorch tensors) gives what the ctypes mirror
+    gives, which the preprocessing tests hold against the checker."""
+    import torch
+    from adop_amd import preprocess, scenes
+
+    mod = _module()
+    g = np.random.default_rng(6)
+    n = 30000
+    p = np.zeros((n, 4), np.float32)
+    p[:, :3] = g.standard_normal((n, 3)) * 0.6
+    p[1000:1300, :3] = p[:300, :3] + np.float32(2e-6)  # near-duplicates for the close-point filter
+    announce("C++ scene data processing: N=30000, 9 frames")
+    pos = torch.from_numpy(p).cuda()
+    assert torch.equal(mod.knn_distance(pos, 4), preprocess.KNearestNeighbourDistance(pos, 4))
+    assert torch.equal(mod.knn_distance(pos, 7), preprocess.KNearestNeighbourDistance(pos, 7))
+    assert torch.equal(mod.morton_codes(pos), preprocess.MortonCodes(pos))
+    assert torch.equal(mod.reorder_morton64(pos), preprocess.ReorderMorton64(pos))
+    views = np.stack([scenes.look_at_view(3.0 * d / np.linalg.norm(d)) for d in g.standard_normal((9, 3))])
+    K = scenes.pinhole_row(300, 300, 160, 120, 0.0, [0.05, -0.01, 0.002, 0.0, 0.0, 0.0, 0.001, 0.0])[None, :]
+    frames = [scenes.make_view(320, 240, image_index=f) for f in range(9)]
+    tuples = [(v.w, v.h, v.image_index, v.camera_index, v.camera_model_type, v.crop_fx, v.crop_fy, v.crop_cx, v.crop_cy,
+               v.crop_s) for v in frames]
+    poses, intr = torch.from_numpy(views).cuda(), torch.from_numpy(K).cuda()
+    cam = mod.point_distance_to_camera(pos, poses, intr, tuples)
+    assert torch.equal(cam, preprocess.PointDistanceToCamera(pos, poses, intr, frames))
+    assert torch.equal(mod.remove_lonely_points(pos, cam, 5, 0.05), preprocess.RemoveLonelyPoints(pos, cam, 5, 0.05))
+    keep = mod.remove_close_points(pos, cam, 0.00005)
+    assert torch.equal(keep, preprocess.RemoveClosePoints(pos, cam, 0.00005))
+    assert 250 <= int((~keep).sum()) <= 320
+    radius = torch.rand(n, device="cuda")
+    assert torch.equal(mod.sort_blocks_by_radius(radius, 256), preprocess.SortBlocksByRadius(radius, 256))
+    with pytest.raises(RuntimeError):
+        mod.knn_distance(pos[:3], 4)
