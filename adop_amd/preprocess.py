@@ -135,8 +135,11 @@ def ComputeRadius(position, rank=4, generator=None):
     n = int(position.shape[0])
     data = torch.zeros(n, 4, dtype=torch.float32, device=position.device)
     data[:, 0] = KNearestNeighbourDistance(position, rank)
-    u = torch.rand(n, generator=generator, dtype=torch.float64, device="cpu").clamp_min_(1e-300).to(position.device)
-    data[:, 2] = torch.sqrt(1.0 / u).to(torch.float32)
+    if generator is not None and generator.device.type == "cpu":  # a host generator: draw there
+        u = torch.rand(n, generator=generator, dtype=torch.float64, device="cpu").to(position.device)
+    else:
+        u = torch.rand(n, generator=generator, dtype=torch.float64, device=position.device)
+    data[:, 2] = torch.sqrt(1.0 / u.clamp_min_(1e-300)).to(torch.float32)
     data[:, 3] = data[:, 0] * data[:, 2]
     return data
 
@@ -156,11 +159,12 @@ def PreprocessPointCloud(position, normal=None, rank=4, block_size=256, seed=0):
     RandomBlockShuffle(256), ComputeRadius, SortBlocksByRadius(256).  Returns (position [N,4] with the drop-out radius in
     w, normal, data [N,4], order) where ``order`` maps new to original point ids."""
     gen = torch.Generator(device="cpu").manual_seed(int(seed))
+    gen_dev = torch.Generator(device=position.device).manual_seed(int(seed))  # the per-point numbers are drawn on the device
     position = position.contiguous()
     order = ReorderMorton64(position)
     order = order[RandomBlockShuffle(int(position.shape[0]), block_size, gen)]
     position = position[order].contiguous()
-    data = ComputeRadius(position, rank, gen)
+    data = ComputeRadius(position, rank, gen_dev)
     by_radius = SortBlocksByRadius(data[:, 3], block_size)
     order = order[by_radius]
     position = position[by_radius].clone()
