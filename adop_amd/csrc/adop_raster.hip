@@ -616,7 +616,7 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     StageScope post("Post Process Gradient", stream);
     launch_finalize(dviews, num_views, C, bg_partial, bg_blocks, pt_partial, pt_blocks, grads, scene->num_poses,
                     scene->num_cameras, scene->intrinsics_cols, params->normalize_mode, scratch,
-                    (double*)((char*)workspace + wl.fin_mini), q.counts + (size_t)num_views * kNumQueues, N, stream);
+                    (double*)((char*)workspace + wl.fin_mini), q.counts + (size_t)num_views * kNumQueues, N, q, stream);
     ADOP_HIP_CHECK(hipGetLastError());
     return ADOP_OK;
 }

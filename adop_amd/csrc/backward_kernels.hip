@@ -641,6 +641,10 @@ struct FinalizeArg
     double* scratch;
     double* mini;      // [kFinalizeParts * kMaxChannels] + [B * kFinalizeParts * kPartialStride]: rows of the first stage
     uint32_t* ticket;  // zero at the start of the kernel
+    // one view: its work queue names exactly the points with a spatial gradient (count > 0); null otherwise
+    const uint32_t* q_counts;
+    const unsigned long long* q_items;
+    uint32_t q_cap;
 };
 
 constexpr int kFinalizeSmall = 1024;  // pose / intrinsics sums of up to this many f64 stay in LDS
@@ -866,6 +870,38 @@ __global__ __launch_bounds__(kFinalizeBlock) void finalize_kernel(FinalizeArg a)
     finalize_body<kFinalizeBlock>(a, nullptr, nullptr, 0, 0);
 }
 
+// One view: the rows to normalise are the items of its work queue (a few percent of the points), which costs so
+// little that the reduction is the whole duration of the kernel; it then runs in one stage (one workgroup of 1024
+// threads: half the dependent round trips of the two stages with their ticket) beside the workgroups that normalise,
+// four sub-queues each.  Element t of the normalisation is point t in either mode.
+constexpr int kQueuesPerBlock = kFinalizeBlock / kBlock;
+
+__global__ __launch_bounds__(kFinalizeBlock) void finalize_queue_kernel(FinalizeArg a, float* __restrict__ g,
+                                                                        const float* __restrict__ count, int mode)
+{
+    if (blockIdx.x == 0)
+    {
+        finalize_body<kFinalizeBlock>(a, nullptr, nullptr, 0, 0);
+        return;
+    }
+    const int q = (blockIdx.x - 1) * kQueuesPerBlock + (threadIdx.x / kBlock);
+    if (q >= kNumQueues) return;
+    const uint32_t items = a.q_counts[q];
+    for (uint32_t e = threadIdx.x % kBlock; e < items; e += kBlock)
+    {
+        const uint32_t t = (uint32_t)__builtin_nontemporal_load(a.q_items + (size_t)q * a.q_cap + e);
+        const float c    = count[t];
+        const size_t o   = (mode == 0) ? 3 * (size_t)t : 4 * (size_t)t;
+        if (c > 0)
+        {
+            const float v0 = g[o + 0], v1 = g[o + 1], v2 = g[o + 2];
+            g[o + 0] = v0 / c;
+            g[o + 1] = v1 / c;
+            g[o + 2] = v2 / c;
+        }
+    }
+}
+
 // 8 waves per SIMD (<= 64 VGPRs): the normalisation lives on memory latency; the registers the reduction would like
 // to take (104) halve its occupancy and cost it 40%.
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) void finalize_normalize_kernel(
@@ -950,14 +986,24 @@ void launch_backward_ghost(const CloudArg& pc, const ViewConst* views, const Lev
 void launch_finalize(const ViewConst* views, int B, int C, const double* bg_partial, int bg_blocks,
                      const double* pt_partial, int pt_blocks, const adop_backward_buffers* g, int num_poses,
                      int num_cameras, int cols, int normalize_mode, double* scratch, double* mini, uint32_t* ticket, int n,
-                     hipStream_t st)
+                     const QueueArg& q, hipStream_t st)
 {
     FinalizeArg a{views, B, C, bg_partial, bg_blocks, pt_partial, pt_blocks, g->grad_background, g->grad_pose,
                   g->grad_pose_count, num_poses, g->grad_intrinsics, g->grad_intrinsics_count, num_cameras, cols,
-                  normalize_mode, scratch, mini, ticket};
+                  normalize_mode, scratch, mini, ticket, nullptr, nullptr, 0};
     if (!g->grad_points || n < 1) n = 0;
+    static const int by_queue = getenv("ADOP_NORMALIZE_BY_QUEUE") ? atoi(getenv("ADOP_NORMALIZE_BY_QUEUE")) : 1;
     if (n == 0)
         hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kFinalizeBlock), 0, st, a);
+    else if (B == 1 && by_queue)
+    {
+        // (with several views a point sits in several queues and would be divided more than once)
+        a.q_counts = q.counts;
+        a.q_items  = q.items;
+        a.q_cap    = q.cap;
+        hipLaunchKernelGGL(finalize_queue_kernel, dim3(1 + kNumQueues / kQueuesPerBlock), dim3(kFinalizeBlock), 0, st, a,
+                           g->grad_points, g->grad_points_count, normalize_mode);
+    }
     else
         hipLaunchKernelGGL(finalize_normalize_kernel, dim3(kFinalizeParts + (n + kBlock * kNormPer - 1) / (kBlock * kNormPer)), dim3(kBlock), 0, st, a,
                            g->grad_points, g->grad_points_count, n, normalize_mode);

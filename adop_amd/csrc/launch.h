@@ -95,7 +95,7 @@ void launch_backward_ghost(const CloudArg& pc, const ViewConst* views, const Lev
 void launch_finalize(const ViewConst* views, int B, int C, const double* bg_partial, int bg_blocks,
                      const double* pt_partial, int pt_blocks, const adop_backward_buffers* g, int num_poses,
                      int num_cameras, int cols, int normalize_mode, double* scratch, double* mini, uint32_t* ticket, int n,
-                     hipStream_t st);
+                     const QueueArg& q, hipStream_t st);
 
 void launch_env_sample(const ViewChunk& chunk, const double* poses, const float* intrinsics, const Levels& lv,
                        const EnvLevels& ev, const float* tex, int eh, int ew, int add_to_out, hipStream_t st);
