@@ -649,8 +649,10 @@ struct FinalizeArg
 
 constexpr int kFinalizeSmall = 1024;  // pose / intrinsics sums of up to this many f64 stay in LDS
 
+// part: 0 = everything, 1 = the background gradient only, 2 = the pose / intrinsics gradients only (the two are
+// independent: two workgroups can share the work)
 template <int NT>
-__device__ static void finalize_block(const FinalizeArg& a, double* sh, double* s_small)
+__device__ static void finalize_block(const FinalizeArg& a, double* sh, double* s_small, int part = 0)
 {
     const ViewConst* __restrict__ views = a.views;
     const int B = a.B, C = a.C, bg_blocks = a.bg_blocks, pt_blocks = a.pt_blocks, num_poses = a.num_poses,
@@ -665,6 +667,7 @@ __device__ static void finalize_block(const FinalizeArg& a, double* sh, double* 
     // flat pointer: LDS when the sums fit (every round trip to memory is on this block's critical path)
     double* scratch = (num_poses * 7 + num_cameras * (cols + 1) <= kFinalizeSmall) ? s_small : a.scratch;
     // background: thread t sums channel t%16 over the partial rows t/16, t/16+16, ...
+    if (part != 2)
     {
         const int c = threadIdx.x % kMaxChannels, k0 = threadIdx.x / kMaxChannels;
         constexpr int GR = NT / kMaxChannels;
@@ -681,7 +684,7 @@ __device__ static void finalize_block(const FinalizeArg& a, double* sh, double* 
         }
         __syncthreads();
     }
-    if (!gpose && !gintr) return;
+    if ((!gpose && !gintr) || part == 1) return;
 
     // scratch: [num_poses*7] pose sums + count, then [num_cameras*(cols+1)] intrinsics sums + count
     double* sp = scratch;
@@ -874,20 +877,23 @@ __global__ __launch_bounds__(kFinalizeBlock) void finalize_kernel(FinalizeArg a)
 // little that the reduction is the whole duration of the kernel; it then runs in one stage (one workgroup of 1024
 // threads: half the dependent round trips of the two stages with their ticket) beside the workgroups that normalise,
 // four sub-queues each.  Element t of the normalisation is point t in either mode.
-constexpr int kQueuesPerBlock = kFinalizeBlock / kBlock;
+constexpr int kQueuesPerBlock = 2;  // 512 threads per sub-queue: about one item per thread
 
 __global__ __launch_bounds__(kFinalizeBlock) void finalize_queue_kernel(FinalizeArg a, float* __restrict__ g,
                                                                         const float* __restrict__ count, int mode)
 {
-    if (blockIdx.x == 0)
+    if (blockIdx.x < 2)
     {
-        finalize_body<kFinalizeBlock>(a, nullptr, nullptr, 0, 0);
+        __shared__ double sh[kFinalizeBlock];
+        __shared__ double s_small[kFinalizeSmall];
+        finalize_block<kFinalizeBlock>(a, sh, s_small, 1 + (int)blockIdx.x);
         return;
     }
-    const int q = (blockIdx.x - 1) * kQueuesPerBlock + (threadIdx.x / kBlock);
+    constexpr int TPQ = kFinalizeBlock / kQueuesPerBlock;  // threads per sub-queue
+    const int q       = (blockIdx.x - 2) * kQueuesPerBlock + (threadIdx.x / TPQ);
     if (q >= kNumQueues) return;
     const uint32_t items = a.q_counts[q];
-    for (uint32_t e = threadIdx.x % kBlock; e < items; e += kBlock)
+    for (uint32_t e = threadIdx.x % TPQ; e < items; e += TPQ)
     {
         const uint32_t t = (uint32_t)__builtin_nontemporal_load(a.q_items + (size_t)q * a.q_cap + e);
         const float c    = count[t];
@@ -1001,7 +1007,7 @@ void launch_finalize(const ViewConst* views, int B, int C, const double* bg_part
         a.q_counts = q.counts;
         a.q_items  = q.items;
         a.q_cap    = q.cap;
-        hipLaunchKernelGGL(finalize_queue_kernel, dim3(1 + kNumQueues / kQueuesPerBlock), dim3(kFinalizeBlock), 0, st, a,
+        hipLaunchKernelGGL(finalize_queue_kernel, dim3(2 + kNumQueues / kQueuesPerBlock), dim3(kFinalizeBlock), 0, st, a,
                            g->grad_points, g->grad_points_count, normalize_mode);
     }
     else
