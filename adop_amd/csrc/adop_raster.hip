@@ -132,6 +132,7 @@ struct WorkspaceLayout
 constexpr int kTileLevels = 2;  // levels the tile path renders in LDS (a point has at most one bin entry per such level)
 constexpr int kTilePathMinPoints = 1 << 16;
 constexpr int kTilePathMaxPointsPerPixel = 16;
+constexpr int kGroupedViewsMaxPoints = 4000000;  // backward: spatial gradients of a group of views in one launch
 
 size_t max_tiles(int B, int w0, int h0)
 {
@@ -595,6 +596,14 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     q.counts = (uint32_t*)((char*)workspace + wl.q_counts);
     q.items  = (unsigned long long*)((char*)workspace + wl.q_items);
     q.cap    = wl.q_cap;
+    // Several views: one spatial-gradient launch per group of views (items carry the level masks of the whole group;
+    // a group's 16-byte items fit where the 8-byte items of its views would be) while the launches per view would be
+    // small; a large cloud fills a launch per view, and the compacted per-view queues then beat the group kernel, whose
+    // wavefronts walk the views in step.  ADOP_GHOST_GROUPS (read at every call): 0 = never, 2 = always.
+    const char* env_groups = getenv("ADOP_GHOST_GROUPS");
+    const int groups_mode  = env_groups ? atoi(env_groups) : 1;
+    const bool grouped     = num_views > 1 && (groups_mode == 2 || (groups_mode == 1 && N <= kGroupedViewsMaxPoints));
+    q.views_per_item       = grouped ? ghost_views_per_item() : 1;
     if (N < 1)
     {
         // nothing writes the partial rows: clear them for finalize
@@ -607,12 +616,23 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
         StageScope sc("RenderBackward/descriptor", stream);
         launch_backward_tex(pc, dviews, lv, rp, half, ig, dw, grads, scene->index_is_identity, q, stats, stream);
     }
-    for (int b = 0; b < num_views; ++b)
+    if (q.views_per_item > 1)
     {
-        StageScope sc("RenderBackward/spatial", stream);
-        launch_backward_ghost(pc, dviews, lv, rp, half, ig, grads, want_pose, want_intr, scene->index_is_identity, b,
-                              q, pt_blocks, pt_partial, stream);
+        for (int first = 0, group = 0; first < num_views; first += q.views_per_item, ++group)
+        {
+            StageScope sc("RenderBackward/spatial", stream);
+            const int count = num_views - first < q.views_per_item ? num_views - first : q.views_per_item;
+            launch_backward_ghost_multi(pc, dviews, lv, rp, half, ig, grads, want_pose, want_intr,
+                                        scene->index_is_identity, group, first, count, q, pt_blocks, pt_partial, stream);
+        }
     }
+    else
+        for (int b = 0; b < num_views; ++b)
+        {
+            StageScope sc("RenderBackward/spatial", stream);
+            launch_backward_ghost(pc, dviews, lv, rp, half, ig, grads, want_pose, want_intr, scene->index_is_identity, b,
+                                  q, pt_blocks, pt_partial, stream);
+        }
     StageScope post("Post Process Gradient", stream);
     launch_finalize(dviews, num_views, C, bg_partial, bg_blocks, pt_partial, pt_blocks, grads, scene->num_poses,
                     scene->num_cameras, scene->intrinsics_cols, params->normalize_mode, scratch,

@@ -126,6 +126,20 @@ def test_more_views_than_one_constant_chunk(oracle_mod):
     _fwd_bwd(hs, oracle_mod)
 
 
+@pytest.mark.parametrize("groups", ["0", "2"], ids=["per_view", "grouped"])
+@pytest.mark.parametrize("batch", [2, 5, 13, 34])
+def test_spatial_gradients_per_view_and_per_group_of_views(oracle_mod, monkeypatch, groups, batch):
+    """With several views the spatial-gradient pass runs once per view (large clouds) or once per group of twelve views
+    (small ones; the library picks by the size of the cloud): both against the checker, with batch sizes on either
+    side of a group and of the 32-view chunk of constants."""
+    from adop_amd import scenes
+
+    monkeypatch.setenv("ADOP_GHOST_GROUPS", groups)
+    announce(f"config2 40k pts B={batch} 96x80 L3 fwd+bwd ghost, ADOP_GHOST_GROUPS={groups}")
+    hs = scenes.config2(n=40_000, w=96, h=80, levels=3, batch=batch, seed=batch)
+    _fwd_bwd(hs, oracle_mod)
+
+
 @pytest.mark.parametrize("mode", [0, 1])
 def test_normalize_modes_and_backward_mode4(oracle_mod, mode):
     from adop_amd import scenes
