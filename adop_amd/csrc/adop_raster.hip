@@ -19,13 +19,14 @@
 //   interleave      per pixel: background-gradient partial sums (CombineAndFillBackward :851-900), the pixel-major
 //                   [image | upstream gradient] array and (depth, weight) pairs the next kernels gather from; one
 //                   workgroup computes the per-view constants
-//   per view:
-//   backward_tex    per point: depth tests, descriptor gradient, which levels get a ghost / spatial gradient
-//                   (RenderBackward :396-489); appends those points to a work queue
-//   backward_ghost  per queue item: four-neighbour gather, image-space gradient, ProjectPoint*Backward (:491-724);
-//                   pose / intrinsics sums per thread in fp32, per workgroup in f64, one partial row per workgroup
-//   finalize_normalize  partial rows -> grad_background / grad_pose / grad_intrinsics, NormalizeGradient
-//                   (:1534-1547) of all outputs
+//   backward_tex    per point, all views in one pass: depth tests, descriptor gradient (written once), which levels get
+//                   a ghost / spatial gradient (RenderBackward :396-489); appends those points to a work queue per
+//                   view, or, for small clouds, per group of twelve views
+//   backward_ghost  per queue item (one launch per view or per group): four-neighbour gather, image-space gradient,
+//                   ProjectPoint*Backward (:491-724); pose / intrinsics sums per thread in fp32, per workgroup in f64,
+//                   one partial row per workgroup and view
+//   finalize        partial rows -> grad_background / grad_pose / grad_intrinsics, NormalizeGradient (:1534-1547) of
+//                   all outputs (one view: the point gradients by walking the work queue)
 //
 // No MFMA anywhere: the path is scan + scatter/gather + atomics, bounded by HBM and atomic transaction rate.
 #include <hip/hip_runtime.h>
