@@ -164,6 +164,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(CT != 0 
     constexpr int CMAX = CT ? CT : 1;  // register arrays exist only for compile-time channel counts
     __shared__ uint32_t s_wave_count[kBlock / 64];
     __shared__ uint32_t s_base;
+    __shared__ unsigned long long s_culled[kBlock / 64];
+    __shared__ unsigned long long s_block_culled;
+    static_assert(kBlock / 64 == 4, "four runs per workgroup");
     const bool STATS    = stats != nullptr;  // counter pass (uniform branch)
     const float accept  = rp.depth_accept + 1;
     const int C         = CT ? CT : lv.C;
@@ -185,128 +188,161 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(CT != 0 
     // item and a queue stands for a group of views
     const int num_views = MULTI ? lv.B : 1;
     unsigned long long masks = 0;
+    // Several views (crops see a small part of the cloud): the first record of the wavefront's run of 64 points says
+    // whether the forward pass culled the whole run for a view (kRunCulledBits); lane b asks for view b, all at once,
+    // and the records of the runs culled are never read.
+    unsigned long long culled_views = 0;
+    if (MULTI && pc.cache)
+    {
+        const int first = i & ~63;
+        bool c          = false;
+        if (lane < num_views && first < pc.n)
+        {
+            const float4 head = pc.cache[(size_t)lane * pc.n + first];
+            c                 = __float_as_uint(head.x) == kRunCulledBits && head.z == 0.f;
+        }
+        culled_views = __ballot(c);
+        // views culled for all four runs of the workgroup: their whole iteration is skipped below
+        if (lane == 0) s_culled[wave] = culled_views;
+        __syncthreads();
+        if (threadIdx.x == 0) s_block_culled = s_culled[0] & s_culled[1] & s_culled[2] & s_culled[3];
+        __syncthreads();
+    }
+    else if (MULTI)
+    {
+        if (threadIdx.x == 0) s_block_culled = 0;
+        __syncthreads();
+    }
     for (int b = 0; b < num_views; ++b)
     {
-        const ViewConst& vc = views[b];
-        bool drop_out;
-        V2 ip = {0.f, 0.f};
-        float z = 0.f, radius_pixels = 0.f;
-        bool ok;
-        if (pc.cache)  // kernel-uniform: the forward pass left the projected points with the caller
+        // a view for which every run of this workgroup was culled has nothing to test (mask stays 0)
+        uint32_t mask = 0;
+        if (!(MULTI && b < 64 && (s_block_culled >> b & 1ull) != 0))
         {
-            // depth 0: culled; negative depth: dropped for this image (:314-315)
-            float4 R = make_float4(0, 0, 0, 0);
-            if (valid)
+            const ViewConst& vc = views[b];
+            bool drop_out;
+            V2 ip = {0.f, 0.f};
+            float z = 0.f, radius_pixels = 0.f;
+            bool ok;
+            if (pc.cache)  // kernel-uniform: the forward pass left the projected points with the caller
             {
-                const v4f r = __builtin_nontemporal_load((const v4f*)pc.cache + (size_t)b * pc.n + i);
-                R           = make_float4(r.x, r.y, r.z, r.w);
-            }
-            ip             = {R.x, R.y};
-            drop_out       = R.z < 0;
-            z              = fabsf(R.z);
-            radius_pixels  = R.w;
-            ok             = valid && z != 0;
-        }
-        else
-        {
-            drop_out = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;
-            float4 P = valid ? pc.position[i] : make_float4(0, 0, 0, 0);
-            V3 pos   = {P.x, P.y, P.z};
-            V3 nrm   = {0, 0, 0};
-            if (valid && pc.normal) nrm = unpack_normal10(pc.normal[i]);
-            V3 view_p;
-            ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff, lv.l[0].w,
-                                        &ip, &z, &radius_pixels, &view_p);
-        }
-        ok = ok && tex_in_range;
-
-        // phase 1: pixel of every level, depth loads (independent)
-        uint32_t pix[ADOP_MAX_LAYERS];
-        bool in[ADOP_MAX_LAYERS];
-        bool edge_ok[ADOP_MAX_LAYERS];
-        float dep[ADOP_MAX_LAYERS];
-        float wgt[ADOP_MAX_LAYERS];
-#pragma unroll
-        for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
-        {
-            in[l]      = false;
-            edge_ok[l] = false;
-            pix[l]     = 0;
-            dep[l]     = 0.f;
-            wgt[l]     = 0.f;
-            if (l < lv.num)
-            {
-                const LevelArg& L = lv.l[l];
-                int px = f2i_rn(ip.x), py = f2i_rn(ip.y);
-                bool lod_skip = rp.drop_by_radius && radius_pixels < rp.drop_threshold;  // continue, :451-454
-                in[l]         = ok && !lod_skip && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h;
-                if (in[l])
+                // depth 0: culled; negative depth: dropped for this image (:314-315)
+                float4 R = make_float4(0, 0, 0, 0);
+                // Several views (crops see a small part of the cloud): the first record of the wavefront's run of 64 points
+                // says whether the forward pass culled the whole run for this view; the other 63 records are then not read.
+                const bool run_culled = MULTI && b < 64 && (culled_views >> b & 1ull) != 0;
+                if (valid && !run_culled)
                 {
-                    pix[l]     = (uint32_t)py * (uint32_t)L.w + (uint32_t)px;
-                    const float2 d_w = dw[ws_pixel(lv, l, b, pix[l])];  // (depth, weight) left by interleave_kernel
-                    dep[l]           = d_w.x;
-                    wgt[l]           = d_w.y;
-                    int ex     = min(px, L.w - 1 - px);
-                    int ey     = min(py, L.h - 1 - py);
-                    edge_ok[l] = min(ex, ey) > 2;  // distanceFromEdge > 2, :489
+                    const v4f r = __builtin_nontemporal_load((const v4f*)pc.cache + (size_t)b * pc.n + i);
+                    R           = make_float4(r.x, r.y, r.z, r.w);
                 }
-                radius_pixels *= 0.5f;
-                ip.x *= 0.5f;
-                ip.y *= 0.5f;
+                ip             = {R.x, R.y};
+                drop_out       = R.z < 0;
+                z              = fabsf(R.z);
+                radius_pixels  = R.w;
+                ok             = valid && z != 0;
             }
-        }
-        // phase 2: depth test in level order, `break` at the first failure (:462)
-        bool pass[ADOP_MAX_LAYERS];
-        {
-            bool alive = true;
-#pragma unroll
+            else
+            {
+                drop_out = valid && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;
+                float4 P = valid ? pc.position[i] : make_float4(0, 0, 0, 0);
+                V3 pos   = {P.x, P.y, P.z};
+                V3 nrm   = {0, 0, 0};
+                if (valid && pc.normal) nrm = unpack_normal10(pc.normal[i]);
+                V3 view_p;
+                ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff, lv.l[0].w,
+                                            &ip, &z, &radius_pixels, &view_p);
+            }
+            ok = ok && tex_in_range;
+
+            // phase 1: pixel of every level, depth loads (independent)
+            uint32_t pix[ADOP_MAX_LAYERS];
+            bool in[ADOP_MAX_LAYERS];
+            bool edge_ok[ADOP_MAX_LAYERS];
+            float dep[ADOP_MAX_LAYERS];
+            float wgt[ADOP_MAX_LAYERS];
+    #pragma unroll
             for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
             {
-                pass[l] = false;
-                if (in[l] && alive)
+                in[l]      = false;
+                edge_ok[l] = false;
+                pix[l]     = 0;
+                dep[l]     = 0.f;
+                wgt[l]     = 0.f;
+                if (l < lv.num)
                 {
-                    if (z > dep[l] * accept)
-                        alive = false;
-                    else
-                        pass[l] = true;
+                    const LevelArg& L = lv.l[l];
+                    int px = f2i_rn(ip.x), py = f2i_rn(ip.y);
+                    bool lod_skip = rp.drop_by_radius && radius_pixels < rp.drop_threshold;  // continue, :451-454
+                    in[l]         = ok && !lod_skip && (unsigned)px < (unsigned)L.w && (unsigned)py < (unsigned)L.h;
+                    if (in[l])
+                    {
+                        pix[l]     = (uint32_t)py * (uint32_t)L.w + (uint32_t)px;
+                        const float2 d_w = dw[ws_pixel(lv, l, b, pix[l])];  // (depth, weight) left by interleave_kernel
+                        dep[l]           = d_w.x;
+                        wgt[l]           = d_w.y;
+                        int ex     = min(px, L.w - 1 - px);
+                        int ey     = min(py, L.h - 1 - py);
+                        edge_ok[l] = min(ex, ey) > 2;  // distanceFromEdge > 2, :489
+                    }
+                    radius_pixels *= 0.5f;
+                    ip.x *= 0.5f;
+                    ip.y *= 0.5f;
                 }
             }
-        }
-        // phase 3: descriptor gradient of the rendered (not dropped) points; spatial-gradient eligibility
-        const bool point_grad = (rp.ghost_gradients && drop_out) | (!rp.ghost_gradients && !drop_out);
-        uint32_t mask         = 0;
-#pragma unroll
-        for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
-        {
-            bool go = pass[l];
-            if (pass[l] && !drop_out)
+            // phase 2: depth test in level order, `break` at the first failure (:462)
+            bool pass[ADOP_MAX_LAYERS];
             {
-                if (wgt[l] == 0)
-                    go = false;  // continue, :473
-                else
+                bool alive = true;
+    #pragma unroll
+                for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
                 {
-                    float iw        = 1.f / wgt[l];
-                    const float* pg = ig + (size_t)ws_pixel(lv, l, b, pix[l]) * (2 * C) + C;  // G of the pixel
-                    if (CT == 0)
+                    pass[l] = false;
+                    if (in[l] && alive)
                     {
-                        // any channel count: one atomic per channel and level (:478-484)
-#pragma unroll 1
-                        for (int c = 0; c < C; ++c)
-                            unsafeAtomicAdd(gtex + (size_t)c * pc.num_texels + tex_index, iw * pg[c]);
-                    }
-                    else
-                    {
-                        float G[CMAX];
-                        load_channels<CT ? CT : 4>(pg, G);
-#pragma unroll
-                        for (int c = 0; c < CMAX; ++c) gt[c] += iw * G[c];
-                        gt_live = true;
+                        if (z > dep[l] * accept)
+                            alive = false;
+                        else
+                            pass[l] = true;
                     }
                 }
             }
-            bool spatial = go && point_grad && edge_ok[l];
-            if (spatial) mask |= 1u << l;
-            if (STATS && l < lv.num) stat_add(&stats->spatial[l], spatial);
+            // phase 3: descriptor gradient of the rendered (not dropped) points; spatial-gradient eligibility
+            const bool point_grad = (rp.ghost_gradients && drop_out) | (!rp.ghost_gradients && !drop_out);
+            mask                  = 0;
+    #pragma unroll
+            for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+            {
+                bool go = pass[l];
+                if (pass[l] && !drop_out)
+                {
+                    if (wgt[l] == 0)
+                        go = false;  // continue, :473
+                    else
+                    {
+                        float iw        = 1.f / wgt[l];
+                        const float* pg = ig + (size_t)ws_pixel(lv, l, b, pix[l]) * (2 * C) + C;  // G of the pixel
+                        if (CT == 0)
+                        {
+                            // any channel count: one atomic per channel and level (:478-484)
+    #pragma unroll 1
+                            for (int c = 0; c < C; ++c)
+                                unsafeAtomicAdd(gtex + (size_t)c * pc.num_texels + tex_index, iw * pg[c]);
+                        }
+                        else
+                        {
+                            float G[CMAX];
+                            load_channels<CT ? CT : 4>(pg, G);
+    #pragma unroll
+                            for (int c = 0; c < CMAX; ++c) gt[c] += iw * G[c];
+                            gt_live = true;
+                        }
+                    }
+                }
+                bool spatial = go && point_grad && edge_ok[l];
+                if (spatial) mask |= 1u << l;
+                if (STATS && l < lv.num) stat_add(&stats->spatial[l], spatial);
+            }
         }
         // Point gradients of the first view: points without a spatial gradient are cleared here (Build(info,false),
         // :922-949), the others are written by backward_ghost_kernel; no separate zero-fill of the two buffers.
@@ -328,6 +364,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(CT != 0 
             masks = mask;
         // queue push: rank inside the workgroup, one returning atomic per workgroup on the sub-queue counter
         bool has               = masks != 0;
+        if (MULTI && !__syncthreads_or(has)) continue;  // nothing in the whole workgroup (masks is 0)
         unsigned long long bal = __ballot(has);
         uint32_t rank_in_wave  = (uint32_t)__popcll(bal & ((1ull << lane) - 1ull));
         if (lane == 0) s_wave_count[wave] = (uint32_t)__popcll(bal);

@@ -117,9 +117,12 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(PPT > 2 
             // (the sign of the depth carries the dropout flag: the readers need no second array)
             // (only the projected points' flags are read: the 55 % outside the image cost no dropout bytes)
             const bool dropped = ok && pc.dropout && __builtin_nontemporal_load(pc.dropout + (size_t)b * pc.n + i) == 1.f;  // :314-315
+            // (a run of 64 points none of which is projected: marked in its first record, see kRunCulledBits)
+            const bool run_culled = !__ballot(ok);
             if (valid)
                 nt_store4(pc.cache + (size_t)b * pc.n + i,
-                          ok ? make_float4(ip.x, ip.y, dropped ? -z : z, radius_pixels) : make_float4(0, 0, 0, 0));
+                          ok ? make_float4(ip.x, ip.y, dropped ? -z : z, radius_pixels)
+                             : make_float4((run_culled && lane == 0) ? __uint_as_float(kRunCulledBits) : 0.f, 0, 0, 0));
             if (STATS) stat_add(&stats->bad_index, ok && !dropped && !tex_ok[k]);
             if (!__ballot(ok) && !STATS)  // wavefront-uniform
             {
@@ -153,7 +156,13 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(PPT > 2 
                 for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
                     if (l < lv.num) stat_add(&stats->visible[l], in[l]);
             }
-            if (!__ballot(any_in)) continue;
+            if (!__ballot(any_in))
+            {
+                // projected, but all outside the image (a crop): the run counts as culled all the same
+                if (valid && lane == 0)
+                    nt_store4(pc.cache + (size_t)b * pc.n + i, make_float4(__uint_as_float(kRunCulledBits), 0, 0, 0));
+                continue;
+            }
             // one atomic per distinct tile of the wavefront, for the primary and for the second entries
             const unsigned long long below = (1ull << lane) - 1ull;
             const unsigned long long pm    = wave_group_mask(any_in, ptile);

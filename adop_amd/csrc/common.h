@@ -20,6 +20,9 @@ constexpr int kAcc           = 21;
 constexpr int kFinalizeParts = 16;    // workgroups of the first stage of the final two-stage reduction
 constexpr int kNumQueues     = 2048;  // sub-queues of the backward work queue (multiple of kBlock)
 constexpr int kMaxIntrinsicsCols = 24;  // 13 pinhole / 5 affine + up to 19 polynomial coefficients
+// Point cache: when a whole run of 64 points (64-aligned) is culled for a view, the record of its first point carries
+// this bit pattern in x (its depth is 0 like every culled record's), so that a reader can skip the other 63 records.
+constexpr uint32_t kRunCulledBits = 0x7FC0C011u;  // a quiet NaN no projection produces
 constexpr uint64_t kClearPacked = (uint64_t(0x47C35000u) << 32) | 0xFFFFFFFFull;  // bits(100000.f), PointRenderer.cu:1045
 
 struct LevelArg

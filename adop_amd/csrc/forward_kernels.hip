@@ -156,6 +156,18 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
                 }
             }
         }
+        // A run of 64 points none of which lands in the image at any level (a crop sees a small part of the cloud):
+        // its first record says so (kRunCulledBits), and the backward pass of several views skips the run.
+        if (pc.cache && !pc.list_ids)
+        {
+#pragma unroll
+            for (int k = 0; k < PPT; ++k)
+            {
+                const int i = base + k * kBlock;
+                if (!__ballot(inmask[k] != 0) && (threadIdx.x & 63) == 0 && i < pc.n)
+                    pc.cache[(size_t)b * pc.n + i] = make_float4(__uint_as_float(kRunCulledBits), 0, 0, 0);
+            }
+        }
         // List mode: the points of every wavefront that may still pass a depth test, compacted into the first slots of
         // the wavefront's own range (no LDS, no barrier, no atomics).  In a dense cloud they are a few percent,
         // scattered over all wavefronts; the blend packs the four lists of a workgroup and runs on full wavefronts of

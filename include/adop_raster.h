@@ -138,7 +138,8 @@ typedef struct adop_forward_buffers
      * dropped for that image, dropout_points) and the LOD
      * radius in pixels.  adop_forward writes it; adop_backward reads it instead of projecting when the same
      * buffer is passed back in `fwd`.  NULL: adop_forward keeps the records in the workspace, adop_backward
-     * projects again. */
+     * projects again.  When none of the points i..i+63 (i a multiple of 64) lands in the image of a view at any
+     * level, record i of that view holds the bits 0x7FC0C011 in x (and depth 0): adop_backward then skips the run. */
     float* point_cache;
 } adop_forward_buffers;
 
