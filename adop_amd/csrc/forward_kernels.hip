@@ -439,8 +439,24 @@ __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewCo
         if (valid && pc.normal) nrm = unpack_normal10(pc.normal[i]);
     }
 
+    // Several views: the prepass marked the runs of 64 points that miss a view entirely in their first record
+    // (kRunCulledBits); lane b asks for view b, all at once, and the records of such runs are not read.
+    unsigned long long culled_views = 0;
+    if (pc.cache && lv.B > 1)
+    {
+        const int lane  = threadIdx.x & 63;
+        const int first = i & ~63;
+        bool c          = false;
+        if (lane < lv.B && first < pc.n)
+        {
+            const float4 head = pc.cache[(size_t)lane * pc.n + first];
+            c                 = __float_as_uint(head.x) == kRunCulledBits && head.z == 0.f;
+        }
+        culled_views = __ballot(c);
+    }
     for (int b = 0; b < lv.B; ++b)
     {
+        if (b < 64 && (culled_views >> b & 1ull) != 0 && !STATS) continue;  // wavefront-uniform
         V2 ip = {0.f, 0.f};
         float z = 0.f, radius_pixels = 0.f;
         bool ok;
