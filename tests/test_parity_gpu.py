@@ -279,3 +279,43 @@ def test_bad_texture_index_is_counted(oracle_mod):
     scene, info, ctx, images, masks = run_hip_forward(hs)
     check_forward(hs, ref, ctx, images, masks, info)
     assert info.cache.read_stats().bad_index == ref.stats.bad_index > 0
+
+
+@pytest.mark.parametrize("forward_path", [1, 2], ids=["direct", "tiles"])
+def test_runs_that_miss_a_view_are_marked_and_skipped(oracle_mod, forward_path):
+    """A batch of crops: most runs of 64 points miss most views.  The forward marks them in the point cache (first
+    record of the run: a NaN bit pattern in x, depth 0), the blend and the backward of the batch skip them, and every
+    result still equals the checker's.  The marks are exactly the runs without a point in the image."""
+    import torch
+    from adop_amd import render, scenes
+
+    n, w, h = 150_000, 256, 192
+    hs = scenes.config2(n=n, w=w, h=h, levels=3, batch=1, seed=9)
+    hs.params.forward_path = forward_path
+    g = np.random.default_rng(2)
+    poses = [hs.poses_se3[0], scenes.look_at_view((0.5, 2.5, -1.5)), scenes.look_at_view((9.0, 0.0, 0.0), (20.0, 0.0, 0.0))]
+    hs.poses_se3 = np.stack(poses)  # the third camera looks away from the cloud
+    hs.views = [scenes.make_view(64, 48, image_index=f, crop=(1.0, 1.0, -float(g.integers(0, w - 64)), -float(g.integers(0, h - 48)), 0.0))
+                for f in (0, 0, 1, 1, 2)]
+    hs.dropout = scenes.bernoulli_mask(4, len(hs.views), n, 0.25)
+    announce(f"crops and a camera that looks away: N={n} B={len(hs.views)} 64x48 L=3 forward_path={forward_path}")
+    ref, refb = _fwd_bwd(hs, oracle_mod)
+    # the marks in the cache of a second forward
+    scene, info, ctx, images, masks = run_hip_forward(hs)
+    cache = info.cache.point_cache.cpu().numpy()  # [B,N,4]
+    bits = cache[:, ::64, 0].view(np.uint32)
+    marked = (bits == 0x7FC0C011) & (cache[:, ::64, 2] == 0)
+    assert marked[4].all()  # nothing of the cloud is in front of the third camera
+    assert 0.3 < marked[:4].mean() < 0.99
+    # a marked run holds no record that lands in the image
+    z = cache[:, :, 2]
+    ipx, ipy = cache[:, :, 0], cache[:, :, 1]
+    with np.errstate(invalid="ignore"):
+        inside = (z != 0) & ~np.isnan(ipx) & (np.rint(ipx) >= 0) & (np.rint(ipx) < 64) & (np.rint(ipy) >= 0) & (np.rint(ipy) < 48)
+    run_of = np.arange(n) // 64
+    for b in range(5):
+        runs_with_points = np.zeros(marked.shape[1], bool)
+        runs_with_points[np.unique(run_of[inside[b]])] = True
+        assert not (marked[b] & runs_with_points).any()
+    # and the unmarked records account for every point the checker counts as visible at the finest level
+    assert int(inside.sum()) == ref.stats.visible[0]
