@@ -113,19 +113,20 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(PPT > 2 
             float z = 0.f, radius_pixels = 0.f;
             bool ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P[k].w, rp.check_normal != 0, rp.dist_cutoff,
                                              lv.l[0].w, &ip, &z, &radius_pixels, &view_p);
-            // the second pass (and the backward pass, if the caller keeps the buffer) read this instead of projecting
-            // (the sign of the depth carries the dropout flag: the readers need no second array)
+            // the second pass (and the backward pass, if the caller keeps the buffer) read the cache instead of
+            // projecting (the sign of the depth carries the dropout flag: the readers need no second array)
             // (only the projected points' flags are read: the 55 % outside the image cost no dropout bytes)
             const bool dropped = ok && pc.dropout && __builtin_nontemporal_load(pc.dropout + (size_t)b * pc.n + i) == 1.f;  // :314-315
-            // (a run of 64 points none of which is projected: marked in its first record, see kRunCulledBits)
-            const bool run_culled = !__ballot(ok);
-            if (valid)
-                nt_store4(pc.cache + (size_t)b * pc.n + i,
-                          ok ? make_float4(ip.x, ip.y, dropped ? -z : z, radius_pixels)
-                             : make_float4((run_culled && lane == 0) ? __uint_as_float(kRunCulledBits) : 0.f, 0, 0, 0));
+            const float4 rec   = ok ? make_float4(ip.x, ip.y, dropped ? -z : z, radius_pixels) : make_float4(0, 0, 0, 0);
+            const float4 mark  = make_float4(__uint_as_float(kRunCulledBits), 0, 0, 0);
+            // A run of 64 points none of which lands in the image at any level is marked in its first record, see
+            // kRunCulledBits.  The readers of a batch of views look at that record first and skip the run: its other
+            // records are not written at all (views 0..63, no counter pass).
+            const bool sparse = lv.B > 1 && b < 64 && !STATS;
             if (STATS) stat_add(&stats->bad_index, ok && !dropped && !tex_ok[k]);
-            if (!__ballot(ok) && !STATS)  // wavefront-uniform
+            if (!__ballot(ok) && !STATS)  // wavefront-uniform: nothing projected
             {
+                if (valid && (lane == 0 || !sparse)) nt_store4(pc.cache + (size_t)b * pc.n + i, lane == 0 ? mark : rec);
                 if (valid) __builtin_nontemporal_store(0u, bin.info + (size_t)b * pc.n + i);
                 continue;
             }
@@ -159,10 +160,10 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(PPT > 2 
             if (!__ballot(any_in))
             {
                 // projected, but all outside the image (a crop): the run counts as culled all the same
-                if (valid && lane == 0)
-                    nt_store4(pc.cache + (size_t)b * pc.n + i, make_float4(__uint_as_float(kRunCulledBits), 0, 0, 0));
+                if (valid && (lane == 0 || !sparse)) nt_store4(pc.cache + (size_t)b * pc.n + i, lane == 0 ? mark : rec);
                 continue;
             }
+            if (valid) nt_store4(pc.cache + (size_t)b * pc.n + i, rec);
             // one atomic per distinct tile of the wavefront, for the primary and for the second entries
             const unsigned long long below = (1ull << lane) - 1ull;
             const unsigned long long pm    = wave_group_mask(any_in, ptile);

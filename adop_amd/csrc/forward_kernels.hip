@@ -116,14 +116,6 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
             float z = 0.f, radius_pixels = 0.f;
             bool ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P[k].w, rp.check_normal != 0, rp.dist_cutoff,
                                              lv.l[0].w, &ip, &z, &radius_pixels, &view_p);
-            // the blend (and the backward pass, if the caller keeps the buffer) read this instead of projecting again
-            if (valid && pc.cache && !pc.list_ids)
-            {
-                // (the sign of the depth carries the dropout flag: the readers need no second array)
-                const bool dropped = pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;
-                pc.cache[(size_t)b * pc.n + i] =
-                    ok ? make_float4(ip.x, ip.y, dropped ? -z : z, radius_pixels) : make_float4(0, 0, 0, 0);
-            }
             zz[k]      = z;
             inmask[k]  = 0;
             rec[k]     = make_float4(ip.x, ip.y, 0.f, radius_pixels);
@@ -156,16 +148,33 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
                 }
             }
         }
-        // A run of 64 points none of which lands in the image at any level (a crop sees a small part of the cloud):
-        // its first record says so (kRunCulledBits), and the backward pass of several views skips the run.
+        // The blend (and the backward pass, if the caller keeps the buffer) read the projected points from the cache
+        // instead of projecting again; the sign of the depth carries the dropout flag (only the flags of points in the
+        // image are read; the counter pass reads those of all projected points).  A run of 64 points none of which
+        // lands in the image at any level (a crop sees a small part of the cloud): its first record says so
+        // (kRunCulledBits).  The readers of a batch of views look at that record first and skip the run, so its other
+        // records are not written at all (views 0..63, no counter pass).
         if (pc.cache && !pc.list_ids)
         {
+            const bool sparse = lv.B > 1 && b < 64 && !STATS;
 #pragma unroll
             for (int k = 0; k < PPT; ++k)
             {
-                const int i = base + k * kBlock;
-                if (!__ballot(inmask[k] != 0) && (threadIdx.x & 63) == 0 && i < pc.n)
-                    pc.cache[(size_t)b * pc.n + i] = make_float4(__uint_as_float(kRunCulledBits), 0, 0, 0);
+                const int i       = base + k * kBlock;
+                const bool culled = !__ballot(inmask[k] != 0);  // wavefront-uniform
+                if (culled && sparse)
+                {
+                    if (lane == 0 && i < pc.n)
+                        pc.cache[(size_t)b * pc.n + i] = make_float4(__uint_as_float(kRunCulledBits), 0, 0, 0);
+                }
+                else if (i < pc.n)
+                {
+                    const bool dropped = (inmask[k] != 0 || (STATS && okk[k])) && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;
+                    float4 r = okk[k] ? make_float4(rec[k].x, rec[k].y, dropped ? -zz[k] : zz[k], rec[k].w)
+                                      : make_float4(0, 0, 0, 0);
+                    if (culled && lane == 0) r = make_float4(__uint_as_float(kRunCulledBits), 0, 0, 0);
+                    pc.cache[(size_t)b * pc.n + i] = r;
+                }
             }
         }
         // List mode: the points of every wavefront that may still pass a depth test, compacted into the first slots of

@@ -139,7 +139,10 @@ typedef struct adop_forward_buffers
      * radius in pixels.  adop_forward writes it; adop_backward reads it instead of projecting when the same
      * buffer is passed back in `fwd`.  NULL: adop_forward keeps the records in the workspace, adop_backward
      * projects again.  When none of the points i..i+63 (i a multiple of 64) lands in the image of a view at any
-     * level, record i of that view holds the bits 0x7FC0C011 in x (and depth 0): adop_backward then skips the run. */
+     * level, record i of that view holds the bits 0x7FC0C011 in x (and depth 0): adop_backward then skips the run.
+     * In a call with several views the other 63 records of such a run are not written (for the first 64 views, and
+     * unless counters are collected): they keep whatever the buffer held.  A point outside the image at every level
+     * carries a positive depth whatever its dropout flag. */
     float* point_cache;
 } adop_forward_buffers;
 
