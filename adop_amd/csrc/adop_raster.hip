@@ -133,6 +133,7 @@ struct WorkspaceLayout
 constexpr int kTileLevels = 2;  // levels the tile path renders in LDS (a point has at most one bin entry per such level)
 constexpr int kTilePathMinPoints = 1 << 16;
 constexpr int kTilePathMaxPointsPerPixel = 16;
+constexpr int kWindowCloudShare = 16;  // a crop window is taken to see 1/16 of the cloud
 constexpr int kGroupedViewsMaxPoints = 4000000;  // backward: spatial gradients of a group of views in one launch
 
 size_t max_tiles(int B, int w0, int h0)
@@ -434,11 +435,19 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
                          max_tiles(num_views, views[0].w, views[0].h) < ((size_t)1 << 24);
     // The tile path bins every projected point; a cloud with very many points per pixel is faster through the direct
     // path, whose early depth test drops most of them before they cost anything.
+    // A batch of windows into their frames (crop offsets: the crops of a training step) counts with the share of the
+    // cloud that a window sees, taken as 1/16: a 512 x 512 window of a 1920 x 1080 frame holds an eighth of the
+    // frame's points, and a frame about half of the cloud.
     if (path == 0)
+    {
+        bool windows = num_views > 1;
+        for (int b = 0; b < num_views; ++b) windows = windows && (views[b].crop_cx != 0.f || views[b].crop_cy != 0.f);
+        const size_t per_pixel = (size_t)kTilePathMaxPointsPerPixel * (windows ? kWindowCloudShare : 1);
         path = (scene->num_points >= kTilePathMinPoints &&
-                (size_t)scene->num_points <= (size_t)kTilePathMaxPointsPerPixel * views[0].w * views[0].h)
+                (size_t)scene->num_points <= per_pixel * views[0].w * views[0].h)
                    ? 2
                    : 1;
+    }
     if (path == 2 && !can_bin) path = 1;
 
     if (path == 2)

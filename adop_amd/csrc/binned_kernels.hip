@@ -98,38 +98,67 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(PPT > 2 
         }
     }
 
+    // (the crops of one frame follow each other in a training batch: the point in the uncropped image is kept from
+    // one view to the next, only the crop transform and the radius are computed per view)
+    V2 frame_p[PPT];
+    float frame_z[PPT];
+    const ImageBox box = image_box(lv);
     for (int b = 0; b < lv.B; ++b)
     {
         const ViewConst& vc = views[b];
+        const bool same_frame = b > 0 && vc.image_index == views[b - 1].image_index &&
+                                vc.camera_index == views[b - 1].camera_index && vc.model == views[b - 1].model;  // uniform
 #pragma unroll
         for (int k = 0; k < PPT; ++k)
         {
             const int i      = base + k * kBlock;
             const bool valid = i < pc.n;
-            V3 pos           = {P[k].x, P[k].y, P[k].z};
-            V3 nrm           = unpack_normal10(nenc[k]);
             V2 ip            = {0.f, 0.f};
-            V3 view_p;
-            float z = 0.f, radius_pixels = 0.f;
-            bool ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P[k].w, rp.check_normal != 0, rp.dist_cutoff,
-                                             lv.l[0].w, &ip, &z, &radius_pixels, &view_p);
-            // the second pass (and the backward pass, if the caller keeps the buffer) read the cache instead of
-            // projecting (the sign of the depth carries the dropout flag: the readers need no second array)
-            // (only the projected points' flags are read: the 55 % outside the image cost no dropout bytes)
-            const bool dropped = ok && pc.dropout && __builtin_nontemporal_load(pc.dropout + (size_t)b * pc.n + i) == 1.f;  // :314-315
-            const float4 rec   = ok ? make_float4(ip.x, ip.y, dropped ? -z : z, radius_pixels) : make_float4(0, 0, 0, 0);
-            const float4 mark  = make_float4(__uint_as_float(kRunCulledBits), 0, 0, 0);
-            // A run of 64 points none of which lands in the image at any level is marked in its first record, see
-            // kRunCulledBits.  The readers of a batch of views look at that record first and skip the run: its other
-            // records are not written at all (views 0..63, no counter pass).
-            const bool sparse = lv.B > 1 && b < 64 && !STATS;
-            if (STATS) stat_add(&stats->bad_index, ok && !dropped && !tex_ok[k]);
-            if (!__ballot(ok) && !STATS)  // wavefront-uniform: nothing projected
+            float radius_pixels = 0.f;
+            if (!same_frame)
             {
-                if (valid && (lane == 0 || !sparse)) nt_store4(pc.cache + (size_t)b * pc.n + i, lane == 0 ? mark : rec);
+                V3 pos = {P[k].x, P[k].y, P[k].z};
+                V3 nrm = unpack_normal10(nenc[k]);
+                V3 view_p;
+                frame_p[k] = {0.f, 0.f};
+                frame_z[k] = 0.f;
+                if (valid)
+                    project_frame(vc, pc.intrinsics, pos, nrm, rp.check_normal != 0, rp.dist_cutoff, &frame_p[k], &frame_z[k],
+                                  &view_p);
+            }
+            const float z = frame_z[k];
+            const bool ok = z != 0;
+            if (ok) ip = k_apply(vc.crop, frame_p[k]);
+            // The second pass (and the backward pass, if the caller keeps the buffer) read the cache instead of
+            // projecting.  A run of 64 points none of which lands in the image at any level is marked in its first
+            // record, see kRunCulledBits.  The readers of a batch of views look at that record first and skip the run:
+            // its other records are not written at all (views 0..63, no counter pass).
+            const bool sparse = lv.B > 1 && b < 64 && !STATS;
+            const float4 mark = make_float4(__uint_as_float(kRunCulledBits), 0, 0, 0);
+            // a crop sees a small part of the cloud: most runs are nowhere near it (or not projected at all)
+            const bool near_image = __ballot(ok && !outside_every_level(box, ip)) != 0;  // wavefront-uniform
+            if (!near_image && !STATS)
+            {
+                if (sparse)
+                {
+                    if (valid && lane == 0) nt_store4(pc.cache + (size_t)b * pc.n + i, mark);
+                }
+                else if (valid)
+                {
+                    const bool dropped = ok && pc.dropout && __builtin_nontemporal_load(pc.dropout + (size_t)b * pc.n + i) == 1.f;
+                    const float4 far   = ok ? make_float4(ip.x, ip.y, dropped ? -z : z, crop_radius(vc, z, P[k].w, lv.l[0].w))
+                                            : make_float4(0, 0, 0, 0);
+                    nt_store4(pc.cache + (size_t)b * pc.n + i, lane == 0 ? mark : far);
+                }
                 if (valid) __builtin_nontemporal_store(0u, bin.info + (size_t)b * pc.n + i);
                 continue;
             }
+            if (ok) radius_pixels = crop_radius(vc, z, P[k].w, lv.l[0].w);
+            // (the sign of the depth carries the dropout flag: the readers need no second array; only the projected
+            // points' flags are read)
+            const bool dropped = ok && pc.dropout && __builtin_nontemporal_load(pc.dropout + (size_t)b * pc.n + i) == 1.f;  // :314-315
+            const float4 rec   = ok ? make_float4(ip.x, ip.y, dropped ? -z : z, radius_pixels) : make_float4(0, 0, 0, 0);
+            if (STATS) stat_add(&stats->bad_index, ok && !dropped && !tex_ok[k]);
 
             bool in[ADOP_MAX_LAYERS];
             bool any_in;

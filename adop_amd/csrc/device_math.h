@@ -270,17 +270,18 @@ __device__ __forceinline__ void ocam_core(V3 p, const float* aff, const float* p
     }
 }
 
-// Head of the three reference point kernels (PointRenderer.cu:227-256, 334-359, 409-438):
-// ProjectPointPinhole / ProjectPointOcam (PointRendererHelper.h:49-106), the LOD radius in pixels and the
-// crop transform.  Returns false when the point is culled (z == 0).
-__device__ __forceinline__ bool project_point(const ViewConst& vc, const float* __restrict__ intrinsics, V3 pos,
-                                              V3 nrm, float radius, bool check_normal, float dist_cutoff, int w0,
-                                              V2* ip, float* z_out, float* radius_pixels, V3* view_p_out)
+// Head of the three reference point kernels (PointRenderer.cu:227-256, 334-359, 409-438), in two parts.
+// First part, the same for every crop of one frame (pose and camera model): ProjectPointPinhole / ProjectPointOcam
+// (PointRendererHelper.h:49-106) up to the point in the uncropped image.  Returns false when the point is culled
+// (z == 0).
+__device__ __forceinline__ bool project_frame(const ViewConst& vc, const float* __restrict__ intrinsics, V3 pos, V3 nrm,
+                                              bool check_normal, float dist_cutoff, V2* image_p_out, float* z_out,
+                                              V3* view_p_out)
 {
     V3 r      = quat_rotate(vc.qx, vc.qy, vc.qz, vc.qw, pos);
     V3 view_p = {r.x + vc.tx, r.y + vc.ty, r.z + vc.tz};
     *view_p_out = view_p;
-    V2 image_p;
+    V2 image_p = {0.f, 0.f};
     float z;
     if (vc.model == 0)
     {
@@ -293,16 +294,15 @@ __device__ __forceinline__ bool project_point(const ViewConst& vc, const float* 
         // culled: nothing below can bring the point back; Morton-ordered clouds cull whole wavefronts here
         if (z == 0)
         {
-            *z_out         = 0;
-            *radius_pixels = 0;
+            *z_out       = 0;
+            *image_p_out = image_p;
             return false;
         }
         float iz  = 1.0f / view_p.z;
         V2 norm_p = {view_p.x * iz, view_p.y * iz};
         V2 dist_p = distort<false>(norm_p, vc.d, dist_cutoff, nullptr, nullptr);
         if (dist_p.x == 100000.f) z = 0;
-        image_p        = k_apply(vc.k, dist_p);
-        *radius_pixels = vc.k[0] * vc.crop[0] * radius / z;
+        image_p = k_apply(vc.k, dist_p);
     }
     else
     {
@@ -310,11 +310,60 @@ __device__ __forceinline__ bool project_point(const ViewConst& vc, const float* 
         ocam_core<false>(view_p, row, row + 5, vc.npoly, dist_cutoff, &image_p, &z, nullptr, nullptr);
         V3 view_n = quat_rotate(vc.qx, vc.qy, vc.qz, vc.qw, nrm);
         if (check_normal & (dot3(view_p, view_n) > 0)) z = 0;
-        *radius_pixels = (float)w0 * vc.crop[0] * radius / z;
     }
-    *z_out = z;
-    if (z == 0) return false;
-    *ip = k_apply(vc.crop, image_p);
+    *z_out       = z;
+    *image_p_out = image_p;
+    return z != 0;
+}
+
+// Second part, per crop: the LOD radius in pixels and the crop transform of a point that project_frame kept.
+__device__ __forceinline__ float crop_radius(const ViewConst& vc, float z, float radius, int w0)
+{
+    return (vc.model == 0 ? vc.k[0] : (float)w0) * vc.crop[0] * radius / z;
+}
+
+__device__ __forceinline__ void project_crop(const ViewConst& vc, V2 image_p, float z, float radius, int w0, V2* ip,
+                                             float* radius_pixels)
+{
+    *radius_pixels = crop_radius(vc, z, radius, w0);
+    *ip            = k_apply(vc.crop, image_p);
+}
+
+// A level-0 image point outside this box lands outside the image at every level: level l takes the pixel
+// rint(ip * 0.5^l) (an exact scaling), which is inside only if -0.5 <= ip * 0.5^l <= w_l - 0.5.  The box is wider than
+// that by a pixel of the coarsest level on every side; a NaN is never outside (its pixel is 0, as in the reference).
+struct ImageBox
+{
+    float lo, hi_x, hi_y;
+};
+
+template <class LevelsT>
+__device__ __forceinline__ ImageBox image_box(const LevelsT& lv)
+{
+    ImageBox box = {-(float)(1 << lv.num), 0.f, 0.f};
+#pragma unroll
+    for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
+        if (l < lv.num)
+        {
+            box.hi_x = fmaxf(box.hi_x, (float)(lv.l[l].w + 1) * (float)(1 << l));
+            box.hi_y = fmaxf(box.hi_y, (float)(lv.l[l].h + 1) * (float)(1 << l));
+        }
+    return box;
+}
+
+__device__ __forceinline__ bool outside_every_level(const ImageBox& box, V2 ip)
+{
+    return ip.x < box.lo || ip.x > box.hi_x || ip.y < box.lo || ip.y > box.hi_y;
+}
+
+__device__ __forceinline__ bool project_point(const ViewConst& vc, const float* __restrict__ intrinsics, V3 pos,
+                                              V3 nrm, float radius, bool check_normal, float dist_cutoff, int w0,
+                                              V2* ip, float* z_out, float* radius_pixels, V3* view_p_out)
+{
+    V2 image_p;
+    *radius_pixels = 0;
+    if (!project_frame(vc, intrinsics, pos, nrm, check_normal, dist_cutoff, &image_p, z_out, view_p_out)) return false;
+    project_crop(vc, image_p, *z_out, radius, w0, ip, radius_pixels);
     return true;
 }
 

@@ -93,9 +93,11 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
         nenc[k] = (i < pc.n && pc.normal) ? pc.normal[i] : 0;
     }
 
+    const ImageBox box = image_box(lv);
     for (int b = 0; b < lv.B; ++b)
     {
         const ViewConst& vc = views[b];
+        const bool sparse = lv.B > 1 && b < 64 && !STATS;  // (the cache records of a run outside the view: see below)
         // phase 1: projection, pixel of every level and the early-z read (PointRenderer.cu:278) of the depth word;
         // the loads are independent.  A stale value only costs a redundant atomic.
         uint32_t pix[PPT][ADOP_MAX_LAYERS];
@@ -112,10 +114,18 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
             V3 pos     = {P[k].x, P[k].y, P[k].z};
             V3 nrm     = unpack_normal10(nenc[k]);
             V2 ip = {0.f, 0.f};
+            float radius_pixels = 0.f;
+            // (keeping the point in the uncropped image from one crop of a frame to the next, as the tile path does,
+            // costs this kernel more in registers than it saves: a single view of 100 M points ran 17 % slower)
             V3 view_p;
-            float z = 0.f, radius_pixels = 0.f;
-            bool ok = valid && project_point(vc, pc.intrinsics, pos, nrm, P[k].w, rp.check_normal != 0, rp.dist_cutoff,
-                                             lv.l[0].w, &ip, &z, &radius_pixels, &view_p);
+            V2 frame_p = {0.f, 0.f};
+            float z    = 0.f;
+            if (valid) project_frame(vc, pc.intrinsics, pos, nrm, rp.check_normal != 0, rp.dist_cutoff, &frame_p, &z, &view_p);
+            const bool ok = z != 0;
+            if (ok) ip = k_apply(vc.crop, frame_p);
+            // a crop sees a small part of the cloud: most runs of 64 points are nowhere near it and skip the levels
+            const bool near_image = __ballot(ok && !outside_every_level(box, ip)) != 0;  // wavefront-uniform
+            if (ok && (near_image || !sparse)) radius_pixels = crop_radius(vc, z, P[k].w, lv.l[0].w);
             zz[k]      = z;
             inmask[k]  = 0;
             rec[k]     = make_float4(ip.x, ip.y, 0.f, radius_pixels);
@@ -126,7 +136,7 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
             {
                 pix[k][l] = 0;
                 cur[k][l] = 0;
-                if (l < lv.num)
+                if (l < lv.num && near_image)
                 {
                     if (rp.drop_by_radius && radius_pixels < rp.drop_threshold) alive = false;  // break, :261-264
                     const LevelArg& L = lv.l[l];
@@ -156,7 +166,6 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
         // records are not written at all (views 0..63, no counter pass).
         if (pc.cache && !pc.list_ids)
         {
-            const bool sparse = lv.B > 1 && b < 64 && !STATS;
 #pragma unroll
             for (int k = 0; k < PPT; ++k)
             {
