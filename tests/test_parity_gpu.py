@@ -316,3 +316,36 @@ def test_runs_that_miss_a_view_are_marked_and_skipped(oracle_mod, forward_path):
         inside = (z != 0) & ~np.isnan(ipx) & (np.rint(ipx) >= 0) & (np.rint(ipx) < 64) & (np.rint(ipy) >= 0) & (np.rint(ipy) < 48)
     inside &= ~np.repeat(marked, 64, axis=1)[:, :n]
     assert int(inside.sum()) == ref.stats.visible[0]
+
+
+@pytest.mark.parametrize("forward_path", [1, 2], ids=["direct", "tiles"])
+def test_runs_left_of_the_image_still_reach_the_coarse_levels(oracle_mod, forward_path):
+    """Level l takes the pixel rint(ip * 0.5^l): a point up to half a coarse pixel left of (or above) the image is
+    outside at level 0 and inside at a coarser level.  The cloud is ordered by image x here, so that whole runs of 64
+    points lie in that band: a forward that drops runs by their level-0 position alone loses them."""
+    from adop_amd import scenes
+
+    n, w, h = 60_000, 250, 186
+    hs = scenes.config2(n=n, w=w, h=h, levels=5, batch=1, seed=3)
+    hs.params.forward_path = 1
+    scene, info, ctx, images, masks = run_hip_forward(hs)
+    cache = info.cache.point_cache.cpu().numpy()[0]  # one view: every record is written
+    x_full = np.where(cache[:, 2] != 0, cache[:, 0], np.inf)
+    order = np.argsort(x_full, kind="stable")
+    hs.position, hs.index = hs.position[order], hs.index[order]
+    if hs.normal is not None:
+        hs.normal = hs.normal[order]
+    x_full, y_full = x_full[order], cache[order, 1]
+    # two windows of 128 x 96 whose left edges cut through the cloud
+    offsets = [(-70.0, -40.0), (-101.0, -60.0)]
+    hs.views = [scenes.make_view(128, 96, image_index=0, crop=(1.0, 1.0, cx, cy, 0.0)) for cx, cy in offsets]
+    hs.dropout = scenes.bernoulli_mask(5, 2, n, 0.2)
+    hs.params.forward_path = forward_path
+    for cx, cy in offsets:
+        band = (x_full + cx >= -7.9) & (x_full + cx < -0.6)
+        runs = np.add.reduceat(band.astype(np.int64), np.arange(0, n, 64))
+        whole = np.repeat(runs == 64, 64)[:n]
+        assert (runs == 64).sum() >= 3, "the scene no longer puts whole runs into the band"
+        assert (whole & (y_full + cy > 0) & (y_full + cy < 95)).sum() >= 64  # and those runs have points at image height
+    announce(f"runs of 64 points in the band left of two windows: N={n} 128x96 L=5 forward_path={forward_path}")
+    _fwd_bwd(hs, oracle_mod)
