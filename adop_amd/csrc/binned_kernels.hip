@@ -141,6 +141,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(PPT > 2 
             {
                 if (sparse)
                 {
+                    // (the second pass sees the mark and reads no tile words of the run)
                     if (valid && lane == 0) nt_store4(pc.cache + (size_t)b * pc.n + i, mark);
                 }
                 else if (valid)
@@ -149,8 +150,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(PPT > 2 
                     const float4 far   = ok ? make_float4(ip.x, ip.y, dropped ? -z : z, crop_radius(vc, z, P[k].w, lv.l[0].w))
                                             : make_float4(0, 0, 0, 0);
                     nt_store4(pc.cache + (size_t)b * pc.n + i, lane == 0 ? mark : far);
+                    __builtin_nontemporal_store(0u, bin.info + (size_t)b * pc.n + i);
                 }
-                if (valid) __builtin_nontemporal_store(0u, bin.info + (size_t)b * pc.n + i);
                 continue;
             }
             if (ok) radius_pixels = crop_radius(vc, z, P[k].w, lv.l[0].w);
@@ -213,15 +214,39 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels
     const int base = blockIdx.x * (kBlock * PPT) + threadIdx.x;
     const unsigned long long below = (1ull << lane) - 1ull;
 
+    // Several views: the first pass marked the runs of 64 points that miss a view entirely in the first record of the
+    // run (kRunCulledBits) and wrote no tile words for them; lane b asks for view b, for all views at once.
+    unsigned long long culled_views[PPT];
+#pragma unroll
+    for (int k = 0; k < PPT; ++k)
+    {
+        culled_views[k] = 0;
+        if (lv.B > 1)  // kernel-uniform
+        {
+            const int first = (base + k * kBlock) & ~63;
+            bool c          = false;
+            if (lane < lv.B && first < pc.n)
+            {
+                const float4 head = pc.cache[(size_t)lane * pc.n + first];
+                c                 = __float_as_uint(head.x) == kRunCulledBits && head.z == 0.f;
+            }
+            culled_views[k] = __ballot(c);
+        }
+    }
+
     for (int b = 0; b < lv.B; ++b)
     {
         uint32_t info[PPT];
+        bool any = false;
 #pragma unroll
         for (int k = 0; k < PPT; ++k)
         {
-            const int i = base + k * kBlock;
-            info[k]     = i < pc.n ? __builtin_nontemporal_load(bin.info + (size_t)b * pc.n + i) : 0u;
+            const int i       = base + k * kBlock;
+            const bool culled = b < 64 && (culled_views[k] >> b & 1ull) != 0;  // wavefront-uniform
+            info[k]           = (i < pc.n && !culled) ? __builtin_nontemporal_load(bin.info + (size_t)b * pc.n + i) : 0u;
+            any |= !culled;
         }
+        if (!any) continue;  // wavefront-uniform
         float4 R[PPT];
 #pragma unroll
         for (int k = 0; k < PPT; ++k)
