@@ -191,6 +191,13 @@ def load_library(path=None):
             "(run `python -c 'import __graft_entry__ as g; g.build()'` or `make -C adop_amd/csrc`). "
             "There is no CPU fallback."
         )
+    # PyTorch ships a HIP runtime of its own.  Loaded after this library it would come up as a second copy beside the
+    # system's one, and only one copy gets the GPU (the other reports "no ROCm-capable device"): import torch first,
+    # so that the library binds to the runtime torch has already loaded.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     lib = C.CDLL(p)
     for name, (restype, argtypes) in ENTRY_POINTS.items():
         fn = getattr(lib, name)

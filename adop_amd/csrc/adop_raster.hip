@@ -661,14 +661,24 @@ static adop_status env_common(const adop_scene* scene, const adop_view* views, i
     if (num_views > 32) return fail(ADOP_INVALID_ARG, "environment map: at most 32 views per call");
     for (int b = 0; b < num_views; ++b)
     {
-        // SAIGA_ASSERT(cam.camera_model_type == CameraModel::PINHOLE_DISTORTION), EnvironmentMap.cu:129
-        if (views[b].camera_model_type != ADOP_CAMERA_PINHOLE_DISTORTION)
-            return fail(ADOP_INVALID_ARG, "environment map needs the pinhole model");
+        // The reference samples pinhole views only (SAIGA_ASSERT(cam.camera_model_type == PINHOLE_DISTORTION),
+        // EnvironmentMap.cu:129); OCam views are an extension here: pixel -> ray through ocam_unproject.
+        if (views[b].camera_model_type == ADOP_CAMERA_PINHOLE_DISTORTION)
+        {
+            if (scene->intrinsics_cols != 13) return fail(ADOP_INVALID_ARG, "pinhole intrinsics need 13 columns");
+        }
+        else if (views[b].camera_model_type == ADOP_CAMERA_OCAM)
+        {
+            if (scene->intrinsics_cols < 6 || scene->intrinsics_cols > kMaxIntrinsicsCols)
+                return fail(ADOP_INVALID_ARG, "OCam intrinsics need 6 .. 24 columns");
+        }
+        else
+            return fail(ADOP_INVALID_ARG, "unknown camera model");
         if (views[b].image_index < 0 || views[b].image_index >= scene->num_poses || views[b].camera_index < 0 ||
             views[b].camera_index >= scene->num_cameras)
             return fail(ADOP_INVALID_ARG, "view index out of range");
     }
-    if (scene->intrinsics_cols != 13) return fail(ADOP_INVALID_ARG, "pinhole intrinsics need 13 columns");
+    if (!scene->poses_se3 || !scene->intrinsics) return fail(ADOP_INVALID_ARG, "poses / intrinsics missing");
     return ADOP_OK;
 }
 
@@ -698,7 +708,8 @@ adop_status adop_env_sample(const adop_scene* scene, const adop_view* views, int
         ev.env[l] = env_levels ? env_levels[l] : nullptr;
         if (add_to_out && !buffers->layers[l].out) return fail(ADOP_INVALID_ARG, "out buffer missing");
     }
-    launch_env_sample(chunk, scene->poses_se3, scene->intrinsics, lv, ev, env_texture, env_h, env_w, add_to_out, stream);
+    launch_env_sample(chunk, scene->poses_se3, scene->intrinsics, lv, ev, env_texture, env_h, env_w, add_to_out,
+                      scene->intrinsics_cols, stream);
     ADOP_HIP_CHECK(hipGetLastError());
     return ADOP_OK;
 }
@@ -722,7 +733,8 @@ adop_status adop_env_sample_backward(const adop_scene* scene, const adop_view* v
     }
     st = fill_async(grad_env, sizeof(float) * (size_t)scene->num_channels * env_h * env_w, 0, stream);
     if (st != ADOP_OK) return st;
-    launch_env_backward(chunk, scene->poses_se3, scene->intrinsics, lv, ev, grad_env, env_h, env_w, stream);
+    launch_env_backward(chunk, scene->poses_se3, scene->intrinsics, lv, ev, grad_env, env_h, env_w, scene->intrinsics_cols,
+                        stream);
     ADOP_HIP_CHECK(hipGetLastError());
     return ADOP_OK;
 }

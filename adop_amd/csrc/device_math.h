@@ -128,6 +128,23 @@ __device__ __forceinline__ float acos_poly(float x)
     return ADOP_HALF_PI - asin_poly(x);
 }
 
+// sine and cosine of an angle in [-pi/2, pi/2] (Cephes single-precision kernels on [-pi/4, pi/4], the rest through
+// the complementary angle), + - * only.
+__device__ __forceinline__ void sincos_poly(float theta, float* s_out, float* c_out)
+{
+    float a     = theta < 0 ? -theta : theta;
+    bool compl_ = a > ADOP_QUART_PI;
+    float x     = compl_ ? ADOP_HALF_PI - a : a;
+    float z     = x * x;
+    float sn    = ((-1.9515295891e-4f * z + 8.3321608736e-3f) * z - 1.6666654611e-1f) * z * x + x;
+    float cs    = ((2.443315711809948e-5f * z - 1.388731625493765e-3f) * z + 4.166664568298827e-2f) * z * z +
+               (1.0f - 0.5f * z);
+    float s = compl_ ? cs : sn;
+    float c = compl_ ? sn : cs;
+    *s_out  = theta < 0 ? -s : s;
+    *c_out  = c;
+}
+
 __device__ __forceinline__ V3 cross3(V3 a, V3 b)
 {
     return {a.y * b.z - a.z * b.y, a.z * b.x - a.x * b.z, a.x * b.y - a.y * b.x};
@@ -268,6 +285,41 @@ __device__ __forceinline__ void ocam_core(V3 p, const float* aff, const float* p
         Ja[0] = uu; Ja[1] = vv; Ja[2] = 0;  Ja[3] = 1; Ja[4] = 0;
         Ja[5] = 0;  Ja[6] = 0;  Ja[7] = uu; Ja[8] = 0; Ja[9] = 1;
     }
+}
+
+// Pixel of the uncropped OCam image -> unit ray in camera space, the inverse of ocam_core (the reference has none: its
+// environment map asserts the pinhole model, EnvironmentMap.cu:129): undo the affine map, solve poly(theta) = rho with
+// kOcamNewtonSteps Newton steps from the axis (theta = -pi/2), theta kept in [-pi/2, pi/2]; the ray is
+// (cos(theta) * (uu,vv)/rho, -sin(theta)), so that theta = atan(-z / |xy|) as in the forward direction.
+constexpr int kOcamNewtonSteps = 8;
+__device__ __forceinline__ V3 ocam_unproject(const float* aff, const float* poly, int npoly, V2 ip)
+{
+    float c = aff[0], d = aff[1], e = aff[2], cx = aff[3], cy = aff[4];
+    float px = ip.x - cx, py = ip.y - cy;
+    float det   = c - d * e;
+    float uu    = (px - d * py) / det;
+    float vv    = (c * py - e * px) / det;
+    float rho   = sqrtf(uu * uu + vv * vv);
+    float theta = -ADOP_HALF_PI;
+    for (int it = 0; it < kOcamNewtonSteps; ++it)
+    {
+        float r   = poly[0];
+        float dr  = 0;
+        float t_i = 1;
+        for (int i = 1; i < npoly; ++i)
+        {
+            dr += (float)i * poly[i] * t_i;
+            t_i *= theta;
+            r += t_i * poly[i];
+        }
+        if (dr != 0) theta = theta - (r - rho) / dr;
+        theta = fminf(fmaxf(theta, -ADOP_HALF_PI), ADOP_HALF_PI);
+    }
+    float sn, cs;
+    sincos_poly(theta, &sn, &cs);
+    float cxn = rho > 0 ? uu / rho : 0.f;
+    float cyn = rho > 0 ? vv / rho : 0.f;
+    return {cxn * cs, cyn * cs, -sn};
 }
 
 // Head of the three reference point kernels (PointRenderer.cu:227-256, 334-359, 409-438), in two parts.

@@ -35,16 +35,27 @@ __device__ __forceinline__ V2 undistort_simple(V2 p, const float* D)
 }
 
 // BuildSphericalUV + SphericalCoordinates for pixel (gx,gy) of a level whose crop is scaled by `sc`.
-__device__ __forceinline__ V2 spherical_uv(const ViewConst& vc, float sc, int gx, int gy)
+__device__ __forceinline__ V2 spherical_uv(const ViewConst& vc, const float* __restrict__ intrinsics, float sc, int gx,
+                                           int gy)
 {
     float cr[5] = {vc.crop[0] * sc, vc.crop[1] * sc, vc.crop[2] * sc, vc.crop[3] * sc, vc.crop[4] * sc};
     V3 t    = {vc.tx, vc.ty, vc.tz};
     V3 rt   = quat_rotate(-vc.qx, -vc.qy, -vc.qz, vc.qw, t);
     V3 tinv = {-rt.x, -rt.y, -rt.z};
     V2 ip   = {(float)gx, (float)gy};
-    V2 dist_p = k_unproject2(vc.k, k_unproject2(cr, ip));
-    V2 np     = undistort_simple(dist_p, vc.d);
-    V3 inp    = {np.x, np.y, 1};
+    V3 inp;
+    if (vc.model == 0)
+    {
+        V2 dist_p = k_unproject2(vc.k, k_unproject2(cr, ip));
+        V2 np     = undistort_simple(dist_p, vc.d);
+        inp       = {np.x, np.y, 1};
+    }
+    else
+    {
+        // OCam views (not in the reference, which asserts the pinhole model, EnvironmentMap.cu:129)
+        const float* row = intrinsics + vc.intr_offset;
+        inp              = ocam_unproject(row, row + 5, vc.npoly, k_unproject2(cr, ip));
+    }
     V3 r      = quat_rotate(-vc.qx, -vc.qy, -vc.qz, vc.qw, inp);
     V3 wp     = {r.x + tinv.x, r.y + tinv.y, r.z + tinv.z};
     V3 d      = {wp.x - tinv.x, wp.y - tinv.y, wp.z - tinv.z};
@@ -89,7 +100,7 @@ __device__ __forceinline__ Bilinear bilinear_setup(V2 uv, int ew, int eh)
 __global__ __launch_bounds__(kBlock) void env_sample_kernel(ViewChunk chunk, const double* __restrict__ poses,
                                                             const float* __restrict__ intrinsics, Levels lv,
                                                             EnvLevels ev, const float* __restrict__ tex, int eh, int ew,
-                                                            int add_to_out)
+                                                            int add_to_out, int cols)
 {
     int per_image = lv.pix_prefix[lv.num];
     size_t total  = (size_t)per_image * lv.B;
@@ -111,7 +122,7 @@ __global__ __launch_bounds__(kBlock) void env_sample_kernel(ViewChunk chunk, con
     if (add_to_out && L.mask) bgw = 1.f - L.mask[(size_t)b * hw + p];
     bool need = ev.uv[l] || ev.env[l] || (add_to_out && bgw != 0.f);
     if (!need) return;
-    V2 uv = spherical_uv(make_view_const(chunk.v[b], poses, intrinsics, 13), sc, gx, gy);
+    V2 uv = spherical_uv(make_view_const(chunk.v[b], poses, intrinsics, cols), intrinsics, sc, gx, gy);
     if (ev.uv[l])
     {
         ev.uv[l][((size_t)b * hw + p) * 2 + 0] = uv.x;
@@ -135,7 +146,8 @@ __global__ __launch_bounds__(kBlock) void env_sample_kernel(ViewChunk chunk, con
 
 __global__ __launch_bounds__(kBlock) void env_backward_kernel(ViewChunk chunk, const double* __restrict__ poses,
                                                               const float* __restrict__ intrinsics, Levels lv,
-                                                              EnvLevels ev, float* __restrict__ genv, int eh, int ew)
+                                                              EnvLevels ev, float* __restrict__ genv, int eh, int ew,
+                                                              int cols)
 {
     int per_image = lv.pix_prefix[lv.num];
     size_t total  = (size_t)per_image * lv.B;
@@ -156,7 +168,7 @@ __global__ __launch_bounds__(kBlock) void env_backward_kernel(ViewChunk chunk, c
     float bgw = 1.f;
     if (L.mask) bgw = 1.f - L.mask[(size_t)b * hw + p];
     if (bgw == 0.f) return;
-    V2 uv      = spherical_uv(make_view_const(chunk.v[b], poses, intrinsics, 13), sc, gx, gy);
+    V2 uv      = spherical_uv(make_view_const(chunk.v[b], poses, intrinsics, cols), intrinsics, sc, gx, gy);
     Bilinear s = bilinear_setup(uv, ew, eh);
     for (int c = 0; c < lv.C; ++c)
     {
@@ -222,23 +234,23 @@ __global__ void apply_tangent_kernel(double* __restrict__ tangent, double* __res
 
 
 void launch_env_sample(const ViewChunk& chunk, const double* poses, const float* intrinsics, const Levels& lv,
-                       const EnvLevels& ev, const float* tex, int eh, int ew, int add_to_out, hipStream_t st)
+                       const EnvLevels& ev, const float* tex, int eh, int ew, int add_to_out, int cols, hipStream_t st)
 {
     size_t total = (size_t)lv.pix_prefix[lv.num] * lv.B;
     int grid     = (int)((total + kBlock - 1) / kBlock);
     if (grid > 0)
         hipLaunchKernelGGL(env_sample_kernel, dim3(grid), dim3(kBlock), 0, st, chunk, poses, intrinsics, lv, ev, tex, eh,
-                           ew, add_to_out);
+                           ew, add_to_out, cols);
 }
 
 void launch_env_backward(const ViewChunk& chunk, const double* poses, const float* intrinsics, const Levels& lv,
-                         const EnvLevels& ev, float* genv, int eh, int ew, hipStream_t st)
+                         const EnvLevels& ev, float* genv, int eh, int ew, int cols, hipStream_t st)
 {
     size_t total = (size_t)lv.pix_prefix[lv.num] * lv.B;
     int grid     = (int)((total + kBlock - 1) / kBlock);
     if (grid > 0)
         hipLaunchKernelGGL(env_backward_kernel, dim3(grid), dim3(kBlock), 0, st, chunk, poses, intrinsics, lv, ev, genv,
-                           eh, ew);
+                           eh, ew, cols);
 }
 
 void launch_apply_tangent(double* tangent, double* poses, int n, hipStream_t st)

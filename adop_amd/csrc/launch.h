@@ -105,8 +105,8 @@ void launch_finalize(const ViewConst* views, int B, int C, const double* bg_part
                      const QueueArg& q, hipStream_t st);
 
 void launch_env_sample(const ViewChunk& chunk, const double* poses, const float* intrinsics, const Levels& lv,
-                       const EnvLevels& ev, const float* tex, int eh, int ew, int add_to_out, hipStream_t st);
+                       const EnvLevels& ev, const float* tex, int eh, int ew, int add_to_out, int cols, hipStream_t st);
 void launch_env_backward(const ViewChunk& chunk, const double* poses, const float* intrinsics, const Levels& lv,
-                         const EnvLevels& ev, float* genv, int eh, int ew, hipStream_t st);
+                         const EnvLevels& ev, float* genv, int eh, int ew, int cols, hipStream_t st);
 void launch_apply_tangent(double* tangent, double* poses, int n, hipStream_t st);
 }  // namespace adop

@@ -192,7 +192,15 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
 /* Replaces EnvironmentMapImpl::Sample (EnvironmentMap.cu:107-157: BuildSphericalUV + grid_sample bilinear /
  * border / align_corners) fused with the composition images += (1-mask)*env (RenderModule.cpp:121-125).
  * env_texture [C,eh,ew] f32. For level l: uv_l [B,h_l,w_l,2] (may be NULL), env_l [B,C,h_l,w_l] (may be NULL),
- * and, if add_to_out != 0, out_l += (1 - mask_l) * env. */
+ * and, if add_to_out != 0, out_l += (1 - mask_l) * env.
+ * Pinhole views: the pixel's ray as in BuildSphericalUV (EnvironmentMap.cu:82-90: unproject2 through crop and K,
+ * undistortNormalizedPointSimple).  OCam views (the reference asserts pinhole, EnvironmentMap.cu:129; this is an
+ * extension): the ray comes from inverting the world2cam polynomial of the intrinsics row itself (no cam2world
+ * polynomial is passed): the affine map (c,d,e,cx,cy) is undone, poly(theta) = rho is solved by 8 Newton steps from
+ * the optical axis (theta = -pi/2) with theta kept in [-pi/2, pi/2], and the camera-space ray is
+ * (cos(theta) * (uu,vv)/rho, -sin(theta)), i.e. the inverse of ProjectOCam (PointRendererHelper.h:85-106) wherever the
+ * polynomial is monotonic; pixels the polynomial does not reach take the ray of the nearest end of that range.
+ * Everything after the ray (rotation to world space, SphericalCoordinates, sampling) is EnvironmentMap.cu:41-105. */
 adop_status adop_env_sample(const adop_scene* scene, const adop_view* views, int32_t num_views,
                             const float* env_texture, int32_t env_h, int32_t env_w, const adop_forward_buffers* buffers,
                             float* const* uv_levels, float* const* env_levels, int32_t add_to_out, void* hip_stream);

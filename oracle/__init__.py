@@ -67,6 +67,12 @@ def lib(omp=False):
         L.oracle_distort.argtypes = [C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p]
         L.oracle_undistort.restype = None
         L.oracle_undistort.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+        L.oracle_sincosf.restype = None
+        L.oracle_sincosf.argtypes = [C.c_float, C.c_void_p]
+        L.oracle_ocam_unproject.restype = None
+        L.oracle_ocam_unproject.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
+        L.oracle_ocam_core.restype = None
+        L.oracle_ocam_core.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_void_p]
         L.oracle_num_threads.restype = C.c_int
         L.oracle_num_threads.argtypes = []
         _libs[key] = L
@@ -209,3 +215,28 @@ def apply_tangent(tangent, poses):
     p = np.array(poses, np.float64, copy=True)
     lib().oracle_apply_tangent(_p(t), _p(p), t.shape[0])
     return t, p
+
+
+def sincos(theta):
+    """(sin, cos) of an angle in [-pi/2, pi/2] as the checker evaluates them."""
+    out = np.empty(2, np.float32)
+    lib().oracle_sincosf(float(theta), _p(out))
+    return float(out[0]), float(out[1])
+
+
+def ocam_unproject(intr_row, ip):
+    """Unit camera-space ray of pixel ``ip`` of the uncropped OCam image (row = c,d,e,cx,cy + world2cam poly)."""
+    row = np.ascontiguousarray(intr_row, np.float32)
+    ipa = np.ascontiguousarray(ip, np.float32)
+    out = np.empty(3, np.float32)
+    lib().oracle_ocam_unproject(_p(row), row.shape[0], _p(ipa), _p(out))
+    return out
+
+
+def ocam_core(intr_row, view_p, cutoff=10.0):
+    """(u, v, z) of a camera-space point through the OCam model alone."""
+    row = np.ascontiguousarray(intr_row, np.float32)
+    pa = np.ascontiguousarray(view_p, np.float32)
+    out = np.empty(3, np.float32)
+    lib().oracle_ocam_core(_p(pa), _p(row), row.shape[0], float(cutoff), _p(out))
+    return out

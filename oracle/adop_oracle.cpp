@@ -172,6 +172,23 @@ inline float o_acosf(float x)
     return kHalfPi - o_asinf(x);
 }
 
+// sine and cosine of an angle in [-pi/2, pi/2] (Cephes single-precision kernels on [-pi/4, pi/4], the rest through
+// the complementary angle), + - * only.
+inline void o_sincosf(float theta, float* s_out, float* c_out)
+{
+    float a    = theta < 0 ? -theta : theta;
+    bool compl_ = a > kQuartPi;
+    float x    = compl_ ? kHalfPi - a : a;
+    float z    = x * x;
+    float sn   = ((-1.9515295891e-4f * z + 8.3321608736e-3f) * z - 1.6666654611e-1f) * z * x + x;
+    float cs   = ((2.443315711809948e-5f * z - 1.388731625493765e-3f) * z + 4.166664568298827e-2f) * z * z +
+               (1.0f - 0.5f * z);
+    float s = compl_ ? cs : sn;
+    float c = compl_ ? sn : cs;
+    *s_out  = theta < 0 ? -s : s;
+    *c_out  = c;
+}
+
 // ------------------------------------------------------------------------------------------------
 // geometry (saiga / Sophus / Eigen restatements)
 // ------------------------------------------------------------------------------------------------
@@ -449,6 +466,42 @@ void project_ocam(V3 p, V3 n, const Pose& V, const float* aff, const float* poly
     V3 view_n = rotate(V, n);
     if (check_normal & (dot(view_p, view_n) > 0)) z = 0;
     *z_out = z;
+}
+
+// Pixel of the uncropped OCam image -> unit ray in camera space: the inverse of project_ocam_core.  The reference
+// has no such routine (its environment map asserts the pinhole model, EnvironmentMap.cu:129, and
+// PointRendererHelper.h:85-106 is the forward direction only); DEFINED here: undo the affine map, then solve
+// poly(theta) = rho with kOcamNewtonSteps Newton steps from the axis (theta = -pi/2), theta kept in [-pi/2, pi/2];
+// the ray is (cos(theta) * (uu,vv)/rho, -sin(theta)), so that theta = atan(-z / |xy|) as in the forward direction.
+const int kOcamNewtonSteps = 8;
+V3 ocam_unproject(const float* aff, const float* poly, int npoly, V2 ip)
+{
+    float c = aff[0], d = aff[1], e = aff[2], cx = aff[3], cy = aff[4];
+    float px = ip.x - cx, py = ip.y - cy;
+    float det = c - d * e;
+    float uu  = (px - d * py) / det;
+    float vv  = (c * py - e * px) / det;
+    float rho = std::sqrt(uu * uu + vv * vv);
+    float theta = -kHalfPi;
+    for (int it = 0; it < kOcamNewtonSteps; ++it)
+    {
+        float r   = poly[0];
+        float dr  = 0;
+        float t_i = 1;
+        for (int i = 1; i < npoly; ++i)
+        {
+            dr += (float)i * poly[i] * t_i;
+            t_i *= theta;
+            r += t_i * poly[i];
+        }
+        if (dr != 0) theta = theta - (r - rho) / dr;
+        theta = std::fmin(std::fmax(theta, -kHalfPi), kHalfPi);
+    }
+    float sn, cs;
+    o_sincosf(theta, &sn, &cs);
+    float cxn = rho > 0 ? uu / rho : 0.f;
+    float cyn = rho > 0 ? vv / rho : 0.f;
+    return {cxn * cs, cyn * cs, -sn};
 }
 
 struct BackwardOut
@@ -1079,10 +1132,16 @@ void oracle_env_uv(const adop_scene* s, const adop_view* view, int level, int w,
     for (int gy = 0; gy < h; ++gy)
         for (int gx = 0; gx < w; ++gx)
         {
-            V2 ip     = {(float)gx, (float)gy};
-            V2 dist_p = k_unproject2(cam.K, k_unproject2(cr, ip));
-            V2 np     = undistort_simple(dist_p, cam.D);
-            V3 inp    = {np.x, np.y, 1};
+            V2 ip = {(float)gx, (float)gy};
+            V3 inp;
+            if (cam.model == ADOP_CAMERA_PINHOLE_DISTORTION)
+            {
+                V2 dist_p = k_unproject2(cam.K, k_unproject2(cr, ip));
+                V2 np     = undistort_simple(dist_p, cam.D);
+                inp       = {np.x, np.y, 1};
+            }
+            else  // OCam views (not in the reference: EnvironmentMap.cu:129 asserts pinhole)
+                inp = ocam_unproject(cam.aff, cam.poly, cam.npoly, k_unproject2(cr, ip));
             V3 r      = rotate_inv(cam.V, inp);
             V3 wp     = {r.x + tinv.x, r.y + tinv.y, r.z + tinv.z};
             V3 d      = {wp.x - tinv.x, wp.y - tinv.y, wp.z - tinv.z};
@@ -1267,6 +1326,25 @@ void oracle_undistort(const float* p, const float* dist8, float* out2)
     V2 r         = undistort_simple({p[0], p[1]}, D);
     out2[0]      = r.x;
     out2[1]      = r.y;
+}
+void oracle_sincosf(float theta, float* out2) { o_sincosf(theta, out2, out2 + 1); }
+// intr: (c,d,e,cx,cy) + world2cam polynomial, cols floats; ip: pixel of the uncropped image; out: unit ray (camera)
+void oracle_ocam_unproject(const float* intr, int cols, const float* ip, float* out3)
+{
+    V3 r    = ocam_unproject(intr, intr + 5, cols - 5, {ip[0], ip[1]});
+    out3[0] = r.x;
+    out3[1] = r.y;
+    out3[2] = r.z;
+}
+// view-space point -> (u, v, z) through the OCam model alone (no pose, no normal test)
+void oracle_ocam_core(const float* p, const float* intr, int cols, float cutoff, float* out3)
+{
+    V2 uv;
+    float z;
+    project_ocam_core({p[0], p[1], p[2]}, intr, intr + 5, cols - 5, cutoff, &uv, &z, nullptr, nullptr);
+    out3[0] = uv.x;
+    out3[1] = uv.y;
+    out3[2] = z;
 }
 int oracle_num_threads(void)
 {

@@ -73,18 +73,77 @@ def test_env_backward_matches_autograd_of_grid_sample():
     assert_norm_close(g_env.cpu().numpy(), tex.grad.numpy(), 2e-5, "grad env texture")
 
 
-def test_env_rejects_ocam():
+def _ocam_env_scene():
+    from adop_amd import _capi, scenes
+
+    hs = scenes.config5(n=60_000, w=176, h=120, levels=3, batch=2, patches=40, env_hw=(48, 96))
+    # an affine part, so that the inverse has to undo it; the second view is a crop window of the same camera
+    hs.intrinsics[0, :3] = [1.03, 0.02, -0.015]
+    hs.views[1] = scenes.make_view(176, 120, image_index=1, model=_capi.CAMERA_OCAM, crop=(1.25, 1.25, -30.0, -12.0, 0.0))
+    hs.params.output_background_mask_value = 0.0
+    hs.dropout = scenes.bernoulli_mask(5, 2, hs.num_points, 0.25)
+    return hs
+
+
+def test_env_on_ocam_views(oracle_mod):
+    """Environment map on OCam views (an extension: the reference asserts pinhole, EnvironmentMap.cu:129): the ray of
+    a pixel comes from the inverted world2cam polynomial."""
+    import torch
+    from adop_amd import render, scenes
+
+    announce("environment map on OCam views: uv, sample, composition, texture gradient")
+    hs = _ocam_env_scene()
+    scene, info, ctx, images, masks = run_hip_forward(hs)
+    before = [im.clone() for im in images]
+    uv, env = render.EnvironmentMapSample(info, add_to_out=True, want_uv=True, want_env=True)
+    torch.cuda.synchronize()
+    empty = 0
+    for l in range(hs.num_layers):
+        for b in range(hs.batch):
+            want_uv = oracle_mod.env_uv(hs, b, l)
+            got_uv = uv[l][b].cpu().numpy()
+            assert np.isfinite(got_uv).all()
+            assert np.abs(got_uv - want_uv).max() <= 1e-6, (l, b, np.abs(got_uv - want_uv).max())
+            want_env = oracle_mod.grid_sample(hs.env_texture, got_uv)
+            assert_close(env[l][b].cpu().numpy(), want_env, 1e-5, 1e-6, f"env level {l} view {b}")
+        m = masks[l].cpu().numpy()
+        empty += int((m == 0).sum())
+        want = before[l].cpu().numpy() + (1 - m) * env[l].cpu().numpy()
+        assert_close(images[l].cpu().numpy(), want, 1e-6, 1e-7, f"composition level {l}")
+    assert empty > 1000  # the scene leaves pixels for the environment map
+    gout = [torch.from_numpy(g).cuda() for g in scenes.upstream_grads(hs, 9)]
+    g_env = render.EnvironmentMapSampleBackward(info, gout)
+    torch.cuda.synchronize()
+    tex = torch.from_numpy(hs.env_texture).double().requires_grad_(True)
+    loss = 0
+    for l in range(hs.num_layers):
+        s = torch.nn.functional.grid_sample(tex[None].repeat(hs.batch, 1, 1, 1), uv[l].cpu().double(), mode="bilinear",
+                                            padding_mode="border", align_corners=True)
+        loss = loss + (s * (1 - masks[l].cpu().double()) * gout[l].cpu().double()).sum()
+    loss.backward()
+    assert_norm_close(g_env.cpu().numpy(), tex.grad.numpy(), 2e-5, "grad env texture (OCam)")
+
+
+def test_env_rejects_unknown_model_and_bad_rows():
     import ctypes as C
     from adop_amd import _capi, scenes
 
-    announce("environment map: OCam views are rejected (reference asserts pinhole)")
+    announce("environment map: argument checks of the camera model")
     hs = scenes.config5(n=1000, w=44, h=30, batch=1, patches=10)
     scene, info, ctx, images, masks = run_hip_forward(hs)
     cache = info.cache
     s = scene.struct()
     fb = cache.forward_struct()
-    rc = cache.lib.adop_env_sample(C.byref(s), cache.views_array(), 1, C.c_void_p(scene.environment_map.data_ptr()),
-                                   512, 1024, C.byref(fb), None, None, 1, None)
+    env = scene.environment_map
+    views = cache.views_array()
+    views[0].camera_model_type = 7
+    rc = cache.lib.adop_env_sample(C.byref(s), views, 1, C.c_void_p(env.data_ptr()), int(env.shape[1]),
+                                   int(env.shape[2]), C.byref(fb), None, None, 1, None)
+    assert rc == _capi.ADOP_INVALID_ARG
+    # a pinhole view needs rows of 13 floats; this scene's rows are OCam rows of 11
+    views[0].camera_model_type = _capi.CAMERA_PINHOLE_DISTORTION
+    rc = cache.lib.adop_env_sample(C.byref(s), views, 1, C.c_void_p(env.data_ptr()), int(env.shape[1]),
+                                   int(env.shape[2]), C.byref(fb), None, None, 1, None)
     assert rc == _capi.ADOP_INVALID_ARG
 
 

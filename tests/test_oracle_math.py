@@ -347,6 +347,71 @@ def test_ocam_equidistant_polynomial(oracle_mod):
     assert project_ocam(L, (0, 0, 2), intr)[:2] == pytest.approx([500, 400])
 
 
+def test_sincos_polynomials_against_libm(oracle_mod):
+    """The fixed sine / cosine polynomials of the OCam pixel-to-ray routine over their whole domain [-pi/2, pi/2]."""
+    for t in np.concatenate([np.linspace(-np.pi / 2, np.pi / 2, 6001), [0.0, np.pi / 4, -np.pi / 4, 1e-9]]):
+        t = np.float32(t)
+        s, c = oracle_mod.sincos(t)
+        assert abs(s - np.sin(np.float64(t))) < 2e-7 and abs(c - np.cos(np.float64(t))) < 2e-7, t
+    assert oracle_mod.sincos(0.0) == (0.0, 1.0)
+
+
+def test_ocam_unproject_equidistant_closed_form(oracle_mod):
+    """rho = f*(theta + pi/2): a pixel at radius r from the centre, direction phi, comes from the ray
+    (sin(a) cos(phi), sin(a) sin(phi), cos(a)) with a = r / f off the optical axis."""
+    f = 200.0
+    intr = f32(1, 0, 0, 500, 400, f * np.pi / 2, f)
+    g = scenes.rng(31)
+    for _ in range(200):
+        a = g.uniform(0.01, np.deg2rad(100))
+        phi = g.uniform(-np.pi, np.pi)
+        ip = (500 + f * a * np.cos(phi), 400 + f * a * np.sin(phi))
+        d = oracle_mod.ocam_unproject(intr, ip)
+        want = (np.sin(a) * np.cos(phi), np.sin(a) * np.sin(phi), np.cos(a))
+        assert d == pytest.approx(want, abs=3e-6)
+        assert np.linalg.norm(d.astype(np.float64)) == pytest.approx(1.0, abs=1e-6)
+    # the centre pixel is the optical axis
+    assert oracle_mod.ocam_unproject(intr, (500, 400)) == pytest.approx([0, 0, 1], abs=1e-7)
+
+
+def test_ocam_unproject_inverts_the_projection(oracle_mod):
+    """project(unproject(pixel)) = pixel for a 5th-order polynomial with an affine part, over the image circle; and
+    unproject(project(p)) is the direction of p."""
+    g = scenes.rng(32)
+    for seed in range(4):
+        intr = scenes.ocam_row(1200, 900, seed=seed)
+        intr[:3] = [1.0 + 0.02 * seed, 0.01 * seed, -0.015 * seed]
+        r0 = oracle_mod.ocam_core(intr, (1e-6, 0, 1.0))  # radius the polynomial gives next to the axis
+        r_min = abs(np.hypot(r0[0] - intr[3], r0[1] - intr[4])) + 2.0
+        for _ in range(300):
+            # a pixel on a ring the polynomial reaches (its value on the axis is not exactly 0)
+            r = g.uniform(r_min, 600.0)
+            phi = g.uniform(-np.pi, np.pi)
+            ip = np.array([intr[3] + r * np.cos(phi), intr[4] + r * np.sin(phi)])
+            d = oracle_mod.ocam_unproject(intr, ip)
+            back = oracle_mod.ocam_core(intr, 3.7 * d)
+            assert back[:2] == pytest.approx(ip, abs=2e-3), (seed, ip, d)
+            assert back[2] == pytest.approx(3.7, rel=1e-6)
+        for _ in range(100):
+            p = g.uniform(-1, 1, 3)
+            p[2] = g.uniform(0.0, 2.0)
+            uvz = oracle_mod.ocam_core(intr, p)
+            if np.hypot(uvz[0] - intr[3], uvz[1] - intr[4]) < r_min:
+                continue
+            d = oracle_mod.ocam_unproject(intr, uvz[:2])
+            assert d == pytest.approx(p / np.linalg.norm(p), abs=2e-5)
+
+
+def test_ocam_unproject_outside_the_polynomial_range(oracle_mod):
+    """Pixels the polynomial does not reach take the ray at the nearest end of theta's range and stay finite."""
+    f = 100.0
+    intr = f32(1, 0, 0, 50, 50, f * np.pi / 2 + 5.0, f)  # rho(-pi/2) = 5: nothing projects inside 5 pixels
+    assert oracle_mod.ocam_unproject(intr, (52, 50)) == pytest.approx([0, 0, 1], abs=1e-6)
+    # far outside: theta stops at +pi/2, the ray points backwards along the axis
+    d = oracle_mod.ocam_unproject(intr, (5000, 50))
+    assert np.isfinite(d).all() and d == pytest.approx([0, 0, -1], abs=1e-6)
+
+
 def test_ocam_backward_by_finite_differences(oracle_mod):
     L = oracle_mod.lib()
     g = scenes.rng(10)

@@ -368,6 +368,37 @@ def test_environment_uv_closed_forms(oracle_mod):
     assert oracle_mod.env_uv(hs, 0, 0) == pytest.approx(uv, abs=2e-6)
 
 
+def test_environment_uv_of_an_ocam_view(oracle_mod):
+    """OCam views: the pixel's ray comes from the inverted world2cam polynomial, the rest is the same spherical
+    mapping.  Equidistant fisheye with f = 8 pixels per radian: the centre pixel looks along +z, a pixel k to the right of
+    it along (sin(k/f), 0, cos(k/f)), a pixel k below it along (0, sin(k/f), cos(k/f))."""
+    from adop_amd import _capi
+
+    f = 8.0
+    w, h = 33, 17
+    hs = scenes.config5(n=1, w=w, h=h, levels=2, batch=1, patches=1)
+    hs.intrinsics = np.array([[1, 0, 0, 16.0, 8.0, f * np.pi / 2, f]], np.float32)
+    hs.poses_se3[0] = [0, 0, 0, 1, 0, 0, 0, 0]
+    assert hs.views[0].camera_model_type == _capi.CAMERA_OCAM
+    uv = oracle_mod.env_uv(hs, 0, 0)
+    assert uv[8, 16] == pytest.approx([0.5, 0.0], abs=1e-6)  # d = (0,0,1): phi = -pi/2 -> x = 0.75
+    for gx in range(17, 33):
+        a = (gx - 16.0) / f
+        d = np.array([np.sin(a), 0.0, np.cos(a)])
+        x = (np.arctan2(-d[2], d[0]) / (2 * np.pi)) % 1.0
+        assert uv[8, gx] == pytest.approx([2 * x - 1, 0.0], abs=2e-6), gx
+    for gy in range(0, 17):
+        a = (gy - 8.0) / f  # towards +y
+        d = np.array([0.0, np.sin(a), np.cos(a)])
+        y = 1 - np.arccos(d[1]) / np.pi
+        assert uv[gy, 16][1] == pytest.approx(2 * y - 1, abs=2e-6), gy
+    # level 1: crop scaled by 1/2 -> its pixel (8,4) is the centre again
+    assert oracle_mod.env_uv(hs, 0, 1)[4, 8] == pytest.approx([0.5, 0.0], abs=1e-6)
+    # a crop window: pixel (0,0) of a view cropped at offset (-10,-3) is pixel (10,3) of the full image
+    hs.views[0] = scenes.make_view(w, h, image_index=0, model=_capi.CAMERA_OCAM, crop=(1.0, 1.0, -10.0, -3.0, 0.0))
+    assert oracle_mod.env_uv(hs, 0, 0)[0, 0] == pytest.approx(uv[3, 10], abs=1e-6)
+
+
 def test_grid_sample_matches_torch(oracle_mod):
     import torch
 
