@@ -162,6 +162,11 @@ ENTRY_POINTS = {
         C.c_int,
         [C.POINTER(Scene), C.POINTER(View), C.c_int32, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p],
     ),
+    "adop_static_max_frames": (C.c_int32, []),
+    "adop_point_distance_to_camera_static": (
+        C.c_int,
+        [C.POINTER(Scene), C.POINTER(View), C.c_int32, C.c_void_p, C.c_void_p],
+    ),
     "adop_close_points": (
         C.c_int,
         [C.c_void_p, C.c_int32, C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_void_p, C.c_void_p,

@@ -36,6 +36,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -384,6 +385,38 @@ int pixel_grid(const Levels& lv, int first_level = 0)
     return (int)(want < 16384 ? (want ? want : 1) : 16384);
 }
 
+}  // namespace adop
+
+// Scratch memory of the one entry point that takes no workspace (adop_point_distance_to_camera_static): the per-frame
+// constants of up to kStaticMaxFrames frames.  Every GPU the library runs on holds its own copy of the array until the
+// process ends.  In host code the name `scratch` is only a handle for hipGetSymbolAddress: the address the kernels get
+// is the one that call returns for the current device, kept per device below.
+constexpr int kStaticMaxFrames = 1024;
+static __device__ __align__(256) unsigned char scratch[sizeof(adop::ViewConst) * kStaticMaxFrames];
+
+namespace adop
+{
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (looked up once per device).
+adop_status scratch_of_current_device(void** out)
+{
+    int dev = -1;
+    ADOP_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(ADOP_HIP_ERROR, "device ordinal out of range");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev])
+    {
+        void* p = nullptr;
+        ADOP_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail(ADOP_HIP_ERROR, "hipGetSymbolAddress returned no address for the scratch array");
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return ADOP_OK;
+}
 }  // namespace adop
 
 using namespace adop;
@@ -902,9 +935,9 @@ size_t adop_frames_workspace_size(int32_t num_frames)
     return num_frames < 1 ? 0 : align_up(sizeof(ViewConst) * (size_t)num_frames, 256);
 }
 
-adop_status adop_point_distance_to_camera(const adop_scene* scene, const adop_view* frames, int32_t num_frames,
-                                          float* out_distance, void* workspace, size_t workspace_bytes,
-                                          void* hip_stream)
+// Argument checks shared by the two camera-distance entry points.
+static adop_status camera_distance_check(const adop_scene* scene, const adop_view* frames, int32_t num_frames,
+                                         const float* out_distance)
 {
     if (!scene || !frames || !out_distance) return fail(ADOP_INVALID_ARG, "null argument");
     if (num_frames < 1) return fail(ADOP_INVALID_ARG, "num_frames must be >= 1");
@@ -922,16 +955,53 @@ adop_status adop_point_distance_to_camera(const adop_scene* scene, const adop_vi
             v.camera_index >= scene->num_cameras || v.w < 1 || v.h < 1)
             return fail(ADOP_INVALID_ARG, "frame out of range");
     }
-    if (!workspace || workspace_bytes < adop_frames_workspace_size(num_frames))
-        return fail(ADOP_WORKSPACE_TOO_SMALL, "workspace too small");
+    return ADOP_OK;
+}
+
+// The per-frame constants go to `dviews` (device memory for num_frames ViewConst), then every point is tested against
+// every frame.
+static adop_status camera_distance_run(const adop_scene* scene, const adop_view* frames, int32_t num_frames,
+                                       float* out_distance, ViewConst* dviews, hipStream_t stream)
+{
     if (scene->num_points == 0) return ADOP_OK;
-    hipStream_t stream = (hipStream_t)hip_stream;
-    ViewConst* dviews  = (ViewConst*)workspace;
-    adop_status st     = upload_views(scene, frames, num_frames, dviews, stream);
+    adop_status st = upload_views(scene, frames, num_frames, dviews, stream);
     if (st != ADOP_OK) return st;
     launch_camera_distance((const float4*)scene->position, scene->num_points, dviews, num_frames, out_distance, stream);
     ADOP_HIP_CHECK(hipGetLastError());
     return ADOP_OK;
+}
+
+adop_status adop_point_distance_to_camera(const adop_scene* scene, const adop_view* frames, int32_t num_frames,
+                                          float* out_distance, void* workspace, size_t workspace_bytes,
+                                          void* hip_stream)
+{
+    adop_status st = camera_distance_check(scene, frames, num_frames, out_distance);
+    if (st != ADOP_OK) return st;
+    if (!workspace || workspace_bytes < adop_frames_workspace_size(num_frames))
+        return fail(ADOP_WORKSPACE_TOO_SMALL, "workspace too small");
+    return camera_distance_run(scene, frames, num_frames, out_distance, (ViewConst*)workspace, (hipStream_t)hip_stream);
+}
+
+int32_t adop_static_max_frames(void)
+{
+    return kStaticMaxFrames;
+}
+
+adop_status adop_point_distance_to_camera_static(const adop_scene* scene, const adop_view* frames, int32_t num_frames,
+                                                 float* out_distance, void* hip_stream)
+{
+    adop_status st = camera_distance_check(scene, frames, num_frames, out_distance);
+    if (st != ADOP_OK) return st;
+    if (num_frames > kStaticMaxFrames)
+        return fail(ADOP_INVALID_ARG, "adop_point_distance_to_camera_static takes at most " +
+                                          std::to_string(kStaticMaxFrames) +
+                                          " frames per call (the size of the library's own scratch array); use "
+                                          "adop_point_distance_to_camera with a workspace for more");
+    void* dviews = nullptr;
+    if ((st = scratch_of_current_device(&dviews)) != ADOP_OK) return st;
+    // Nothing of the array has to start at zero: the constants of frames 0 .. num_frames-1 are written before the
+    // distance kernel reads them, and it reads no others.
+    return camera_distance_run(scene, frames, num_frames, out_distance, (ViewConst*)dviews, (hipStream_t)hip_stream);
 }
 
 adop_status adop_morton_codes(const float* position, int32_t num_points, const float* bbox_min, const float* bbox_max,

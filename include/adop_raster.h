@@ -237,6 +237,17 @@ adop_status adop_point_distance_to_camera(const adop_scene* scene, const adop_vi
                                           float* out_distance, void* workspace, size_t workspace_bytes,
                                           void* hip_stream);
 
+/* adop_point_distance_to_camera without a workspace, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The
+ * per-frame constants live in an array inside the library (132 bytes per frame, adop_static_max_frames() = 1024
+ * frames = 132 KiB per GPU, held until the process ends); more frames are rejected with ADOP_INVALID_ARG.  The call
+ * allocates and frees nothing; the first call on a device looks the array's address up (make that call outside a
+ * stream capture).  All calls on one GPU share the array: calls that overlap on one GPU (different streams or
+ * threads) race; calls on one stream are ordered and safe.  Results equal adop_point_distance_to_camera's. */
+int32_t adop_static_max_frames(void);
+adop_status adop_point_distance_to_camera_static(const adop_scene* scene, const adop_view* frames, int32_t num_frames,
+                                                 float* out_distance, void* hip_stream);
+
 /* Replaces the sequential sweep of SceneData::RemoveClosePoints (SceneData.cpp:598-642): state[i] = 2 (erased) when a
  * point j < i with state[j] = 1 (kept) lies closer than radius[i] (d2 < radius^2 in fp32), else 1; the result equals
  * the sweep in index order.  The points are decided in rounds (a point waits for its earlier neighbours):
