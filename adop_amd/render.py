@@ -238,10 +238,12 @@ def _stream_ptr():
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
-def BlendPointCloudForward(ctx, info):
-    """PointRenderer.cu:1389-1531.  Returns (images per level, masks per level)."""
+def BlendPointCloudForward(ctx, info, build=True):
+    """PointRenderer.cu:1389-1531.  Returns (images per level, masks per level).  ``build=False``: the caller has
+    already run ``cache.Build(info, True)`` (the reference calls it first thing, :1407)."""
     cache = info.cache
-    cache.Build(info, True)
+    if build:
+        cache.Build(info, True)
     s = info.scene.struct()
     fb = cache.forward_struct()
     stats = C.c_void_p(cache.stats.data_ptr()) if info.collect_stats else None
@@ -258,6 +260,9 @@ def BlendPointCloudForward(ctx, info):
         ctx.point_cache = cache.point_cache
         ctx.depth_index = [L.depth_index_tensor for L in cache.layers_cuda]
         ctx.masks = list(cache.output_forward_background_mask)
+        # depth / weight / packed depth now belong to the graph (the kernels write them through raw pointers, autograd
+        # would not notice a later forward overwriting them): the next forward allocates fresh ones
+        cache.cache_size = None
     return list(cache.output_forward), list(cache.output_forward_background_mask)
 
 

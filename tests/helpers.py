@@ -14,7 +14,12 @@ def announce(msg):
 FORWARD_PATH = 0
 
 
-def run_hip_forward(hs, collect_stats=True, forward_path=None, train=True):
+# Pattern the poisoned runs fill the point cache and the workspace with before a forward: whatever the forward does
+# not write still holds it afterwards, and a kernel that reads an unwritten record computes with garbage.
+POISON_BITS = 0xDEADBEEF
+
+
+def run_hip_forward(hs, collect_stats=True, forward_path=None, train=True, poison=False):
     import torch
     from adop_amd import render
 
@@ -31,7 +36,14 @@ def run_hip_forward(hs, collect_stats=True, forward_path=None, train=True):
             self.saved_tensors = t
 
     ctx = Ctx()
-    images, masks = render.BlendPointCloudForward(ctx, info)
+    if poison:
+        cache.Build(info, True)
+        cache.workspace.view(torch.int32).fill_(POISON_BITS - (1 << 32))
+        if cache.point_cache is not None:
+            cache.point_cache.view(torch.int32).fill_(POISON_BITS - (1 << 32))
+        images, masks = render.BlendPointCloudForward(ctx, info, build=False)
+    else:
+        images, masks = render.BlendPointCloudForward(ctx, info)
     torch.cuda.synchronize()
     return scene, info, ctx, images, masks
 
@@ -104,7 +116,17 @@ def check_forward(hs, ref, ctx, images, masks, info, stats=True):
         assert st.accepted[l] == ref.stats.accepted[l], ("accepted", l, st.accepted[l], ref.stats.accepted[l])
 
 
-def check_backward(hs, refb, grads, info):
+def count_misses(got, want, rel=1e-4, abs_tol=1e-6):
+    """Elements outside |got-want| <= max(rel*|want|, abs_tol): (number, size, largest miss relative to max|want|)."""
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    err = np.abs(got - want)
+    bad = err > np.maximum(rel * np.abs(want), abs_tol)
+    worst = float(err[bad].max() / max(np.abs(want).max(), 1e-30)) if bad.any() else 0.0
+    return int(bad.sum()), int(bad.size), worst
+
+
+def check_backward(hs, refb, grads, info, stats=True):
     """gradients within 1e-4 relative or 1e-6 absolute (float atomics reorder the sums)."""
     g_tex, g_bg, g_pts, g_pose, g_intr = grads
     cache = info.cache
@@ -121,6 +143,8 @@ def check_backward(hs, refb, grads, info):
         assert np.array_equal(cache.output_gradient_intrinsics_count.cpu().numpy(), refb.grad_intrinsics_count)
         scale = np.abs(refb.grad_intrinsics).max() + 1e-30
         assert_close(g_intr.cpu().numpy(), refb.grad_intrinsics, 1e-4, 1e-6 * max(scale, 1.0), "grad_intrinsics")
+    if not stats:
+        return
     st = cache.read_stats()
     for l in range(hs.num_layers):
         assert st.spatial[l] == refb.stats.spatial[l], ("spatial", l, st.spatial[l], refb.stats.spatial[l])

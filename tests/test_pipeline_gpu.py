@@ -9,7 +9,8 @@ from helpers import announce, check_backward, check_forward, download_forward
 pytestmark = pytest.mark.gpu
 
 
-def test_scene_directory_to_gradients(oracle_mod, tmp_path):
+@pytest.mark.parametrize("collect_stats", [True, False], ids=["counters", "plain"])
+def test_scene_directory_to_gradients(oracle_mod, tmp_path, collect_stats):
     import torch
     from adop_amd import preprocess, render, scene_io, scenes
 
@@ -59,10 +60,10 @@ def test_scene_directory_to_gradients(oracle_mod, tmp_path):
     scene.texture.requires_grad_(True)
     scene.tangent_poses.requires_grad_(True)
     info = render.NeuralRenderInfo(scene=scene, images=list(views), params=params, num_layers=3,
-                                   cache=render.PointRendererCache(), collect_stats=True, train=True)
+                                   cache=render.PointRendererCache(), collect_stats=collect_stats, train=True)
     images = render.BlendPointCloud(info)[:3]
     ref = oracle_mod.forward(hs)
-    check_forward(hs, ref, None, [im.detach() for im in images], [], info)
+    check_forward(hs, ref, None, [im.detach() for im in images], [], info, stats=collect_stats)
     assert all(float((L.weight > 0).float().mean()) > 0.05 for L in info.cache.layers_cuda)  # the crops see the blob
     gout = scenes.upstream_grads(hs, 3)
     loss = sum((im * torch.from_numpy(go).cuda()).sum() for im, go in zip(images, gout))

@@ -88,15 +88,18 @@ def test_random_scene(oracle_mod, seed, forward_path):
     scene, info, ctx, images, masks = run_hip_forward(hs, collect_stats=seed % 2 == 0, forward_path=forward_path,
                                                       train=False)
     check_forward(hs, ref, ctx, images, masks, info, stats=seed % 2 == 0)
-    # training forward + backward
-    scene, info, ctx, images, masks = run_hip_forward(hs, forward_path=forward_path)
-    check_forward(hs, ref, ctx, images, masks, info)
+    # training forward + backward; every third seed without the counters (the kernels' production variants), from a
+    # poisoned point cache and workspace
+    counters = seed % 3 != 0
+    scene, info, ctx, images, masks = run_hip_forward(hs, collect_stats=counters, forward_path=forward_path,
+                                                      poison=not counters)
+    check_forward(hs, ref, ctx, images, masks, info, stats=counters)
     gout = scenes.upstream_grads(hs, seed + 11)
     grads = render.BlendPointCloudBackward(ctx, info, [torch.from_numpy(g).cuda() for g in gout], needs)
     torch.cuda.synchronize()
     saved = download_forward(hs, info, images, masks)
     refb = oracle_mod.backward(hs, saved, gout, *needs)
-    check_backward(hs, refb, grads, info)
+    check_backward(hs, refb, grads, info, stats=counters)
     refb2 = oracle_mod.backward(hs, ref, gout, *needs)
     names = ["grad_texture", "grad_background", "grad_points", "grad_pose", "grad_intrinsics"]
     for name, gr in zip(names, grads):

@@ -6,7 +6,7 @@ import sys
 import numpy as np
 import pytest
 
-from helpers import announce, assert_close, assert_norm_close
+from helpers import count_misses, announce, assert_close, assert_norm_close
 
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -80,9 +80,15 @@ def test_point_render_autograd_matches_checker(oracle_mod):
     refb = oracle_mod.backward(hs, ref, gout)
     assert_close(t["texture"].grad.cpu().numpy(), refb.grad_texture, 1e-4, 1e-5, "grad texture")
     assert_close(t["background"].grad.cpu().numpy(), refb.grad_background, 1e-4, 1e-4, "grad background")
-    assert_norm_close(t["position"].grad.cpu().numpy(), refb.grad_points, 1e-4, "grad points")
-    assert_norm_close(t["tangent_poses"].grad.cpu().numpy(), refb.grad_pose, 1e-4, "grad pose")
-    assert_norm_close(t["intrinsics"].grad.cpu().numpy(), refb.grad_intrinsics, 1e-4, "grad intrinsics")
+    # The checker ran its own forward here (the wrapper keeps its depth / weight buffers to itself), so the spatial
+    # gradients see images that differ by summation order: tensor-level bound, and the element-wise bar (1e-4 relative
+    # / 1e-6 absolute) with the ceilings of tests/test_parity_gpu.py on how many elements miss it and by how much.
+    for name, got, want in (("grad points", t["position"].grad, refb.grad_points),
+                            ("grad pose", t["tangent_poses"].grad, refb.grad_pose),
+                            ("grad intrinsics", t["intrinsics"].grad, refb.grad_intrinsics)):
+        assert_norm_close(got.cpu().numpy(), want, 1e-4, name)
+        misses, size, worst = count_misses(got.cpu().numpy(), want)
+        assert misses <= max(1, int(1e-4 * size)) and worst <= 1e-6, (name, misses, size, worst)
 
 
 def test_dropout_is_drawn_like_the_reference_and_eval_disables_it(oracle_mod):
