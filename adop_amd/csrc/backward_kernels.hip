@@ -237,7 +237,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(CT != 0 
                     R           = make_float4(r.x, r.y, r.z, r.w);
                 }
                 ip             = {R.x, R.y};
-                drop_out       = R.z < 0;
+                drop_out       = depth_is_dropped(R.z);
                 z              = fabsf(R.z);
                 radius_pixels  = R.w;
                 ok             = valid && z != 0;

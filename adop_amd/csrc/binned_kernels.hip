@@ -147,7 +147,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(PPT > 2 
                 else if (valid)
                 {
                     const bool dropped = ok && pc.dropout && __builtin_nontemporal_load(pc.dropout + (size_t)b * pc.n + i) == 1.f;
-                    const float4 far   = ok ? make_float4(ip.x, ip.y, dropped ? -z : z, crop_radius(vc, z, P[k].w, lv.l[0].w))
+                    const float4 far   = ok ? make_float4(ip.x, ip.y, signed_depth(z, dropped), crop_radius(vc, z, P[k].w, lv.l[0].w))
                                             : make_float4(0, 0, 0, 0);
                     nt_store4(pc.cache + (size_t)b * pc.n + i, lane == 0 ? mark : far);
                     __builtin_nontemporal_store(0u, bin.info + (size_t)b * pc.n + i);
@@ -158,7 +158,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(PPT > 2 
             // (the sign of the depth carries the dropout flag: the readers need no second array; only the projected
             // points' flags are read)
             const bool dropped = ok && pc.dropout && __builtin_nontemporal_load(pc.dropout + (size_t)b * pc.n + i) == 1.f;  // :314-315
-            const float4 rec   = ok ? make_float4(ip.x, ip.y, dropped ? -z : z, radius_pixels) : make_float4(0, 0, 0, 0);
+            const float4 rec   = ok ? make_float4(ip.x, ip.y, signed_depth(z, dropped), radius_pixels) : make_float4(0, 0, 0, 0);
             if (STATS) stat_add(&stats->bad_index, ok && !dropped && !tex_ok[k]);
 
             bool in[ADOP_MAX_LAYERS];

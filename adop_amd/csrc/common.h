@@ -25,6 +25,25 @@ constexpr int kMaxIntrinsicsCols = 24;  // 13 pinhole / 5 affine + up to 19 poly
 constexpr uint32_t kRunCulledBits = 0x7FC0C011u;  // a quiet NaN no projection produces
 constexpr uint64_t kClearPacked = (uint64_t(0x47C35000u) << 32) | 0xFFFFFFFFull;  // bits(100000.f), PointRenderer.cu:1045
 
+// The depth kept in the point cache and in the bin entries: 0 = culled, sign bit set = dropped for this image
+// (PointRenderer.cu:314-315).  Tested on the bits, so that a NaN depth (a point with NaN coordinates seen through an
+// OCam) counts as a depth like any other, as in the reference, where every comparison with it is false and the point
+// is blended.
+__device__ __forceinline__ float signed_depth(float z, bool dropped)
+{
+    // (a NaN may come with either sign: only the dropout flag decides the sign bit)
+    const uint32_t bits = __float_as_uint(z) & 0x7FFFFFFFu;
+    return __uint_as_float(dropped ? bits | 0x80000000u : bits);
+}
+__device__ __forceinline__ bool depth_is_rendered(float zs)
+{
+    return (int32_t)__float_as_uint(zs) > 0;
+}
+__device__ __forceinline__ bool depth_is_dropped(float zs)
+{
+    return (int32_t)__float_as_uint(zs) < 0;
+}
+
 struct LevelArg
 {
     int32_t w, h;

@@ -179,7 +179,7 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
                 else if (i < pc.n)
                 {
                     const bool dropped = (inmask[k] != 0 || (STATS && okk[k])) && pc.dropout && pc.dropout[(size_t)b * pc.n + i] == 1.f;
-                    float4 r = okk[k] ? make_float4(rec[k].x, rec[k].y, dropped ? -zz[k] : zz[k], rec[k].w)
+                    float4 r = okk[k] ? make_float4(rec[k].x, rec[k].y, signed_depth(zz[k], dropped), rec[k].w)
                                       : make_float4(0, 0, 0, 0);
                     if (culled && lane == 0) r = make_float4(__uint_as_float(kRunCulledBits), 0, 0, 0);
                     pc.cache[(size_t)b * pc.n + i] = r;
@@ -438,7 +438,7 @@ __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewCo
                 bool tex_ok        = (unsigned)tex_index < (unsigned)pc.num_texels;  // device assert :362
                 bool staged        = false;
                 wave_lds_sync();  // the staged descriptors of the previous round are no longer read
-                blend_point(b, valid && R.z > 0, V2{R.x, R.y}, R.z, R.w, tex_index, tex_ok, staged);
+                blend_point(b, valid && depth_is_rendered(R.z), V2{R.x, R.y}, R.z, R.w, tex_index, tex_ok, staged);
             }
         }
         return;
@@ -485,7 +485,7 @@ __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewCo
             ip             = {R.x, R.y};
             z              = R.z;
             radius_pixels  = R.w;
-            ok             = valid && z > 0;
+            ok             = valid && depth_is_rendered(z);
         }
         else
         {

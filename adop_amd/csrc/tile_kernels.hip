@@ -286,7 +286,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu((CT != 0
             for (int k = 0; k < K; ++k)
             {
                 const uint32_t id = __float_as_uint(E[k].w) & kEntryIdMask;
-                ok[k]             = E[k].z > 0;  // dropped points carry -z (:314-315), padding too
+                ok[k]             = depth_is_rendered(E[k].z);  // dropped points carry -z (:314-315), padding too
                 int tex_index     = 0;
                 if (ok[k]) tex_index = identity_index ? (int)id : pc.index[id];
                 ok[k] = ok[k] && (unsigned)tex_index < (unsigned)pc.num_texels;  // device assert :362

@@ -18,7 +18,10 @@ def lib(omp=False):
     key = bool(omp)
     if key not in _libs:
         path = _build.LIB_OMP if omp else _build.LIB
-        if not os.path.exists(path):
+        if os.environ.get("ADOP_ORACLE_SANITIZE") == "1":
+            # the ASan / UBSan build (tests/test_sanitizers.py runs the pinning tests on it in a child process)
+            path = _build.build_sanitized(force=False)
+        elif not os.path.exists(path):
             _build.build(force=False)
         L = C.CDLL(path)
         L.oracle_forward.restype = C.c_int

@@ -10,6 +10,7 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    config.addinivalue_line("markers", "sanitize: CPU sanitizer builds in child processes (compiles for ~30 s)")
 
 
 @pytest.fixture(scope="session")

@@ -48,19 +48,20 @@ def test_forward_backward_replayed_from_a_graph(forward_path):
             g_images, _ = render.BlendPointCloudForward(ctx, info)
             g_gout = [torch.ones_like(im) * (l + 1) for l, im in enumerate(g_images)]
             g_grads = render.BlendPointCloudBackward(ctx, info, g_gout)
+            g_layers = list(info.cache.layers_cuda)  # the buffers the recorded kernels write (a later forward takes new ones)
     torch.cuda.synchronize()
     for rep in range(4):
         # new inputs in place: descriptors, and the camera pose (the view constants are computed on the device)
         scene.texture.copy_(tex0 * (1.0 + 0.25 * rep) + 0.125 * rep)
         scene.poses_se3[0, 4:7] += 0.01 * rep
         want_images, want_grads, want_packed = eager()
-        for L in info.cache.layers_cuda:  # scribble over what the replay must rewrite
+        for L in g_layers:  # scribble over what the replay must rewrite
             L.depth_index_tensor.fill_(7)
             L.weight.fill_(-1)
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
-        for l, L in enumerate(info.cache.layers_cuda):
+        for l, L in enumerate(g_layers):
             assert bool((L.depth_index_tensor == want_packed[l]).all()), (rep, l)
             a, b = g_images[l], want_images[l]
             assert float((a - b).abs().max()) <= 1e-5 * float(b.abs().max()), (rep, l)
