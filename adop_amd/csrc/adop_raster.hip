@@ -1065,6 +1065,8 @@ const char* adop_last_error_string(void)
 
 const char* adop_version(void)
 {
-    return "adop_raster 0.1 (gfx950)";
+    // "kernels N" names the state of the kernels' memory behaviour: it goes up whenever a change moves a kernel's bytes,
+    // so that traffic figures measured for one state (rocprofv3 counters) are not quoted for another.
+    return "adop_raster 0.2 (gfx950) kernels 1";
 }
 }  // extern "C"

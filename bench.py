@@ -1,21 +1,28 @@
 #!/usr/bin/env python3
 """Benchmark of the point-rasterizer hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config3|config2|config4|config5]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config3|config1|config2|config4|config5|crops]
 
 A step is one pass of the hot path over one batch of synthetic input that already sits in HBM:
-``adop_forward`` + ``adop_backward`` through the C-ABI (forward only for the viewer workload config4).
-Prints ONE JSON line.  Default workload: BASELINE config 3 (10 M points, 1920x1080, 4 levels, 8 channels,
-forward + backward with descriptor / point / pose / intrinsics gradients) -> points/s.
+``adop_forward`` + ``adop_backward`` through the C-ABI (forward only for configs 1 and 4; config 5 adds the
+environment-map pass on its OCam views and its texture gradient).  Prints ONE JSON line.
+
+Default workload: BASELINE config 3 (10 M points, 1920x1080, 4 levels, 8 channels, forward + backward with
+descriptor / point / pose / intrinsics gradients) -> points/s.  The default run then also measures the second
+headline figure, config 4 (100 M points, 5 levels, fp16 descriptors, forward over the 300-frame orbit -> frames/s),
+and reports it under ``step.config4`` (``--no-config4`` leaves it out).
 
 ``roofline`` describes the slowest kernel of the step: algorithmic bytes of that kernel (byte model below, with
 the point-level counts V/A/G measured by the kernels' own counters in an untimed pass) divided by its average
-duration measured with HIP events on the launch stream, against the 8 TB/s HBM peak.
+duration measured with HIP events on the launch stream, against the 8 TB/s HBM peak.  ``roofline.traffic`` and
+``step.hbm_frac_measured`` use HBM bytes per launch measured with rocprofv3 counters (MEASURED_TRAFFIC below: each
+table names the profile it comes from and the kernel state it was measured on; for any other state they are null).
 ``cpu_baseline`` times the CPU checker (OpenMP build) on the host cores for the same workload (or a bounded
 sample of it).
 """
 import argparse
 import ctypes as C
+import gc
 import json
 import os
 import sys
@@ -28,7 +35,21 @@ HBM_PEAK_GBS = 8000.0
 KERNEL_OF_STAGE = {"BinCount": "bin_count_kernel", "BinScatter": "bin_scatter_kernel", "TileDepth": "tile_depth_kernel", "TileBlend": "tile_blend_kernel",
                    "DepthPrepass": "prepass_kernel", "RenderForward": "blend_kernel", "CombineAndFill": "resolve_kernel",
                    "CombineAndFillBackward": "interleave_kernel", "RenderBackward/descriptor": "backward_tex_kernel",
-                   "RenderBackward/spatial": "backward_ghost_kernel"}
+                   "RenderBackward/spatial": "backward_ghost_kernel", "EnvironmentMap": "env_sample_kernel",
+                   "EnvironmentMapBackward": "env_backward_kernel"}
+
+# HBM bytes per launch (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, KiB per dispatch; FETCH_SIZE x 2.0 and WRITE_SIZE
+# x 1.0 after calibration with plain device copies of known size), per workload.  "kernels" is the state of the library
+# (the number adop_version() ends in) the profile was taken on: the figures are quoted for that state only.
+MEASURED_TRAFFIC = {
+    "config3": {"kernels": 1, "profile": "profiles/config3_tile_path_fwd_bwd_kernels_traffic_instructions.md",
+                "bytes": {"RenderBackward/descriptor": 911.8e6, "RenderBackward/spatial": 486.2e6, "TileBlend": 436.6e6,
+                          "BinCount": 430.3e6, "BinScatter": 197.0e6, "TileDepth": 101.0e6,
+                          "CombineAndFillBackward": 397.3e6, "Initialize": 11.7e6, "CombineAndFill": 18.2e6,
+                          "Post Process Gradient": 90.8e6}},
+    "config4": {"kernels": 1, "profile": "profiles/config4_direct_path_forward_kernels_traffic_instructions.md",
+                "bytes": {"DepthPrepass": 5053.5e6, "RenderForward": 1548.3e6}},
+}
 
 
 def byte_model(N, B, C_, S_d, P, V, A, G, has_mask, has_dropout):
@@ -61,6 +82,21 @@ def tile_path_model(k, N, B, C_, P_levels, V, has_dropout, lt=2):
     k["CombineAndFill"] = caf * frac_coarse
     assert abs(sum((k[n] for n in ("BinCount", "BinScatter", "TileDepth", "TileBlend", "CombineAndFill"))) - (prepass + blend + caf)) < 1
     return k
+
+
+def kernel_state(lib):
+    """The number adop_version() ends in ("... kernels N")."""
+    words = lib.adop_version().decode().split()
+    return int(words[-1]) if len(words) >= 2 and words[-2] == "kernels" and words[-1].isdigit() else None
+
+
+def host_threads():
+    """Threads of the CPU baseline: the share of the host this process is given (OMP_NUM_THREADS where the
+    environment sets it, as the GPU boxes do for their one-GPU share; otherwise every core the OS shows)."""
+    env = os.environ.get("OMP_NUM_THREADS", "")
+    n = int(env) if env.isdigit() and int(env) > 0 else (os.cpu_count() or 1)
+    os.environ["OMP_NUM_THREADS"] = str(n)
+    return n
 
 
 def bench_preprocess(args):
@@ -129,7 +165,7 @@ def bench_preprocess(args):
         cpu = {"value": m / sec, "unit": "points/s", "cores": 1, "kind": "port",
                "sample": f"brute-force neighbour search among the first {m} of {N} points + their Morton codes",
                "seconds": round(sec, 3)}
-    print(json.dumps({
+    return {
         "metric": "preprocess points/s", "value": N / (ms_per_step * 1e-3), "unit": "points/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
@@ -143,54 +179,58 @@ def bench_preprocess(args):
         "step": {"stage_ms": {"knn_distance": round(t_knn, 4), "morton_codes": round(t_mor, 4)},
                  "filters_ms": filt,
                  "scene_gen_s": round(gen_s, 1)},
-    }))
+    }
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="config3", choices=["config2", "config3", "config4", "config5", "preprocess"])
-    ap.add_argument("--points", type=int, default=0, help="override the point count (0 = the configuration's)")
-    ap.add_argument("--point-order", default="morton", choices=["morton", "random"])
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-point-cache", action="store_true",
-                    help="do not keep the projected points for the backward pass (it projects again)")
-    ap.add_argument("--cpu-points", type=int, default=0, help="point count of the CPU sample (0 = automatic)")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run a plain 1 GiB device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build runs on one GPU only (one process, one MI355X); "
-              "a figure at several GPUs is not produced. Use --gpus 1.", file=sys.stderr)
-        sys.exit(2)
+def crops_scene(args):
+    """A training batch as the reference forms it (configs/train_boat.ini:5-6, Dataset.cpp:107-227): 4 frames x 4
+    random crops of 512 x 512 (zoom 0.75 .. 1.5) of the config-3 scene."""
+    import numpy as np
+    from adop_amd import scenes
 
+    kw = {"n": args.points} if args.points else {}
+    hs = scenes.config3(point_order=args.point_order, **kw)
+    g = np.random.default_rng(1)
+    frames, per_frame, cw = 4, 4, 512
+    hs.poses_se3 = np.stack([scenes.orbit_pose(f, radius=3.0, deg_per_frame=20.0) for f in range(frames)])
+    views = []
+    for f in range(frames):
+        for _ in range(per_frame):
+            zoom = float(g.uniform(0.75, 1.5))
+            # window of cw / zoom source pixels somewhere inside the 1920 x 1080 frame
+            src = cw / zoom
+            x0 = float(g.uniform(0, 1920 - src))
+            y0 = float(g.uniform(0, 1080 - src))
+            views.append(scenes.make_view(cw, cw, image_index=f, crop=(zoom, zoom, -x0 * zoom, -y0 * zoom, 0.0)))
+    hs.views = views
+    hs.dropout = scenes.bernoulli_mask(2, len(views), hs.num_points, 0.25)
+    hs.name = "crops"
+    return hs
+
+
+def run_workload(args, workload, steps, warmup, lib):
+    """Measures one render workload; returns the JSON object of its bench line."""
     import numpy as np
     import torch
     from adop_amd import _capi, render, scenes
 
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(3)
-    lib = _capi.load_library()
     dev = "cuda:0"
-    torch.cuda.set_device(0)
-    if args.workload == "preprocess":
-        bench_preprocess(args)
-        return
-
     t0 = time.time()
     kw = {"n": args.points} if args.points else {}
-    if args.workload == "config3":
+    if workload == "config3":
         hs = scenes.config3(point_order=args.point_order, **kw)
-    elif args.workload == "config2":
+    elif workload == "config1":
+        hs = scenes.config1(**kw)
+    elif workload == "config2":
         hs = scenes.config2(point_order=args.point_order, **kw)
-    elif args.workload == "config4":
+    elif workload == "config4":
         hs = scenes.config4(point_order=args.point_order, **kw)
+    elif workload == "crops":
+        hs = crops_scene(args)
     else:
         hs = scenes.config5(point_order=args.point_order, **kw)
-    backward = args.workload != "config4"
+    backward = workload not in ("config1", "config4")
+    with_env = workload == "config5" and hs.env_texture is not None and not args.no_env
     gen_s = time.time() - t0
 
     scene = render.NeuralScene.from_host(hs, dev)
@@ -225,24 +265,54 @@ def main():
         keep = [gout, g_tex, g_bg, g_pts, g_pts_c, g_pose, g_pose_c, g_intr, g_intr_c]
         gb.grad_texture, gb.grad_background = g_tex.data_ptr(), g_bg.data_ptr()
         gb.grad_points, gb.grad_points_count = g_pts.data_ptr(), g_pts_c.data_ptr()
-        if args.workload in ("config3",):
+        if workload in ("config3", "crops"):
             gb.grad_pose, gb.grad_pose_count = g_pose.data_ptr(), g_pose_c.data_ptr()
             gb.grad_intrinsics, gb.grad_intrinsics_count = g_intr.data_ptr(), g_intr_c.data_ptr()
+    env_args = None
+    if with_env:
+        env = scene.environment_map
+        g_env = torch.empty_like(env)
+        gout_arr = (C.c_void_p * L)(*[g.data_ptr() for g in gout])
+        env_args = (C.c_void_p(env.data_ptr()), int(env.shape[1]), int(env.shape[2]), gout_arr, C.c_void_p(g_env.data_ptr()))
+        keep += [g_env]
 
     frame = [0]
+    env_events = []  # (name, start, stop) torch events around the environment-map calls while profiling
 
-    def step(stats=None):
-        if args.workload == "config4":
-            views[0].image_index = frame[0] % scene.poses_se3.shape[0]  # orbit
+    def fail():
+        raise RuntimeError(lib.adop_last_error_string().decode())
+
+    def step(stats=None, timed_env=False):
+        if workload == "config4":
+            views[0].image_index = frame[0] % scene.poses_se3.shape[0]  # the orbit: 1.2 degrees per frame
             frame[0] += 1
-        rc = lib.adop_forward(C.byref(s), views, B, C.byref(hs.params), C.byref(fb), ws, ws_n, stats, stream_of[0])
-        if rc != 0:
-            raise RuntimeError(lib.adop_last_error_string().decode())
+        if lib.adop_forward(C.byref(s), views, B, C.byref(hs.params), C.byref(fb), ws, ws_n, stats, stream_of[0]) != 0:
+            fail()
+        if with_env:
+            # spherical environment map sampled at the empty pixels of the OCam views, added to the images
+            if timed_env:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+            if lib.adop_env_sample(C.byref(s), views, B, env_args[0], env_args[1], env_args[2], C.byref(fb), None, None,
+                                   1, stream_of[0]) != 0:
+                fail()
+            if timed_env:
+                e1.record()
+                env_events.append(("EnvironmentMap", e0, e1))
         if backward:
-            rc = lib.adop_backward(C.byref(s), views, B, C.byref(hs.params), C.byref(fb), C.byref(gb), ws, ws_n,
-                                   stats, stream_of[0])
-            if rc != 0:
-                raise RuntimeError(lib.adop_last_error_string().decode())
+            if lib.adop_backward(C.byref(s), views, B, C.byref(hs.params), C.byref(fb), C.byref(gb), ws, ws_n, stats,
+                                 stream_of[0]) != 0:
+                fail()
+        if with_env:
+            if timed_env:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+            if lib.adop_env_sample_backward(C.byref(s), views, B, env_args[1], env_args[2], C.byref(fb), env_args[3],
+                                            env_args[4], stream_of[0]) != 0:
+                fail()
+            if timed_env:
+                e1.record()
+                env_events.append(("EnvironmentMapBackward", e0, e1))
 
     copy_gbs = None
     if args.calibrate_copy:
@@ -265,32 +335,38 @@ def main():
     torch.cuda.synchronize()
     st = cache.read_stats()
     V, A, G = list(st.visible)[:L], list(st.accepted)[:L], list(st.spatial)[:L]
+    empty_pixels = 0
+    if with_env:
+        empty_pixels = int(sum(int((m == 0).sum().item()) for m in cache.output_forward_background_mask))
 
     frame[0] = 0
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     torch.cuda.synchronize()
     t2 = time.perf_counter()
-    ms_per_step = (t2 - t1) * 1e3 / args.steps
+    ms_per_step = (t2 - t1) * 1e3 / steps
 
     # per-stage durations from HIP events on the launch stream
     lib.adop_profile_enable(1)
-    for _ in range(args.steps):
-        step()
+    prof_steps = min(steps, 50)
+    for _ in range(prof_steps):
+        step(timed_env=True)
     torch.cuda.synchronize()
     arr = (_capi.StageTime * 16)()
     n = lib.adop_profile_read(arr, 16)
     lib.adop_profile_enable(0)
-    stages = {arr[i].name.decode(): arr[i].total_ms / args.steps for i in range(n)}  # ms per step
+    stages = {arr[i].name.decode(): arr[i].total_ms / prof_steps for i in range(n)}  # ms per step
+    for name, e0, e1 in env_events:
+        stages[name] = stages.get(name, 0.0) + e0.elapsed_time(e1) / prof_steps
 
     # the same step recorded once into a HIP graph and replayed (outside the timed region above: what the host-side
     # launches cost); configuration 4 changes a host-side argument every frame and is not recorded
     graph_ms = None
-    if args.workload != "config4":
+    if workload != "config4" and not args.no_graph:
         side = torch.cuda.Stream()
         graph = torch.cuda.CUDAGraph()
         eager_stream = stream_of[0]
@@ -299,85 +375,116 @@ def main():
                 stream_of[0] = C.c_void_p(side.cuda_stream)
                 step()
         stream_of[0] = eager_stream
-        for _ in range(max(args.warmup, 1)):
+        for _ in range(max(warmup, 1)):
             graph.replay()
         torch.cuda.synchronize()
         tg = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(steps):
             graph.replay()
         torch.cuda.synchronize()
-        graph_ms = (time.perf_counter() - tg) * 1e3 / args.steps
+        graph_ms = (time.perf_counter() - tg) * 1e3 / steps
+        del graph
 
-    P = sum(w * h for (w, h) in hs.level_sizes())
+    P_levels = [w * h for (w, h) in hs.level_sizes()]
+    P = sum(P_levels)
     S_d = 2 if hs.texture.dtype == np.float16 else 4
     model = byte_model(N, B, Cn, S_d, P, V, A, G, bool(hs.params.output_background_mask), hs.dropout is not None)
     if "TileBlend" in stages:
-        model = tile_path_model(model, N, B, Cn, [w * h for (w, h) in hs.level_sizes()], V, hs.dropout is not None)
+        model = tile_path_model(model, N, B, Cn, P_levels, V, hs.dropout is not None)
     if not backward:
         model = {k: v for k, v in model.items() if k in ("DepthPrepass", "RenderForward", "CombineAndFill", "BinCount",
                                                          "BinScatter", "TileDepth", "TileBlend")}
+    if with_env:
+        # uv is not stored; every pixel reads its mask, an empty one its four taps per channel and adds to the image
+        model["EnvironmentMap"] = B * P * 4 + empty_pixels * (16 * Cn + 8 * Cn)
+        model["EnvironmentMapBackward"] = B * P * 4 + empty_pixels * (4 * Cn + 2 * 16 * Cn)
     total_bytes = sum(model.values())
     dom = max((k for k in model if k in stages), key=lambda k: stages[k])
     dom_gbs = model[dom] / (stages[dom] * 1e-3) / 1e9
-    # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
-    # FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 after calibration with plain device copies); measured for the default
-    # workload only
-    measured_traffic = {}
-    if args.workload == "config3" and not args.points and args.point_order == "morton" and not args.no_point_cache:
-        # profiles/config3_tile_path_fwd_bwd_kernels_traffic_instructions.md, profiles/config3_direct_path_fwd_bwd_kernels_traffic_instructions.md
-        measured_traffic = {"RenderBackward/descriptor": 912.7e6, "RenderBackward/spatial": 486.2e6, "TileBlend": 438.1e6,
-                            "BinCount": 436.4e6, "BinScatter": 196.9e6, "TileDepth": 101.0e6,
-                            "CombineAndFillBackward": 397.3e6, "RenderForward": 611.0e6, "DepthPrepass": 578.9e6}
-    if args.workload == "config4" and not args.points and args.point_order == "morton":
-        # profiles/config4_direct_path_forward_kernels_traffic_instructions.md
-        measured_traffic = {"DepthPrepass": 5053.5e6, "RenderForward": 1548.3e6}
+
+    # measured HBM traffic (rocprofv3 counters), for the exact workload and kernel state the profile was taken on
+    measured, measured_from = {}, None
+    tab = MEASURED_TRAFFIC.get(workload)
+    if (tab and not args.points and args.point_order == "morton" and not args.no_point_cache
+            and tab["kernels"] == kernel_state(lib)):
+        measured = {k: v for k, v in tab["bytes"].items() if k in stages}
+        measured_from = {"profile": tab["profile"], "kernels": tab["kernels"]}
+    step_measured = None  # every stage of the step that moves memory has a figure
+    if measured and all(k in measured for k in stages if k != "Prepare Backward"):
+        step_measured = sum(measured.values())
     roofline = {"bound": "hbm", "kernel": KERNEL_OF_STAGE.get(dom, dom), "stage": dom, "achieved": round(dom_gbs, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
-                "traffic": measured_traffic.get(dom),
+                "traffic": measured.get(dom), "traffic_from": measured_from if dom in measured else None,
                 "kernel_ms": round(stages[dom], 4), "algorithmic_bytes": int(model[dom])}
     step_gbs = total_bytes / (ms_per_step * 1e-3) / 1e9
+    # a stage whose algorithmic bytes exceed what it moves (neighbouring points share lines through the L2) is charged
+    # its measured bytes in hbm_frac_dedup, so that no stage is credited with more than it moves
+    dedup_bytes = sum(min(model[k], measured.get(k, model[k])) for k in model) if measured else None
 
-    if args.workload == "config4":
-        metric, unit, value = "forward frames/s at 100M points 1920x1080 x5 levels", "frames/s", 1e3 / ms_per_step
+    if workload in ("config4", "config1"):
+        what = "100M" if workload == "config4" else str(N)
+        metric, unit, value = f"forward frames/s at {what} points {hs.views[0].w}x{hs.views[0].h} x{L} levels", "frames/s", 1e3 / ms_per_step
     else:
         metric, unit = "fwd+bwd points/s", "points/s"
         value = N * B / (ms_per_step * 1e-3)
 
     cpu = None
     if not args.no_cpu_baseline:
+        import copy
         import oracle
-        cores = min(os.cpu_count() or 1, 16)
-        os.environ["OMP_NUM_THREADS"] = str(cores)
-        chs, sample = hs, "the full workload, one step"
-        cpu_n = args.cpu_points or (20_000_000 if N > 20_000_000 else 0)
-        if cpu_n and cpu_n < N:
-            # bounded sample: the first cpu_n points of the same cloud at the same resolution
-            import copy
+        nthreads = host_threads()
+        chs, sample, reps = hs, "the full workload, one step", 1
+        cpu_n = args.cpu_points or 0
+        if workload == "config5":
+            # one of the 8 views (the others cost the same per view: stated, not measured)
             chs = copy.copy(hs)
+            chs.views, chs.dropout = hs.views[:1], None if hs.dropout is None else np.ascontiguousarray(hs.dropout[:1])
+            sample = f"view 0 of {B} at the full point count and resolution, forward + backward (points/s counts that one view)"
+        if workload == "crops":
+            chs = copy.copy(hs)
+            chs.views, chs.dropout = hs.views[:4], np.ascontiguousarray(hs.dropout[:4])
+            sample = f"the 4 crops of frame 0 (of {B}) at the full point count, forward + backward"
+        if cpu_n and cpu_n < N:
+            chs = copy.copy(chs)
             chs.position, chs.index = hs.position[:cpu_n], hs.index[:cpu_n]
             chs.normal = None if hs.normal is None else hs.normal[:cpu_n]
-            chs.dropout = None if hs.dropout is None else np.ascontiguousarray(hs.dropout[:, :cpu_n])
-            sample = f"first {cpu_n} of {N} points, same resolution, one step"
+            chs.dropout = None if chs.dropout is None else np.ascontiguousarray(chs.dropout[:, :cpu_n])
+            sample = f"first {cpu_n} of {N} points; " + sample
+        frames_cpu = [0]
+        if workload == "config4":
+            frames_cpu, reps = [0, 100, 200], 3
+            sample = "the full cloud, orbit frames 0, 100 and 200, forward"
+        cgout = scenes.upstream_grads(chs) if backward else None
+        oracle.lib(True)  # load outside the timed region
         tc0 = time.perf_counter()
-        ref = oracle.forward(chs, omp=True)
-        if backward:
-            oracle.backward(chs, ref, scenes.upstream_grads(chs), omp=True)
+        for f in frames_cpu:
+            if workload == "config4":
+                chs.views[0].image_index = f
+            ref = oracle.forward(chs, omp=True)
+            if backward:
+                oracle.backward(chs, ref, cgout, omp=True)
         tc = time.perf_counter() - tc0
-        nthreads = oracle.lib(True).oracle_num_threads()
-        if args.workload == "config4":
-            cpu_val, cpu_unit = (chs.num_points / N) / tc, "frames/s"
-            sample += " (frames/s scaled linearly to the full point count)"
+        if workload == "config4":
+            chs.views[0].image_index = 0
+        used = oracle.lib(True).oracle_num_threads()
+        if workload in ("config4", "config1"):
+            cpu_val, cpu_unit = reps * (chs.num_points / N) / tc, "frames/s"
         else:
-            cpu_val, cpu_unit = chs.num_points * B / tc, "points/s"
-        cpu = {"value": cpu_val, "unit": cpu_unit, "cores": nthreads, "kind": "port", "sample": sample,
-               "seconds": round(tc, 3)}
+            cpu_val, cpu_unit = chs.num_points * chs.batch / tc, "points/s"
+        cpu = {"value": cpu_val, "unit": cpu_unit, "cores": used, "kind": "port", "sample": sample,
+               "seconds": round(tc, 3), "host_cpus": os.cpu_count(),
+               "threads_from": "OMP_NUM_THREADS" if os.environ.get("OMP_NUM_THREADS") else "os.cpu_count()"}
+        assert used == nthreads or used >= 1
 
     out = {
-        "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32" if S_d == 4 else "f16-stored/f32-accumulated", "data": "synthetic",
-        "config": {"workload": f"BASELINE {hs.name}: {N} points, B={B}, {hs.views[0].w}x{hs.views[0].h}, "
-                               f"{L} levels, C={Cn}, " + ("forward+backward" if backward else "forward only"),
+        "config": {"workload": (f"BASELINE {hs.name}" if hs.name.startswith("config") else "training batch of 4 frames x 4 crops of config3") +
+                               f": {N} points, B={B}, {hs.views[0].w}x{hs.views[0].h}, "
+                               f"{L} levels, C={Cn}, " + ("forward+backward" if backward else "forward only") +
+                               (", spherical environment map on the OCam views with its gradient" if with_env else "") +
+                               (", 300-pose orbit of radius 12, 1.2 degrees per frame" if workload == "config4" else ""),
                    "point_order": hs.meta.get("point_order", "as generated"), "lod_radius_test": False,
                    "dropout": 0.25 if hs.dropout is not None else 0.0,
                    "ghost_gradients": bool(hs.params.ghost_gradients)},
@@ -385,12 +492,77 @@ def main():
         "cpu_baseline": cpu,
         "step": {"algorithmic_bytes": int(total_bytes), "achieved_GBps": round(step_gbs, 1),
                  "hbm_frac": round(step_gbs / HBM_PEAK_GBS, 4),
+                 "measured_bytes": None if step_measured is None else int(step_measured),
+                 "hbm_frac_measured": None if step_measured is None else round(step_measured / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                 "hbm_frac_dedup": None if dedup_bytes is None else round(dedup_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                 "measured_from": measured_from,
                  "stage_ms": {k: round(v, 4) for k, v in stages.items()},
                  "stage_GBps": {k: round(model[k] / (stages[k] * 1e-3) / 1e9, 1) for k in model if k in stages},
+                 "stage_GBps_measured": {k: round(measured[k] / (stages[k] * 1e-3) / 1e9, 1) for k in measured} or None,
+                 "stages_model_above_peak": [k for k in model if k in stages and model[k] / (stages[k] * 1e-3) / 1e9 > HBM_PEAK_GBS],
                  "visible": V, "accepted": A, "spatial": G, "scene_gen_s": round(gen_s, 1),
                  "graph_replay_ms_per_step": None if graph_ms is None else round(graph_ms, 4),
                  "device_copy_GBps": None if copy_gbs is None else round(copy_gbs, 1)},
     }
+    if with_env:
+        out["step"]["empty_pixels"] = empty_pixels
+    del keep, cache, scene, info, hs
+    gc.collect()
+    torch.cuda.empty_cache()
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=0, help="timed steps (default 20; 300 = the whole orbit for config4)")
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="config3",
+                    choices=["config1", "config2", "config3", "config4", "config5", "crops", "preprocess"])
+    ap.add_argument("--points", type=int, default=0, help="override the point count (0 = the configuration's)")
+    ap.add_argument("--point-order", default="morton", choices=["morton", "random"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-config4", action="store_true",
+                    help="default workload only: do not measure the 100 M-point orbit after config3")
+    ap.add_argument("--no-env", action="store_true", help="config5 without the environment-map passes")
+    ap.add_argument("--no-graph", action="store_true", help="do not replay the step from a HIP graph as well")
+    ap.add_argument("--no-point-cache", action="store_true",
+                    help="do not keep the projected points for the backward pass (it projects again)")
+    ap.add_argument("--cpu-points", type=int, default=0, help="point count of the CPU sample (0 = the full cloud)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (one process, one MI355X); "
+              "a figure at several GPUs is not produced. Use --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from adop_amd import _capi
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    lib = _capi.load_library()
+    torch.cuda.set_device(0)
+    if args.workload == "preprocess":
+        args.steps = args.steps or 20
+        print(json.dumps(bench_preprocess(args)))
+        return
+
+    steps = args.steps or (300 if args.workload == "config4" else 20)
+    out = run_workload(args, args.workload, steps, args.warmup, lib)
+    if args.workload == "config3" and not args.no_config4 and not args.points:
+        # the second headline figure: forward frames/s at 100 M points over the whole 300-frame orbit
+        c4 = run_workload(args, "config4", 300, args.warmup, lib)
+        out["step"]["config4"] = {
+            "metric": c4["metric"], "value": round(c4["value"], 2), "unit": c4["unit"], "frames": c4["steps"],
+            "ms_per_frame": round(c4["ms_per_step"], 4), "target_frames_per_s": 60, "workload": c4["config"]["workload"],
+            "dtype": c4["dtype"], "roofline": c4["roofline"], "cpu_baseline": c4["cpu_baseline"],
+            "hbm_frac": c4["step"]["hbm_frac"], "hbm_frac_measured": c4["step"]["hbm_frac_measured"],
+            "achieved_GBps": c4["step"]["achieved_GBps"], "stage_ms": c4["step"]["stage_ms"],
+            "stage_GBps": c4["step"]["stage_GBps"], "scene_gen_s": c4["step"]["scene_gen_s"],
+        }
     print(json.dumps(out))
 
 
