@@ -144,7 +144,7 @@ ENTRY_POINTS = {
     "adop_env_sample_backward": (
         C.c_int,
         [C.POINTER(Scene), C.POINTER(View), C.c_int32, C.c_int32, C.c_int32, C.POINTER(ForwardBuffers),
-         C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p],
+         C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p],
     ),
     "adop_apply_tangent": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "adop_knn_workspace_size": (C.c_size_t, [C.c_int32]),

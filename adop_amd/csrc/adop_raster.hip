@@ -749,7 +749,8 @@ adop_status adop_env_sample(const adop_scene* scene, const adop_view* views, int
 
 adop_status adop_env_sample_backward(const adop_scene* scene, const adop_view* views, int32_t num_views, int32_t env_h,
                                      int32_t env_w, const adop_forward_buffers* buffers,
-                                     const float* const* grad_out_levels, float* grad_env, void* hip_stream)
+                                     const float* const* grad_out_levels, const float* const* uv_levels,
+                                     float* grad_env, void* hip_stream)
 {
     adop_status st = env_common(scene, views, num_views, buffers, env_h, env_w);
     if (st != ADOP_OK) return st;
@@ -763,6 +764,9 @@ adop_status adop_env_sample_backward(const adop_scene* scene, const adop_view* v
     {
         if (!grad_out_levels[l]) return fail(ADOP_INVALID_ARG, "upstream gradient missing");
         ev.gout[l] = grad_out_levels[l];
+        // (the texture coordinates the forward call stored, if the caller kept them; every level or none)
+        if (uv_levels && !uv_levels[l]) return fail(ADOP_INVALID_ARG, "uv_levels: a level is missing");
+        ev.uv[l] = uv_levels ? const_cast<float*>(uv_levels[l]) : nullptr;
     }
     st = fill_async(grad_env, sizeof(float) * (size_t)scene->num_channels * env_h * env_w, 0, stream);
     if (st != ADOP_OK) return st;
@@ -1067,6 +1071,6 @@ const char* adop_version(void)
 {
     // "kernels N" names the state of the kernels' memory behaviour: it goes up whenever a change moves a kernel's bytes,
     // so that traffic figures measured for one state (rocprofv3 counters) are not quoted for another.
-    return "adop_raster 0.2 (gfx950) kernels 1";
+    return "adop_raster 0.2 (gfx950) kernels 2";
 }
 }  // extern "C"

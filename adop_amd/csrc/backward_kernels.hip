@@ -2,8 +2,10 @@
 //
 // The ghost gradient of one point-level reads the image I and the upstream gradient G at four neighbour pixels for
 // every channel.  In the planar [B,C,h,w] layout that is 8C scattered 4-byte loads (plus C for the centre); the
-// interleave kernel therefore first builds a pixel-major array IG[pixel][I_0..I_{C-1}, G_0..G_{C-1}] in the
-// workspace (one 64-byte line per pixel for C = 8), while it sums the background gradient in the same pass.
+// interleave kernel therefore first builds two pixel-major arrays in the workspace, I[pixel][C] and, behind it,
+// G[pixel][C] (32 bytes per pixel each for C = 8), while it sums the background gradient in the same pass.  Two arrays
+// and not one record [I | G] per pixel: the descriptor pass gathers G alone, and with I in the same 64-byte line it
+// fetched twice the bytes it used.
 #include "common.h"
 #include "launch.h"
 
@@ -48,7 +50,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
         dw[ws_pixel(lv, l, b, (uint32_t)p)] = make_float2(L.depth[(size_t)b * hw + p], wgt);
         const float* g    = L.gin + (size_t)b * C * hw + p;
         const float* im   = L.out + (size_t)b * C * hw + p;
-        float* dst        = ig + (size_t)ws_pixel(lv, l, b, (uint32_t)p) * (2 * C);
+        float* dst        = ig + (size_t)ws_pixel(lv, l, b, (uint32_t)p) * C;  // I record; the G record at dst + goff
+        const size_t goff = total * (size_t)C;
         float I[CMAX], G[CMAX];
 #pragma unroll
         for (int c = 0; c < CMAX; ++c)
@@ -63,7 +66,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
             // The 64 pixels of a wavefront are 64 consecutive records of the pixel-major array when they lie in one
             // level of one image: transposed through LDS, every store instruction then writes 1 KB of consecutive
             // bytes instead of a quarter (half) of 64 separate lines.
-            constexpr int V     = CT / 2;  // float4 per record
+            constexpr int V     = CT / 4;  // float4 per record of either array
             const int lane      = threadIdx.x & 63;
             const size_t t_wave = t - lane;
             const int r_last    = (int)((t_wave + 63) - (size_t)b * per_image);
@@ -72,28 +75,32 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
                                level_of(lv, r - lane) == l;
             if (whole)  // wavefront-uniform
             {
+                // s_tr: the I records of the 64 pixels, then their G records
                 float4* sw = s_tr[threadIdx.x >> 6];
                 wave_lds_sync();
 #pragma unroll
-                for (int q = 0; q < CT / 4; ++q)
+                for (int q = 0; q < V; ++q)
                 {
                     sw[lane * V + q]          = make_float4(I[4 * q], I[4 * q + 1], I[4 * q + 2], I[4 * q + 3]);
-                    sw[lane * V + CT / 4 + q] = make_float4(G[4 * q], G[4 * q + 1], G[4 * q + 2], G[4 * q + 3]);
+                    sw[64 * V + lane * V + q] = make_float4(G[4 * q], G[4 * q + 1], G[4 * q + 2], G[4 * q + 3]);
                 }
                 wave_lds_sync();
-                float4* d4 = (float4*)(dst - (size_t)lane * (2 * CT));  // record of the wavefront's first pixel
+                float* d0 = dst - (size_t)lane * CT;  // I record of the wavefront's first pixel
 #pragma unroll
                 for (int k = 0; k < V; ++k)
-                    __builtin_nontemporal_store(((const v4f*)sw)[k * 64 + lane], (v4f*)d4 + k * 64 + lane);
+                {
+                    __builtin_nontemporal_store(((const v4f*)sw)[k * 64 + lane], (v4f*)d0 + k * 64 + lane);
+                    __builtin_nontemporal_store(((const v4f*)sw)[64 * V + k * 64 + lane], (v4f*)(d0 + goff) + k * 64 + lane);
+                }
             }
             else
             {
                 float4* d4 = (float4*)dst;
+                float4* g4 = (float4*)(dst + goff);
 #pragma unroll
-                for (int q = 0; q < CT / 4; ++q) d4[q] = make_float4(I[4 * q], I[4 * q + 1], I[4 * q + 2], I[4 * q + 3]);
+                for (int q = 0; q < V; ++q) d4[q] = make_float4(I[4 * q], I[4 * q + 1], I[4 * q + 2], I[4 * q + 3]);
 #pragma unroll
-                for (int q = 0; q < CT / 4; ++q)
-                    d4[CT / 4 + q] = make_float4(G[4 * q], G[4 * q + 1], G[4 * q + 2], G[4 * q + 3]);
+                for (int q = 0; q < V; ++q) g4[q] = make_float4(G[4 * q], G[4 * q + 1], G[4 * q + 2], G[4 * q + 3]);
             }
         }
         else
@@ -102,8 +109,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
             for (int c = 0; c < CMAX; ++c)
                 if (c < C)
                 {
-                    dst[c]     = I[c];
-                    dst[C + c] = G[c];
+                    dst[c]        = I[c];
+                    dst[goff + c] = G[c];
                 }
         }
     }
@@ -321,7 +328,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(CT != 0 
                     else
                     {
                         float iw        = 1.f / wgt[l];
-                        const float* pg = ig + (size_t)ws_pixel(lv, l, b, pix[l]) * (2 * C) + C;  // G of the pixel
+                        const float* pg = ig + gradient_array_offset(lv, C) + (size_t)ws_pixel(lv, l, b, pix[l]) * C;  // G of the pixel
                         if (CT == 0)
                         {
                             // any channel count: one atomic per channel and level (:478-484)
@@ -536,7 +543,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
                 int px = f2i_rn(ip.x), py = f2i_rn(ip.y);
                 size_t hw             = (size_t)L.w * L.h;
                 size_t p              = (size_t)py * L.w + px;
-                const float* pg       = ig + (size_t)ws_pixel(lv, l, b, (uint32_t)p) * (2 * C);  // [I | G] of the pixel
+                const float* pg       = ig + (size_t)ws_pixel(lv, l, b, (uint32_t)p) * C;  // I of the pixel, its G at + goff
+                const size_t goff     = gradient_array_offset(lv, C);
                 const ptrdiff_t nb[4] = {-1, 1, -(ptrdiff_t)L.w, (ptrdiff_t)L.w};
                 float Wn[4] = {0, 0, 0, 0}, Dn[4] = {0, 0, 0, 0};
                 if (rp.test_backward_mode == 4)
@@ -571,8 +579,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
 #pragma unroll
                         for (int k = 0; k < 4; ++k)
                         {
-                            const float* q = pg + nb[k] * (2 * C);
-                            v[k]           = dI_of(T_c, q[c], Wn[k], Dn[k]) * q[C + c];
+                            const float* q = pg + nb[k] * C;
+                            v[k]           = dI_of(T_c, q[c], Wn[k], Dn[k]) * q[goff + c];
                         }
                         float a0 = -v[0], a1 = v[1], b0 = -v[2], b1 = v[3];
                         dR_dpx += 0.5f * (a0 + a1);
@@ -585,10 +593,10 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
 #pragma unroll
                     for (int k = 0; k < 4; ++k)
                     {
-                        const float* q = pg + nb[k] * (2 * C);
+                        const float* q = pg + nb[k] * C;
                         float In[CMAX], Gn[CMAX];
                         load_channels<CT ? CT : 4>(q, In);
-                        load_channels<CT ? CT : 4>(q + C, Gn);
+                        load_channels<CT ? CT : 4>(q + goff, Gn);
 #pragma unroll
                         for (int c = 0; c < CMAX; ++c) v[k][c] = dI_of(T[c], In[c], Wn[k], Dn[k]) * Gn[c];
                     }
@@ -806,7 +814,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
                     int px = f2i_rn(ip.x), py = f2i_rn(ip.y);
                     size_t hw             = (size_t)L.w * L.h;
                     size_t p              = (size_t)py * L.w + px;
-                    const float* pg       = ig + (size_t)ws_pixel(lv, l, b, (uint32_t)p) * (2 * C);  // [I | G] of the pixel
+                    const float* pg       = ig + (size_t)ws_pixel(lv, l, b, (uint32_t)p) * C;  // I of the pixel, its G at + goff
+                    const size_t goff     = gradient_array_offset(lv, C);
                     const ptrdiff_t nb[4] = {-1, 1, -(ptrdiff_t)L.w, (ptrdiff_t)L.w};
                     float Wn[4] = {0, 0, 0, 0}, Dn[4] = {0, 0, 0, 0};
                     if (rp.test_backward_mode == 4)
@@ -841,8 +850,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
     #pragma unroll
                             for (int k = 0; k < 4; ++k)
                             {
-                                const float* q = pg + nb[k] * (2 * C);
-                                v[k]           = dI_of(T_c, q[c], Wn[k], Dn[k]) * q[C + c];
+                                const float* q = pg + nb[k] * C;
+                                v[k]           = dI_of(T_c, q[c], Wn[k], Dn[k]) * q[goff + c];
                             }
                             float a0 = -v[0], a1 = v[1], b0 = -v[2], b1 = v[3];
                             dR_dpx += 0.5f * (a0 + a1);
@@ -855,10 +864,10 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
     #pragma unroll
                         for (int k = 0; k < 4; ++k)
                         {
-                            const float* q = pg + nb[k] * (2 * C);
+                            const float* q = pg + nb[k] * C;
                             float In[CMAX], Gn[CMAX];
                             load_channels<CT ? CT : 4>(q, In);
-                            load_channels<CT ? CT : 4>(q + C, Gn);
+                            load_channels<CT ? CT : 4>(q + goff, Gn);
     #pragma unroll
                             for (int c = 0; c < CMAX; ++c) v[k][c] = dI_of(T[c], In[c], Wn[k], Dn[k]) * Gn[c];
                         }

@@ -135,6 +135,13 @@ __device__ __forceinline__ uint32_t ws_pixel(const Levels& lv, int l, int b, uin
     return (uint32_t)lv.pix_prefix[l] * (uint32_t)lv.B + (uint32_t)b * (uint32_t)(lv.l[l].w * lv.l[l].h) + p;
 }
 
+// Backward workspace: the resolved image and the upstream gradient in pixel-major order as two arrays [pixel][C], the
+// image first; this is where the gradient array starts (in floats).
+__device__ __forceinline__ size_t gradient_array_offset(const Levels& lv, int C)
+{
+    return (size_t)lv.pix_prefix[lv.num] * (size_t)lv.B * (size_t)C;
+}
+
 // Streamed data (read or written once per kernel) goes past the caches with the nontemporal hint, so that the lines
 // the gathers of the same kernel reuse stay resident.
 typedef float v4f __attribute__((ext_vector_type(4)));

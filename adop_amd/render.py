@@ -390,8 +390,10 @@ def EnvironmentMapSample(info, fb_struct=None, add_to_out=True, want_uv=False, w
     return uv, ev
 
 
-def EnvironmentMapSampleBackward(info, grad_out, fb_struct=None):
-    """Gradient of the fused sample-and-add w.r.t. the environment texture."""
+def EnvironmentMapSampleBackward(info, grad_out, fb_struct=None, uv=None):
+    """Gradient of the fused sample-and-add w.r.t. the environment texture.  ``uv``: the per-level texture coordinates
+    ``EnvironmentMapSample(..., want_uv=True)`` returned for the same views (the kernel then reads them instead of
+    computing every pixel's ray again)."""
     cache = info.cache
     scene = info.scene
     env = scene.environment_map
@@ -401,8 +403,9 @@ def EnvironmentMapSampleBackward(info, grad_out, fb_struct=None):
     g_arr = (C.c_void_p * L)(*[g.data_ptr() for g in grad_out])
     g_env = torch.empty_like(env)
     s = scene.struct()
+    uv_arr = None if uv is None else (C.c_void_p * L)(*[t.data_ptr() for t in uv[:L]])
     rc = cache.lib.adop_env_sample_backward(C.byref(s), cache.views_array(), cache.num_batches, int(env.shape[1]),
-                                            int(env.shape[2]), C.byref(fb), g_arr, C.c_void_p(g_env.data_ptr()),
+                                            int(env.shape[2]), C.byref(fb), g_arr, uv_arr, C.c_void_p(g_env.data_ptr()),
                                             _stream_ptr())
     _check(rc, cache.lib)
     return g_env

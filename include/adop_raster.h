@@ -205,11 +205,15 @@ adop_status adop_env_sample(const adop_scene* scene, const adop_view* views, int
                             const float* env_texture, int32_t env_h, int32_t env_w, const adop_forward_buffers* buffers,
                             float* const* uv_levels, float* const* env_levels, int32_t add_to_out, void* hip_stream);
 
-/* Gradient of adop_env_sample w.r.t. env_texture: grad_env [C,eh,ew] += sum over pixels of
- * (1-mask) * grad_out * bilinear weights (torch autograd of grid_sample in the reference). */
+/* Gradient of adop_env_sample w.r.t. env_texture: grad_env [C,eh,ew] = sum over pixels of
+ * (1-mask) * grad_out * bilinear weights (torch autograd of grid_sample in the reference; grad_env is cleared first).
+ * uv_levels: NULL, or per level the uv_l [B,h_l,w_l,2] that adop_env_sample wrote for these views (the reference's
+ * autograd keeps the sampling grid the same way): the kernel then reads the texture coordinates instead of computing
+ * each pixel's ray again. */
 adop_status adop_env_sample_backward(const adop_scene* scene, const adop_view* views, int32_t num_views,
                                      int32_t env_h, int32_t env_w, const adop_forward_buffers* buffers,
-                                     const float* const* grad_out_levels, float* grad_env, void* hip_stream);
+                                     const float* const* grad_out_levels, const float* const* uv_levels,
+                                     float* grad_env, void* hip_stream);
 
 /* Replaces ApplyTangentToPose / ApplyTangent (PointRenderer.cu:1646-1665): pose = se3_exp(tangent) * pose,
  * tangent = 0; f64. tangent [F,6], poses_se3 [F,8]. */

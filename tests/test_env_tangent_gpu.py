@@ -59,7 +59,7 @@ def test_env_backward_matches_autograd_of_grid_sample():
     scene, info, ctx, images, masks = run_hip_forward(hs)
     uv, env = render.EnvironmentMapSample(info, add_to_out=False, want_uv=True, want_env=False)
     gout = [torch.from_numpy(g).cuda() for g in scenes.upstream_grads(hs, 9)]
-    g_env = render.EnvironmentMapSampleBackward(info, gout)
+    g_env = render.EnvironmentMapSampleBackward(info, gout, uv=uv)
     torch.cuda.synchronize()
     tex = torch.from_numpy(hs.env_texture).double().requires_grad_(True)
     loss = 0
@@ -113,6 +113,7 @@ def test_env_on_ocam_views(oracle_mod):
     assert empty > 1000  # the scene leaves pixels for the environment map
     gout = [torch.from_numpy(g).cuda() for g in scenes.upstream_grads(hs, 9)]
     g_env = render.EnvironmentMapSampleBackward(info, gout)
+    g_env_uv = render.EnvironmentMapSampleBackward(info, gout, uv=uv)  # the coordinates kept from the forward call
     torch.cuda.synchronize()
     tex = torch.from_numpy(hs.env_texture).double().requires_grad_(True)
     loss = 0
@@ -122,6 +123,9 @@ def test_env_on_ocam_views(oracle_mod):
         loss = loss + (s * (1 - masks[l].cpu().double()) * gout[l].cpu().double()).sum()
     loss.backward()
     assert_norm_close(g_env.cpu().numpy(), tex.grad.numpy(), 2e-5, "grad env texture (OCam)")
+    assert_norm_close(g_env_uv.cpu().numpy(), tex.grad.numpy(), 2e-5, "grad env texture (OCam, uv from the forward call)")
+    # the sums are integer sums per tile: the same inputs give the same bits, and the kept coordinates are the inputs
+    assert_norm_close(g_env_uv.cpu().numpy(), g_env.cpu().numpy(), 1e-6, "grad env texture: kept uv vs computed uv")
 
 
 def test_env_rejects_unknown_model_and_bad_rows():

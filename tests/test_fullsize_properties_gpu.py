@@ -169,3 +169,63 @@ def test_backward_sums(full):
     g_tex2 = render.BlendPointCloudBackward(ctx, info, [3.0 * x for x in gout])[0]
     torch.cuda.synchronize()
     assert float((g_tex2 - 3.0 * g_tex).abs().max()) <= 1e-5 * float(g_tex.abs().max()) * 3
+
+
+def test_environment_map_on_the_ocam_views_at_full_size(full_scene):
+    """Configuration 5 as written: the spherical environment map sampled at the empty pixels of the 8 OCam views
+    (2200 x 1500, 4 levels: 35 M pixels) and its gradient.  Properties that hold whatever the scene: the texture
+    coordinates are finite and inside [-1, 1] and equal the checker's on two sampled windows of 64 x 64 pixels; the composition
+    changes empty pixels only and is linear in the texture; the texture gradient is the adjoint of the sampling
+    (<g_env, dT> = <grad_out, (1 - mask) * sample(dT)>), equal with the coordinates kept from the forward call, and
+    bit-identical from run to run (its sums are integer sums per tile, flushed with one float atomic per texel)."""
+    import torch
+    from adop_amd import render
+
+    if full_scene.name != "config5":
+        pytest.skip("the environment map belongs to configuration 5")
+    import oracle
+
+    hs = full_scene
+    announce("config5 full size: environment map on 8 OCam views of 2200x1500, forward and texture gradient")
+    scene, info, ctx, images, masks = run_hip_forward(hs, collect_stats=False, forward_path=2)
+    before = [im.clone() for im in images]
+    uv, env = render.EnvironmentMapSample(info, add_to_out=True, want_uv=True, want_env=True)
+    torch.cuda.synchronize()
+    L = hs.num_layers
+    for l in range(L):
+        assert bool(torch.isfinite(uv[l]).all()) and float(uv[l].abs().max()) <= 1.0
+        m = masks[l]
+        want = before[l] + (1 - m) * env[l]
+        assert float((images[l] - want).abs().max()) <= 1e-6
+        assert bool((images[l] == before[l])[(m == 1).expand_as(images[l])].all())  # rendered pixels untouched
+    # a sample of pixels against the checker: 64 x 64 windows of view 3 at levels 0 and 2
+    for l, (y0, x0) in ((0, (700, 1000)), (2, (100, 200))):
+        want = oracle.env_uv(hs, 3, l)[y0:y0 + 64, x0:x0 + 64]
+        got = uv[l][3, y0:y0 + 64, x0:x0 + 64].cpu().numpy()
+        assert np.abs(got - want).max() <= 1e-6, l
+    # linearity in the texture: sample(2 T) = 2 sample(T)
+    tex = scene.environment_map
+    scene.environment_map = tex * 2
+    _, env2 = render.EnvironmentMapSample(info, add_to_out=False, want_uv=False, want_env=True)
+    scene.environment_map = tex
+    for l in range(L):
+        assert float((env2[l] - 2 * env[l]).abs().max()) <= 1e-6
+    # the gradient: adjoint identity against the forward sampling of a random texture perturbation
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    gout = [torch.randn(im.shape, device="cuda", generator=gen) for im in images]
+    g_env = render.EnvironmentMapSampleBackward(info, gout)
+    g_env_uv = render.EnvironmentMapSampleBackward(info, gout, uv=uv)
+    g_env_again = render.EnvironmentMapSampleBackward(info, gout)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(g_env).all())
+    dT = torch.randn(tex.shape, device="cuda", generator=gen)
+    scene.environment_map = dT
+    _, env_d = render.EnvironmentMapSample(info, add_to_out=False, want_uv=False, want_env=True)
+    scene.environment_map = tex
+    lhs = float((g_env.double() * dT.double()).sum())
+    rhs = sum(float((gout[l].double() * (1 - masks[l].double()) * env_d[l].double()).sum()) for l in range(L))
+    scale = sum(float((gout[l].double() * (1 - masks[l].double()) * env_d[l].double()).abs().sum()) for l in range(L))
+    assert abs(lhs - rhs) <= 2e-6 * scale, (lhs, rhs, scale)
+    assert float((g_env_uv - g_env).abs().max()) <= 1e-6 * float(g_env.abs().max())
+    # run to run: the only float additions are the per-tile flushes, whose order across tiles may change
+    assert float((g_env_again - g_env).abs().max()) <= 1e-6 * float(g_env.abs().max())
