@@ -147,14 +147,15 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(PPT > 2 
                 else if (valid)
                 {
                     const bool dropped = ok && pc.dropout && __builtin_nontemporal_load(pc.dropout + (size_t)b * pc.n + i) == 1.f;
-                    const float4 far   = ok ? make_float4(ip.x, ip.y, signed_depth(z, dropped), crop_radius(vc, z, P[k].w, lv.l[0].w))
+                    const float4 far   = ok ? make_float4(ip.x, ip.y, signed_depth(z, dropped), rp.drop_by_radius ? crop_radius(vc, z, P[k].w, lv.l[0].w) : 0.f)
                                             : make_float4(0, 0, 0, 0);
                     nt_store4(pc.cache + (size_t)b * pc.n + i, lane == 0 ? mark : far);
                     __builtin_nontemporal_store(0u, bin.info + (size_t)b * pc.n + i);
                 }
                 continue;
             }
-            if (ok) radius_pixels = crop_radius(vc, z, P[k].w, lv.l[0].w);
+            // (the LOD radius costs a correctly rounded division: computed only when the LOD test reads it)
+            if (ok && rp.drop_by_radius) radius_pixels = crop_radius(vc, z, P[k].w, lv.l[0].w);
             // (the sign of the depth carries the dropout flag: the readers need no second array; only the projected
             // points' flags are read)
             const bool dropped = ok && pc.dropout && __builtin_nontemporal_load(pc.dropout + (size_t)b * pc.n + i) == 1.f;  // :314-315
@@ -300,12 +301,13 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels
     }
 }
 
-// Exclusive prefix sum of the tile counts (one workgroup): offset[0..T].  Chunks of 8192 tiles; the eight counts of a
-// thread are consecutive (two 16-byte loads, one memory round trip per chunk).
+// Exclusive prefix sum of the tile counts (one workgroup): offset[0..T].  Chunks of 1024 * PER tiles; the PER counts of
+// a thread are consecutive (16-byte loads, one memory round trip per chunk).  PER = 8 covers one view of 1920 x 1080 in
+// one chunk; batches of views take PER = 32 (a chunk costs three barriers and a round trip whatever its size).
+template <int PER>
 __global__ __launch_bounds__(1024) void tile_scan_kernel(const uint32_t* __restrict__ count, uint32_t* __restrict__ offset,
                                                          int T)
 {
-    constexpr int PER = 8;
     __shared__ uint32_t s_wave[16];
     __shared__ uint32_t s_carry;
     const int tid = threadIdx.x;
@@ -315,8 +317,20 @@ __global__ __launch_bounds__(1024) void tile_scan_kernel(const uint32_t* __restr
     {
         const int t0 = c0 + tid * PER;
         uint32_t v[PER];
+        if (t0 + PER <= T)  // (count is 256-byte aligned and t0 a multiple of PER)
+        {
 #pragma unroll
-        for (int k = 0; k < PER; ++k) v[k] = t0 + k < T ? count[t0 + k] : 0u;
+            for (int k = 0; k < PER; k += 4)
+            {
+                const uint4 q = *(const uint4*)(count + t0 + k);
+                v[k] = q.x, v[k + 1] = q.y, v[k + 2] = q.z, v[k + 3] = q.w;
+            }
+        }
+        else
+        {
+#pragma unroll
+            for (int k = 0; k < PER; ++k) v[k] = t0 + k < T ? count[t0 + k] : 0u;
+        }
         uint32_t sum = 0;
 #pragma unroll
         for (int k = 0; k < PER; ++k) sum += v[k];
@@ -380,7 +394,10 @@ void launch_bin(int pass, const CloudArg& pc, const ViewConst* views, const Leve
 
 void launch_tile_scan(const BinArg& bin, int num_tiles, hipStream_t st)
 {
-    hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, st, bin.count, bin.offset, num_tiles);
+    if (num_tiles <= 8192)
+        hipLaunchKernelGGL(tile_scan_kernel<8>, dim3(1), dim3(1024), 0, st, bin.count, bin.offset, num_tiles);
+    else
+        hipLaunchKernelGGL(tile_scan_kernel<32>, dim3(1), dim3(1024), 0, st, bin.count, bin.offset, num_tiles);
 }
 
 }  // namespace adop

@@ -291,7 +291,7 @@ __device__ __forceinline__ void ocam_core(V3 p, const float* aff, const float* p
 // environment map asserts the pinhole model, EnvironmentMap.cu:129): undo the affine map, solve poly(theta) = rho with
 // kOcamNewtonSteps Newton steps from the axis (theta = -pi/2), theta kept in [-pi/2, pi/2]; the ray is
 // (cos(theta) * (uu,vv)/rho, -sin(theta)), so that theta = atan(-z / |xy|) as in the forward direction.
-constexpr int kOcamNewtonSteps = 8;
+constexpr int kOcamNewtonSteps = 5;
 __device__ __forceinline__ V3 ocam_unproject(const float* aff, const float* poly, int npoly, V2 ip)
 {
     float c = aff[0], d = aff[1], e = aff[2], cx = aff[3], cy = aff[4];

@@ -125,7 +125,7 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
             if (ok) ip = k_apply(vc.crop, frame_p);
             // a crop sees a small part of the cloud: most runs of 64 points are nowhere near it and skip the levels
             const bool near_image = __ballot(ok && !outside_every_level(box, ip)) != 0;  // wavefront-uniform
-            if (ok && (near_image || !sparse)) radius_pixels = crop_radius(vc, z, P[k].w, lv.l[0].w);
+            if (ok && rp.drop_by_radius && (near_image || !sparse)) radius_pixels = crop_radius(vc, z, P[k].w, lv.l[0].w);
             zz[k]      = z;
             inmask[k]  = 0;
             rec[k]     = make_float4(ip.x, ip.y, 0.f, radius_pixels);

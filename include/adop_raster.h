@@ -134,10 +134,10 @@ typedef struct adop_forward_buffers
      * that both sides of a parity test see the same mask. */
     const float* dropout_points;
     /* Optional [B,N,4] f32 (no counterpart in the reference, which projects every point again in each of its
-     * three kernels): per view and point the level-0 image point (x,y), the depth (0 = culled; negative = the point is
-     * dropped for that image, dropout_points) and the LOD
-     * radius in pixels.  adop_forward writes it; adop_backward reads it instead of projecting when the same
-     * buffer is passed back in `fwd`.  NULL: adop_forward keeps the records in the workspace, adop_backward
+     * three kernels): per view and point the level-0 image point (x,y), the depth (0 = culled; sign bit set = the
+     * point is dropped for that image, dropout_points) and the LOD radius in pixels (0 when
+     * drop_out_points_by_radius is off: nothing reads it then).  adop_forward writes it; adop_backward reads it
+     * instead of projecting when the same buffer is passed back in `fwd`, with the same render parameters.  NULL: adop_forward keeps the records in the workspace, adop_backward
      * projects again.  When none of the points i..i+63 (i a multiple of 64) lands in the image of a view at any
      * level, record i of that view holds the bits 0x7FC0C011 in x (and depth 0): adop_backward then skips the run.
      * In a call with several views the other 63 records of such a run are not written (for the first 64 views, and
@@ -196,7 +196,7 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
  * Pinhole views: the pixel's ray as in BuildSphericalUV (EnvironmentMap.cu:82-90: unproject2 through crop and K,
  * undistortNormalizedPointSimple).  OCam views (the reference asserts pinhole, EnvironmentMap.cu:129; this is an
  * extension): the ray comes from inverting the world2cam polynomial of the intrinsics row itself (no cam2world
- * polynomial is passed): the affine map (c,d,e,cx,cy) is undone, poly(theta) = rho is solved by 8 Newton steps from
+ * polynomial is passed): the affine map (c,d,e,cx,cy) is undone, poly(theta) = rho is solved by 5 Newton steps from
  * the optical axis (theta = -pi/2) with theta kept in [-pi/2, pi/2], and the camera-space ray is
  * (cos(theta) * (uu,vv)/rho, -sin(theta)), i.e. the inverse of ProjectOCam (PointRendererHelper.h:85-106) wherever the
  * polynomial is monotonic; pixels the polynomial does not reach take the ray of the nearest end of that range.

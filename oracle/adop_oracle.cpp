@@ -473,7 +473,9 @@ void project_ocam(V3 p, V3 n, const Pose& V, const float* aff, const float* poly
 // PointRendererHelper.h:85-106 is the forward direction only); DEFINED here: undo the affine map, then solve
 // poly(theta) = rho with kOcamNewtonSteps Newton steps from the axis (theta = -pi/2), theta kept in [-pi/2, pi/2];
 // the ray is (cos(theta) * (uu,vv)/rho, -sin(theta)), so that theta = atan(-z / |xy|) as in the forward direction.
-const int kOcamNewtonSteps = 8;
+// (Five steps: on fisheye polynomials with up to 5 % of higher-order terms the fourth step no longer changes the
+// round trip project(unproject(pixel)) - pixel, which stays below 4e-4 pixels; tests/test_oracle_math.py.)
+const int kOcamNewtonSteps = 5;
 V3 ocam_unproject(const float* aff, const float* poly, int npoly, V2 ip)
 {
     float c = aff[0], d = aff[1], e = aff[2], cx = aff[3], cy = aff[4];

@@ -378,9 +378,11 @@ def test_ocam_unproject_inverts_the_projection(oracle_mod):
     """project(unproject(pixel)) = pixel for a 5th-order polynomial with an affine part, over the image circle; and
     unproject(project(p)) is the direction of p."""
     g = scenes.rng(32)
-    for seed in range(4):
+    for seed in range(6):
         intr = scenes.ocam_row(1200, 900, seed=seed)
         intr[:3] = [1.0 + 0.02 * seed, 0.01 * seed, -0.015 * seed]
+        if seed >= 4:
+            intr[7:] *= 6.0  # six times the higher-order terms: the fixed number of Newton steps still converges
         r0 = oracle_mod.ocam_core(intr, (1e-6, 0, 1.0))  # radius the polynomial gives next to the axis
         r_min = abs(np.hypot(r0[0] - intr[3], r0[1] - intr[4])) + 2.0
         for _ in range(300):
