@@ -369,11 +369,36 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(CT != 0 
         }
         else
             masks = mask;
-        // queue push: rank inside the workgroup, one returning atomic per workgroup on the sub-queue counter
         bool has               = masks != 0;
-        if (MULTI && !__syncthreads_or(has)) continue;  // nothing in the whole workgroup (masks is 0)
         unsigned long long bal = __ballot(has);
         uint32_t rank_in_wave  = (uint32_t)__popcll(bal & ((1ull << lane) - 1ull));
+        if (MULTI)
+        {
+            // Several views: every wavefront pushes for itself (one returning atomic per wavefront with items, onto the
+            // sub-queue of its workgroup), so that the loop over the views has no barrier in it: most views do not see
+            // the run at all.
+            if (bal)
+            {
+                const uint32_t q = blockIdx.x % kNumQueues;
+                uint32_t base    = 0;
+                if (lane == 0) base = atomicAdd(&q_counts[(size_t)set * kNumQueues + q], (uint32_t)__popcll(bal));
+                base = (uint32_t)__shfl((int)base, 0, 64);
+                if (has)
+                {
+                    const size_t at = ((size_t)set * kNumQueues + q) * q_cap + base + rank_in_wave;
+                    if (views_per_item > 1)
+                    {
+                        q_items[2 * at]     = (unsigned long long)(uint32_t)i;
+                        q_items[2 * at + 1] = masks;
+                    }
+                    else
+                        q_items[at] = (unsigned long long)(uint32_t)i | (masks << 32);
+                }
+            }
+            masks = 0;
+            continue;
+        }
+        // one view: rank inside the workgroup, one returning atomic per workgroup on the sub-queue counter
         if (lane == 0) s_wave_count[wave] = (uint32_t)__popcll(bal);
         __syncthreads();
         uint32_t before = 0, total = 0;
