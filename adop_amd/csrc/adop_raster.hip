@@ -135,7 +135,6 @@ constexpr int kTileLevels = 2;  // levels the tile path renders in LDS (a point 
 constexpr int kTilePathMinPoints = 1 << 16;
 constexpr int kTilePathMaxPointsPerPixel = 16;
 constexpr int kWindowCloudShare = 16;  // a crop window is taken to see 1/16 of the cloud
-constexpr int kGroupedViewsMaxPoints = 4000000;  // backward: spatial gradients of a group of views in one launch
 
 size_t max_tiles(int B, int w0, int h0)
 {
@@ -639,14 +638,12 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     q.counts = (uint32_t*)((char*)workspace + wl.q_counts);
     q.items  = (unsigned long long*)((char*)workspace + wl.q_items);
     q.cap    = wl.q_cap;
-    // Several views: one spatial-gradient launch per group of views (items carry the level masks of the whole group;
-    // a group's 16-byte items fit where the 8-byte items of its views would be) while the launches per view would be
-    // small; a large cloud fills a launch per view, and the compacted per-view queues then beat the group kernel, whose
-    // wavefronts walk the views in step.  ADOP_GHOST_GROUPS (read at every call): 0 = never, 2 = always.
-    const char* env_groups = getenv("ADOP_GHOST_GROUPS");
-    const int groups_mode  = env_groups ? atoi(env_groups) : 1;
-    const bool grouped     = num_views > 1 && (groups_mode == 2 || (groups_mode == 1 && N <= kGroupedViewsMaxPoints));
-    q.views_per_item       = grouped ? ghost_views_per_item() : 1;
+    // Several views (up to kConcurrentViews): the spatial gradients of all views run side by side in one launch; the
+    // descriptor pass tells every item whether other views add to the same point's gradient row (those rows are summed
+    // with float atomics, all others written by their one owner).  More views, or ADOP_GHOST_CONCURRENT=0 (read at
+    // every call): one launch per view, each adding to the point gradients in the order of the views.
+    const char* env_conc = getenv("ADOP_GHOST_CONCURRENT");
+    q.concurrent = num_views > 1 && num_views <= kConcurrentViews && !(env_conc && atoi(env_conc) == 0) ? 1 : 0;
     if (N < 1)
     {
         // nothing writes the partial rows: clear them for finalize
@@ -659,15 +656,11 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
         StageScope sc("RenderBackward/descriptor", stream);
         launch_backward_tex(pc, dviews, lv, rp, half, ig, dw, grads, scene->index_is_identity, q, stats, stream);
     }
-    if (q.views_per_item > 1)
+    if (q.concurrent)
     {
-        for (int first = 0, group = 0; first < num_views; first += q.views_per_item, ++group)
-        {
-            StageScope sc("RenderBackward/spatial", stream);
-            const int count = num_views - first < q.views_per_item ? num_views - first : q.views_per_item;
-            launch_backward_ghost_multi(pc, dviews, lv, rp, half, ig, grads, want_pose, want_intr,
-                                        scene->index_is_identity, group, first, count, q, pt_blocks, pt_partial, stream);
-        }
+        StageScope sc("RenderBackward/spatial", stream);
+        launch_backward_ghost(pc, dviews, lv, rp, half, ig, grads, want_pose, want_intr, scene->index_is_identity, -1, q,
+                              pt_blocks, pt_partial, stream);
     }
     else
         for (int b = 0; b < num_views; ++b)
@@ -1071,6 +1064,6 @@ const char* adop_version(void)
 {
     // "kernels N" names the state of the kernels' memory behaviour: it goes up whenever a change moves a kernel's bytes,
     // so that traffic figures measured for one state (rocprofv3 counters) are not quoted for another.
-    return "adop_raster 0.2 (gfx950) kernels 2";
+    return "adop_raster 0.2 (gfx950) kernels 3";
 }
 }  // extern "C"

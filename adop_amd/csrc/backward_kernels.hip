@@ -13,6 +13,8 @@
 
 namespace adop
 {
+// Work-queue items of one view: point id (32 bits) | level mask (5 bits) | kItemSharedBit.
+constexpr int kItemSharedBit = 37;  // set when the point has items in other views of the call too
 
 // CombineAndFillBackward (:851-900) fused with the I/G interleave.  One thread per pixel of every level/image.
 // Background gradient: per-thread fp32 partial over a handful of pixels, wave/block reduction in f64, one f64
@@ -166,7 +168,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(CT != 0 
                                                                float* __restrict__ gpoints_count, int identity_index,
                                                                uint32_t* __restrict__ q_counts,
                                                                unsigned long long* __restrict__ q_items,
-                                                               uint32_t q_cap, int views_per_item, adop_stats* stats)
+                                                               uint32_t q_cap, int concurrent, adop_stats* stats)
 {
     constexpr int CMAX = CT ? CT : 1;  // register arrays exist only for compile-time channel counts
     __shared__ uint32_t s_wave_count[kBlock / 64];
@@ -190,11 +192,14 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(CT != 0 
     for (int c = 0; c < CMAX; ++c) gt[c] = 0.f;
     bool gt_live = false;
 
-    // the views one after the other: view b appends to work queue b (MULTI = false: one view, no loop); with
-    // views_per_item = kGhostViews the level masks of that many consecutive views (5 bits each) travel in one 16-byte
-    // item and a queue stands for a group of views
+    // the views one after the other: view b appends to work queue b (MULTI = false: one view, no loop)
     const int num_views = MULTI ? lv.B : 1;
     unsigned long long masks = 0;
+    // `concurrent` (at most kConcurrentViews views): the level masks of all views are kept (5 bits each) and the items
+    // are pushed after the loop, when the thread knows whether its point has items in several views; the
+    // spatial-gradient kernel then runs all views in one launch, see backward_ghost_kernel
+    const bool deferred = MULTI && concurrent != 0;
+    unsigned long long kept[2] = {0ull, 0ull};
     // Several views (crops see a small part of the cloud): the first record of the wavefront's run of 64 points says
     // whether the forward pass culled the whole run for a view (kRunCulledBits); lane b asks for view b, all at once,
     // and the records of the runs culled are never read.
@@ -353,22 +358,19 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(CT != 0 
         }
         // Point gradients of the first view: points without a spatial gradient are cleared here (Build(info,false),
         // :922-949), the others are written by backward_ghost_kernel; no separate zero-fill of the two buffers.
+        if (deferred)
+        {
+            kept[b / 12] |= (unsigned long long)mask << (5 * (b % 12));
+            continue;
+        }
         if (b == 0 && gpoints && valid && mask == 0)
         {
             nt_store4((float4*)gpoints + i, make_float4(0, 0, 0, 0));
             __builtin_nontemporal_store(0.f, gpoints_count + i);
         }
 
-        int set = b;  // queue set the item goes to
-        if (MULTI && views_per_item > 1)
-        {
-            const int slot = b % views_per_item;
-            masks |= (unsigned long long)mask << (5 * slot);
-            if (slot != views_per_item - 1 && b != num_views - 1) continue;  // workgroup-uniform
-            set = b / views_per_item;
-        }
-        else
-            masks = mask;
+        const int set = b;  // queue set the item goes to
+        masks         = mask;
         bool has               = masks != 0;
         unsigned long long bal = __ballot(has);
         uint32_t rank_in_wave  = (uint32_t)__popcll(bal & ((1ull << lane) - 1ull));
@@ -386,13 +388,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(CT != 0 
                 if (has)
                 {
                     const size_t at = ((size_t)set * kNumQueues + q) * q_cap + base + rank_in_wave;
-                    if (views_per_item > 1)
-                    {
-                        q_items[2 * at]     = (unsigned long long)(uint32_t)i;
-                        q_items[2 * at + 1] = masks;
-                    }
-                    else
-                        q_items[at] = (unsigned long long)(uint32_t)i | (masks << 32);
+                    q_items[at]     = (unsigned long long)(uint32_t)i | (masks << 32);
                 }
             }
             masks = 0;
@@ -415,17 +411,38 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(CT != 0 
         if (has)
         {
             const size_t at = ((size_t)set * kNumQueues + q) * q_cap + s_base + before + rank_in_wave;
-            if (MULTI && views_per_item > 1)
-            {
-                q_items[2 * at]     = (unsigned long long)(uint32_t)i;
-                q_items[2 * at + 1] = masks;
-            }
-            else
-                q_items[at] = (unsigned long long)(uint32_t)i | (masks << 32);
+            q_items[at]     = (unsigned long long)(uint32_t)i | (masks << 32);
         }
         masks = 0;
         __syncthreads();  // s_wave_count and s_base are reused by the next view
     }  // views
+
+    if (deferred)
+    {
+        int nitems = 0;
+        for (int b = 0; b < num_views; ++b) nitems += (kept[b / 12] >> (5 * (b % 12)) & 31ull) != 0;
+        // A point with one item gets its gradient row from that item's thread; a row nobody writes, or one that several
+        // views add to with atomics, starts at zero (Build(info,false), :922-949).
+        if (gpoints && valid && nitems != 1)
+        {
+            nt_store4((float4*)gpoints + i, make_float4(0, 0, 0, 0));
+            __builtin_nontemporal_store(0.f, gpoints_count + i);
+        }
+        const unsigned long long shared = nitems > 1 ? 1ull << kItemSharedBit : 0ull;
+        for (int b = 0; b < num_views; ++b)
+        {
+            const unsigned long long m = kept[b / 12] >> (5 * (b % 12)) & 31ull;
+            const unsigned long long bal = __ballot(m != 0);
+            if (!bal) continue;  // wavefront-uniform
+            const uint32_t q = blockIdx.x % kNumQueues;
+            uint32_t base    = 0;
+            if (lane == 0) base = atomicAdd(&q_counts[(size_t)b * kNumQueues + q], (uint32_t)__popcll(bal));
+            base = (uint32_t)__shfl((int)base, 0, 64);
+            if (m != 0)
+                q_items[((size_t)b * kNumQueues + q) * q_cap + base + (uint32_t)__popcll(bal & ((1ull << lane) - 1ull))] =
+                    (unsigned long long)(uint32_t)i | (m << 32) | shared;
+        }
+    }
 
     if (CT != 0)
     {
@@ -467,7 +484,15 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
     constexpr int CMAX = CT ? CT : 1;
     __shared__ float s_red[kAcc * kBlock];
     __shared__ uint32_t s_prefix[kNumQueues + 1];
-    const int b         = view_b;
+    // view_b < 0: all views in one launch, view = blockIdx.y (the queues of the views follow each other); an item's
+    // kItemSharedBit then says whether other views add to the same point's gradient row
+    const bool concurrent = view_b < 0;
+    const int b           = concurrent ? (int)blockIdx.y : view_b;
+    if (concurrent)
+    {
+        q_counts += (size_t)b * kNumQueues;
+        q_items += (size_t)b * kNumQueues * q_cap;
+    }
     const ViewConst& vc = views[b];
     const float accept  = rp.depth_accept + 1;
     const int C         = CT ? CT : lv.C;
@@ -528,7 +553,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
         // (the item and the point record are read once by this kernel: past the caches, which hold the [I|G] lines)
         unsigned long long item = __builtin_nontemporal_load(q_items + (size_t)lo * q_cap + (t - s_prefix[lo]));
         const int i             = (int)(uint32_t)item;
-        const uint32_t mask     = (uint32_t)(item >> 32);
+        const uint32_t mask     = (uint32_t)(item >> 32) & 31u;
+        const bool shared       = (item >> kItemSharedBit & 1ull) != 0;
 
         float4 P = nt_load4(pc.position + i);
         V3 pos   = {P.x, P.y, P.z};
@@ -550,7 +576,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
         // view, level after level); this thread owns point i for this view
         float gp[3] = {0, 0, 0};
         float gp_n  = 0;
-        if (gpoints && !first_view)
+        if (gpoints && !first_view && !concurrent)
         {
             const float* g = gpoints + 4 * (size_t)i;
             gp[0]          = g[0];
@@ -683,15 +709,28 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
         if (gpoints)
         {
             float* g = gpoints + 4 * (size_t)i;
-            if (first_view)
-                *(float4*)g = make_float4(gp[0], gp[1], gp[2], 0.f);  // nothing has cleared the row
+            if (concurrent && shared)
+            {
+                // the point has items in several views, which run side by side: the row was cleared by the descriptor
+                // pass and every view adds its part (the order of these float additions is the one thing of the
+                // gradients that is not fixed from run to run)
+                unsafeAtomicAdd(g + 0, gp[0]);
+                unsafeAtomicAdd(g + 1, gp[1]);
+                unsafeAtomicAdd(g + 2, gp[2]);
+                unsafeAtomicAdd(gpoints_count + i, gp_n);
+            }
             else
             {
-                g[0] = gp[0];
-                g[1] = gp[1];
-                g[2] = gp[2];
+                if (first_view || concurrent)
+                    *(float4*)g = make_float4(gp[0], gp[1], gp[2], 0.f);  // nothing has cleared the row
+                else
+                {
+                    g[0] = gp[0];
+                    g[1] = gp[1];
+                    g[2] = gp[2];
+                }
+                gpoints_count[i] = gp_n;
             }
-            gpoints_count[i] = gp_n;
         }
     }
 
@@ -711,288 +750,6 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
     }
 }
 
-// The same for a batch of views in one launch.  An item names a point and carries the level masks of up to
-// kGhostViews consecutive views (backward_tex_kernel, views_per_item); the thread that takes it walks the views in
-// order, so a point's gradient row is summed view after view, level after level as the reference does, in registers,
-// and written once.  The views are walked in step by the whole workgroup (the view constants stay uniform): after each
-// view the per-thread pose / intrinsics columns are summed into that view's row of s_view (f64) and cleared.  The
-// points of a wavefront are neighbours in space, so they mostly meet the same few views.
-constexpr int kGhostViews = 12;  // 5 mask bits each in a 64-bit word
-
-template <int CT, bool HALF>
-__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) void backward_ghost_multi_kernel(
-    CloudArg pc, const ViewConst* __restrict__ views, Levels lv, ParamArg rp, const float* __restrict__ ig,
-    float* __restrict__ gpoints, float* __restrict__ gpoints_count, int want_pose, int want_intr, int identity_index,
-    int first_view_index, int num_group_views, const uint32_t* __restrict__ q_counts,
-    const unsigned long long* __restrict__ q_items, uint32_t q_cap, double* __restrict__ partial)
-{
-    constexpr int CMAX = CT ? CT : 1;
-    __shared__ float s_red[kAcc * kBlock];
-    __shared__ uint32_t s_prefix[kNumQueues + 1];
-    __shared__ double s_view[kGhostViews * kAcc];
-    const float accept     = rp.depth_accept + 1;
-    const int C            = CT ? CT : lv.C;
-    const bool first_view  = first_view_index == 0;  // nothing has written the point-gradient rows yet
-    {
-        constexpr int PER = kNumQueues / kBlock;
-        static_assert(PER == 8, "two 16-byte loads per thread");
-        __shared__ uint32_t s_wave[kBlock / 64];
-        const uint4 c0 = *(const uint4*)(q_counts + threadIdx.x * PER);
-        const uint4 c1 = *(const uint4*)(q_counts + threadIdx.x * PER + 4);
-        const uint32_t v[PER] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
-        uint32_t sum = 0;
-#pragma unroll
-        for (int k = 0; k < PER; ++k) sum += v[k];
-        uint32_t inc = sum;
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1)
-        {
-            uint32_t u = __shfl_up(inc, off, 64);
-            if ((int)(threadIdx.x & 63) >= off) inc += u;
-        }
-        if ((threadIdx.x & 63) == 63) s_wave[threadIdx.x >> 6] = inc;
-        __syncthreads();
-        uint32_t run = inc - sum;
-        for (int w = 0; w < (int)(threadIdx.x >> 6); ++w) run += s_wave[w];
-#pragma unroll
-        for (int k = 0; k < PER; ++k)
-        {
-            s_prefix[threadIdx.x * PER + k] = run;
-            run += v[k];
-        }
-        if (threadIdx.x == kBlock - 1) s_prefix[kNumQueues] = run;
-        for (int k = threadIdx.x; k < kGhostViews * kAcc; k += kBlock) s_view[k] = 0;
-        __syncthreads();
-    }
-    const uint32_t total = s_prefix[kNumQueues];
-    float* acc = s_red + threadIdx.x;  // acc[k * kBlock]
-#pragma unroll
-    for (int k = 0; k < kAcc; ++k) acc[k * kBlock] = 0;
-
-    for (uint32_t t0 = blockIdx.x * kBlock; t0 < total; t0 += gridDim.x * kBlock)  // workgroup-uniform
-    {
-        const uint32_t t  = t0 + threadIdx.x;
-        const bool active = t < total;
-        int i = 0;
-        unsigned long long masks = 0;
-        float4 P = make_float4(0, 0, 0, 0);
-        V3 nrm   = {0, 0, 0};
-        int tex_index = 0;
-        float T[CMAX];
-#pragma unroll
-        for (int c = 0; c < CMAX; ++c) T[c] = 0.f;
-        float gp[3] = {0, 0, 0};
-        float gp_n  = 0;
-        if (active)
-        {
-            uint32_t lo = 0, hi = kNumQueues;
-            while (hi - lo > 1)
-            {
-                uint32_t mid = (lo + hi) >> 1;
-                if (s_prefix[mid] <= t)
-                    lo = mid;
-                else
-                    hi = mid;
-            }
-            const size_t at = (size_t)lo * q_cap + (t - s_prefix[lo]);
-            i               = (int)(uint32_t)__builtin_nontemporal_load(q_items + 2 * at);
-            masks           = __builtin_nontemporal_load(q_items + 2 * at + 1);
-            P               = nt_load4(pc.position + i);
-            if (pc.normal) nrm = unpack_normal10(__builtin_nontemporal_load(pc.normal + i));
-            tex_index = identity_index ? i : pc.index[i];
-            if (CT != 0)
-            {
-#pragma unroll
-                for (int c = 0; c < CMAX; ++c)
-                    T[c] = tex_fetch_stream<HALF>(pc.texture, (size_t)c * pc.num_texels + tex_index);
-            }
-            if (gpoints && !first_view)
-            {
-                const float* g = gpoints + 4 * (size_t)i;
-                gp[0]          = g[0];
-                gp[1]          = g[1];
-                gp[2]          = g[2];
-                gp_n           = gpoints_count[i];
-            }
-        }
-        const V3 pos = {P.x, P.y, P.z};
-        for (int v = 0; v < num_group_views; ++v)  // workgroup-uniform
-        {
-            const uint32_t mask = (uint32_t)(masks >> (5 * v)) & 31u;
-            if (!__syncthreads_or(mask != 0)) continue;
-            if (mask)
-            {
-                const int b         = first_view_index + v;
-                const ViewConst& vc = views[b];
-                V2 ip;
-                V3 view_p;
-                float z, radius_pixels;
-                project_point(vc, pc.intrinsics, pos, nrm, P.w, rp.check_normal != 0, rp.dist_cutoff, lv.l[0].w, &ip, &z,
-                              &radius_pixels, &view_p);
-            float scale = 1;
-    #pragma unroll 1
-            for (int l = 0; l < lv.num; ++l)
-            {
-                if (mask & (1u << l))
-                {
-                    const LevelArg& L = lv.l[l];
-                    int px = f2i_rn(ip.x), py = f2i_rn(ip.y);
-                    size_t hw             = (size_t)L.w * L.h;
-                    size_t p              = (size_t)py * L.w + px;
-                    const float* pg       = ig + (size_t)ws_pixel(lv, l, b, (uint32_t)p) * C;  // I of the pixel, its G at + goff
-                    const size_t goff     = gradient_array_offset(lv, C);
-                    const ptrdiff_t nb[4] = {-1, 1, -(ptrdiff_t)L.w, (ptrdiff_t)L.w};
-                    float Wn[4] = {0, 0, 0, 0}, Dn[4] = {0, 0, 0, 0};
-                    if (rp.test_backward_mode == 4)
-                    {
-                        const float* Wp = L.weight + (size_t)b * hw + p;
-                        const float* Dp = L.depth + (size_t)b * hw + p;
-    #pragma unroll
-                        for (int k = 0; k < 4; ++k)
-                        {
-                            Wn[k] = Wp[nb[k]];
-                            Dn[k] = Dp[nb[k]];
-                        }
-                    }
-                    auto dI_of = [&](float T_c, float I_x, float W_x, float D_x) -> float
-                    {
-                        if (rp.test_backward_mode == 4)
-                        {
-                            if (W_x == 0 || z * accept < D_x) return T_c - I_x;          // full override
-                            if (z > D_x * accept) return 0.f;                            // discard
-                            return (W_x / (W_x + 1) * I_x + 1 / (W_x + 1) * T_c - I_x);  // blend
-                        }
-                        return T_c - I_x;
-                    };
-                    float dR_dpx = 0, dR_dpy = 0;
-                    if (CT == 0)
-                    {
-    #pragma unroll 1
-                        for (int c = 0; c < C; ++c)
-                        {
-                            float T_c = tex_fetch<HALF>(pc.texture, (size_t)c * pc.num_texels + tex_index);
-                            float v[4];
-    #pragma unroll
-                            for (int k = 0; k < 4; ++k)
-                            {
-                                const float* q = pg + nb[k] * C;
-                                v[k]           = dI_of(T_c, q[c], Wn[k], Dn[k]) * q[goff + c];
-                            }
-                            float a0 = -v[0], a1 = v[1], b0 = -v[2], b1 = v[3];
-                            dR_dpx += 0.5f * (a0 + a1);
-                            dR_dpy += 0.5f * (b0 + b1);
-                        }
-                    }
-                    else
-                    {
-                        float v[4][CMAX];  // dI * G per neighbour and channel
-    #pragma unroll
-                        for (int k = 0; k < 4; ++k)
-                        {
-                            const float* q = pg + nb[k] * C;
-                            float In[CMAX], Gn[CMAX];
-                            load_channels<CT ? CT : 4>(q, In);
-                            load_channels<CT ? CT : 4>(q + goff, Gn);
-    #pragma unroll
-                            for (int c = 0; c < CMAX; ++c) v[k][c] = dI_of(T[c], In[c], Wn[k], Dn[k]) * Gn[c];
-                        }
-    #pragma unroll
-                        for (int c = 0; c < CMAX; ++c)
-                        {
-                            float a0 = -v[0][c], a1 = v[1][c], b0 = -v[2][c], b1 = v[3][c];
-                            dR_dpx += 0.5f * (a0 + a1);
-                            dR_dpy += 0.5f * (b0 + b1);
-                        }
-                    }
-                    V2 dR_dp       = {dR_dpx / (float)C, dR_dpy / (float)C};
-                    float crop2[5] = {vc.crop[0] * scale, vc.crop[1] * scale, vc.crop[2] * scale, vc.crop[3] * scale,
-                                      vc.crop[4] * scale};  // crop.scale(scale), :616
-                    BackwardOut bo;
-                    project_point_backward(vc, pc.intrinsics, view_p, dR_dp, crop2, rp.dist_cutoff, &bo);
-                    gp[0] += bo.g_point[0];
-                    gp[1] += bo.g_point[1];
-                    gp[2] += bo.g_point[2];
-                    gp_n += 1.f;
-                    if (want_pose)
-                    {
-    #pragma unroll
-                        for (int k = 0; k < 6; ++k) acc[k * kBlock] += bo.g_pose[k];
-                        acc[6 * kBlock] += 1.0f;
-                    }
-                    if (want_intr)
-                    {
-                        if (vc.model == 0)
-                        {
-                            float kf = rp.K_gradient_factor;
-                            bo.g_k[4] *= 0.1f;
-                            bo.g_k[4] *= 0;  // :653-654
-    #pragma unroll
-                            for (int k = 0; k < 5; ++k) acc[(8 + k) * kBlock] += kf * bo.g_k[k];
-                            float df = rp.distortion_gradient_factor;
-                            bo.g_dis[2] *= 0.25f;
-                            bo.g_dis[3] *= 0.1f;
-                            bo.g_dis[4] *= 0.1f;
-                            bo.g_dis[5] *= 0.1f;
-                            bo.g_dis[6] *= 0.1f;
-                            bo.g_dis[7] *= 0.1f;
-    #pragma unroll
-                            for (int k = 0; k < 8; ++k) acc[(13 + k) * kBlock] += df * bo.g_dis[k];
-                            acc[7 * kBlock] += 1.0f / 1024.0f;  // :680-681
-                        }
-                        else
-                        {
-    #pragma unroll
-                            for (int k = 0; k < 5; ++k) acc[(8 + k) * kBlock] += bo.g_k[k];
-                            acc[7 * kBlock] += 1.0f;  // :718
-                        }
-                    }
-                }
-                scale *= 0.5f;
-                ip.x *= 0.5f;
-                ip.y *= 0.5f;
-            }
-            }
-            if (want_pose || want_intr)
-            {
-                // the columns of this view -> its row of s_view, then cleared for the next view
-                __syncthreads();
-                const int k = threadIdx.x >> 3, part = threadIdx.x & 7;
-                double sum  = 0;
-                if (k < kAcc)
-                    for (int c = part; c < kBlock; c += 8) sum += (double)s_red[k * kBlock + c];
-                sum += __shfl_xor(sum, 1, 64);
-                sum += __shfl_xor(sum, 2, 64);
-                sum += __shfl_xor(sum, 4, 64);
-                if (k < kAcc && part == 0) s_view[v * kAcc + k] += sum;
-                __syncthreads();
-#pragma unroll
-                for (int q = 0; q < kAcc; ++q) acc[q * kBlock] = 0;
-            }
-        }
-        if (active && gpoints)
-        {
-            float* g = gpoints + 4 * (size_t)i;
-            if (first_view)
-                *(float4*)g = make_float4(gp[0], gp[1], gp[2], 0.f);  // nothing has cleared the row
-            else
-            {
-                g[0] = gp[0];
-                g[1] = gp[1];
-                g[2] = gp[2];
-            }
-            gpoints_count[i] = gp_n;
-        }
-    }
-    if (want_pose || want_intr)
-    {
-        __syncthreads();
-        for (int k = threadIdx.x; k < num_group_views * kAcc; k += kBlock)
-        {
-            const int v = k / kAcc, q = k - v * kAcc;
-            partial[((size_t)(first_view_index + v) * gridDim.x + blockIdx.x) * kPartialStride + q] = s_view[k];
-        }
-    }
-}
 
 constexpr int kFinalizeBlock = 1024;  // the reduction as a kernel of its own: one workgroup, 16 loads in flight per thread
 
@@ -1314,11 +1071,11 @@ static void launch_bwd_tex_t(const CloudArg& pc, const ViewConst* views, const L
     if (lv.B > 1)
         hipLaunchKernelGGL((backward_tex_kernel<CT, HALF, true>), dim3(grid), dim3(kBlock), 0, st, pc, views, lv, rp, ig,
                            dw, g->grad_texture, g->grad_points, g->grad_points_count, identity_index, q.counts, q.items,
-                           q.cap, q.views_per_item, stats);
+                           q.cap, q.concurrent, stats);
     else
         hipLaunchKernelGGL((backward_tex_kernel<CT, HALF, false>), dim3(grid), dim3(kBlock), 0, st, pc, views, lv, rp, ig,
                            dw, g->grad_texture, g->grad_points, g->grad_points_count, identity_index, q.counts, q.items,
-                           q.cap, 1, stats);
+                           q.cap, 0, stats);
 }
 
 template <int CT, bool HALF>
@@ -1327,22 +1084,14 @@ static void launch_bwd_ghost_t(const CloudArg& pc, const ViewConst* views, const
                                int identity_index, int b, const QueueArg& q, int ghost_blocks, double* partial,
                                hipStream_t st)
 {
-    hipLaunchKernelGGL((backward_ghost_kernel<CT, HALF>), dim3(ghost_blocks), dim3(kBlock), 0, st, pc, views, lv, rp,
-                       ig, g->grad_points, g->grad_points_count, want_pose, want_intr, identity_index, b, b == 0,
-                       q.counts + (size_t)b * kNumQueues, q.items + (size_t)b * kNumQueues * q.cap, q.cap, partial);
-}
-
-// group of views [first, first + count): queue set `group`, 16-byte items
-template <int CT, bool HALF>
-static void launch_bwd_ghost_multi_t(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp,
-                                     const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr,
-                                     int identity_index, int group, int first, int count, const QueueArg& q,
-                                     int ghost_blocks, double* partial, hipStream_t st)
-{
-    hipLaunchKernelGGL((backward_ghost_multi_kernel<CT, HALF>), dim3(ghost_blocks), dim3(kBlock), 0, st, pc, views, lv,
-                       rp, ig, g->grad_points, g->grad_points_count, want_pose, want_intr, identity_index, first, count,
-                       q.counts + (size_t)group * kNumQueues, q.items + 2 * (size_t)group * kNumQueues * q.cap, q.cap,
-                       partial);
+    if (b < 0)  // every view at once: view = blockIdx.y
+        hipLaunchKernelGGL((backward_ghost_kernel<CT, HALF>), dim3(ghost_blocks, lv.B), dim3(kBlock), 0, st, pc, views, lv,
+                           rp, ig, g->grad_points, g->grad_points_count, want_pose, want_intr, identity_index, -1, 0,
+                           q.counts, q.items, q.cap, partial);
+    else
+        hipLaunchKernelGGL((backward_ghost_kernel<CT, HALF>), dim3(ghost_blocks), dim3(kBlock), 0, st, pc, views, lv, rp,
+                           ig, g->grad_points, g->grad_points_count, want_pose, want_intr, identity_index, b, b == 0,
+                           q.counts + (size_t)b * kNumQueues, q.items + (size_t)b * kNumQueues * q.cap, q.cap, partial);
 }
 
 #define ADOP_DISPATCH_C_HALF(FN, ...)                                   \
@@ -1376,17 +1125,6 @@ void launch_backward_ghost(const CloudArg& pc, const ViewConst* views, const Lev
                          ghost_blocks, partial, st);
 }
 
-int ghost_views_per_item() { return kGhostViews; }
-
-void launch_backward_ghost_multi(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp,
-                                 bool half, const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr,
-                                 int identity_index, int group, int first, int count, const QueueArg& q,
-                                 int ghost_blocks, double* partial, hipStream_t st)
-{
-    if (pc.n < 1) return;
-    ADOP_DISPATCH_C_HALF(launch_bwd_ghost_multi_t, pc, views, lv, rp, ig, g, want_pose, want_intr, identity_index, group,
-                         first, count, q, ghost_blocks, partial, st);
-}
 #undef ADOP_DISPATCH_C_HALF
 
 void launch_finalize(const ViewConst* views, int B, int C, const double* bg_partial, int bg_blocks,

@@ -84,8 +84,9 @@ struct QueueArg
     uint32_t* counts;           // [B][kNumQueues]: one set per view
     unsigned long long* items;  // [B][kNumQueues * cap]
     uint32_t cap;
-    int views_per_item;         // 1: u64 items (point | level mask << 32), one queue set per view; more: 16-byte items
-                                // (point, level masks of that many views), one queue set per group of views
+    int concurrent;             // several views: 1 = the items of all views are pushed when the descriptor pass knows
+                                // which points several views share, and the spatial-gradient kernel runs every view
+                                // in one launch; 0 = items pushed view by view, one spatial-gradient launch per view
 };
 void launch_backward_tex(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
                          const float* ig, const float2* dw, const adop_backward_buffers* g, int identity_index,
@@ -94,11 +95,7 @@ void launch_backward_ghost(const CloudArg& pc, const ViewConst* views, const Lev
                            const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr,
                            int identity_index, int b, const QueueArg& q, int ghost_blocks, double* partial,
                            hipStream_t st);
-int ghost_views_per_item();
-void launch_backward_ghost_multi(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp,
-                                 bool half, const float* ig, const adop_backward_buffers* g, int want_pose, int want_intr,
-                                 int identity_index, int group, int first, int count, const QueueArg& q,
-                                 int ghost_blocks, double* partial, hipStream_t st);
+constexpr int kConcurrentViews = 24;  // views whose level masks a descriptor-pass thread can keep (2 x 12 x 5 bits)
 void launch_finalize(const ViewConst* views, int B, int C, const double* bg_partial, int bg_blocks,
                      const double* pt_partial, int pt_blocks, const adop_backward_buffers* g, int num_poses,
                      int num_cameras, int cols, int normalize_mode, double* scratch, double* mini, uint32_t* ticket, int n,

@@ -149,16 +149,18 @@ def test_more_views_than_one_constant_chunk(oracle_mod):
     _fwd_bwd(hs, oracle_mod)
 
 
-@pytest.mark.parametrize("groups", ["0", "2"], ids=["per_view", "grouped"])
-@pytest.mark.parametrize("batch", [2, 5, 13, 34])
-def test_spatial_gradients_per_view_and_per_group_of_views(oracle_mod, monkeypatch, groups, batch):
-    """With several views the spatial-gradient pass runs once per view (large clouds) or once per group of twelve views
-    (small ones; the library picks by the size of the cloud): both against the checker, with batch sizes on either
-    side of a group and of the 32-view chunk of constants."""
+@pytest.mark.parametrize("concurrent", ["0", "1"], ids=["per_view", "concurrent"])
+@pytest.mark.parametrize("batch", [2, 5, 13, 24, 25, 34])
+def test_spatial_gradients_per_view_and_of_all_views_at_once(oracle_mod, monkeypatch, concurrent, batch):
+    """With several views the spatial-gradient pass runs all views side by side in one launch (up to 24 views: a point
+    that several views see is summed with atomics, every other row has one owner) or once per view, in the order of
+    the views (more views, or ADOP_GHOST_CONCURRENT=0): both against the checker, with batch sizes on either side of
+    the limit and of the 32-view chunk of constants.  The views of this scene look at one small cloud, so that most
+    points are shared by several views."""
     from adop_amd import scenes
 
-    monkeypatch.setenv("ADOP_GHOST_GROUPS", groups)
-    announce(f"config2 40k pts B={batch} 96x80 L3 fwd+bwd ghost, ADOP_GHOST_GROUPS={groups}")
+    monkeypatch.setenv("ADOP_GHOST_CONCURRENT", concurrent)
+    announce(f"config2 40k pts B={batch} 96x80 L3 fwd+bwd ghost, ADOP_GHOST_CONCURRENT={concurrent}")
     hs = scenes.config2(n=40_000, w=96, h=80, levels=3, batch=batch, seed=batch)
     _fwd_bwd(hs, oracle_mod)
 
