@@ -723,6 +723,7 @@ adop_status adop_env_sample(const adop_scene* scene, const adop_view* views, int
     adop_status st = env_common(scene, views, num_views, buffers, env_h, env_w);
     if (st != ADOP_OK) return st;
     if (!env_texture) return fail(ADOP_INVALID_ARG, "env_texture missing");
+    if (add_to_out < 0 || add_to_out > 2) return fail(ADOP_INVALID_ARG, "add_to_out must be 0, 1 or 2");
     hipStream_t stream = (hipStream_t)hip_stream;
     ViewChunk chunk    = make_chunk(views, num_views);
     Levels lv = make_levels(scene, num_views, buffers, nullptr);
@@ -733,6 +734,7 @@ adop_status adop_env_sample(const adop_scene* scene, const adop_view* views, int
         ev.uv[l]  = uv_levels ? uv_levels[l] : nullptr;
         ev.env[l] = env_levels ? env_levels[l] : nullptr;
         if (add_to_out && !buffers->layers[l].out) return fail(ADOP_INVALID_ARG, "out buffer missing");
+        if (add_to_out == 2 && !ev.env[l]) return fail(ADOP_INVALID_ARG, "add_to_out = 2 writes the composed image to env_levels");
     }
     launch_env_sample(chunk, scene->poses_se3, scene->intrinsics, lv, ev, env_texture, env_h, env_w, add_to_out,
                       scene->intrinsics_cols, stream);

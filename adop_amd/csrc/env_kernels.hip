@@ -157,7 +157,20 @@ __global__ __launch_bounds__(kBlock) void env_sample_kernel(ViewChunk chunk, con
     for (int k = 0; k < l; ++k) sc /= 2;
     float bgw = 1.f;
     if (add_to_out && L.mask) bgw = 1.f - L.mask[(size_t)b * hw + p];
-    bool need = ev.uv[l] || ev.env[l] || (add_to_out && bgw != 0.f);
+    if (add_to_out && bgw == 0.f)
+    {
+        // a rendered pixel: the composition does not sample it (and its uv is not written); out of place it is a copy
+        if (add_to_out == 2)
+            for (int c = 0; c < lv.C; ++c)
+            {
+                const size_t o = ((size_t)b * lv.C + c) * hw + p;
+                ev.env[l][o]   = L.out[o];
+            }
+        else if (ev.env[l])
+            for (int c = 0; c < lv.C; ++c) ev.env[l][((size_t)b * lv.C + c) * hw + p] = 0.f;
+        return;
+    }
+    bool need = ev.uv[l] || ev.env[l] || add_to_out;
     if (!need) return;
     V2 uv = spherical_uv(vc, intrinsics, sc, e.gx, e.gy);
     if (ev.uv[l])
@@ -175,8 +188,13 @@ __global__ __launch_bounds__(kBlock) void env_sample_kernel(ViewChunk chunk, con
         if (s.y1ok) a += tc[(size_t)(s.y0 + 1) * ew + s.x0] * s.w10;
         if (s.x1ok && s.y1ok) a += tc[(size_t)(s.y0 + 1) * ew + s.x0 + 1] * s.w11;
         size_t o = ((size_t)b * lv.C + c) * hw + p;
-        if (ev.env[l]) ev.env[l][o] = a;
-        if (add_to_out) L.out[o] = L.out[o] + bgw * a;
+        if (add_to_out == 2)
+            ev.env[l][o] = L.out[o] + bgw * a;  // the composed image, out_l itself stays as the rasterizer left it
+        else
+        {
+            if (ev.env[l]) ev.env[l][o] = a;
+            if (add_to_out) L.out[o] = L.out[o] + bgw * a;
+        }
     }
 }
 

@@ -369,7 +369,10 @@ def ApplyTangentToPose(tangent, pose):
 
 def EnvironmentMapSample(info, fb_struct=None, add_to_out=True, want_uv=False, want_env=False):
     """EnvironmentMapImpl::Sample (EnvironmentMap.cu:107-157) fused with ``images += (1-mask)*env``
-    (RenderModule.cpp:121-125).  Operates on the cache's current forward outputs."""
+    (RenderModule.cpp:121-125).  Operates on the cache's current forward outputs.  ``add_to_out``: False / 0 = sample
+    only, True / 1 = add in place, 2 = the second return value holds the composed images and the rasterizer's outputs
+    stay untouched (what the backward pass should see, as in the reference)."""
+    want_env = want_env or add_to_out == 2
     cache = info.cache
     scene = info.scene
     env = scene.environment_map
@@ -384,7 +387,7 @@ def EnvironmentMapSample(info, fb_struct=None, add_to_out=True, want_uv=False, w
     ev_arr = (C.c_void_p * L)(*[t.data_ptr() for t in ev]) if ev else None
     s = scene.struct()
     rc = cache.lib.adop_env_sample(C.byref(s), cache.views_array(), B, C.c_void_p(env.data_ptr()), int(env.shape[1]),
-                                   int(env.shape[2]), C.byref(fb), uv_arr, ev_arr, 1 if add_to_out else 0,
+                                   int(env.shape[2]), C.byref(fb), uv_arr, ev_arr, int(add_to_out),
                                    _stream_ptr())
     _check(rc, cache.lib)
     return uv, ev

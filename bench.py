@@ -276,9 +276,13 @@ def run_workload(args, workload, steps, warmup, lib):
         # the texture coordinates travel from the forward to the backward call (the reference's autograd saves them too)
         uvs = [torch.empty(B, h, w, 2, dtype=torch.float32, device=dev) for (w, h) in hs.level_sizes()]
         uv_arr = (C.c_void_p * L)(*[t.data_ptr() for t in uvs])
+        # the composed images go to buffers of their own (the reference composes out of place, RenderModule.cpp:121-125):
+        # the backward pass sees the rasterizer's own output
+        composed = [torch.empty_like(o) for o in cache.output_forward]
+        comp_arr = (C.c_void_p * L)(*[t.data_ptr() for t in composed])
         env_args = (C.c_void_p(env.data_ptr()), int(env.shape[1]), int(env.shape[2]), gout_arr, C.c_void_p(g_env.data_ptr()),
-                    uv_arr)
-        keep += [g_env, uvs]
+                    uv_arr, comp_arr)
+        keep += [g_env, uvs, composed]
 
     frame = [0]
     env_events = []  # (name, start, stop) torch events around the environment-map calls while profiling
@@ -298,7 +302,7 @@ def run_workload(args, workload, steps, warmup, lib):
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record()
             if lib.adop_env_sample(C.byref(s), views, B, env_args[0], env_args[1], env_args[2], C.byref(fb), env_args[5],
-                                   None, 1, stream_of[0]) != 0:
+                                   env_args[6], 2, stream_of[0]) != 0:
                 fail()
             if timed_env:
                 e1.record()
@@ -399,9 +403,9 @@ def run_workload(args, workload, steps, warmup, lib):
         model = {k: v for k, v in model.items() if k in ("DepthPrepass", "RenderForward", "CombineAndFill", "BinCount",
                                                          "BinScatter", "TileDepth", "TileBlend")}
     if with_env:
-        # every pixel reads its mask, an empty one stores its uv, reads its four taps per channel and adds to the image;
-        # backward: mask, uv, upstream gradient and the read-modify-write of the four taps per channel
-        model["EnvironmentMap"] = B * P * 4 + empty_pixels * (8 + 16 * Cn + 8 * Cn)
+        # every pixel reads its mask and the image and writes the composed image, an empty one also stores its uv and
+        # reads its four taps per channel; backward: mask, uv, upstream gradient and the read-modify-write of the taps
+        model["EnvironmentMap"] = B * P * (4 + 8 * Cn) + empty_pixels * (8 + 16 * Cn)
         model["EnvironmentMapBackward"] = B * P * 4 + empty_pixels * (8 + 4 * Cn + 2 * 16 * Cn)
     total_bytes = sum(model.values())
     dom = max((k for k in model if k in stages), key=lambda k: stages[k])

@@ -191,8 +191,14 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
 
 /* Replaces EnvironmentMapImpl::Sample (EnvironmentMap.cu:107-157: BuildSphericalUV + grid_sample bilinear /
  * border / align_corners) fused with the composition images += (1-mask)*env (RenderModule.cpp:121-125).
- * env_texture [C,eh,ew] f32. For level l: uv_l [B,h_l,w_l,2] (may be NULL), env_l [B,C,h_l,w_l] (may be NULL),
- * and, if add_to_out != 0, out_l += (1 - mask_l) * env.
+ * env_texture [C,eh,ew] f32. For level l: uv_l [B,h_l,w_l,2] (may be NULL), env_l [B,C,h_l,w_l] (may be NULL).
+ * add_to_out = 0: env_l receives the samples, uv_l the coordinates of every pixel.  With 1 or 2 only the pixels the
+ * composition samples (mask_l != 1) are computed: uv_l is written there only (the rest keeps what the buffer held;
+ * adop_env_sample_backward reads no other), env_l is 0 elsewhere.
+ * 1: out_l += (1 - mask_l) * env in place (env_l, if given, the samples).
+ * 2: env_l receives the composed image out_l + (1 - mask_l) * env and out_l is left alone, as the reference composes
+ * (RenderModule.cpp:121-125): adop_backward reads out_l as the image its spatial gradients see, so a training step
+ * that composes in place before its backward pass shows them the environment at the empty pixels as well.
  * Pinhole views: the pixel's ray as in BuildSphericalUV (EnvironmentMap.cu:82-90: unproject2 through crop and K,
  * undistortNormalizedPointSimple).  OCam views (the reference asserts pinhole, EnvironmentMap.cu:129; this is an
  * extension): the ray comes from inverting the world2cam polynomial of the intrinsics row itself (no cam2world

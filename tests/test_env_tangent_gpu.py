@@ -23,31 +23,66 @@ def _env_scene():
     return hs
 
 
-def test_env_uv_sample_and_composition(oracle_mod):
+def _check_sampling_and_composition(oracle_mod, hs):
+    """uv and samples of every pixel against the checker; the composition in place and out of place."""
     import torch
     from adop_amd import render
 
-    announce("environment map: uv, bilinear sample, out += (1-mask)*env")
-    hs = _env_scene()
     scene, info, ctx, images, masks = run_hip_forward(hs)
     before = [im.clone() for im in images]
-    uv, env = render.EnvironmentMapSample(info, add_to_out=True, want_uv=True, want_env=True)
+    uv, env = render.EnvironmentMapSample(info, add_to_out=False, want_uv=True, want_env=True)
     torch.cuda.synchronize()
+    empty = 0
     for l in range(hs.num_layers):
+        assert bool((images[l] == before[l]).all())
         for b in range(hs.batch):
             want_uv = oracle_mod.env_uv(hs, b, l)
             got_uv = uv[l][b].cpu().numpy()
-            assert np.abs(got_uv - want_uv).max() <= 1e-6, (l, b)
+            assert np.isfinite(got_uv).all()
+            assert np.abs(got_uv - want_uv).max() <= 1e-6, (l, b, np.abs(got_uv - want_uv).max())
             # sampling of the HIP uv with the checker's bilinear rule
             want_env = oracle_mod.grid_sample(hs.env_texture, got_uv)
             assert_close(env[l][b].cpu().numpy(), want_env, 1e-5, 1e-6, f"env level {l} view {b}")
-        m = masks[l].cpu().numpy()
-        want = before[l].cpu().numpy() + (1 - m) * env[l].cpu().numpy()
-        assert_close(images[l].cpu().numpy(), want, 1e-6, 1e-7, f"composition level {l}")
         # library cross-check: torch grid_sample on the same uv
         ref = torch.nn.functional.grid_sample(torch.from_numpy(hs.env_texture)[None].repeat(hs.batch, 1, 1, 1),
                                               uv[l].cpu(), mode="bilinear", padding_mode="border", align_corners=True)
         assert_close(env[l].cpu().numpy(), ref.numpy(), 1e-5, 2e-6, f"env vs torch level {l}")
+        empty += int((masks[l] == 0).sum())
+    assert empty > 1000  # the scene leaves pixels for the environment map
+    # out of place (as the reference composes, RenderModule.cpp:121-125): the rasterizer's images stay as they are
+    _, composed = render.EnvironmentMapSample(info, add_to_out=2)
+    torch.cuda.synchronize()
+    for l in range(hs.num_layers):
+        m = masks[l].cpu().numpy()
+        want = before[l].cpu().numpy() + (1 - m) * env[l].cpu().numpy()
+        assert_close(composed[l].cpu().numpy(), want, 1e-6, 1e-7, f"composition out of place, level {l}")
+        assert bool((images[l] == before[l]).all())
+    # in place: the same numbers in the images; uv and samples only where the composition samples
+    uv1 = [torch.full_like(u, float("nan")) for u in uv]
+    fb = info.cache.forward_struct()
+    import ctypes as C
+    L = hs.num_layers
+    env1 = [torch.full_like(e, 7.0) for e in env]
+    s = scene.struct()
+    tex = scene.environment_map
+    rc = info.cache.lib.adop_env_sample(C.byref(s), info.cache.views_array(), hs.batch, C.c_void_p(tex.data_ptr()),
+                                        int(tex.shape[1]), int(tex.shape[2]), C.byref(fb),
+                                        (C.c_void_p * L)(*[t.data_ptr() for t in uv1]),
+                                        (C.c_void_p * L)(*[t.data_ptr() for t in env1]), 1, None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    for l in range(L):
+        assert bool((images[l] == composed[l]).all()), l
+        m = masks[l]
+        sampled = (m == 0)
+        assert bool(torch.isnan(uv1[l][~sampled[:, 0]]).all()) and bool((uv1[l][sampled[:, 0]] == uv[l][sampled[:, 0]]).all())
+        assert bool((env1[l] == torch.where(sampled.expand_as(env[l]), env[l], torch.zeros_like(env[l]))).all())
+    return scene, info, masks, uv1
+
+
+def test_env_uv_sample_and_composition(oracle_mod):
+    announce("environment map: uv, bilinear sample, composition in place and out of place")
+    _check_sampling_and_composition(oracle_mod, _env_scene())
 
 
 def test_env_backward_matches_autograd_of_grid_sample():
@@ -93,24 +128,8 @@ def test_env_on_ocam_views(oracle_mod):
 
     announce("environment map on OCam views: uv, sample, composition, texture gradient")
     hs = _ocam_env_scene()
-    scene, info, ctx, images, masks = run_hip_forward(hs)
-    before = [im.clone() for im in images]
-    uv, env = render.EnvironmentMapSample(info, add_to_out=True, want_uv=True, want_env=True)
-    torch.cuda.synchronize()
-    empty = 0
-    for l in range(hs.num_layers):
-        for b in range(hs.batch):
-            want_uv = oracle_mod.env_uv(hs, b, l)
-            got_uv = uv[l][b].cpu().numpy()
-            assert np.isfinite(got_uv).all()
-            assert np.abs(got_uv - want_uv).max() <= 1e-6, (l, b, np.abs(got_uv - want_uv).max())
-            want_env = oracle_mod.grid_sample(hs.env_texture, got_uv)
-            assert_close(env[l][b].cpu().numpy(), want_env, 1e-5, 1e-6, f"env level {l} view {b}")
-        m = masks[l].cpu().numpy()
-        empty += int((m == 0).sum())
-        want = before[l].cpu().numpy() + (1 - m) * env[l].cpu().numpy()
-        assert_close(images[l].cpu().numpy(), want, 1e-6, 1e-7, f"composition level {l}")
-    assert empty > 1000  # the scene leaves pixels for the environment map
+    scene, info, masks, uv = _check_sampling_and_composition(oracle_mod, hs)
+    # (uv holds coordinates at the sampled pixels only, NaN elsewhere: the backward pass must not read those)
     gout = [torch.from_numpy(g).cuda() for g in scenes.upstream_grads(hs, 9)]
     g_env = render.EnvironmentMapSampleBackward(info, gout)
     g_env_uv = render.EnvironmentMapSampleBackward(info, gout, uv=uv)  # the coordinates kept from the forward call
@@ -118,7 +137,8 @@ def test_env_on_ocam_views(oracle_mod):
     tex = torch.from_numpy(hs.env_texture).double().requires_grad_(True)
     loss = 0
     for l in range(hs.num_layers):
-        s = torch.nn.functional.grid_sample(tex[None].repeat(hs.batch, 1, 1, 1), uv[l].cpu().double(), mode="bilinear",
+        grid = torch.nan_to_num(uv[l].cpu().double(), nan=0.0)
+        s = torch.nn.functional.grid_sample(tex[None].repeat(hs.batch, 1, 1, 1), grid, mode="bilinear",
                                             padding_mode="border", align_corners=True)
         loss = loss + (s * (1 - masks[l].cpu().double()) * gout[l].cpu().double()).sum()
     loss.backward()

@@ -189,15 +189,23 @@ def test_environment_map_on_the_ocam_views_at_full_size(full_scene):
     announce("config5 full size: environment map on 8 OCam views of 2200x1500, forward and texture gradient")
     scene, info, ctx, images, masks = run_hip_forward(hs, collect_stats=False, forward_path=2)
     before = [im.clone() for im in images]
-    uv, env = render.EnvironmentMapSample(info, add_to_out=True, want_uv=True, want_env=True)
+    uv, env = render.EnvironmentMapSample(info, add_to_out=False, want_uv=True, want_env=True)
+    _, composed = render.EnvironmentMapSample(info, add_to_out=2)  # out of place, as the reference composes
     torch.cuda.synchronize()
     L = hs.num_layers
     for l in range(L):
         assert bool(torch.isfinite(uv[l]).all()) and float(uv[l].abs().max()) <= 1.0
         m = masks[l]
         want = before[l] + (1 - m) * env[l]
-        assert float((images[l] - want).abs().max()) <= 1e-6
-        assert bool((images[l] == before[l])[(m == 1).expand_as(images[l])].all())  # rendered pixels untouched
+        assert float((composed[l] - want).abs().max()) <= 1e-6
+        assert bool((images[l] == before[l]).all())  # the rasterizer's output is left alone
+        assert bool((composed[l] == before[l])[(m == 1).expand_as(images[l])].all())  # rendered pixels: a copy
+    uv_in_place, _ = render.EnvironmentMapSample(info, add_to_out=True, want_uv=True)
+    torch.cuda.synchronize()
+    for l in range(L):
+        assert bool((images[l] == composed[l]).all())  # in place: the same numbers
+        sampled = (masks[l] == 0)[:, 0]
+        assert bool((uv_in_place[l][sampled] == uv[l][sampled]).all())
     # a sample of pixels against the checker: 64 x 64 windows of view 3 at levels 0 and 2
     for l, (y0, x0) in ((0, (700, 1000)), (2, (100, 200))):
         want = oracle.env_uv(hs, 3, l)[y0:y0 + 64, x0:x0 + 64]
