@@ -135,6 +135,7 @@ constexpr int kTileLevels = 2;  // levels the tile path renders in LDS (a point 
 constexpr int kTilePathMinPoints = 1 << 16;
 constexpr int kTilePathMaxPointsPerPixel = 16;
 constexpr int kWindowCloudShare = 16;  // a crop window is taken to see 1/16 of the cloud
+constexpr int kConcurrentMaxPoints = 4000000;  // backward: full views of a larger cloud get a spatial-gradient launch each
 
 size_t max_tiles(int B, int w0, int h0)
 {
@@ -640,10 +641,17 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     q.cap    = wl.q_cap;
     // Several views (up to kConcurrentViews): the spatial gradients of all views run side by side in one launch; the
     // descriptor pass tells every item whether other views add to the same point's gradient row (those rows are summed
-    // with float atomics, all others written by their one owner).  More views, or ADOP_GHOST_CONCURRENT=0 (read at
-    // every call): one launch per view, each adding to the point gradients in the order of the views.
+    // with float atomics, all others written by their one owner).  Otherwise: one launch per view, each adding to the
+    // point gradients in the order of the views.
+    // Side by side pays while a launch per view would be small or the views share few points (the crop windows of a
+    // training batch; a cloud of at most kConcurrentMaxPoints points); full views of a large cloud, which share most
+    // of their points, fill a launch each and need no atomics that way (8 views of 20 M points: 1.76 against 1.82 ms).
+    // ADOP_GHOST_CONCURRENT=1 forces the one launch, 0 the launch per view.
     const char* env_conc = getenv("ADOP_GHOST_CONCURRENT");
-    q.concurrent = num_views > 1 && num_views <= kConcurrentViews && !(env_conc && atoi(env_conc) == 0) ? 1 : 0;
+    bool windows         = num_views > 1;
+    for (int b = 0; b < num_views; ++b) windows = windows && (views[b].crop_cx != 0.f || views[b].crop_cy != 0.f);
+    const bool want_conc = env_conc ? atoi(env_conc) != 0 : (windows || N <= kConcurrentMaxPoints);
+    q.concurrent         = num_views > 1 && num_views <= kConcurrentViews && want_conc ? 1 : 0;
     if (N < 1)
     {
         // nothing writes the partial rows: clear them for finalize
