@@ -125,6 +125,7 @@ struct WorkspaceLayout
     size_t list_count;  // uint32[B * 4 * ceil(N / 256)]
     size_t bin_count;   // uint32[max tiles]           tile bins of the forward pass
     size_t bin_offset;  // uint32[max tiles + 1]
+    size_t bin_order;   // uint4[max tiles]
     size_t bin_info;    // uint32[B * N]
     size_t bin_entries; // float4[kTileLevels * B * N]
     size_t bin_cap;     // entries
@@ -212,6 +213,8 @@ WorkspaceLayout layout(const adop_scene* s, int B, int L, int w0, int h0)
     o            = align_up(o + sizeof(uint32_t) * T, 256);
     w.bin_offset = o;
     o            = align_up(o + sizeof(uint32_t) * (T + 1), 256);
+    w.bin_order  = o;
+    o            = align_up(o + sizeof(uint4) * T, 256);
     w.bin_cap    = (size_t)kTileLevels * (size_t)B * (size_t)(s->num_points > 0 ? s->num_points : 0);
     w.bin_info   = o;
     o            = align_up(o + sizeof(uint32_t) * (size_t)B * (size_t)(s->num_points > 0 ? s->num_points : 0), 256);
@@ -492,6 +495,7 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
         bin.tiles_y = ((views[0].h - 1) >> kTileShiftY) + 1;
         bin.count   = (uint32_t*)((char*)workspace + wl.bin_count);
         bin.offset  = (uint32_t*)((char*)workspace + wl.bin_offset);
+        bin.order   = (uint4*)((char*)workspace + wl.bin_order);
         bin.entries = (float4*)((char*)workspace + wl.bin_entries);
         bin.info    = (uint32_t*)((char*)workspace + wl.bin_info);
         const int T = bin.tiles_x * bin.tiles_y * num_views;
@@ -1074,6 +1078,6 @@ const char* adop_version(void)
 {
     // "kernels N" names the state of the kernels' memory behaviour: it goes up whenever a change moves a kernel's bytes,
     // so that traffic figures measured for one state (rocprofv3 counters) are not quoted for another.
-    return "adop_raster 0.2 (gfx950) kernels 3";
+    return "adop_raster 0.2 (gfx950) kernels 4";
 }
 }  // extern "C"

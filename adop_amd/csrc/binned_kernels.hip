@@ -205,14 +205,67 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(PPT > 2 
     }
 }
 
+// The order in which the tile kernels take the tiles: order[i] = (tile, first entry, end, 0), the fullest bins first.
+// The bins of a view differ by two orders of magnitude (a surface seen at a grazing angle beside empty sky), a tile is one
+// workgroup from its first entry to its last, and the hardware starts workgroups in the order of their index: with the
+// tiles in image order a full bin may start late and run on alone (config 3: tile_blend_kernel 129 -> 102 us).
+// Computed by the first order_groups(T) workgroups of the bin_scatter launch, beside the scatter (nothing waits for it
+// before the tile kernels): workgroup g classes the tiles g, g + G, g + 2G, ... by entries / 128 (classes of equal cost
+// in batches of the tile kernels) and puts the r-th of them, fullest class first, at order[g + G * r].  Inside a class the
+// order is whatever the LDS atomics make it, which changes no result.
+constexpr int kOrderClasses       = 64;
+constexpr int kOrderTilesPerGroup = 1024;
+
+static int order_groups(int T) { return T > 0 ? (T + kOrderTilesPerGroup - 1) / kOrderTilesPerGroup : 0; }
+
+__device__ __forceinline__ void order_tiles(const BinArg& bin, int T, int g, int G)
+{
+    __shared__ uint32_t s_class[kOrderClasses];  // tiles per class, then the next free rank of the class
+    static_assert(kOrderClasses == 64, "one wavefront scans the classes");
+    const int tid = threadIdx.x;
+    if (tid < kOrderClasses) s_class[tid] = 0;
+    __syncthreads();
+    auto class_of = [](uint32_t entries) -> uint32_t
+    {
+        const uint32_t c = entries >> 7;
+        return (uint32_t)(kOrderClasses - 1) - (c < (uint32_t)(kOrderClasses - 1) ? c : (uint32_t)(kOrderClasses - 1));  // 0 = fullest
+    };
+    for (int t = g + G * tid; t < T; t += G * kBlock) atomicAdd(&s_class[class_of(bin.offset[t + 1] - bin.offset[t])], 1u);
+    __syncthreads();
+    if (tid < 64)
+    {
+        const uint32_t h = s_class[tid];
+        uint32_t inc     = h;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1)
+        {
+            uint32_t u = __shfl_up(inc, off, 64);
+            if (tid >= off) inc += u;
+        }
+        s_class[tid] = inc - h;
+    }
+    __syncthreads();
+    for (int t = g + G * tid; t < T; t += G * kBlock)
+    {
+        const uint32_t start = bin.offset[t], end = bin.offset[t + 1];
+        const uint32_t rank  = atomicAdd(&s_class[class_of(end - start)], 1u);
+        bin.order[(size_t)g + (size_t)G * rank] = make_uint4((uint32_t)t, start, end, 0u);
+    }
+}
+
 // Second pass: PPT points per thread, so that the cache loads, the slot reservations (one returning atomic per
 // distinct tile of a wavefront, for the primary entries and for the second entries alike) and the entry stores of PPT
 // runs of 64 points are in flight together — the kernel is a chain of three dependent memory round trips.
 template <int PPT>
-__global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels lv, ParamArg rp, BinArg bin)
+__global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels lv, ParamArg rp, BinArg bin, int T, int G)
 {
+    if ((int)blockIdx.x < G)  // the first G workgroups order the T tiles for the tile kernels
+    {
+        order_tiles(bin, T, (int)blockIdx.x, G);
+        return;
+    }
     const int lane = threadIdx.x & 63;
-    const int base = blockIdx.x * (kBlock * PPT) + threadIdx.x;
+    const int base = ((int)blockIdx.x - G) * (kBlock * PPT) + threadIdx.x;
     const unsigned long long below = (1ull << lane) - 1ull;
 
     // Several views: the first pass marked the runs of 64 points that miss a view entirely in the first record of the
@@ -381,15 +434,17 @@ void launch_bin(int pass, const CloudArg& pc, const ViewConst* views, const Leve
                                lv, rp, bin, stats);
         return;
     }
+    const int T = bin.tiles_x * bin.tiles_y * lv.B;
+    const int G = order_groups(T);
     static const int ppt = getenv("ADOP_SCATTER_PPT") ? atoi(getenv("ADOP_SCATTER_PPT")) : 2;
     if (ppt == 1)
-        hipLaunchKernelGGL((bin_scatter_kernel<1>), dim3((pc.n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, pc, lv, rp, bin);
+        hipLaunchKernelGGL((bin_scatter_kernel<1>), dim3(G + (pc.n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, pc, lv, rp, bin, T, G);
     else if (ppt == 2)
-        hipLaunchKernelGGL((bin_scatter_kernel<2>), dim3((pc.n + kBlock * 2 - 1) / (kBlock * 2)), dim3(kBlock), 0, st, pc,
-                           lv, rp, bin);
+        hipLaunchKernelGGL((bin_scatter_kernel<2>), dim3(G + (pc.n + kBlock * 2 - 1) / (kBlock * 2)), dim3(kBlock), 0, st, pc,
+                           lv, rp, bin, T, G);
     else
-        hipLaunchKernelGGL((bin_scatter_kernel<4>), dim3((pc.n + kBlock * 4 - 1) / (kBlock * 4)), dim3(kBlock), 0, st, pc,
-                           lv, rp, bin);
+        hipLaunchKernelGGL((bin_scatter_kernel<4>), dim3(G + (pc.n + kBlock * 4 - 1) / (kBlock * 4)), dim3(kBlock), 0, st, pc,
+                           lv, rp, bin, T, G);
 }
 
 void launch_tile_scan(const BinArg& bin, int num_tiles, hipStream_t st)

@@ -58,6 +58,7 @@ struct BinArg
     uint32_t* count;   // [T] entries per tile after the first pass; the second pass counts it down to zero to hand
                        // out the slots of a bin
     uint32_t* offset;  // [T + 1] exclusive prefix sum
+    uint4* order;      // [T] (tile, first entry, end, 0): the tiles as the tile kernels take them, the fullest bins first
     float4* entries;   // (ip.x, ip.y, +-depth, point id | flags), at most lt per point and view
     uint32_t* info;    // [B * N] written by the first pass for the second: tile of the primary entry (bits 0..23),
                        // levels before the LOD break (24..26), second entry one tile to the right / below (27, 28),

@@ -75,13 +75,14 @@ __global__ __launch_bounds__(kBlock) void tile_depth_kernel(Levels lv, BinArg bi
 {
     __shared__ unsigned long long s_depth[kTileMaxPixels];
     const int tiles_per_view = bin.tiles_x * bin.tiles_y;
-    const int tile           = blockIdx.x;
+    const uint4 mine         = bin.order[blockIdx.x];  // (tile, first entry, end): the fullest bins come first
+    const int tile           = (int)mine.x;
     const int b              = tile / tiles_per_view;
     const int tr             = tile - b * tiles_per_view;
     const int ty             = tr / bin.tiles_x;
     const int tx             = tr - ty * bin.tiles_x;
-    const uint32_t start     = bin.offset[tile];
-    const uint32_t end       = bin.offset[tile + 1];
+    const uint32_t start     = mine.y;
+    const uint32_t end       = mine.z;
     const TileLayout T       = tile_layout(lv, tx, ty, bin.lt, lv.num);
     const int npix           = T.base[ADOP_MAX_LAYERS];
 
@@ -214,13 +215,14 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu((CT != 0
     const int tid    = threadIdx.x;
 
     const int tiles_per_view = bin.tiles_x * bin.tiles_y;
-    const int tile           = blockIdx.x;
+    const uint4 mine         = bin.order[blockIdx.x];  // (tile, first entry, end): the fullest bins come first
+    const int tile           = (int)mine.x;
     const int b              = tile / tiles_per_view;
     const int tr             = tile - b * tiles_per_view;
     const int ty             = tr / bin.tiles_x;
     const int tx             = tr - ty * bin.tiles_x;
-    const uint32_t start     = bin.offset[tile];
-    const uint32_t end       = bin.offset[tile + 1];
+    const uint32_t start     = mine.y;
+    const uint32_t end       = mine.z;
     const int lt             = bin.lt;
     const TileLayout T       = tile_layout(lv, tx, ty, lt, lv.num);
     const int npix           = T.base[ADOP_MAX_LAYERS];
