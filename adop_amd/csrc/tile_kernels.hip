@@ -71,7 +71,9 @@ __host__ __device__ inline int tile_pixels(int lt, int upto)
 
 constexpr int kTileMaxPixels = 512;  // 256 + 64 own pixels and the coarse windows (9x3 + 5x2 + 3x2)
 
-__global__ __launch_bounds__(kBlock) void tile_depth_kernel(Levels lv, BinArg bin)
+// 8 waves per SIMD: the kernel is a chain of round trips per tile (bin range, entries, stores) with little arithmetic,
+// and its 100 scalar registers allow only 6.
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) void tile_depth_kernel(Levels lv, BinArg bin)
 {
     __shared__ unsigned long long s_depth[kTileMaxPixels];
     const int tiles_per_view = bin.tiles_x * bin.tiles_y;
@@ -114,8 +116,11 @@ __global__ __launch_bounds__(kBlock) void tile_depth_kernel(Levels lv, BinArg bi
                     // Early depth test on the LDS copy from level 1 on: the entries of a tile share few coarse pixels,
                     // LDS atomics of one instruction on one address run one after the other, and after the first
                     // batches most entries lose against the value already there (a plain read is a broadcast).
+                    // (builtins that keep the LDS address space: with the register limit of 8 waves per SIMD the
+                    // compiler fails on the generic-pointer forms)
                     unsigned long long* dst = &s_depth[T.base[l] + cy * T.wx[l] + cx];
-                    if (l == 0 || pk < *(volatile unsigned long long*)dst) atomicMin(dst, (unsigned long long)pk);
+                    if (l == 0 || pk < __hip_atomic_load(dst, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP))
+                        __hip_atomic_fetch_min(dst, (unsigned long long)pk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 }
                 if (l >= bin.lt && live && !hit) miss |= 1u << l;
                 x *= 0.5f;
