@@ -656,6 +656,10 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     for (int b = 0; b < num_views; ++b) windows = windows && (views[b].crop_cx != 0.f || views[b].crop_cy != 0.f);
     const bool want_conc = env_conc ? atoi(env_conc) != 0 : (windows || N <= kConcurrentMaxPoints);
     q.concurrent         = num_views > 1 && num_views <= kConcurrentViews && want_conc ? 1 : 0;
+    // One view: the spatial-gradient kernel normalises the point gradients itself (ADOP_NORMALIZE_FUSED=0: a pass of
+    // the finalize kernel over the work queue does).
+    static const int fused_norm = getenv("ADOP_NORMALIZE_FUSED") ? atoi(getenv("ADOP_NORMALIZE_FUSED")) : 1;
+    q.normalize = (num_views == 1 && grads->grad_points && fused_norm) ? (params->normalize_mode == 0 ? 1 : 2) : 0;
     if (N < 1)
     {
         // nothing writes the partial rows: clear them for finalize

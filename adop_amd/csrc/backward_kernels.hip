@@ -363,10 +363,14 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(CT != 0 
             kept[b / 12] |= (unsigned long long)mask << (5 * (b % 12));
             continue;
         }
-        if (b == 0 && gpoints && valid && mask == 0)
+        if (b == 0 && gpoints && valid && (mask == 0 || !MULTI))
         {
-            nt_store4((float4*)gpoints + i, make_float4(0, 0, 0, 0));
-            __builtin_nontemporal_store(0.f, gpoints_count + i);
+            if (mask == 0) nt_store4((float4*)gpoints + i, make_float4(0, 0, 0, 0));
+            // One view: the number of contributions of a point is the number of its levels with a spatial gradient, known
+            // here for every point; the spatial-gradient kernel then normalises its rows itself (NormalizeGradient,
+            // :1534-1547), for which it needs the counts of other points (normalize_mode 0 divides the floats 3t..3t+2 of
+            // the [N,4] buffer by count[t]).
+            __builtin_nontemporal_store(MULTI ? 0.f : (float)__popc(mask), gpoints_count + i);
         }
 
         const int set = b;  // queue set the item goes to
@@ -476,7 +480,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
                                                                  float* __restrict__ gpoints,
                                                                  float* __restrict__ gpoints_count, int want_pose,
                                                                  int want_intr, int identity_index, int view_b,
-                                                                 int first_view,
+                                                                 int first_view, int normalize,
                                                                  const uint32_t* __restrict__ q_counts,
                                                                  const unsigned long long* __restrict__ q_items,
                                                                  uint32_t q_cap, double* __restrict__ partial)
@@ -721,15 +725,46 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
             }
             else
             {
-                if (first_view || concurrent)
-                    *(float4*)g = make_float4(gp[0], gp[1], gp[2], 0.f);  // nothing has cleared the row
+                if (normalize)
+                {
+                    // One view: the descriptor pass left the final count of every point, and this thread writes the
+                    // normalised row (NormalizeGradient<float,3>, :1534-1547, launched on the [N,4] buffer, :1620-1627).
+                    // normalize = 1 (the reference's launch): float f of the buffer belongs to element f / 3 and is
+                    // divided by that point's count when it is positive and f / 3 < N; 2: row i by count[i].
+                    if (normalize == 2)
+                    {
+                        gp[0] = gp[0] / gp_n;
+                        gp[1] = gp[1] / gp_n;
+                        gp[2] = gp[2] / gp_n;
+                    }
+                    else
+                    {
+                        const uint32_t f0 = 4u * (uint32_t)i;  // (N <= 2^30)
+#pragma unroll
+                        for (int k = 0; k < 3; ++k)
+                        {
+                            const uint32_t t = (f0 + (uint32_t)k) / 3u;
+                            if (t < (uint32_t)pc.n)
+                            {
+                                const float c = t == (uint32_t)i ? gp_n : gpoints_count[t];
+                                if (c > 0) gp[k] = gp[k] / c;
+                            }
+                        }
+                    }
+                    *(float4*)g = make_float4(gp[0], gp[1], gp[2], 0.f);
+                }
+                else if (first_view || concurrent)
+                {
+                    *(float4*)g      = make_float4(gp[0], gp[1], gp[2], 0.f);  // nothing has cleared the row
+                    gpoints_count[i] = gp_n;
+                }
                 else
                 {
-                    g[0] = gp[0];
-                    g[1] = gp[1];
-                    g[2] = gp[2];
+                    g[0]             = gp[0];
+                    g[1]             = gp[1];
+                    g[2]             = gp[2];
+                    gpoints_count[i] = gp_n;
                 }
-                gpoints_count[i] = gp_n;
             }
         }
     }
@@ -1086,12 +1121,13 @@ static void launch_bwd_ghost_t(const CloudArg& pc, const ViewConst* views, const
 {
     if (b < 0)  // every view at once: view = blockIdx.y
         hipLaunchKernelGGL((backward_ghost_kernel<CT, HALF>), dim3(ghost_blocks, lv.B), dim3(kBlock), 0, st, pc, views, lv,
-                           rp, ig, g->grad_points, g->grad_points_count, want_pose, want_intr, identity_index, -1, 0,
+                           rp, ig, g->grad_points, g->grad_points_count, want_pose, want_intr, identity_index, -1, 0, 0,
                            q.counts, q.items, q.cap, partial);
     else
         hipLaunchKernelGGL((backward_ghost_kernel<CT, HALF>), dim3(ghost_blocks), dim3(kBlock), 0, st, pc, views, lv, rp,
                            ig, g->grad_points, g->grad_points_count, want_pose, want_intr, identity_index, b, b == 0,
-                           q.counts + (size_t)b * kNumQueues, q.items + (size_t)b * kNumQueues * q.cap, q.cap, partial);
+                           q.normalize, q.counts + (size_t)b * kNumQueues, q.items + (size_t)b * kNumQueues * q.cap, q.cap,
+                           partial);
 }
 
 #define ADOP_DISPATCH_C_HALF(FN, ...)                                   \
@@ -1139,6 +1175,10 @@ void launch_finalize(const ViewConst* views, int B, int C, const double* bg_part
     static const int by_queue = getenv("ADOP_NORMALIZE_BY_QUEUE") ? atoi(getenv("ADOP_NORMALIZE_BY_QUEUE")) : 1;
     if (n == 0)
         hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kFinalizeBlock), 0, st, a);
+    else if (q.normalize)
+        // one view: the spatial-gradient kernel has normalised the rows; two workgroups reduce the partial sums
+        hipLaunchKernelGGL(finalize_queue_kernel, dim3(2), dim3(kFinalizeBlock), 0, st, a, g->grad_points,
+                           g->grad_points_count, normalize_mode);
     else if (B == 1 && by_queue)
     {
         // (with several views a point sits in several queues and would be divided more than once)

@@ -85,6 +85,9 @@ struct QueueArg
     uint32_t* counts;           // [B][kNumQueues]: one set per view
     unsigned long long* items;  // [B][kNumQueues * cap]
     uint32_t cap;
+    int normalize;              // one view: 0 = the point gradients are normalised by the finalize kernel; 1, 2 = by the
+                                // spatial-gradient kernel, as normalize_mode 0 / 1 (the descriptor pass then writes
+                                // the final count of every point)
     int concurrent;             // several views: 1 = the items of all views are pushed when the descriptor pass knows
                                 // which points several views share, and the spatial-gradient kernel runs every view
                                 // in one launch; 0 = items pushed view by view, one spatial-gradient launch per view
