@@ -71,8 +71,11 @@ __host__ __device__ inline int tile_pixels(int lt, int upto)
 
 constexpr int kTileMaxPixels = 512;  // 256 + 64 own pixels and the coarse windows (9x3 + 5x2 + 3x2)
 
+// LT = LT as a compile-time constant: the extents and offsets of the tile's pixel windows are then constants instead
+// of scalar registers (the kernel is short: a tile's set-up is a third of it).
 // 8 waves per SIMD: the kernel is a chain of round trips per tile (bin range, entries, stores) with little arithmetic,
 // and its 100 scalar registers allow only 6.
+template <int LT>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) void tile_depth_kernel(Levels lv, BinArg bin)
 {
     __shared__ unsigned long long s_depth[kTileMaxPixels];
@@ -85,7 +88,25 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
     const int tx             = tr - ty * bin.tiles_x;
     const uint32_t start     = mine.y;
     const uint32_t end       = mine.z;
-    const TileLayout T       = tile_layout(lv, tx, ty, bin.lt, lv.num);
+    if (end == start)  // (workgroup-uniform) an empty bin, four tiles in ten of a typical view: the tile's own pixels are
+    {                  // cleared and nothing else happens
+#pragma unroll
+        for (int l = 0; l < LT; ++l)
+        {
+            if (l < lv.num)
+            {
+                const LevelArg& L = lv.l[l];
+                const int W       = 1 << (kTileShiftX - l);
+                const int q       = threadIdx.x;
+                const int cy = q / W, cx = q - cy * W;
+                const int px = (tx << (kTileShiftX - l)) + cx, py = (ty << (kTileShiftY - l)) + cy;
+                if (q < W * (1 << (kTileShiftY - l)) && px < L.w && py < L.h)
+                    L.depth_index[(size_t)b * L.w * L.h + (size_t)py * L.w + px] = kClearPacked;
+            }
+        }
+        return;
+    }
+    const TileLayout T       = tile_layout(lv, tx, ty, LT, lv.num);
     const int npix           = T.base[ADOP_MAX_LAYERS];
 
     for (int p = threadIdx.x; p < npix; p += kBlock) s_depth[p] = kClearPacked;
@@ -109,7 +130,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
             {
                 const int px = f2i_rn(x), py = f2i_rn(y);
                 const int cx = px - T.ox[l], cy = py - T.oy[l];
-                const bool live = l < nlev && (l < bin.lt || primary);
+                const bool live = l < nlev && (l < LT || primary);
                 const bool hit  = live && (unsigned)cx < (unsigned)T.cwx[l] && (unsigned)cy < (unsigned)T.cwy[l];
                 if (hit)
                 {
@@ -122,7 +143,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
                     if (l == 0 || pk < __hip_atomic_load(dst, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP))
                         __hip_atomic_fetch_min(dst, (unsigned long long)pk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 }
-                if (l >= bin.lt && live && !hit) miss |= 1u << l;
+                if (l >= LT && live && !hit) miss |= 1u << l;
                 x *= 0.5f;
                 y *= 0.5f;
             }
@@ -160,7 +181,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
                 {
                     unsigned long long v = s_depth[T.base[l] + q];
                     uint64_t* dst        = L.depth_index + (size_t)b * L.w * L.h + (size_t)py * L.w + px;
-                    if (l < bin.lt)
+                    if (l < LT)
                         *dst = v;  // the tile owns the pixel
                     else if (v != kClearPacked)
                         atomicMin((unsigned long long*)dst, v);
@@ -179,14 +200,15 @@ constexpr int kL1Bucket0     = 256;
 constexpr int kCoarseBucket0 = 384;
 constexpr uint32_t kListEnd = 0xFFFFu;
 
-template <int CT>
+template <int CT, int BATCH>
 __device__ __forceinline__ void add_staged(float* acc, const float* s_stage, int slot, int C)
 {
     constexpr int CMAX = CT ? CT : kMaxChannels;
     if (CT == 8)
     {
-        const float4* d = (const float4*)(s_stage + slot * 8);
-        float4 u = d[0], v = d[1];
+        // (two planes of float4, [half][slot]: the lanes of a wavefront store consecutive 16-byte words)
+        const float4* d = (const float4*)s_stage + slot;
+        float4 u = d[0], v = d[BATCH];
         acc[0] += u.x; acc[1] += u.y; acc[2] += u.z; acc[3] += u.w;
         acc[4] += v.x; acc[5] += v.y; acc[6] += v.z; acc[7] += v.w;
     }
@@ -396,9 +418,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu((CT != 0
                 {
                     if (CT == 8)
                     {
-                        float4* d = (float4*)(s_stage + slot * 8);
+                        float4* d = (float4*)s_stage + slot;
                         d[0]      = make_float4(t[k][0], t[k][1], t[k][2], t[k][3]);
-                        d[1]      = make_float4(t[k][4], t[k][5], t[k][6], t[k][7]);
+                        d[BATCH]  = make_float4(t[k][4], t[k][5], t[k][6], t[k][7]);
                     }
                     else if (CT == 4)
                         *(float4*)(s_stage + slot * 4) = make_float4(t[k][0], t[k][1], t[k][2], t[k][3]);
@@ -417,7 +439,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu((CT != 0
                 float n       = 0.f;
                 while (node != kListEnd)
                 {
-                    add_staged<CT>(acc0, s_stage, (int)(node & (BATCH - 1)), C);
+                    add_staged<CT, BATCH>(acc0, s_stage, (int)(node & (BATCH - 1)), C);
                     n += 1.f;
                     node = s_next[node];
                 }
@@ -427,7 +449,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu((CT != 0
                 n           = 0.f;
                 while (node != kListEnd)
                 {
-                    add_staged<CT>(acc1, s_stage, (int)(node & (BATCH - 1)), C);
+                    add_staged<CT, BATCH>(acc1, s_stage, (int)(node & (BATCH - 1)), C);
                     n += 1.f;
                     node = s_next[node];
                 }
@@ -548,7 +570,10 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu((CT != 0
 // ------------------------------------------------------------------------------------------------
 void launch_tile_depth(const Levels& lv, const BinArg& bin, int num_tiles, hipStream_t st)
 {
-    hipLaunchKernelGGL(tile_depth_kernel, dim3(num_tiles), dim3(kBlock), 0, st, lv, bin);
+    if (bin.lt == 1)
+        hipLaunchKernelGGL(tile_depth_kernel<1>, dim3(num_tiles), dim3(kBlock), 0, st, lv, bin);
+    else
+        hipLaunchKernelGGL(tile_depth_kernel<2>, dim3(num_tiles), dim3(kBlock), 0, st, lv, bin);
 }
 
 template <int K>
