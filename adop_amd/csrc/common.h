@@ -283,7 +283,8 @@ __device__ __forceinline__ ViewConst make_view_const(const adop_view& v, const d
     c.model        = v.camera_model_type;
     c.intr_offset  = cols * v.camera_index;
     c.npoly        = cols - 5;
-    c.pad          = 0;
+    c.no_distortion = v.camera_model_type == ADOP_CAMERA_PINHOLE_DISTORTION;
+    for (int i = 0; i < 8; ++i) c.no_distortion = c.no_distortion && c.d[i] == 0.f;
     return c;
 }
 

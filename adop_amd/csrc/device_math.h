@@ -34,7 +34,7 @@ struct ViewConst
     int32_t model;        // 0 pinhole+distortion, 1 OCam
     int32_t intr_offset;  // first float of this camera's row in `intrinsics`
     int32_t npoly;        // OCam: number of world2cam coefficients
-    int32_t pad;
+    int32_t no_distortion;  // pinhole: all eight distortion coefficients are zero
 };
 
 __device__ __forceinline__ uint32_t f2u(float f)
@@ -352,7 +352,18 @@ __device__ __forceinline__ bool project_frame(const ViewConst& vc, const float* 
         }
         float iz  = 1.0f / view_p.z;
         V2 norm_p = {view_p.x * iz, view_p.y * iz};
-        V2 dist_p = distort<false>(norm_p, vc.d, dist_cutoff, nullptr, nullptr);
+        // A camera without distortion (the coefficients all zero): distortNormalizedPoint returns its argument, bit for
+        // bit up to the sign of a zero, as long as r^6 is finite (0 * inf would make the polynomial NaN).  Taken when
+        // that holds for every lane of the wavefront: a third of the projection's instructions.
+        const float r2 = norm_p.x * norm_p.x + norm_p.y * norm_p.y;
+        V2 dist_p;
+        if (vc.no_distortion && __ballot(!(r2 < 1.0e12f)) == 0)
+        {
+            dist_p = norm_p;
+            if (r2 > dist_cutoff * dist_cutoff) dist_p = {100000.f, 100000.f};
+        }
+        else
+            dist_p = distort<false>(norm_p, vc.d, dist_cutoff, nullptr, nullptr);
         if (dist_p.x == 100000.f) z = 0;
         image_p = k_apply(vc.k, dist_p);
     }
