@@ -85,7 +85,8 @@ typedef struct adop_render_params
     int32_t normalize_mode;
     /* How adop_forward renders (same results either way; no counterpart in the reference):
      * 0: the library chooses; 1: direct (depth prepass and blend with global atomics, PointRenderer.cu:203-393
-     * as written); 2: through screen-space tile bins (the fine levels are rendered in LDS). */
+     * as written); 2: through screen-space tile bins (the fine levels are rendered in LDS).  0 decides by the number
+     * of points per pixel of the whole image; when the cloud covers only a small part of the image, 1 is the faster. */
     int32_t forward_path;
 } adop_render_params;
 
