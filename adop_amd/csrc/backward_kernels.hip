@@ -225,11 +225,36 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(CT != 0 
         if (threadIdx.x == 0) s_block_culled = 0;
         __syncthreads();
     }
+    // Views 0..63 for which every run of this workgroup was culled have nothing to test: the loop jumps from one live view
+    // to the next (a crop sees a small part of the cloud: 2 to 3 of 16 views are live for a workgroup, and the loop
+    // is scalar control flow that the scalar unit of the CU has to issue for every wavefront).
+    unsigned long long live_views = ~0ull;
+    if (MULTI)
+    {
+        const unsigned long long bc = s_block_culled;
+        live_views = ~(((unsigned long long)(uint32_t)__builtin_amdgcn_readfirstlane((int)(bc >> 32)) << 32) |
+                       (unsigned long long)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)bc));
+        // view 0 culled for the whole workgroup: its iteration, which clears the point-gradient rows, is skipped
+        if (!deferred && (live_views & 1ull) == 0 && gpoints && valid)
+        {
+            nt_store4((float4*)gpoints + i, make_float4(0, 0, 0, 0));
+            __builtin_nontemporal_store(0.f, gpoints_count + i);
+        }
+    }
     for (int b = 0; b < num_views; ++b)
     {
-        // a view for which every run of this workgroup was culled has nothing to test (mask stays 0)
+        if (MULTI && b < 64)
+        {
+            const unsigned long long rest = live_views >> b;  // (uniform)
+            if (rest == 0)
+            {
+                b = 63;  // the views from 64 on carry no marks
+                continue;
+            }
+            b += __builtin_ctzll(rest);
+            if (b >= num_views) break;
+        }
         uint32_t mask = 0;
-        if (!(MULTI && b < 64 && (s_block_culled >> b & 1ull) != 0))
         {
             const ViewConst& vc = views[b];
             bool drop_out;
@@ -423,8 +448,15 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(CT != 0 
 
     if (deferred)
     {
+        // number of views with an item: the non-zero 5-bit fields of the two words (bit 0 of a field = the OR of its bits)
+        constexpr unsigned long long kField0 = 0x0084210842108421ull;  // bits 0, 5, ..., 55: twelve fields
         int nitems = 0;
-        for (int b = 0; b < num_views; ++b) nitems += (kept[b / 12] >> (5 * (b % 12)) & 31ull) != 0;
+#pragma unroll
+        for (int w = 0; w < 2; ++w)
+        {
+            const unsigned long long k = kept[w];
+            nitems += __popcll((k | k >> 1 | k >> 2 | k >> 3 | k >> 4) & kField0);
+        }
         // A point with one item gets its gradient row from that item's thread; a row nobody writes, or one that several
         // views add to with atomics, starts at zero (Build(info,false), :922-949).
         if (gpoints && valid && nitems != 1)
@@ -435,6 +467,12 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(CT != 0 
         const unsigned long long shared = nitems > 1 ? 1ull << kItemSharedBit : 0ull;
         for (int b = 0; b < num_views; ++b)
         {
+            {
+                const unsigned long long rest = live_views >> b;  // (uniform; at most kConcurrentViews < 64 views here)
+                if (rest == 0) break;
+                b += __builtin_ctzll(rest);
+                if (b >= num_views) break;
+            }
             const unsigned long long m = kept[b / 12] >> (5 * (b % 12)) & 31ull;
             const unsigned long long bal = __ballot(m != 0);
             if (!bal) continue;  // wavefront-uniform

@@ -288,8 +288,24 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels
         }
     }
 
+    // (views 0..63 that every run of this wavefront missed are jumped over: the loop is scalar control flow, and a crop
+    // sees a small part of the cloud)
+    unsigned long long all_culled = ~0ull;
+#pragma unroll
+    for (int k = 0; k < PPT; ++k) all_culled &= culled_views[k];
     for (int b = 0; b < lv.B; ++b)
     {
+        if (b < 64)
+        {
+            const unsigned long long rest = ~all_culled >> b;  // (wavefront-uniform)
+            if (rest == 0)
+            {
+                b = 63;  // the views from 64 on carry no marks
+                continue;
+            }
+            b += __builtin_ctzll(rest);
+            if (b >= lv.B) break;
+        }
         uint32_t info[PPT];
         bool any = false;
 #pragma unroll
