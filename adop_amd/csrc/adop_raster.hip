@@ -125,7 +125,8 @@ struct WorkspaceLayout
     size_t list_count;  // uint32[B * 4 * ceil(N / 256)]
     size_t bin_count;   // uint32[max tiles]           tile bins of the forward pass
     size_t bin_offset;  // uint32[max tiles + 1]
-    size_t bin_order;   // uint4[max tiles]
+    size_t bin_order;   // uint4[max tiles + slice_rows()]
+    size_t bin_rows;    // float[slice_rows()][slice_row_floats()]: partial results of the slices of split bins
     size_t bin_info;    // uint32[B * N]
     size_t bin_entries; // float4[kTileLevels * B * N]
     size_t bin_cap;     // entries
@@ -209,12 +210,15 @@ WorkspaceLayout layout(const adop_scene* s, int B, int L, int w0, int h0)
     w.list_count = o;
     o = align_up(o + 4 * sizeof(uint32_t) * (size_t)B * (((size_t)(s->num_points > 0 ? s->num_points : 0) + kBlock - 1) / kBlock), 256);
     size_t T     = max_tiles(B, w0, h0);
-    w.bin_count  = o;
-    o            = align_up(o + sizeof(uint32_t) * T, 256);
+    w.bin_count  = o;  // followed by the row counter and the tickets of the split bins: one range to clear
+    const size_t max_rows = (size_t)slice_rows(s->num_points > 0 ? s->num_points : 0, B);
+    o            = align_up(o + sizeof(uint32_t) * (T + 1 + 2 * max_rows), 256);
     w.bin_offset = o;
     o            = align_up(o + sizeof(uint32_t) * (T + 1), 256);
     w.bin_order  = o;
-    o            = align_up(o + sizeof(uint4) * T, 256);
+    o            = align_up(o + sizeof(uint4) * (T + max_rows), 256);
+    w.bin_rows   = o;
+    o            = align_up(o + sizeof(float) * max_rows * (size_t)slice_row_floats(s->num_channels > 0 ? s->num_channels : 1), 256);
     w.bin_cap    = (size_t)kTileLevels * (size_t)B * (size_t)(s->num_points > 0 ? s->num_points : 0);
     w.bin_info   = o;
     o            = align_up(o + sizeof(uint32_t) * (size_t)B * (size_t)(s->num_points > 0 ? s->num_points : 0), 256);
@@ -496,16 +500,24 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
         bin.count   = (uint32_t*)((char*)workspace + wl.bin_count);
         bin.offset  = (uint32_t*)((char*)workspace + wl.bin_offset);
         bin.order   = (uint4*)((char*)workspace + wl.bin_order);
+        bin.rows    = (float*)((char*)workspace + wl.bin_rows);
         bin.entries = (float4*)((char*)workspace + wl.bin_entries);
         bin.info    = (uint32_t*)((char*)workspace + wl.bin_info);
         const int T = bin.tiles_x * bin.tiles_y * num_views;
+        bin.row_count = bin.count + T;
+        bin.tickets   = bin.count + T + 1;
+        bin.max_rows   = slice_rows(scene->num_points, num_views);
+        bin.row_floats = slice_row_floats(scene->num_channels);
+        // (read at every call: the tests split small bins)
+        const char* env_slice = getenv("ADOP_TILE_SLICE");
+        bin.slice_entries     = env_slice && atoi(env_slice) > 0 ? (uint32_t)atoi(env_slice) : 8192u;
         {
             StageScope sc("Initialize", stream);
             // tile counters, and for the coarse levels the packed depth and the global accumulators of the direct path
             size_t first   = (size_t)lv.pix_prefix[bin.lt] * lv.B * S;
             size_t accum_n = (size_t)lv.pix_prefix[lv.num] * lv.B * S - first;
             int grid       = pixel_grid(lv, bin.lt) > 32 ? pixel_grid(lv, bin.lt) : 32;
-            launch_clear(lv, bin.lt, grid, accum + first, S % 4 == 0 ? accum_n : 0, bin.count, T, vp, stream);
+            launch_clear(lv, bin.lt, grid, accum + first, S % 4 == 0 ? accum_n : 0, bin.count, T + 1 + 2 * bin.max_rows, vp, stream);
             if (S % 4 != 0 && (st = fill_async(accum + first, accum_n * sizeof(float), 0, stream)) != ADOP_OK) return st;
         }
         {
@@ -1082,6 +1094,6 @@ const char* adop_version(void)
 {
     // "kernels N" names the state of the kernels' memory behaviour: it goes up whenever a change moves a kernel's bytes,
     // so that traffic figures measured for one state (rocprofv3 counters) are not quoted for another.
-    return "adop_raster 0.2 (gfx950) kernels 5";
+    return "adop_raster 0.2 (gfx950) kernels 6";
 }
 }  // extern "C"

@@ -249,7 +249,32 @@ __device__ __forceinline__ void order_tiles(const BinArg& bin, int T, int g, int
     {
         const uint32_t start = bin.offset[t], end = bin.offset[t + 1];
         const uint32_t rank  = atomicAdd(&s_class[class_of(end - start)], 1u);
-        bin.order[(size_t)g + (size_t)G * rank] = make_uint4((uint32_t)t, start, end, 0u);
+        uint32_t first_end = end, word = 0;
+        const uint32_t n   = end - start;
+        if (n > bin.slice_entries)
+        {
+            // a bin too full for one workgroup: K slices (at most 1023, and as many as rows are left)
+            uint32_t K = (n + bin.slice_entries - 1) / bin.slice_entries;
+            if (K > 1023u) K = 1023u;
+            const uint32_t row = atomicAdd(bin.row_count, K);
+            if (row >= (uint32_t)bin.max_rows)
+                K = 1;
+            else if (row + K > (uint32_t)bin.max_rows)
+                K = (uint32_t)bin.max_rows - row;
+            // (every row below max_rows that was handed out has a workgroup that reads its place of the order)
+            if (row < (uint32_t)bin.max_rows && K == 1) bin.order[(size_t)T + row] = make_uint4(0u, 0u, 0u, 0u);
+            if (K > 1)
+            {
+                // slice sl = entries [n * sl / K, n * (sl + 1) / K) of the bin: none is empty (K <= n)
+                auto cut = [&](uint32_t sl) { return start + (uint32_t)((unsigned long long)n * sl / K); };
+                bin.order[(size_t)T + row] = make_uint4(0u, 0u, 0u, 0u);  // (slice 0 sits in the tile's own place)
+                for (uint32_t sl = 1; sl < K; ++sl)
+                    bin.order[(size_t)T + row + sl] = make_uint4((uint32_t)t, cut(sl), cut(sl + 1), K | sl << 10 | row << 20);
+                first_end = cut(1);
+                word      = K | row << 20;
+            }
+        }
+        bin.order[(size_t)g + (size_t)G * rank] = make_uint4((uint32_t)t, start, first_end, word);
     }
 }
 

@@ -58,7 +58,19 @@ struct BinArg
     uint32_t* count;   // [T] entries per tile after the first pass; the second pass counts it down to zero to hand
                        // out the slots of a bin
     uint32_t* offset;  // [T + 1] exclusive prefix sum
-    uint4* order;      // [T] (tile, first entry, end, 0): the tiles as the tile kernels take them, the fullest bins first
+    uint4* order;      // [T + max_rows] (tile, first entry, end, slice word): the tiles as the tile kernels take them,
+                       // the fullest bins first; behind them the further slices of the bins that are split
+    // A bin with more than slice_entries entries (a cloud that covers a few tiles only) is split in K slices that as
+    // many workgroups take: slice 0 in the tile's own place of the order, the others in order[T + row + s].  The slices
+    // leave their partial results of the tile's own pixels in rows[row + s]; the one that finishes last (ticket) merges
+    // the K rows in their fixed order and writes the pixels.  Slice word: K | s << 10 | row << 20 (0: not split).
+    uint32_t* row_count;   // rows handed out (zero at the start of the call; may run past max_rows: bins that get no
+                           // rows stay whole)
+    uint32_t* tickets;     // [2][max_rows] depth pass, blend pass (zero at the start of the call)
+    float* rows;           // [max_rows][row_floats]
+    uint32_t slice_entries;
+    int32_t max_rows;      // 16 .. kMaxSlices, by the size of the cloud (slice_rows())
+    int32_t row_floats;    // two accumulators of C + 1 floats per thread (slice_row_floats())
     float4* entries;   // (ip.x, ip.y, +-depth, point id | flags), at most lt per point and view
     uint32_t* info;    // [B * N] written by the first pass for the second: tile of the primary entry (bits 0..23),
                        // levels before the LOD break (24..26), second entry one tile to the right / below (27, 28),
@@ -66,6 +78,14 @@ struct BinArg
     int32_t tiles_x, tiles_y;  // tiles of one view
     int32_t lt;                // levels rendered in the tile's LDS (1 or 2); the others go through global atomics
 };
+constexpr int kMaxSlices = 1024;  // (10 bits of the slice word)
+inline int slice_row_floats(int C) { return (1 << (kTileShiftX + kTileShiftY)) * 2 * (C + 1); }
+// rows for the slices of split bins: what a cloud of n points in B views can fill at the default slice size
+inline int slice_rows(long long n, int B)
+{
+    const long long r = (2 * n * B + 8191) / 8192;
+    return (int)(r < 16 ? 16 : (r > kMaxSlices ? kMaxSlices : r));
+}
 constexpr uint32_t kEntryIdMask  = 0x0FFFFFFFu;  // entry word: point id; bits 28..30: levels before the LOD break;
 constexpr uint32_t kEntryPrimary = 0x80000000u;  // bit 31: entry of the tile that owns the (clamped) level-0 pixel
 void launch_bin(int pass, const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp,

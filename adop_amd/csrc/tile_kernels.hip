@@ -76,11 +76,17 @@ constexpr int kTileMaxPixels = 512;  // 256 + 64 own pixels and the coarse windo
 // 8 waves per SIMD: the kernel is a chain of round trips per tile (bin range, entries, stores) with little arithmetic,
 // and its 100 scalar registers allow only 6.
 template <int LT>
-__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) void tile_depth_kernel(Levels lv, BinArg bin)
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) void tile_depth_kernel(Levels lv, BinArg bin, int num_tiles)
 {
     __shared__ unsigned long long s_depth[kTileMaxPixels];
     const int tiles_per_view = bin.tiles_x * bin.tiles_y;
-    const uint4 mine         = bin.order[blockIdx.x];  // (tile, first entry, end): the fullest bins come first
+    // the workgroups behind the tiles take the further slices of the bins that are split; most calls have none
+    if ((int)blockIdx.x >= num_tiles && blockIdx.x - (uint32_t)num_tiles >= *bin.row_count) return;
+    const uint4 mine         = bin.order[blockIdx.x];  // (tile, first entry, end, slice word): the fullest bins come first
+    const int slices         = (int)(mine.w & 1023u);  // K > 1: this workgroup has slice `slice` of K of the tile's bin
+    const int slice          = (int)(mine.w >> 10 & 1023u);
+    const int row0           = (int)(mine.w >> 20);
+    if ((int)blockIdx.x >= num_tiles && slices == 0) return;  // (the place of a slice 0, which sits among the tiles)
     const int tile           = (int)mine.x;
     const int b              = tile / tiles_per_view;
     const int tr             = tile - b * tiles_per_view;
@@ -88,7 +94,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
     const int tx             = tr - ty * bin.tiles_x;
     const uint32_t start     = mine.y;
     const uint32_t end       = mine.z;
-    if (end == start)  // (workgroup-uniform) an empty bin, four tiles in ten of a typical view: the tile's own pixels are
+    if (end == start && slices <= 1)  // (workgroup-uniform) an empty bin, four tiles in ten of a typical view: the tile's own pixels are
     {                  // cleared and nothing else happens
 #pragma unroll
         for (int l = 0; l < LT; ++l)
@@ -166,6 +172,38 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
     }
     __syncthreads();
 
+    // A slice of a split bin leaves the minima of the tile's own pixels in its row; the slice that finishes last takes
+    // the minimum over the K rows and stores it (the coarse windows go through atomics anyway).
+    bool store_own = true;
+    if (slices > 1)  // (workgroup-uniform)
+    {
+        __shared__ uint32_t s_ticket;
+        const int own = T.base[LT];  // local pixels of the levels the tile owns (LT <= lv.num)
+        unsigned long long* rows = (unsigned long long*)bin.rows;
+        const size_t kRow        = (size_t)bin.row_floats / 2;  // 64-bit words per row
+        for (int p = threadIdx.x; p < own; p += kBlock) rows[(size_t)(row0 + slice) * kRow + p] = s_depth[p];
+        __threadfence();
+        __syncthreads();
+        if (threadIdx.x == 0) s_ticket = atomicAdd(&bin.tickets[row0], 1u);
+        __syncthreads();
+        store_own = s_ticket == (uint32_t)(slices - 1);
+        if (store_own)
+        {
+            __threadfence();
+            for (int p = threadIdx.x; p < own; p += kBlock)
+            {
+                unsigned long long v = kClearPacked;
+                for (int sl = 0; sl < slices; ++sl)
+                {
+                    const unsigned long long u = __builtin_nontemporal_load(&rows[(size_t)(row0 + sl) * kRow + p]);
+                    v                          = u < v ? u : v;
+                }
+                s_depth[p] = v;
+            }
+            __syncthreads();
+        }
+    }
+
 #pragma unroll
     for (int l = 0; l < ADOP_MAX_LAYERS; ++l)
     {
@@ -182,7 +220,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
                     unsigned long long v = s_depth[T.base[l] + q];
                     uint64_t* dst        = L.depth_index + (size_t)b * L.w * L.h + (size_t)py * L.w + px;
                     if (l < LT)
-                        *dst = v;  // the tile owns the pixel
+                    {
+                        if (store_own) *dst = v;  // the tile owns the pixel
+                    }
                     else if (v != kClearPacked)
                         atomicMin((unsigned long long*)dst, v);
                 }
@@ -230,7 +270,7 @@ template <int CT, bool HALF, int K>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu((CT != 0 && K == 1) ? 8 : 4, 8))) void tile_blend_kernel(CloudArg pc, Levels lv, ParamArg rp, BinArg bin,
                                                             float* __restrict__ accum, int S,
                                                             const float* __restrict__ background, int write_mask,
-                                                            float mask_value, int identity_index, adop_stats* stats)
+                                                            float mask_value, int identity_index, adop_stats* stats, int num_tiles)
 {
     constexpr int CMAX  = CT ? CT : kMaxChannels;
     constexpr int BATCH = K * kBlock;
@@ -242,7 +282,11 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu((CT != 0
     const int tid    = threadIdx.x;
 
     const int tiles_per_view = bin.tiles_x * bin.tiles_y;
-    const uint4 mine         = bin.order[blockIdx.x];  // (tile, first entry, end): the fullest bins come first
+    // the workgroups behind the tiles take the further slices of the bins that are split; most calls have none
+    if ((int)blockIdx.x >= num_tiles && blockIdx.x - (uint32_t)num_tiles >= *bin.row_count) return;
+    const uint4 mine         = bin.order[blockIdx.x];  // (tile, first entry, end, slice word): the fullest bins come first
+    const int slices         = (int)(mine.w & 1023u);  // > 1: this workgroup has slice `slice` of the tile's bin
+    if ((int)blockIdx.x >= num_tiles && slices == 0) return;  // (the place of a slice 0, which sits among the tiles)
     const int tile           = (int)mine.x;
     const int b              = tile / tiles_per_view;
     const int tr             = tile - b * tiles_per_view;
@@ -460,8 +504,64 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu((CT != 0
         }
     }
 
+    // A slice of a split bin leaves its sums for the tile's own pixels in its row; the slice that finishes last adds the
+    // K rows in their order and resolves the pixels (the coarse windows go through the global accumulators anyway).
+    // Row: per thread the C sums and the count of its first accumulator, then of its second.
+    bool resolve_own = true;
+    if (slices > 1)  // (workgroup-uniform)
+    {
+        const int slice = (int)(mine.w >> 10 & 1023u), row0 = (int)(mine.w >> 20);
+        const bool l1   = tid < kCoarseBucket0 - kL1Bucket0;  // second accumulator: a part of a level-1 pixel
+        const int W     = C + 1;
+        float* mine_row = bin.rows + (size_t)(row0 + slice) * bin.row_floats + (size_t)tid * 2 * W;
+#pragma unroll
+        for (int c = 0; c < CMAX; ++c)
+            if (c < C) mine_row[c] = acc0[c];
+        mine_row[C] = acc0[CMAX];
+        if (l1)
+        {
+#pragma unroll
+            for (int c = 0; c < CMAX; ++c)
+                if (c < C) mine_row[W + c] = acc1[c];
+            mine_row[W + C] = acc1[CMAX];
+        }
+        __threadfence();
+        __syncthreads();
+        if (tid == 0) s_head[0] = atomicAdd(&bin.tickets[bin.max_rows + row0], 1u);  // (the lists are empty by now)
+        __syncthreads();
+        resolve_own = s_head[0] == (uint32_t)(slices - 1);
+        if (resolve_own)
+        {
+            __threadfence();
+#pragma unroll
+            for (int c = 0; c <= CMAX; ++c) acc0[c] = 0.f;
+            if (l1)
+            {
+#pragma unroll
+                for (int c = 0; c <= CMAX; ++c) acc1[c] = 0.f;
+            }
+            for (int sl = 0; sl < slices; ++sl)
+            {
+                const float* r = bin.rows + (size_t)(row0 + sl) * bin.row_floats + (size_t)tid * 2 * W;
+#pragma unroll
+                for (int c = 0; c < CMAX; ++c)
+                    if (c < C) acc0[c] += __builtin_nontemporal_load(r + c);
+                acc0[CMAX] += __builtin_nontemporal_load(r + C);
+                if (l1)
+                {
+#pragma unroll
+                    for (int c = 0; c < CMAX; ++c)
+                        if (c < C) acc1[c] += __builtin_nontemporal_load(r + W + c);
+                    acc1[CMAX] += __builtin_nontemporal_load(r + W + C);
+                }
+            }
+        }
+        __syncthreads();  // (s_head[0] is read by all before anything else may use the LDS)
+    }
+
     // -- resolve (CombineAndFill :726-754, CreateMask :828-847) ----------------------------------------------------
     // level 0: bucket tid is pixel tid of the tile
+    if (resolve_own)
     {
         const LevelArg& L = lv.l[0];
         const int px = T.ox[0] + (tid & (TX - 1)), py = T.oy[0] + (tid >> kTileShiftX);
@@ -486,7 +586,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu((CT != 0
     {
 #pragma unroll
         for (int c = 0; c <= CMAX; ++c) acc1[c] += (tid < kCoarseBucket0 - kL1Bucket0) ? __shfl_xor(acc1[c], 1, 64) : 0.f;
-        if (tid < kCoarseBucket0 - kL1Bucket0 && (tid & 1) == 0)
+        if (resolve_own && tid < kCoarseBucket0 - kL1Bucket0 && (tid & 1) == 0)
         {
             constexpr int T1  = TX / 2;
             const LevelArg& L = lv.l[1];
@@ -571,9 +671,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu((CT != 0
 void launch_tile_depth(const Levels& lv, const BinArg& bin, int num_tiles, hipStream_t st)
 {
     if (bin.lt == 1)
-        hipLaunchKernelGGL(tile_depth_kernel<1>, dim3(num_tiles), dim3(kBlock), 0, st, lv, bin);
+        hipLaunchKernelGGL(tile_depth_kernel<1>, dim3(num_tiles + bin.max_rows), dim3(kBlock), 0, st, lv, bin, num_tiles);
     else
-        hipLaunchKernelGGL(tile_depth_kernel<2>, dim3(num_tiles), dim3(kBlock), 0, st, lv, bin);
+        hipLaunchKernelGGL(tile_depth_kernel<2>, dim3(num_tiles + bin.max_rows), dim3(kBlock), 0, st, lv, bin, num_tiles);
 }
 
 template <int K>
@@ -602,8 +702,8 @@ static hipError_t launch_tile_blend_k(const CloudArg& pc, const Levels& lv, cons
         if (e != hipSuccess) return e;
         allowed = lds;
     }
-    hipLaunchKernelGGL((tile_blend_kernel<CT, HALF, K>), dim3(num_tiles), dim3(kBlock), lds, st, pc, lv, rp, bin,
-                       accum, S, background, write_mask, mask_value, identity_index, stats);
+    hipLaunchKernelGGL((tile_blend_kernel<CT, HALF, K>), dim3(num_tiles + bin.max_rows), dim3(kBlock), lds, st, pc, lv, rp, bin,
+                       accum, S, background, write_mask, mask_value, identity_index, stats, num_tiles);
     return hipSuccess;
 }
 

@@ -468,6 +468,31 @@ def test_tile_path_images_are_bit_identical_from_run_to_run():
     assert same >= 0.9 * total
 
 
+@pytest.mark.parametrize("slice_entries", ["64", "7", "1"], ids=["slices_of_64", "slices_of_7", "no_rows_left"])
+@pytest.mark.parametrize("channels,collect_stats", [(8, True), (8, False), (4, False), (3, True)],
+                         ids=["C8-counters", "C8-plain", "C4-plain", "C3-counters"])
+def test_full_bins_are_split_between_workgroups(oracle_mod, monkeypatch, forward_path, slice_entries, channels,
+                                                collect_stats):
+    """A cloud that covers a few tiles only (the camera far away) puts tens of thousands of entries into one bin; bins
+    above ADOP_TILE_SLICE entries (8192 by default, read at every call) are split in slices that as many workgroups take,
+    the last of which merges their rows.  Forced here on small scenes: with 64 and 7 entries per slice nearly every bin
+    is split (up to 1023 slices a bin), with 1 the 1024 rows run out and most bins stay whole.  Forward and backward
+    through the tile path still equal the checker (packed depth bit for bit), with and without the counters, for the
+    vectorised channel counts and the generic one."""
+    from adop_amd import scenes
+
+    if forward_path != 2:
+        pytest.skip("the tile path only")
+    monkeypatch.setenv("ADOP_TILE_SLICE", slice_entries)
+    announce(f"tile path with split bins: ADOP_TILE_SLICE={slice_entries}, C={channels}, counters={collect_stats}")
+    hs = scenes.config3(n=150_000, w=160, h=96, channels=channels)
+    _fwd_bwd(hs, oracle_mod, collect_stats=collect_stats, poison=not collect_stats)
+    # the camera ten times as far: the cloud lands in a handful of tiles
+    el, az = np.deg2rad(20.0), np.deg2rad(30.0)
+    hs.poses_se3 = scenes.look_at_view(30.0 * np.array([np.cos(el) * np.sin(az), np.sin(el), -np.cos(el) * np.cos(az)]))[None, :]
+    _fwd_bwd(hs, oracle_mod, collect_stats=collect_stats, poison=not collect_stats)
+
+
 def test_zz_report_end_to_end_misses():
     """Prints what the end-to-end element-wise check of every case above found (the asserts are in _fwd_bwd)."""
     for case, rec in end_to_end_misses.items():
