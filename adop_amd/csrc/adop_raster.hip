@@ -510,7 +510,7 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
         bin.row_floats = slice_row_floats(scene->num_channels);
         // (read at every call: the tests split small bins)
         const char* env_slice = getenv("ADOP_TILE_SLICE");
-        bin.slice_entries     = env_slice && atoi(env_slice) > 0 ? (uint32_t)atoi(env_slice) : 8192u;
+        bin.slice_entries     = env_slice && atoi(env_slice) > 0 ? (uint32_t)atoi(env_slice) : (uint32_t)kSliceEntries;
         {
             StageScope sc("Initialize", stream);
             // tile counters, and for the coarse levels the packed depth and the global accumulators of the direct path

@@ -79,11 +79,16 @@ struct BinArg
     int32_t lt;                // levels rendered in the tile's LDS (1 or 2); the others go through global atomics
 };
 constexpr int kMaxSlices = 1024;  // (10 bits of the slice word)
+// Entries above which a bin is split.  A split costs more than it brings while the bin is not the longest piece of work
+// of the launch by far: every slice pays a tile's set-up, and the release / acquire around its ticket writes back and
+// invalidates the L2 of its XCD (config 5, whose fullest bins hold 10 to 30 thousand entries: tile_blend 1.16 -> 1.46 ms
+// with 8 192, 1.24 with 16 384, unchanged with 32 768).
+constexpr int kSliceEntries = 32768;
 inline int slice_row_floats(int C) { return (1 << (kTileShiftX + kTileShiftY)) * 2 * (C + 1); }
 // rows for the slices of split bins: what a cloud of n points in B views can fill at the default slice size
 inline int slice_rows(long long n, int B)
 {
-    const long long r = (2 * n * B + 8191) / 8192;
+    const long long r = (2 * n * B + kSliceEntries - 1) / kSliceEntries;
     return (int)(r < 16 ? 16 : (r > kMaxSlices ? kMaxSlices : r));
 }
 constexpr uint32_t kEntryIdMask  = 0x0FFFFFFFu;  // entry word: point id; bits 28..30: levels before the LOD break;

@@ -80,13 +80,16 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
 {
     __shared__ unsigned long long s_depth[kTileMaxPixels];
     const int tiles_per_view = bin.tiles_x * bin.tiles_y;
-    // the workgroups behind the tiles take the further slices of the bins that are split; most calls have none
-    if ((int)blockIdx.x >= num_tiles && blockIdx.x - (uint32_t)num_tiles >= *bin.row_count) return;
-    const uint4 mine         = bin.order[blockIdx.x];  // (tile, first entry, end, slice word): the fullest bins come first
+    // the first max_rows workgroups take the further slices of the bins that are split (they are the longest pieces of
+    // work of the launch: first, so that they do not form its tail); most calls have none
+    const bool extra = (int)blockIdx.x < bin.max_rows;
+    if (extra && blockIdx.x >= *bin.row_count) return;
+    // (tile, first entry, end, slice word): the tiles fullest bin first, behind them the places of the slices
+    const uint4 mine = bin.order[extra ? (uint32_t)num_tiles + blockIdx.x : blockIdx.x - (uint32_t)bin.max_rows];
     const int slices         = (int)(mine.w & 1023u);  // K > 1: this workgroup has slice `slice` of K of the tile's bin
     const int slice          = (int)(mine.w >> 10 & 1023u);
     const int row0           = (int)(mine.w >> 20);
-    if ((int)blockIdx.x >= num_tiles && slices == 0) return;  // (the place of a slice 0, which sits among the tiles)
+    if (extra && slices == 0) return;  // (the place of a slice 0, which sits among the tiles)
     const int tile           = (int)mine.x;
     const int b              = tile / tiles_per_view;
     const int tr             = tile - b * tiles_per_view;
@@ -282,11 +285,14 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu((CT != 0
     const int tid    = threadIdx.x;
 
     const int tiles_per_view = bin.tiles_x * bin.tiles_y;
-    // the workgroups behind the tiles take the further slices of the bins that are split; most calls have none
-    if ((int)blockIdx.x >= num_tiles && blockIdx.x - (uint32_t)num_tiles >= *bin.row_count) return;
-    const uint4 mine         = bin.order[blockIdx.x];  // (tile, first entry, end, slice word): the fullest bins come first
+    // the first max_rows workgroups take the further slices of the bins that are split (they are the longest pieces of
+    // work of the launch: first, so that they do not form its tail); most calls have none
+    const bool extra = (int)blockIdx.x < bin.max_rows;
+    if (extra && blockIdx.x >= *bin.row_count) return;
+    // (tile, first entry, end, slice word): the tiles fullest bin first, behind them the places of the slices
+    const uint4 mine = bin.order[extra ? (uint32_t)num_tiles + blockIdx.x : blockIdx.x - (uint32_t)bin.max_rows];
     const int slices         = (int)(mine.w & 1023u);  // > 1: this workgroup has slice `slice` of the tile's bin
-    if ((int)blockIdx.x >= num_tiles && slices == 0) return;  // (the place of a slice 0, which sits among the tiles)
+    if (extra && slices == 0) return;  // (the place of a slice 0, which sits among the tiles)
     const int tile           = (int)mine.x;
     const int b              = tile / tiles_per_view;
     const int tr             = tile - b * tiles_per_view;
