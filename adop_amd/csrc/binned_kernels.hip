@@ -251,7 +251,7 @@ __device__ __forceinline__ void order_tiles(const BinArg& bin, int T, int g, int
         const uint32_t rank  = atomicAdd(&s_class[class_of(end - start)], 1u);
         uint32_t first_end = end, word = 0;
         const uint32_t n   = end - start;
-        if (n > bin.slice_entries)
+        if (n > (uint32_t)kSplitFrom * bin.slice_entries)
         {
             // a bin too full for one workgroup: K slices (at most 1023, and as many as rows are left)
             uint32_t K = (n + bin.slice_entries - 1) / bin.slice_entries;

@@ -79,11 +79,13 @@ struct BinArg
     int32_t lt;                // levels rendered in the tile's LDS (1 or 2); the others go through global atomics
 };
 constexpr int kMaxSlices = 1024;  // (10 bits of the slice word)
-// Entries above which a bin is split.  A split costs more than it brings while the bin is not the longest piece of work
-// of the launch by far: every slice pays a tile's set-up, and the release / acquire around its ticket writes back and
-// invalidates the L2 of its XCD (config 5, whose fullest bins hold 10 to 30 thousand entries: tile_blend 1.16 -> 1.46 ms
-// with 8 192, 1.24 with 16 384, unchanged with 32 768).
-constexpr int kSliceEntries = 32768;
+// A bin with more than kSplitFrom slices' worth of entries is split in slices of kSliceEntries.  Splitting a bin that is
+// not by far the longest piece of work of its launch only costs (a tile's set-up per slice, and the release / acquire
+// around its ticket, which writes back and invalidates the L2 of its XCD: config 5, whose fullest bins hold 10 to 30
+// thousand entries, lost 0.3 ms per tile kernel when they were split), and the rows are handed out as the bins come:
+// those bins would take them from the ones that need them.
+constexpr int kSliceEntries = 8192;
+constexpr int kSplitFrom    = 4;
 inline int slice_row_floats(int C) { return (1 << (kTileShiftX + kTileShiftY)) * 2 * (C + 1); }
 // rows for the slices of split bins: what a cloud of n points in B views can fill at the default slice size
 inline int slice_rows(long long n, int B)

@@ -474,9 +474,9 @@ def test_tile_path_images_are_bit_identical_from_run_to_run():
 def test_full_bins_are_split_between_workgroups(oracle_mod, monkeypatch, forward_path, slice_entries, channels,
                                                 collect_stats):
     """A cloud that covers a few tiles only (the camera far away) puts tens of thousands of entries into one bin; bins
-    above ADOP_TILE_SLICE entries (32768 by default, read at every call) are split in slices that as many workgroups take,
-    the last of which merges their rows.  Forced here on small scenes: with 64 and 7 entries per slice nearly every bin
-    is split (up to 1023 slices a bin), with 1 the 1024 rows run out and most bins stay whole.  Forward and backward
+    above four times ADOP_TILE_SLICE entries (8192 by default, read at every call) are split in slices of that size that
+    as many workgroups take, the last of which merges their rows.  Forced here on small scenes: with 64 and 7 entries
+    per slice most bins are split (up to 1023 slices a bin), with 1 the rows run out and most bins stay whole.  Forward and backward
     through the tile path still equal the checker (packed depth bit for bit), with and without the counters, for the
     vectorised channel counts and the generic one."""
     from adop_amd import scenes
