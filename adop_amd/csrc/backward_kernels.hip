@@ -962,17 +962,112 @@ __device__ static void finalize_block(const FinalizeArg& a, double* sh, double* 
 // vec3 view (element t = floats 3t..3t+2 divided by count[t]); mode 1 normalises row t by count[t].
 // Fused with the reduction of the partial rows, which then costs no launch of its own and hides behind the
 // normalisation.  One workgroup reads the ~400 KB of partial rows in 16 us when nothing else runs and in ~50 us next
-// to the normalisation's traffic, so with point gradients the reduction has two stages: workgroups 0..kFinalizeParts-1
-// each reduce a slice of the rows to one row, and the one that finishes last (ticket counter) reduces those rows, in
-// their fixed order, and writes the outputs.  The other workgroups normalise.  Without point gradients (n = 0) a
-// single workgroup of NT = kFinalizeBlock threads does the whole reduction.
+// to the normalisation's traffic, so with point gradients the reduction has two stages: kFinalizeParts workgroups for
+// the background sums and as many for every view each reduce a slice of the partial rows to one row (a workgroup
+// that walked the views one after the other spent 2 to 3 us on each: 40 us for a batch of 16), and the one that
+// finishes last (ticket counter) reduces those rows, in their fixed order, and writes the outputs.  The other
+// workgroups normalise.  Without point gradients (n = 0) a single workgroup of NT = kFinalizeBlock threads does the
+// whole reduction.
+// The rows of the first stage go from their writers to the last workgroup through agent-scope atomic stores and
+// loads (past the L2 of the XCD, which is not coherent with the others'), the stores waited for before the ticket is
+// taken: a release / acquire pair around the ticket would write back and invalidate the whole L2 of the XCD, once per
+// workgroup, under the normalisation's traffic.
 constexpr int kNormPer = 4;  // point-gradient rows per thread of the normalisation
+
+__device__ __forceinline__ void mini_store(double* p, double v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ double mini_load(const double* p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Second stage: the kFinalizeParts rows of the background sums and of every view -> the outputs (as finalize_block).
+template <int NT>
+__device__ static void finalize_last(const FinalizeArg& a, const double* bg_m, const double* pt_m, double* sh,
+                                     double* s_small)
+{
+    const int B = a.B, C = a.C, num_poses = a.num_poses, num_cameras = a.num_cameras, cols = a.cols;
+    double* scratch = (num_poses * 7 + num_cameras * (cols + 1) <= kFinalizeSmall) ? s_small : a.scratch;
+    if ((int)threadIdx.x < kMaxChannels)
+    {
+        double t = 0;
+        for (int r = 0; r < kFinalizeParts; ++r) t += mini_load(bg_m + r * kMaxChannels + threadIdx.x);
+        if ((int)threadIdx.x < C) a.gbg[threadIdx.x] = (float)t;
+    }
+    if (!a.gpose && !a.gintr) return;
+    double* sp = scratch;
+    double* si = scratch + (size_t)num_poses * 7;
+    for (int k = threadIdx.x; k < num_poses * 7 + num_cameras * (cols + 1); k += NT) scratch[k] = 0;
+    __syncthreads();
+    constexpr int VIEWS = NT / 32;  // views summed side by side: thread = (view, value)
+    for (int b0 = 0; b0 < B; b0 += VIEWS)
+    {
+        const int b = b0 + (int)threadIdx.x / 32, q = threadIdx.x % 32;
+        double t = 0;
+        if (b < B && q < kAcc)
+            for (int r = 0; r < kFinalizeParts; ++r) t += mini_load(pt_m + ((size_t)b * kFinalizeParts + r) * kPartialStride + q);
+        sh[threadIdx.x] = t;
+        __syncthreads();
+        // the views of the chunk one after the other: distinct threads write distinct addresses, the order of the
+        // additions to a pose or camera shared by views is that of the views
+        if ((int)threadIdx.x < kAcc)
+        {
+            const int qq = threadIdx.x;
+            for (int v = 0; v < VIEWS && b0 + v < B; ++v)
+            {
+                const double tv     = sh[v * 32 + qq];
+                const ViewConst& vc = a.views[b0 + v];
+                if (qq < 7)
+                    sp[(size_t)vc.image_index * 7 + qq] += tv;
+                else if (qq == 7)
+                    si[(size_t)vc.camera_index * (cols + 1) + cols] += tv;
+                else if (qq - 8 < cols)
+                    si[(size_t)vc.camera_index * (cols + 1) + (qq - 8)] += tv;
+            }
+        }
+        __syncthreads();
+    }
+    if (a.gpose)
+    {
+        for (int f = threadIdx.x; f < num_poses; f += NT)
+        {
+            float c          = (float)sp[(size_t)f * 7 + 6];
+            a.gpose_count[f] = c;
+            for (int k = 0; k < 6; ++k)
+            {
+                double t                   = sp[(size_t)f * 7 + k];
+                a.gpose[(size_t)f * 6 + k] = (c > 0) ? t / (double)c : t;
+            }
+        }
+    }
+    if (a.gintr)
+    {
+        const int total = num_cameras * cols;
+        for (int k = threadIdx.x; k < total; k += NT)
+        {
+            float v     = (float)si[(size_t)(k / cols) * (cols + 1) + (k % cols)];
+            const int t = a.normalize_mode == 0 ? k / 13 : k / cols;
+            if (t < num_cameras)
+            {
+                const float c = (float)si[(size_t)t * (cols + 1) + cols];
+                if (c > 0) v = v / c;
+            }
+            a.gintr[k] = v;
+        }
+        for (int k = threadIdx.x; k < num_cameras; k += NT) a.gintr_count[k] = (float)si[(size_t)k * (cols + 1) + cols];
+    }
+}
+
+// workgroups of the first stage of finalize_body for a batch of B views
+static int finalize_first_stage(int B) { return kFinalizeParts * (1 + B); }
 
 template <int NT>
 __device__ __forceinline__ void finalize_body(FinalizeArg a, float* __restrict__ g, const float* __restrict__ count, int n,
                                               int mode)
 {
-    const int first_stage = n > 0 ? kFinalizeParts : 0;
+    const int first_stage = n > 0 ? kFinalizeParts * (1 + a.B) : 0;
     if ((int)blockIdx.x < (first_stage ? first_stage : 1))
     {
         __shared__ double sh[NT];
@@ -980,9 +1075,11 @@ __device__ __forceinline__ void finalize_body(FinalizeArg a, float* __restrict__
         __shared__ int s_last;
         if (first_stage)
         {
-            const int r  = blockIdx.x;
-            double* bg_m = a.mini;
-            double* pt_m = a.mini + kFinalizeParts * kMaxChannels;
+            const int r     = blockIdx.x % kFinalizeParts;
+            const int which = blockIdx.x / kFinalizeParts;  // 0: background sums; 1 + b: view b
+            double* bg_m    = a.mini;
+            double* pt_m    = a.mini + kFinalizeParts * kMaxChannels;
+            if (which == 0)
             {
                 const int c = threadIdx.x % kMaxChannels, k0 = threadIdx.x / kMaxChannels;
                 constexpr int GR = NT / kMaxChannels;
@@ -997,12 +1094,12 @@ __device__ __forceinline__ void finalize_body(FinalizeArg a, float* __restrict__
                 {
                     double t = 0;
                     for (int q = 0; q < GR; ++q) t += sh[q * kMaxChannels + threadIdx.x];
-                    bg_m[r * kMaxChannels + threadIdx.x] = t;
+                    mini_store(bg_m + r * kMaxChannels + threadIdx.x, t);
                 }
-                __syncthreads();
             }
-            for (int b = 0; b < a.B; ++b)
+            else
             {
+                const int b = which - 1;
                 const int q = threadIdx.x % 32, k0 = threadIdx.x / 32;
                 constexpr int GR = NT / 32;
                 const int lo = (int)((long long)a.pt_blocks * r / kFinalizeParts);
@@ -1018,20 +1115,16 @@ __device__ __forceinline__ void finalize_body(FinalizeArg a, float* __restrict__
                 {
                     double t = 0;
                     for (int w = 0; w < GR; ++w) t += sh[w * 32 + threadIdx.x];
-                    pt_m[((size_t)b * kFinalizeParts + r) * kPartialStride + threadIdx.x] = t;
+                    mini_store(pt_m + ((size_t)b * kFinalizeParts + r) * kPartialStride + threadIdx.x, t);
                 }
-                __syncthreads();
             }
-            __threadfence();  // the rows of this workgroup are visible before its ticket is
-            __syncthreads();
-            if (threadIdx.x == 0) s_last = atomicAdd(a.ticket, 1u) == (uint32_t)(kFinalizeParts - 1);
+            __builtin_amdgcn_s_waitcnt(0);  // the stores of this lane have been acknowledged ...
+            __syncthreads();                // ... and those of the workgroup, before its ticket is taken
+            if (threadIdx.x == 0) s_last = atomicAdd(a.ticket, 1u) == (uint32_t)(first_stage - 1);
             __syncthreads();
             if (!s_last) return;
-            __threadfence();
-            a.bg_partial = bg_m;
-            a.bg_blocks  = kFinalizeParts;
-            a.pt_partial = pt_m;
-            a.pt_blocks  = kFinalizeParts;
+            finalize_last<NT>(a, bg_m, pt_m, sh, s_small);
+            return;
         }
         finalize_block<NT>(a, sh, s_small);
         return;
@@ -1227,7 +1320,7 @@ void launch_finalize(const ViewConst* views, int B, int C, const double* bg_part
                            g->grad_points, g->grad_points_count, normalize_mode);
     }
     else
-        hipLaunchKernelGGL(finalize_normalize_kernel, dim3(kFinalizeParts + (n + kBlock * kNormPer - 1) / (kBlock * kNormPer)), dim3(kBlock), 0, st, a,
+        hipLaunchKernelGGL(finalize_normalize_kernel, dim3(finalize_first_stage(B) + (n + kBlock * kNormPer - 1) / (kBlock * kNormPer)), dim3(kBlock), 0, st, a,
                            g->grad_points, g->grad_points_count, n, normalize_mode);
 }
 
