@@ -1094,6 +1094,6 @@ const char* adop_version(void)
 {
     // "kernels N" names the state of the kernels' memory behaviour: it goes up whenever a change moves a kernel's bytes,
     // so that traffic figures measured for one state (rocprofv3 counters) are not quoted for another.
-    return "adop_raster 0.2 (gfx950) kernels 6";
+    return "adop_raster 0.2 (gfx950) kernels 7";
 }
 }  // extern "C"
