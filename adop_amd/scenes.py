@@ -306,6 +306,27 @@ def orbit_pose(frame, radius=12.0, deg_per_frame=1.2):
     return look_at_view((radius * np.sin(a), 0.0, -radius * np.cos(a)))
 
 
+def training_batch(n=10_000_000, frames=4, per_frame=4, crop=512, seed=1, point_order="morton"):
+    """A training batch as the reference forms it (configs/train_boat.ini:5-6, Dataset.cpp:107-227): `frames` frames
+    x `per_frame` random crops of crop x crop (zoom 0.75 .. 1.5) of the config-3 scene, all gradients."""
+    hs = config3(n=n, point_order=point_order)
+    g = np.random.default_rng(seed)
+    hs.poses_se3 = np.stack([orbit_pose(f, radius=3.0, deg_per_frame=20.0) for f in range(frames)])
+    views = []
+    for f in range(frames):
+        for _ in range(per_frame):
+            zoom = float(g.uniform(0.75, 1.5))
+            # window of crop / zoom source pixels somewhere inside the 1920 x 1080 frame
+            src = crop / zoom
+            x0 = float(g.uniform(0, 1920 - src))
+            y0 = float(g.uniform(0, 1080 - src))
+            views.append(make_view(crop, crop, image_index=f, crop=(zoom, zoom, -x0 * zoom, -y0 * zoom, 0.0)))
+    hs.views = views
+    hs.dropout = bernoulli_mask(2, len(views), hs.num_points, 0.25)
+    hs.name = "crops"
+    return hs
+
+
 def config4(n=100_000_000, w=1920, h=1080, levels=5, frames=300, seed=0, point_order="morton"):
     """Viewer path: uniform points in a 10^3 volume, fp16-stored descriptors, 300-frame orbit of radius 12."""
     g = rng(seed)

@@ -197,29 +197,11 @@ def bench_preprocess(args):
 
 
 def crops_scene(args):
-    """A training batch as the reference forms it (configs/train_boat.ini:5-6, Dataset.cpp:107-227): 4 frames x 4
-    random crops of 512 x 512 (zoom 0.75 .. 1.5) of the config-3 scene."""
-    import numpy as np
+    """A training batch as the reference forms it: 4 frames x 4 random crops of 512 x 512 of the config-3 scene."""
     from adop_amd import scenes
 
     kw = {"n": args.points} if args.points else {}
-    hs = scenes.config3(point_order=args.point_order, **kw)
-    g = np.random.default_rng(1)
-    frames, per_frame, cw = 4, 4, 512
-    hs.poses_se3 = np.stack([scenes.orbit_pose(f, radius=3.0, deg_per_frame=20.0) for f in range(frames)])
-    views = []
-    for f in range(frames):
-        for _ in range(per_frame):
-            zoom = float(g.uniform(0.75, 1.5))
-            # window of cw / zoom source pixels somewhere inside the 1920 x 1080 frame
-            src = cw / zoom
-            x0 = float(g.uniform(0, 1920 - src))
-            y0 = float(g.uniform(0, 1080 - src))
-            views.append(scenes.make_view(cw, cw, image_index=f, crop=(zoom, zoom, -x0 * zoom, -y0 * zoom, 0.0)))
-    hs.views = views
-    hs.dropout = scenes.bernoulli_mask(2, len(views), hs.num_points, 0.25)
-    hs.name = "crops"
-    return hs
+    return scenes.training_batch(point_order=args.point_order, **kw)
 
 
 def run_workload(args, workload, steps, warmup, lib):
