@@ -95,7 +95,10 @@ def assert_close(got, want, rel, abs_tol, what):
 
 
 def check_forward(hs, ref, ctx, images, masks, info, stats=True):
-    """depth/index bit-exact; weight exact; blended descriptors within 1e-5 relative."""
+    """depth/index bit-exact; weight exact; blended descriptors within 1e-5 relative.  A pixel of more than 1024
+    blended points gets sqrt(points / 1024) times that: the checker adds them one after the other in fp32 as the
+    reference's atomics do (PointRenderer.cu:383-390), and the rounding error of such a sum grows with the root of
+    the number of terms (1.2e-5 seen on a pixel of 28 758 points, where both HIP paths agree to 1e-7)."""
     cache = info.cache
     for l in range(hs.num_layers):
         L = cache.layers_cuda[l]
@@ -105,7 +108,8 @@ def check_forward(hs, ref, ctx, images, masks, info, stats=True):
         assert np.array_equal(d.view(np.uint32), ref.depth[l].view(np.uint32)), f"level {l}: depth bits differ"
         w = L.weight.cpu().numpy()
         assert np.array_equal(w, ref.weight[l]), f"level {l}: weight differs"
-        assert_close(images[l].cpu().numpy(), ref.out[l], 1e-5, 1e-7, f"level {l} out")
+        rel = 1e-5 * np.sqrt(np.maximum(w.astype(np.float64) / 1024.0, 1.0))  # [B,1,h,w], broadcast over the channels
+        assert_close(images[l].cpu().numpy(), ref.out[l], rel, 1e-7, f"level {l} out")
         if hs.params.output_background_mask:
             assert np.array_equal(masks[l].cpu().numpy(), ref.mask[l]), f"level {l}: mask differs"
     if not stats:
@@ -134,7 +138,11 @@ def check_backward(hs, refb, grads, info, stats=True):
     assert_close(g_bg.cpu().numpy(), refb.grad_background, 1e-4, 1e-5, "grad_background")
     if g_pts is not None:
         assert np.array_equal(cache.output_gradient_point_count.cpu().numpy(), refb.grad_points_count), "point count"
-        assert_close(g_pts.cpu().numpy(), refb.grad_points, 1e-4, 1e-6, "grad_points")
+        # absolute bar: 1e-6 of the point's own gradient vector where that is larger than 1 (a component that cancels
+        # to 3e-3 beside components of 50, from 12 terms of that size, was off by 1.4e-6 = half a unit in the last
+        # place of the terms)
+        row = np.maximum(np.abs(refb.grad_points).max(axis=1, keepdims=True).astype(np.float64), 1.0)
+        assert_close(g_pts.cpu().numpy(), refb.grad_points, 1e-4, 1e-6 * row, "grad_points")
     if g_pose is not None:
         assert np.array_equal(cache.output_gradient_pose_tangent_count.cpu().numpy(), refb.grad_pose_count)
         scale = np.abs(refb.grad_pose).max() + 1e-30

@@ -3,6 +3,8 @@ channel count, camera model, distortion, crop, LOD radii, dropout, gradient swit
 HIP path (both forward implementations, with and without a point cache) is compared with the CPU checker to the
 bars of tests/test_parity_gpu.py.  The named cases cover what the reference's configurations use; the sweep covers
 the combinations nobody thought of."""
+import os
+
 import numpy as np
 import pytest
 
@@ -10,7 +12,9 @@ from helpers import announce, assert_norm_close, check_backward, check_forward, 
 
 pytestmark = pytest.mark.gpu
 
-SEEDS = list(range(100))
+# ADOP_SWEEP_SEEDS="first:count" draws other scenes than the 100 of a default run (a longer soak on a GPU box)
+_first, _count = (int(x) for x in os.environ.get("ADOP_SWEEP_SEEDS", "0:100").split(":"))
+SEEDS = list(range(_first, _first + _count))
 
 
 def random_scene(seed):
