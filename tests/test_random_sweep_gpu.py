@@ -41,7 +41,7 @@ def random_scene(seed):
             hs.intrinsics[0, 4] = g.uniform(-0.3, 0.3)  # shear
         hs.params.dist_cutoff = float(g.choice([1.0e6, 1.5, 0.8]))
     # descriptors: channel count, storage, texel index
-    C = int(g.choice([1, 3, 4, 8]))
+    C = int(g.choice([1, 3, 4, 8, 1, 3, 4, 8, 2, 5, 7, 12, 16]))  # 4 and 8 have kernels of their own; 16 is the limit
     kind = str(g.choice(["identity", "permuted", "shared"]))
     ntex = n if kind != "shared" else max(1, n // 2)
     tex = g.random((C, ntex), dtype=np.float32)
