@@ -149,6 +149,22 @@ def test_more_views_than_one_constant_chunk(oracle_mod):
     _fwd_bwd(hs, oracle_mod)
 
 
+@pytest.mark.parametrize("collect_stats", [True, False], ids=["counters", "plain"])
+def test_more_views_than_bits_of_the_view_masks(oracle_mod, collect_stats):
+    """70 crop windows: the runs of 64 points that miss a window are marked (and their records left unwritten) for the
+    first 64 views of a call only; the loops that jump from one live view to the next keep their masks in 64 bits."""
+    from adop_amd import scenes
+
+    announce(f"config2 20k pts B=70 crop windows 96x80 L3 fwd+bwd ghost, counters={collect_stats}")
+    hs = scenes.config2(n=20_000, w=96, h=80, levels=3, batch=70, seed=70)
+    g = np.random.default_rng(70)
+    for v in hs.views:
+        s = float(g.uniform(0.8, 3.0))
+        v.crop_fx, v.crop_fy = s, s
+        v.crop_cx, v.crop_cy = float(g.uniform(-2.0, 0.2) * 96), float(g.uniform(-2.0, 0.2) * 80)
+    _fwd_bwd(hs, oracle_mod, collect_stats=collect_stats, poison=not collect_stats)
+
+
 @pytest.mark.parametrize("concurrent", ["0", "1"], ids=["per_view", "concurrent"])
 @pytest.mark.parametrize("batch", [2, 5, 13, 24, 25, 34])
 def test_spatial_gradients_per_view_and_of_all_views_at_once(oracle_mod, monkeypatch, concurrent, batch):
