@@ -1,6 +1,8 @@
 """Random sweep over the preprocessing kernels: every seed draws a cloud (size, shape, exact duplicates, stray points,
 degenerate axes), a neighbour rank and radii, and the device results are compared with the CPU checker: neighbour
 distances and Morton codes bit for bit, the close-point filter equal to the sequential sweep."""
+import os
+
 import numpy as np
 import pytest
 
@@ -42,7 +44,11 @@ def random_cloud(seed):
     return g, p, rank, what
 
 
-@pytest.mark.parametrize("seed", range(60))
+# (ADOP_PREPROCESS_SWEEP_SEEDS="first:count" draws other clouds than the 60 of a default run)
+_first, _count = (int(x) for x in os.environ.get("ADOP_PREPROCESS_SWEEP_SEEDS", "0:60").split(":"))
+
+
+@pytest.mark.parametrize("seed", range(_first, _first + _count))
 def test_random_cloud(seed):
     import torch
     import oracle.preprocess as op
