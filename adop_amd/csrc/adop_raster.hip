@@ -137,6 +137,14 @@ constexpr int kTileLevels = 2;  // levels the tile path renders in LDS (a point 
 constexpr int kTilePathMinPoints = 1 << 16;
 constexpr int kTilePathMaxPointsPerPixel = 16;
 constexpr int kWindowCloudShare = 16;  // a crop window is taken to see 1/16 of the cloud
+// A tile is one workgroup from its first entry to its last: a call with few tiles leaves most of the GPU idle in the
+// tile kernels, whose time per point then grows like 1 / tiles (measured on Morton-ordered clouds, forward:
+// 18 us per million points from ~4 000 tiles up, 75 us at 1 024 tiles, 180 us at 256; the direct path: 25 us whatever
+// the image), while the direct path pays ~50 us more per call for its accumulators of all levels.
+constexpr int kTilePathMinTiles = 512;       // below: the direct path (256 tiles: equal on an ordered cloud, 1.7 x faster on an unordered one)
+constexpr int kTilePathEnoughTiles = 2800;   // from here on the tile path is the faster one per point
+constexpr double kTilePathUsPerMTiles = 73728.0;  // us per million points x tiles of the call
+constexpr double kDirectPathUsPerM = 25.0, kDirectPathFixedUs = 50.0;
 constexpr int kConcurrentMaxPoints = 4000000;  // backward: full views of a larger cloud get a spatial-gradient launch each
 
 size_t max_tiles(int B, int w0, int h0)
@@ -483,8 +491,13 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
         bool windows = num_views > 1;
         for (int b = 0; b < num_views; ++b) windows = windows && (views[b].crop_cx != 0.f || views[b].crop_cy != 0.f);
         const size_t per_pixel = (size_t)kTilePathMaxPointsPerPixel * (windows ? kWindowCloudShare : 1);
+        const size_t tiles     = max_tiles(num_views, views[0].w, views[0].h);
+        const double seen      = (double)scene->num_points / (windows ? kWindowCloudShare : 1);  // points a view handles
+        const bool filled      = tiles >= (size_t)kTilePathEnoughTiles ||
+                            seen * 1e-6 * (kTilePathUsPerMTiles / (double)tiles - kDirectPathUsPerM) <= kDirectPathFixedUs;
         path = (scene->num_points >= kTilePathMinPoints &&
-                (size_t)scene->num_points <= per_pixel * views[0].w * views[0].h)
+                (size_t)scene->num_points <= per_pixel * views[0].w * views[0].h && tiles >= (size_t)kTilePathMinTiles &&
+                filled)
                    ? 2
                    : 1;
     }
