@@ -2,6 +2,8 @@
 // top of libadop_raster.so.  Replaces src/lib/rendering/PointRenderer.cu in an ADOP build for ROCm.
 #include "PointRendererHip.h"
 
+#include <iostream>
+
 #include <c10/hip/HIPStream.h>
 
 namespace
@@ -232,6 +234,13 @@ std::pair<std::vector<torch::Tensor>, std::vector<torch::Tensor>> BlendPointClou
     }
     Check(adop_forward(&scene, views.data(), (int)views.size(), &rp, &fb, cache.workspace.data_ptr(),
                        (size_t)cache.workspace.numel(), nullptr, CurrentStream()));
+
+    if (info->params.debug_print_num_rendered_points)  // PointRenderer.cu:1502-1512
+    {
+        double weight_sum = 0;
+        for (auto& l : cache.layers_cuda) weight_sum += l.weight.sum().item().toFloat();
+        std::cout << "# Rasterized Points = " << (int)weight_sum << std::endl;
+    }
 
     if (ctx)
     {

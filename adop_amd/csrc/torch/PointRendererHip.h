@@ -53,6 +53,7 @@ struct RenderParams
     float dist_cutoff                    = 2;
     bool output_background_mask          = false;
     float output_background_mask_value   = 0;
+    bool debug_print_num_rendered_points = false;  // prints the sum of the weights after a forward (:1502-1512)
     // not in the reference: 0 = NormalizeGradient exactly as the reference launches it, 1 = row-wise
     int normalize_mode = 0;
 };

@@ -57,6 +57,7 @@ static RenderParams ParamsFromDict(const py::dict& d)
     GET(output_background_mask, bool);
     GET(output_background_mask_value, float);
     GET(normalize_mode, int);
+    GET(debug_print_num_rendered_points, bool);
 #undef GET
     return p;
 }

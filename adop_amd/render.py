@@ -123,6 +123,8 @@ class NeuralRenderInfo:
     dropout_points: Optional[torch.Tensor] = None
     dropout: float = 0.0
     collect_stats: bool = False
+    # RenderParams::debug_print_num_rendered_points (Settings.h:43): the sum of the weights after a forward pass
+    debug_print_num_rendered_points: bool = False
     # NeuralRenderInfo::train (RenderInfo.h): a backward pass may follow, so the forward pass leaves the projected
     # points in a tensor of its own (saved like depth / weight) instead of the workspace
     train: bool = True
@@ -250,6 +252,11 @@ def BlendPointCloudForward(ctx, info, build=True):
     rc = cache.lib.adop_forward(C.byref(s), cache.views_array(), cache.num_batches, C.byref(info.params), C.byref(fb),
                                 C.c_void_p(cache.workspace.data_ptr()), cache.workspace.numel(), stats, _stream_ptr())
     _check(rc, cache.lib)
+    if info.debug_print_num_rendered_points:  # PointRenderer.cu:1502-1512
+        weight_sum = 0.0
+        for L in cache.layers_cuda:
+            weight_sum += float(L.weight.sum().item())
+        print(f"# Rasterized Points = {int(weight_sum)}", flush=True)
     if ctx is not None:
         save = []
         for L in cache.layers_cuda:

@@ -139,6 +139,27 @@ def test_backward_without_point_gradients(oracle_mod):
     _fwd_bwd(hs, oracle_mod, needs=(False, True, True))
 
 
+def test_debug_print_num_rendered_points(oracle_mod, capsys):
+    """RenderParams::debug_print_num_rendered_points (PointRenderer.cu:1502-1512): the sum of the weights after a
+    forward pass, printed as the reference prints it."""
+    import torch
+    import helpers
+    from adop_amd import render, scenes
+
+    announce("debug_print_num_rendered_points")
+    hs = scenes.config3(n=100_000, w=240, h=136, channels=4)
+    ref = oracle_mod.forward(hs)
+    hs.params.forward_path = helpers.FORWARD_PATH
+    info = render.NeuralRenderInfo(scene=render.NeuralScene.from_host(hs, "cuda"), images=list(hs.views),
+                                   params=hs.params, num_layers=hs.num_layers, cache=render.PointRendererCache(),
+                                   dropout_points=torch.from_numpy(hs.dropout), train=False,
+                                   debug_print_num_rendered_points=True)
+    capsys.readouterr()
+    render.BlendPointCloudForward(None, info)
+    want = sum(int(a) for a in ref.stats.accepted[: hs.num_layers])
+    assert f"# Rasterized Points = {want}" in capsys.readouterr().out
+
+
 def test_more_views_than_one_constant_chunk(oracle_mod):
     """34 views: the per-view constants take the chunked path (32 per launch), the descriptor pass fills 34 work
     queues, every view accumulates into the same point / pose / intrinsics gradients."""

@@ -55,7 +55,7 @@ def _scene(mod, hs, env=None):
     return s, t
 
 
-def test_point_render_autograd_matches_checker(oracle_mod):
+def test_point_render_autograd_matches_checker(oracle_mod, capfd):
     import torch
     from adop_amd import scenes
 
@@ -67,8 +67,11 @@ def test_point_render_autograd_matches_checker(oracle_mod):
     hs.params.output_background_mask = 1
     ref = oracle_mod.forward(hs)
     s, t = _scene(mod, hs)
-    outs = mod.render(s, _views(hs), _params(hs, dropout=0.0), hs.num_layers)
+    capfd.readouterr()
+    outs = mod.render(s, _views(hs), _params(hs, dropout=0.0, debug_print_num_rendered_points=True), hs.num_layers)
     L = hs.num_layers
+    # RenderParams::debug_print_num_rendered_points (PointRenderer.cu:1502-1512): the sum of the weights of all levels
+    assert f"# Rasterized Points = {sum(int(a) for a in ref.stats.accepted[:L])}" in capfd.readouterr().out
     assert len(outs) == 2 * L  # images then masks (RenderInfo.cpp:39-41)
     for l in range(L):
         assert_close(outs[l].detach().cpu().numpy(), ref.out[l], 1e-5, 1e-7, f"out {l}")
