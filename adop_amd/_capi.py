@@ -52,6 +52,7 @@ class RenderParams(C.Structure):
         ("output_background_mask_value", C.c_float),
         ("normalize_mode", C.c_int32),
         ("forward_path", C.c_int32),
+        ("skip_points", C.c_int32),
     ]
 
 

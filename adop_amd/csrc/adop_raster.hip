@@ -243,9 +243,10 @@ adop_status validate(const adop_scene* s, const adop_view* views, int B, const a
     if (B < 1) return fail(ADOP_INVALID_ARG, "num_views must be >= 1");  // SAIGA_ASSERT(num_batches > 0), :909
     if (fb->num_layers < 1 || fb->num_layers > ADOP_MAX_LAYERS)
         return fail(ADOP_UNSUPPORTED_LAYERS, "invalid number of layers");  // :1199
-    if (s->num_points < 0 || !s->position || !s->index) return fail(ADOP_INVALID_ARG, "point cloud missing");
+    if (s->num_points < 0 || (s->num_points > 0 && (!s->position || !s->index)))
+        return fail(ADOP_INVALID_ARG, "point cloud missing");
     if (s->num_points > (1 << 30)) return fail(ADOP_INVALID_ARG, "at most 2^30 points per call");
-    if (rp->check_normal && !s->normal)
+    if (rp->check_normal && !s->normal && s->num_points > 0)
         return fail(ADOP_INVALID_ARG, "check_normal requires normals");  // NeuralScene.cpp:28
     if (s->num_channels < 1 || s->num_channels > kMaxChannels)
         return fail(ADOP_INVALID_ARG, "num_channels must be in [1,16]");
@@ -445,12 +446,24 @@ size_t adop_workspace_size(const adop_scene* scene, int32_t num_views, int32_t n
     return layout(scene, num_views, num_layers, w, h).total;
 }
 
+// RenderParams::render_points == false (PointRenderer.cu:1417,1433): the forward pass runs on an empty cloud (its
+// workspace layout lies inside the one the caller sized for the whole cloud).
+static const adop_scene* leave_out_points(const adop_scene* scene, adop_scene* copy)
+{
+    *copy                   = *scene;
+    copy->num_points        = 0;
+    copy->index_is_identity = 0;
+    return copy;
+}
+
 adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_t num_views,
                          const adop_render_params* params, const adop_forward_buffers* buffers, void* workspace,
                          size_t workspace_bytes, adop_stats* stats, void* hip_stream)
 {
     adop_status st = validate(scene, views, num_views, params, buffers);
     if (st != ADOP_OK) return st;
+    adop_scene without_points;
+    if (params->skip_points) scene = leave_out_points(scene, &without_points);
     WorkspaceLayout wl = layout(scene, num_views, buffers->num_layers, views[0].w, views[0].h);
     if (!workspace || workspace_bytes < wl.total) return fail(ADOP_WORKSPACE_TOO_SMALL, "workspace too small");
     hipStream_t stream = (hipStream_t)hip_stream;
@@ -629,6 +642,9 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     if (st != ADOP_OK) return st;
     Levels lv   = make_levels(scene, num_views, fwd, grads);
     CloudArg pc = make_cloud(scene, fwd);
+    // (a forward pass that left the points out wrote no projected points; the backward pass runs over the cloud all
+    // the same, as the reference's does, PointRenderer.cu:1598-1604, against the empty depth and weight buffers)
+    if (params->skip_points) pc.cache = nullptr;
     ParamArg rp = make_params(params);
     const int C = scene->num_channels;
     const int N = scene->num_points;

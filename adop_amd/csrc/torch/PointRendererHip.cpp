@@ -66,6 +66,7 @@ adop_render_params MakeParams(const RenderParams& p)
     o.output_background_mask       = p.output_background_mask;
     o.output_background_mask_value = p.output_background_mask_value;
     o.normalize_mode               = p.normalize_mode;
+    o.skip_points                  = p.render_points ? 0 : 1;  // PointRenderer.cu:1417,1433
     return o;
 }
 

@@ -45,6 +45,7 @@ static RenderParams ParamsFromDict(const py::dict& d)
     if (d.contains(#name)) p.name = d[#name].cast<type>()
     GET(test_backward_mode, int);
     GET(check_normal, bool);
+    GET(render_points, bool);
     GET(super_sampling, bool);
     GET(dropout, float);
     GET(depth_accept, float);

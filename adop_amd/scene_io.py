@@ -72,6 +72,8 @@ def RenderParamsFromIni(path):
             setattr(p, key, float(sec[key]))
     if "test_backward_mode" in sec:
         p.test_backward_mode = int(sec["test_backward_mode"])
+    if "render_points" in sec:
+        p.skip_points = 0 if _bool(sec["render_points"]) else 1
     return p, float(sec.get("dropout", 0.25))
 
 

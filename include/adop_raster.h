@@ -88,6 +88,12 @@ typedef struct adop_render_params
      * as written); 2: through screen-space tile bins (the fine levels are rendered in LDS).  0 decides by the number
      * of points per pixel of the whole image; when the cloud covers only a small part of the image, 1 is the faster. */
     int32_t forward_path;
+    /* 1: adop_forward leaves the point cloud out (RenderParams::render_points == false, Settings.h:25;
+     * PointRenderer.cu:1417,1433 skip DepthPrepassMulti and RenderForwardMulti): every pixel is empty and holds the
+     * background colour.  adop_backward still runs over the cloud, as the reference's does (:1598-1604), against those
+     * empty buffers (and ignores point_cache, which such a forward does not write).  0 (the reference's default,
+     * render_points = true): rendered.  A cloud may also be empty (num_points == 0, its pointers may be NULL). */
+    int32_t skip_points;
 } adop_render_params;
 
 /* Inputs owned by NeuralScene: NeuralPointCloudCuda + NeuralTexture + PoseModule + IntrinsicsModule. */

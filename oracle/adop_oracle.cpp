@@ -710,7 +710,7 @@ int oracle_forward(const adop_scene* s, const adop_view* views, int B, const ado
 {
     const int L = fb->num_layers;
     const int C = s->num_channels;
-    const int N = s->num_points;
+    const int N = rp->skip_points ? 0 : s->num_points;  // if (params.render_points), :1417,1433
     if (L < 1 || L > ADOP_MAX_LAYERS) return ADOP_UNSUPPORTED_LAYERS;
     if (stats) std::memset(stats, 0, sizeof(*stats));
 

@@ -67,6 +67,9 @@ def assert_norm_close(got, want, tol, what):
     """tensor-level bound: max|got-want| <= tol * max|want| (for sums whose terms cancel)."""
     got = np.asarray(got, np.float64)
     want = np.asarray(want, np.float64)
+    assert got.shape == want.shape, (what, got.shape, want.shape)
+    if want.size == 0:
+        return
     assert np.isfinite(got).all(), what + ": non-finite values"
     scale = np.abs(want).max()
     err = np.abs(got - want).max()
@@ -124,6 +127,8 @@ def count_misses(got, want, rel=1e-4, abs_tol=1e-6):
     """Elements outside |got-want| <= max(rel*|want|, abs_tol): (number, size, largest miss relative to max|want|)."""
     got = np.asarray(got, np.float64)
     want = np.asarray(want, np.float64)
+    if want.size == 0:
+        return 0, 0, 0.0
     err = np.abs(got - want)
     bad = err > np.maximum(rel * np.abs(want), abs_tol)
     worst = float(err[bad].max() / max(np.abs(want).max(), 1e-30)) if bad.any() else 0.0

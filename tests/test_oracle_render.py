@@ -340,6 +340,42 @@ def test_empty_and_degenerate_inputs(oracle_mod):
     assert all((o == 0).all() for o in r.out)
 
 
+def test_render_points_switched_off_and_empty_cloud(oracle_mod):
+    """render_points = false (PointRenderer.cu:1417,1433): the forward pass skips both point passes, so every pixel
+    is empty: clear depth, weight 0, background colour, mask value; the backward pass (which the reference runs over
+    the cloud all the same, :1598-1604) gives the closed form of CombineAndFillBackward for the background, nothing
+    for rendered points (w == 0 -> continue, :473) and a spatial gradient only to dropped points.  An empty cloud
+    renders the same images."""
+    hs = scenes.config3(n=3000, w=48, h=27, channels=3, levels=3, seed=4)
+    hs.params.output_background_mask = 1
+    hs.params.output_background_mask_value = 0.25
+    hs.background[:] = [0.1, 0.2, 0.3]
+    hs.params.skip_points = 1
+    r = oracle_mod.forward(hs)
+    for l in range(hs.num_layers):
+        assert (r.depth[l] == 100000.0).all() and (r.depth_index[l] == CLEAR).all() and (r.weight[l] == 0).all()
+        assert (r.mask[l] == 0.25).all()
+        for c in range(3):
+            assert (r.out[l][:, c] == hs.background[c]).all()
+    assert list(r.stats.visible[:3]) == [0, 0, 0] and list(r.stats.accepted[:3]) == [0, 0, 0]
+    G = scenes.upstream_grads(hs, 3)
+    b = oracle_mod.backward(hs, r, G)
+    want_bg = sum(g.astype(np.float64).sum(axis=(0, 2, 3)) for g in G)
+    assert b.grad_background == pytest.approx(want_bg, rel=1e-5)
+    assert (b.grad_texture == 0).all()
+    dropped = hs.dropout[0] == 1
+    assert (b.grad_points_count[~dropped] == 0).all() and b.grad_points_count[dropped].max() >= 1
+    # the same images from a cloud without points
+    hs.params.skip_points = 0
+    hs.position, hs.normal, hs.index = hs.position[:0].copy(), hs.normal[:0].copy(), hs.index[:0].copy()
+    hs.dropout = None
+    e = oracle_mod.forward(hs)
+    for l in range(hs.num_layers):
+        assert np.array_equal(e.out[l], r.out[l]) and np.array_equal(e.depth_index[l], r.depth_index[l])
+    be = oracle_mod.backward(hs, e, G)
+    assert be.grad_background == pytest.approx(want_bg, rel=1e-5) and be.grad_points.shape == (0, 4)
+
+
 # --------------------------------------------------------------------------------------------------
 # environment map
 # --------------------------------------------------------------------------------------------------

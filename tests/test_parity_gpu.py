@@ -139,6 +139,37 @@ def test_backward_without_point_gradients(oracle_mod):
     _fwd_bwd(hs, oracle_mod, needs=(False, True, True))
 
 
+@pytest.mark.parametrize("collect_stats", [True, False], ids=["counters", "plain"])
+def test_render_points_switched_off(oracle_mod, collect_stats):
+    """RenderParams::render_points = false (PointRenderer.cu:1417,1433): the forward pass leaves the cloud out, every
+    pixel holds the background; the backward pass still runs over the cloud (:1598-1604) against the empty depth and
+    weight buffers, where only dropped points receive a (ghost) gradient."""
+    from adop_amd import scenes
+
+    announce(f"config3 reduced 100k pts 240x136, render_points = false, counters={collect_stats}")
+    hs = scenes.config3(n=100_000, w=240, h=136, channels=4)
+    hs.params.skip_points = 1
+    hs.params.output_background_mask = 1
+    hs.background[:] = [0.1, 0.2, 0.3, 0.4]
+    ref = oracle_mod.forward(hs)
+    assert all(float(w.max()) == 0.0 for w in ref.weight) and float(ref.out[0][0, 2].min()) == np.float32(0.3)
+    _fwd_bwd(hs, oracle_mod, collect_stats=collect_stats, poison=not collect_stats)
+
+
+def test_empty_cloud(oracle_mod):
+    """No points at all (the pointers of the cloud are NULL): background images, background gradient, empty gradients."""
+    from adop_amd import scenes
+
+    announce("config2 without points, B=2 96x80 L3 fwd+bwd")
+    hs = scenes.config2(n=1000, w=96, h=80, levels=3, batch=2)
+    hs.position, hs.normal, hs.index = hs.position[:0].copy(), hs.normal[:0].copy(), hs.index[:0].copy()
+    hs.dropout = None
+    hs.params.output_background_mask = 1
+    hs.background[:] = [0.5, 0.25, 0.125, 1.0]
+    assert hs.num_points == 0
+    _fwd_bwd(hs, oracle_mod)
+
+
 def test_debug_print_num_rendered_points(oracle_mod, capsys):
     """RenderParams::debug_print_num_rendered_points (PointRenderer.cu:1502-1512): the sum of the weights after a
     forward pass, printed as the reference prints it."""

@@ -94,6 +94,26 @@ def test_point_render_autograd_matches_checker(oracle_mod, capfd):
         assert misses <= max(1, int(1e-4 * size)) and worst <= 1e-6, (name, misses, size, worst)
 
 
+def test_render_points_switched_off():
+    """RenderParams::render_points = false (PointRenderer.cu:1417,1433): background images, masks of the mask value."""
+    from adop_amd import scenes
+
+    announce("libTorch wrapper: render_points = false")
+    mod = _module()
+    hs = scenes.config3(n=50_000, w=160, h=90, channels=4)
+    hs.background[:] = [0.1, 0.2, 0.3, 0.4]
+    hs.params.output_background_mask = 1
+    hs.params.output_background_mask_value = 0.25
+    s, t = _scene(mod, hs)
+    outs = mod.render(s, _views(hs), _params(hs, dropout=0.25, render_points=False), hs.num_layers)
+    L = hs.num_layers
+    for l in range(L):
+        o = outs[l].detach().cpu().numpy()
+        for c in range(4):
+            assert (o[:, c] == hs.background[c]).all()
+        assert (outs[L + l].detach().cpu().numpy() == 0.25).all()
+
+
 def test_dropout_is_drawn_like_the_reference_and_eval_disables_it(oracle_mod):
     import torch
     from adop_amd import scenes
