@@ -119,7 +119,8 @@ class NeuralRenderInfo:
     num_layers: int = 0
     cache: "PointRendererCache" = None
     # The reference draws the dropout mask inside the cache (bernoulli_, PointRenderer.cu:1083).  Passing it here
-    # makes a run reproducible; None + dropout>0 draws it with torch.
+    # makes a run reproducible; None + dropout>0 draws it with torch.  A host tensor is copied to the device by every
+    # forward pass (4 bytes per point and view): hand in a device tensor where that matters.
     dropout_points: Optional[torch.Tensor] = None
     dropout: float = 0.0
     collect_stats: bool = False
