@@ -94,6 +94,7 @@ class ForwardBuffers(C.Structure):
         ("layers", Layer * ADOP_MAX_LAYERS),
         ("dropout_points", C.c_void_p),
         ("point_cache", C.c_void_p),
+        ("pixel_cache", C.c_void_p),
     ]
 
 

@@ -318,6 +318,8 @@ Levels make_levels(const adop_scene* s, int B, const adop_forward_buffers* fb, c
         lv.l[l].gin         = gb ? gb->grad_out[l] : nullptr;
     }
     for (int l = fb->num_layers; l <= ADOP_MAX_LAYERS; ++l) lv.pix_prefix[l] = acc;
+    lv.irec       = fb->pixel_cache;  // (adop_backward: the workspace when the caller kept none)
+    lv.irec_ready = fb->pixel_cache != nullptr;
     return lv;
 }
 
@@ -669,6 +671,7 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
 
     float* ig     = (float*)((char*)workspace + wl.pixels);
     float2* dw    = (float2*)((char*)workspace + wl.dw);
+    if (!lv.irec) lv.irec = ig;  // interleave_kernel leaves the image records in front of the gradient records
     int bg_blocks = pixel_grid(lv) < kBgBlocks ? pixel_grid(lv) : kBgBlocks;
     {
         StageScope sc("CombineAndFillBackward", stream);
@@ -1123,6 +1126,6 @@ const char* adop_version(void)
 {
     // "kernels N" names the state of the kernels' memory behaviour: it goes up whenever a change moves a kernel's bytes,
     // so that traffic figures measured for one state (rocprofv3 counters) are not quoted for another.
-    return "adop_raster 0.2 (gfx950) kernels 7";
+    return "adop_raster 0.2 (gfx950) kernels 8";
 }
 }  // extern "C"

@@ -54,12 +54,14 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
         const float* im   = L.out + (size_t)b * C * hw + p;
         float* dst        = ig + (size_t)ws_pixel(lv, l, b, (uint32_t)p) * C;  // I record; the G record at dst + goff
         const size_t goff = total * (size_t)C;
+        // (the forward pass may have left the I records with the caller: then only G is transposed here)
+        const bool with_I = !lv.irec_ready;  // kernel-uniform
         float I[CMAX], G[CMAX];
 #pragma unroll
         for (int c = 0; c < CMAX; ++c)
             if (c < C)
             {
-                I[c] = __builtin_nontemporal_load(im + (size_t)c * hw);
+                I[c] = with_I ? __builtin_nontemporal_load(im + (size_t)c * hw) : 0.f;
                 G[c] = __builtin_nontemporal_load(g + (size_t)c * hw);
                 if (empty) acc[c] += G[c];
             }
@@ -83,7 +85,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
 #pragma unroll
                 for (int q = 0; q < V; ++q)
                 {
-                    sw[lane * V + q]          = make_float4(I[4 * q], I[4 * q + 1], I[4 * q + 2], I[4 * q + 3]);
+                    if (with_I) sw[lane * V + q] = make_float4(I[4 * q], I[4 * q + 1], I[4 * q + 2], I[4 * q + 3]);
                     sw[64 * V + lane * V + q] = make_float4(G[4 * q], G[4 * q + 1], G[4 * q + 2], G[4 * q + 3]);
                 }
                 wave_lds_sync();
@@ -91,7 +93,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
 #pragma unroll
                 for (int k = 0; k < V; ++k)
                 {
-                    __builtin_nontemporal_store(((const v4f*)sw)[k * 64 + lane], (v4f*)d0 + k * 64 + lane);
+                    if (with_I) __builtin_nontemporal_store(((const v4f*)sw)[k * 64 + lane], (v4f*)d0 + k * 64 + lane);
                     __builtin_nontemporal_store(((const v4f*)sw)[64 * V + k * 64 + lane], (v4f*)(d0 + goff) + k * 64 + lane);
                 }
             }
@@ -99,8 +101,11 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
             {
                 float4* d4 = (float4*)dst;
                 float4* g4 = (float4*)(dst + goff);
+                if (with_I)
+                {
 #pragma unroll
-                for (int q = 0; q < V; ++q) d4[q] = make_float4(I[4 * q], I[4 * q + 1], I[4 * q + 2], I[4 * q + 3]);
+                    for (int q = 0; q < V; ++q) d4[q] = make_float4(I[4 * q], I[4 * q + 1], I[4 * q + 2], I[4 * q + 3]);
+                }
 #pragma unroll
                 for (int q = 0; q < V; ++q) g4[q] = make_float4(G[4 * q], G[4 * q + 1], G[4 * q + 2], G[4 * q + 3]);
             }
@@ -111,7 +116,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
             for (int c = 0; c < CMAX; ++c)
                 if (c < C)
                 {
-                    dst[c]        = I[c];
+                    if (with_I) dst[c] = I[c];
                     dst[goff + c] = G[c];
                 }
         }
@@ -636,8 +641,10 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
                 int px = f2i_rn(ip.x), py = f2i_rn(ip.y);
                 size_t hw             = (size_t)L.w * L.h;
                 size_t p              = (size_t)py * L.w + px;
-                const float* pg       = ig + (size_t)ws_pixel(lv, l, b, (uint32_t)p) * C;  // I of the pixel, its G at + goff
-                const size_t goff     = gradient_array_offset(lv, C);
+                // I of the pixel (where the forward pass or interleave_kernel left it) and its G at + goff
+                const size_t rec      = (size_t)ws_pixel(lv, l, b, (uint32_t)p) * C;
+                const float* pg       = lv.irec + rec;
+                const float* pgg      = ig + gradient_array_offset(lv, C) + rec;
                 const ptrdiff_t nb[4] = {-1, 1, -(ptrdiff_t)L.w, (ptrdiff_t)L.w};
                 float Wn[4] = {0, 0, 0, 0}, Dn[4] = {0, 0, 0, 0};
                 if (rp.test_backward_mode == 4)
@@ -673,7 +680,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
                         for (int k = 0; k < 4; ++k)
                         {
                             const float* q = pg + nb[k] * C;
-                            v[k]           = dI_of(T_c, q[c], Wn[k], Dn[k]) * q[goff + c];
+                            v[k]           = dI_of(T_c, q[c], Wn[k], Dn[k]) * pgg[nb[k] * C + c];
                         }
                         float a0 = -v[0], a1 = v[1], b0 = -v[2], b1 = v[3];
                         dR_dpx += 0.5f * (a0 + a1);
@@ -689,7 +696,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
                         const float* q = pg + nb[k] * C;
                         float In[CMAX], Gn[CMAX];
                         load_channels<CT ? CT : 4>(q, In);
-                        load_channels<CT ? CT : 4>(q + goff, Gn);
+                        load_channels<CT ? CT : 4>(pgg + nb[k] * C, Gn);
 #pragma unroll
                         for (int c = 0; c < CMAX; ++c) v[k][c] = dI_of(T[c], In[c], Wn[k], Dn[k]) * Gn[c];
                     }

@@ -62,6 +62,11 @@ struct Levels
     int32_t C;
     int32_t pix_prefix[ADOP_MAX_LAYERS + 1];  // prefix sum of w*h over levels (one image)
     LevelArg l[ADOP_MAX_LAYERS];
+    // The resolved image in pixel-major order, [ws_pixel][C] (what the spatial gradients read at four neighbours of a
+    // pixel).  Forward: where the resolve leaves it beside the planar images (the caller's pixel_cache), or null.
+    // Backward: where it lies, and whether the forward wrote it (else interleave_kernel transposes `out`).
+    float* irec;
+    int32_t irec_ready;
 };
 
 struct CloudArg
@@ -140,6 +145,26 @@ __device__ __forceinline__ uint32_t ws_pixel(const Levels& lv, int l, int b, uin
 __device__ __forceinline__ size_t gradient_array_offset(const Levels& lv, int C)
 {
     return (size_t)lv.pix_prefix[lv.num] * (size_t)lv.B * (size_t)C;
+}
+
+// One record of the pixel-major image: C consecutive floats (16-byte stores for C = 4 and 8: the records are aligned).
+// Plain stores: with the nontemporal hint tile_blend_kernel, which writes most of them, ran 4 us longer.
+template <int CT>
+__device__ __forceinline__ void store_pixel_record(float* __restrict__ dst, const float* v, int C)
+{
+    if (CT == 8)
+    {
+        ((float4*)dst)[0] = make_float4(v[0], v[1], v[2], v[3]);
+        ((float4*)dst)[1] = make_float4(v[4], v[5], v[6], v[7]);
+    }
+    else if (CT == 4)
+        ((float4*)dst)[0] = make_float4(v[0], v[1], v[2], v[3]);
+    else
+    {
+#pragma unroll
+        for (int c = 0; c < kMaxChannels; ++c)  // (unrolled: v stays in registers)
+            if (c < C) dst[c] = v[c];
+    }
 }
 
 // Streamed data (read or written once per kernel) goes past the caches with the nontemporal hint, so that the lines

@@ -551,8 +551,13 @@ __global__ __launch_bounds__(kBlock) void resolve_kernel(Levels lv, int first_le
         float* out  = L.out + (size_t)b * C * hw + p;
 #pragma unroll
         for (int c = 0; c < CMAX; ++c)
-            if (c < C) out[(size_t)c * hw] = (cou == 0) ? background[c] : v[c] / cou;
+            if (c < C)
+            {
+                v[c]               = (cou == 0) ? background[c] : v[c] / cou;
+                out[(size_t)c * hw] = v[c];
+            }
         if (write_mask && L.mask) L.mask[o] = (cou == 0) ? mask_value : 1.f;
+        if (lv.irec) store_pixel_record<CT>(lv.irec + (size_t)ws_pixel(lv, l, b, (uint32_t)p) * C, v, C);
     }
 }
 

@@ -583,8 +583,13 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu((CT != 0
             float* out = L.out + (size_t)b * C * hw + pix;
 #pragma unroll
             for (int c = 0; c < CMAX; ++c)
-                if (c < C) __builtin_nontemporal_store((cou == 0) ? background[c] : acc0[c] / cou, out + (size_t)c * hw);
+                if (c < C)
+                {
+                    acc0[c] = (cou == 0) ? background[c] : acc0[c] / cou;
+                    __builtin_nontemporal_store(acc0[c], out + (size_t)c * hw);
+                }
             if (write_mask && L.mask) __builtin_nontemporal_store((cou == 0) ? mask_value : 1.f, L.mask + o);
+            if (lv.irec) store_pixel_record<CT>(lv.irec + (size_t)ws_pixel(lv, 0, b, (uint32_t)pix) * C, acc0, C);
         }
     }
     // level 1: buckets kBlock + 2*q and kBlock + 2*q + 1 (adjacent lanes) are the two parts of pixel q
@@ -609,8 +614,13 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu((CT != 0
                 float* out       = L.out + (size_t)b * C * hw + pix;
 #pragma unroll
                 for (int c = 0; c < CMAX; ++c)
-                    if (c < C) out[(size_t)c * hw] = (cou == 0) ? background[c] : acc1[c] / cou;
+                    if (c < C)
+                    {
+                        acc1[c]            = (cou == 0) ? background[c] : acc1[c] / cou;
+                        out[(size_t)c * hw] = acc1[c];
+                    }
                 if (write_mask && L.mask) L.mask[o] = (cou == 0) ? mask_value : 1.f;
+                if (lv.irec) store_pixel_record<CT>(lv.irec + (size_t)ws_pixel(lv, 1, b, (uint32_t)pix) * C, acc1, C);
             }
         }
     }

@@ -227,11 +227,16 @@ std::pair<std::vector<torch::Tensor>, std::vector<torch::Tensor>> BlendPointClou
     adop_forward_buffers fb =
         MakeForwardBuffers(info, di, d, w, cache.output_forward, cache.output_forward_background_mask, cache.dropout_points);
     // projected points: a saved tensor of the backward pass (no counterpart in the reference, which projects again)
-    torch::Tensor point_cache;
+    // ... and the resolved images pixel by pixel, which the spatial gradients read at four neighbours of a pixel
+    torch::Tensor point_cache, pixel_cache;
     if (ctx)
     {
         point_cache    = torch::empty({(long)views.size(), (long)scene.num_points, 4}, d[0].options());
         fb.point_cache = point_cache.data_ptr<float>();
+        long pixels    = 0;
+        for (auto& l : cache.layers_cuda) pixels += (long)views.size() * l.w * l.h;
+        pixel_cache    = torch::empty({pixels, (long)scene.num_channels}, d[0].options());
+        fb.pixel_cache = pixel_cache.data_ptr<float>();
     }
     Check(adop_forward(&scene, views.data(), (int)views.size(), &rp, &fb, cache.workspace.data_ptr(),
                        (size_t)cache.workspace.numel(), nullptr, CurrentStream()));
@@ -257,6 +262,7 @@ std::pair<std::vector<torch::Tensor>, std::vector<torch::Tensor>> BlendPointClou
         save.push_back(cache.dropout_points.defined() ? cache.dropout_points : torch::empty({0}, d[0].options()));
         for (auto& l : cache.layers_cuda) save.push_back(l.depth_index_tensor);
         save.push_back(point_cache);
+        save.push_back(pixel_cache);
         ctx->save_for_backward(save);
         ctx->saved_data["num_masks"] = (int64_t)cache.output_forward_background_mask.size();
         // the cache buffers are handed to the graph: allocate fresh ones on the next forward
@@ -284,7 +290,7 @@ torch::autograd::variable_list BlendPointCloudBackward(torch::autograd::Autograd
         cache.image_gradients.push_back(_image_gradients[i].contiguous());
     }
     auto saved = ctx->get_saved_variables();
-    TORCH_CHECK((int)saved.size() == L * 4 + 2);
+    TORCH_CHECK((int)saved.size() == L * 4 + 3);
     std::vector<torch::Tensor> di, d, w, out;
     for (int i = 0; i < L; ++i)
     {
@@ -347,6 +353,7 @@ torch::autograd::variable_list BlendPointCloudBackward(torch::autograd::Autograd
     std::vector<torch::Tensor> no_mask;
     adop_forward_buffers fb = MakeForwardBuffers(info, di, d, w, out, no_mask, dropout);
     fb.point_cache          = saved[L * 4 + 1].data_ptr<float>();
+    fb.pixel_cache          = saved[L * 4 + 2].data_ptr<float>();
     if (!cache.workspace.defined() ||
         (size_t)cache.workspace.numel() < adop_workspace_size(&s, (int)views.size(), L, views[0].w, views[0].h))
         cache.workspace = torch::empty({(long)adop_workspace_size(&s, (int)views.size(), L, views[0].w, views[0].h)},

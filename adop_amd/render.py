@@ -129,6 +129,9 @@ class NeuralRenderInfo:
     # NeuralRenderInfo::train (RenderInfo.h): a backward pass may follow, so the forward pass leaves the projected
     # points in a tensor of its own (saved like depth / weight) instead of the workspace
     train: bool = True
+    # with train: the forward pass also leaves the resolved images pixel by pixel for the backward pass (one more
+    # saved tensor of the size of the images); False: the backward pass builds those records from the images itself
+    keep_pixel_records: bool = True
 
 
 class PointRendererCache:
@@ -141,6 +144,7 @@ class PointRendererCache:
         self.cache_size = None
         self.dropout_points = None
         self.point_cache = None
+        self.pixel_cache = None
         self.output_forward = []
         self.output_forward_background_mask = []
         self.workspace = None
@@ -209,6 +213,10 @@ class PointRendererCache:
         # without a backward pass the library keeps them in its workspace
         self.point_cache = (torch.empty(B, N, 4, dtype=torch.float32, device=dev)
                             if (forward and info.train) else None)
+        # the resolved images pixel by pixel, for the spatial gradients of the backward pass (saved like the outputs)
+        pixels = B * sum(L.size[0] * L.size[1] for L in self.layers_cuda)
+        self.pixel_cache = (torch.empty(pixels, Cn, dtype=torch.float32, device=dev)
+                            if (forward and info.train and info.keep_pixel_records) else None)
 
     # -- C-ABI structs -----------------------------------------------------------------------
     def forward_struct(self):
@@ -224,6 +232,7 @@ class PointRendererCache:
             S.mask = _ptr(self.output_forward_background_mask[l]) if self.output_forward_background_mask else None
         fb.dropout_points = _ptr(self.dropout_points)
         fb.point_cache = _ptr(self.point_cache)
+        fb.pixel_cache = _ptr(self.pixel_cache)
         return fb
 
     def views_array(self):
@@ -266,6 +275,7 @@ def BlendPointCloudForward(ctx, info, build=True):
         ctx.save_for_backward(*save)
         ctx.dropout_points = cache.dropout_points
         ctx.point_cache = cache.point_cache
+        ctx.pixel_cache = cache.pixel_cache
         ctx.depth_index = [L.depth_index_tensor for L in cache.layers_cuda]
         ctx.masks = list(cache.output_forward_background_mask)
         # depth / weight / packed depth now belong to the graph (the kernels write them through raw pointers, autograd
@@ -299,6 +309,7 @@ def BlendPointCloudBackward(ctx, info, image_gradients, needs=(True, True, True)
         S.mask = _ptr(ctx.masks[l]) if ctx.masks else None
     fb.dropout_points = _ptr(ctx.dropout_points)
     fb.point_cache = _ptr(getattr(ctx, "point_cache", None))
+    fb.pixel_cache = _ptr(getattr(ctx, "pixel_cache", None))
 
     need_points, need_pose, need_intr = needs
     N = scene.point_cloud_cuda.Size()

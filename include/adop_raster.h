@@ -151,6 +151,13 @@ typedef struct adop_forward_buffers
      * unless counters are collected): they keep whatever the buffer held.  A point outside the image at every level
      * carries a positive depth whatever its dropout flag. */
     float* point_cache;
+    /* Optional [B * (w_0 h_0 + ... + w_{L-1} h_{L-1}), C] f32 (no counterpart in the reference): the resolved images
+     * once more, pixel by pixel (C consecutive floats; the pixels of level 0 of all B images first, then level 1, ...;
+     * inside an image row by row).  The spatial gradients read the image at the four neighbours of a pixel in all
+     * channels (PointRenderer.cu:576-611), which the planar [B,C,h,w] layout serves badly.  adop_forward writes it;
+     * adop_backward reads it when the same buffer is passed back in `fwd` (its image I is then what that forward pass
+     * rendered, whatever happened to `out` since).  NULL: adop_backward builds the records from `out` itself. */
+    float* pixel_cache;
 } adop_forward_buffers;
 
 /* DeviceBackwardParams (PointRenderer.cu:124-137) + the tensors PointRendererCache::Build(.., false)

@@ -19,7 +19,7 @@ FORWARD_PATH = 0
 POISON_BITS = 0xDEADBEEF
 
 
-def run_hip_forward(hs, collect_stats=True, forward_path=None, train=True, poison=False):
+def run_hip_forward(hs, collect_stats=True, forward_path=None, train=True, poison=False, pixel_records=True):
     import torch
     from adop_amd import render
 
@@ -29,6 +29,7 @@ def run_hip_forward(hs, collect_stats=True, forward_path=None, train=True, poiso
     cache = render.PointRendererCache()
     info = render.NeuralRenderInfo(scene=scene, images=list(hs.views), params=hs.params, num_layers=hs.num_layers,
                                    cache=cache, collect_stats=collect_stats, train=train,
+                                   keep_pixel_records=pixel_records,
                                    dropout_points=None if hs.dropout is None else torch.from_numpy(hs.dropout))
 
     class Ctx:
@@ -41,6 +42,8 @@ def run_hip_forward(hs, collect_stats=True, forward_path=None, train=True, poiso
         cache.workspace.view(torch.int32).fill_(POISON_BITS - (1 << 32))
         if cache.point_cache is not None:
             cache.point_cache.view(torch.int32).fill_(POISON_BITS - (1 << 32))
+        if cache.pixel_cache is not None:
+            cache.pixel_cache.view(torch.int32).fill_(POISON_BITS - (1 << 32))
         images, masks = render.BlendPointCloudForward(ctx, info, build=False)
     else:
         images, masks = render.BlendPointCloudForward(ctx, info)

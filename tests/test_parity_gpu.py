@@ -37,14 +37,15 @@ END_TO_END_MISS_SIZE = 1e-6
 end_to_end_misses = {}  # case -> {tensor: (misses, size, worst)}: printed by the last test of the file
 
 
-def _fwd_bwd(hs, oracle_mod, needs=(True, True, True), seed=5, collect_stats=True, poison=False):
+def _fwd_bwd(hs, oracle_mod, needs=(True, True, True), seed=5, collect_stats=True, poison=False, pixel_records=True):
     import torch
     from adop_amd import render, scenes
 
     from helpers import count_misses
 
     ref = oracle_mod.forward(hs)
-    scene, info, ctx, images, masks = run_hip_forward(hs, collect_stats=collect_stats, poison=poison)
+    scene, info, ctx, images, masks = run_hip_forward(hs, collect_stats=collect_stats, poison=poison,
+                                                      pixel_records=pixel_records)
     check_forward(hs, ref, ctx, images, masks, info, stats=collect_stats)
     gout = scenes.upstream_grads(hs, seed)
     grads = render.BlendPointCloudBackward(ctx, info, _torch_grads(gout), needs)
@@ -120,13 +121,44 @@ def test_config2_no_ghost(oracle_mod):
     _fwd_bwd(hs, oracle_mod, needs=(True, False, False))
 
 
+@pytest.mark.parametrize("pixel_records", [True, False], ids=["records_from_forward", "records_from_out"])
 @pytest.mark.parametrize("collect_stats", [True, False], ids=["counters", "plain"])
-def test_config3_reduced_all_grads(oracle_mod, collect_stats):
+def test_config3_reduced_all_grads(oracle_mod, collect_stats, pixel_records):
+    """pixel_records: the forward pass leaves the resolved images pixel by pixel for the spatial gradients
+    (adop_forward_buffers.pixel_cache), or the backward pass builds those records from `out`."""
     from adop_amd import scenes
 
-    announce(f"config3 reduced 500k pts 480x270 C=8 all grads, counters={collect_stats}")
+    announce(f"config3 reduced 500k pts 480x270 C=8 all grads, counters={collect_stats}, pixel records from the "
+             f"forward pass={pixel_records}")
     hs = scenes.config3(n=500_000, w=480, h=270)
-    _fwd_bwd(hs, oracle_mod, collect_stats=collect_stats, poison=not collect_stats)
+    _fwd_bwd(hs, oracle_mod, collect_stats=collect_stats, poison=not collect_stats, pixel_records=pixel_records)
+
+
+@pytest.mark.parametrize("channels", [3, 4])
+def test_backward_reads_the_image_the_forward_rendered(oracle_mod, channels):
+    """With pixel records kept from the forward pass, the image I of the spatial gradients is what that forward
+    rendered, whatever happened to `out` since (the reference composes the environment map out of place,
+    RenderModule.cpp:121-125, so its backward sees the rasterizer's own output too); without them it is `out` as it
+    is when the backward pass runs.  Three views, so that the records of all images and levels are addressed."""
+    import torch
+    from adop_amd import render, scenes
+
+    announce(f"backward after `out` was changed in place, C={channels}")
+    hs = scenes.config2(n=60_000, w=160, h=120, levels=3, batch=3, seed=6)
+    hs.texture = np.ascontiguousarray(np.random.default_rng(1).random((channels, hs.num_points), dtype=np.float32))
+    hs.background = np.zeros(channels, np.float32)
+    gout = scenes.upstream_grads(hs, 5)
+    for kept in (True, False):
+        scene, info, ctx, images, masks = run_hip_forward(hs, pixel_records=kept)
+        rendered = download_forward(hs, info, images, masks)
+        for im in images:
+            im.mul_(0.5).add_(0.25)  # (an environment map added in place, a tone curve, ...)
+        torch.cuda.synchronize()
+        changed = download_forward(hs, info, images, masks)
+        grads = render.BlendPointCloudBackward(ctx, info, _torch_grads(gout), (True, True, True))
+        torch.cuda.synchronize()
+        refb = oracle_mod.backward(hs, rendered if kept else changed, gout, True, True, True)
+        check_backward(hs, refb, grads, info)
 
 
 def test_backward_without_point_gradients(oracle_mod):

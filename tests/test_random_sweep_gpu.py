@@ -96,7 +96,7 @@ def test_random_scene(oracle_mod, seed, forward_path):
     # poisoned point cache and workspace
     counters = seed % 3 != 0
     scene, info, ctx, images, masks = run_hip_forward(hs, collect_stats=counters, forward_path=forward_path,
-                                                      poison=not counters)
+                                                      poison=not counters, pixel_records=seed % 4 != 1)
     check_forward(hs, ref, ctx, images, masks, info, stats=counters)
     gout = scenes.upstream_grads(hs, seed + 11)
     grads = render.BlendPointCloudBackward(ctx, info, [torch.from_numpy(g).cuda() for g in gout], needs)
