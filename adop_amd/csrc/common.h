@@ -147,12 +147,33 @@ __device__ __forceinline__ size_t gradient_array_offset(const Levels& lv, int C)
     return (size_t)lv.pix_prefix[lv.num] * (size_t)lv.B * (size_t)C;
 }
 
+// Streamed data (read or written once per kernel) goes past the caches with the nontemporal hint, so that the lines
+// the gathers of the same kernel reuse stay resident.
+typedef float v4f __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 nt_load4(const float4* p)
+{
+    const v4f r = __builtin_nontemporal_load((const v4f*)p);
+    return make_float4(r.x, r.y, r.z, r.w);
+}
+__device__ __forceinline__ void nt_store4(float4* p, float4 v)
+{
+    v4f r = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(r, (v4f*)p);
+}
+
 // One record of the pixel-major image: C consecutive floats (16-byte stores for C = 4 and 8: the records are aligned).
 // Plain stores: with the nontemporal hint tile_blend_kernel, which writes most of them, ran 4 us longer.
-template <int CT>
+template <int CT, bool NT = false>
 __device__ __forceinline__ void store_pixel_record(float* __restrict__ dst, const float* v, int C)
 {
-    if (CT == 8)
+    if (CT == 8 && NT)
+    {
+        nt_store4((float4*)dst, make_float4(v[0], v[1], v[2], v[3]));
+        nt_store4((float4*)dst + 1, make_float4(v[4], v[5], v[6], v[7]));
+    }
+    else if (CT == 4 && NT)
+        nt_store4((float4*)dst, make_float4(v[0], v[1], v[2], v[3]));
+    else if (CT == 8)
     {
         ((float4*)dst)[0] = make_float4(v[0], v[1], v[2], v[3]);
         ((float4*)dst)[1] = make_float4(v[4], v[5], v[6], v[7]);
@@ -167,19 +188,6 @@ __device__ __forceinline__ void store_pixel_record(float* __restrict__ dst, cons
     }
 }
 
-// Streamed data (read or written once per kernel) goes past the caches with the nontemporal hint, so that the lines
-// the gathers of the same kernel reuse stay resident.
-typedef float v4f __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ float4 nt_load4(const float4* p)
-{
-    const v4f r = __builtin_nontemporal_load((const v4f*)p);
-    return make_float4(r.x, r.y, r.z, r.w);
-}
-__device__ __forceinline__ void nt_store4(float4* p, float4 v)
-{
-    v4f r = {v.x, v.y, v.z, v.w};
-    __builtin_nontemporal_store(r, (v4f*)p);
-}
 
 template <typename T>
 __device__ __forceinline__ T wave_sum(T v)

@@ -557,7 +557,7 @@ __global__ __launch_bounds__(kBlock) void resolve_kernel(Levels lv, int first_le
                 out[(size_t)c * hw] = v[c];
             }
         if (write_mask && L.mask) L.mask[o] = (cou == 0) ? mask_value : 1.f;
-        if (lv.irec) store_pixel_record<CT>(lv.irec + (size_t)ws_pixel(lv, l, b, (uint32_t)p) * C, v, C);
+        if (lv.irec) store_pixel_record<CT, true>(lv.irec + (size_t)ws_pixel(lv, l, b, (uint32_t)p) * C, v, C);
     }
 }
 
