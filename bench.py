@@ -46,6 +46,8 @@ MEASURED_TRAFFIC = {
                 "bytes": {"RenderBackward/descriptor": 860.1e6, "RenderBackward/spatial": 572.1e6, "TileBlend": 528.9e6,
                           "BinCount": 430.3e6, "CombineAndFillBackward": 220.8e6, "TileDepth": 101.5e6, "Initialize": 11.8e6,
                           "CombineAndFill": 23.5e6, "BinScatter": 197.4e6, "Post Process Gradient": 0.5e6}},
+    "config1": {"kernels": 8, "profile": "profiles/config1_direct_path_forward_kernels_traffic_instructions.md",
+                "bytes": {"DepthPrepass": 13.1e6, "RenderForward": 8.4e6, "CombineAndFill": 5.6e6, "Initialize": 3.5e6}},
     "config2": {"kernels": 8, "profile": "profiles/config2_fwd_bwd_kernels_traffic_instructions.md",
                 "bytes": {"RenderBackward/descriptor": 200.8e6, "BinCount": 64.6e6, "TileBlend": 163.5e6,
                           "RenderBackward/spatial": 146.3e6, "CombineAndFillBackward": 67.2e6, "TileDepth": 37.9e6,
