@@ -585,7 +585,7 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
         pc.cache      = (float4*)((char*)workspace + wl.proj);
         pc.list_ids   = (uint32_t*)((char*)workspace + wl.list_ids);
         pc.list_count = (uint32_t*)((char*)workspace + wl.list_count);
-        pc.list_span  = prepass_points_per_block();
+        pc.list_span  = prepass_points_per_block(scene->num_points);
         pc.list_stride = wl.list_stride;
     }
     size_t accum_n   = (size_t)lv.pix_prefix[lv.num] * lv.B * S;  // floats, multiple of 4 unless S < 4
@@ -1126,6 +1126,6 @@ const char* adop_version(void)
 {
     // "kernels N" names the state of the kernels' memory behaviour: it goes up whenever a change moves a kernel's bytes,
     // so that traffic figures measured for one state (rocprofv3 counters) are not quoted for another.
-    return "adop_raster 0.2 (gfx950) kernels 8";
+    return "adop_raster 0.2 (gfx950) kernels 9";
 }
 }  // extern "C"

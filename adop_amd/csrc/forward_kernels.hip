@@ -243,9 +243,10 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
                 if (!__ballot(cand)) continue;
                 const LevelArg& L = lv.l[l];
                 uint64_t* dst     = L.depth_index + (size_t)b * L.w * L.h;
-                if (l < group_from)
+                if (l < group_from || !wave_shares_keys(cand, pix[k][l]))
                 {
-                    // fine levels: few lanes of a wavefront share a pixel, grouping would cost more than it saves
+                    // fine levels, or a cloud without order / with few points per pixel: few lanes of the wavefront
+                    // share a pixel, grouping would cost more than it saves
                     if (cand) atomicMin((unsigned long long*)(dst + pix[k][l]), (unsigned long long)pk);
                     continue;
                 }
@@ -376,9 +377,10 @@ __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewCo
             if (!bal) continue;
             wave_lds_sync();
             int G;
-            if (l < group_from)
+            if (l < group_from || !wave_shares_keys(acc[l], gp[l]))
             {
-                // fine level: few lanes of a wavefront share a pixel; every accepted lane is its own entry
+                // fine level, or a cloud without order / with few points per pixel: few lanes of the wavefront share a
+                // pixel; every accepted lane is its own entry
                 G = __popcll(bal);
                 if (acc[l])
                 {
@@ -585,20 +587,25 @@ void launch_clear(const Levels& lv, int first_level, int grid, float* accum, siz
                        zero_u32, zero_n, vp);
 }
 
-static int prepass_ppt()
+// Points per thread of prepass_kernel: two for the clouds of a hundred million points that reach the direct path by
+// their density (more loads in flight per wavefront: config 4 1.10 -> 1.04 ms), one below 2^24 points, where the
+// launch is a few workgroups per CU and the shorter chain per thread counts (1 M points in 256 x 256, unordered:
+// 0.17 -> 0.10 ms; 100 k points: 0.096 -> 0.073 ms).
+static int prepass_ppt(int n)
 {
-    static const int ppt = getenv("ADOP_PREPASS_PPT") ? atoi(getenv("ADOP_PREPASS_PPT")) : 2;
+    static const int env = getenv("ADOP_PREPASS_PPT") ? atoi(getenv("ADOP_PREPASS_PPT")) : 0;
+    const int ppt        = env ? env : (n >= (1 << 24) ? 2 : 1);
     return ppt == 4 ? 4 : (ppt == 2 ? 2 : 1);
 }
 
-int prepass_points_per_block() { return kBlock * prepass_ppt(); }
+int prepass_points_per_block(int n) { return kBlock * prepass_ppt(n); }
 
 void launch_prepass(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, adop_stats* stats,
                     hipStream_t st)
 {
     if (pc.n < 1) return;
     static const int group_from = getenv("ADOP_PREPASS_GROUP_FROM") ? atoi(getenv("ADOP_PREPASS_GROUP_FROM")) : 1;
-    const int ppt               = prepass_ppt();
+    const int ppt               = prepass_ppt(pc.n);
     if (ppt == 4)
         hipLaunchKernelGGL((prepass_kernel<4>), dim3((pc.n + kBlock * 4 - 1) / (kBlock * 4)), dim3(kBlock), 0, st, pc,
                            views, lv, rp, group_from, stats);

@@ -40,7 +40,7 @@ void launch_close_points(const float4* sorted, int n, const KnnGrid* g, const ui
                          int32_t* state, uint32_t* round_count, int round, hipStream_t st);
 void launch_morton(const float4* position, int n, const float* mn, const float* scale, unsigned long long* code,
                    hipStream_t st);
-int prepass_points_per_block();  // points per workgroup of prepass_kernel (the unit of its candidate lists)
+int prepass_points_per_block(int n);  // points per workgroup of prepass_kernel on a cloud of n points (the unit of its candidate lists)
 void launch_prepass(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, adop_stats* stats,
                     hipStream_t st);
 void launch_blend(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
