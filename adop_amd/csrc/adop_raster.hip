@@ -139,12 +139,12 @@ constexpr int kTilePathMaxPointsPerPixel = 16;
 constexpr int kWindowCloudShare = 16;  // a crop window is taken to see 1/16 of the cloud
 // A tile is one workgroup from its first entry to its last: a call with few tiles leaves most of the GPU idle in the
 // tile kernels, whose time per point then grows like 1 / tiles (measured on Morton-ordered clouds, forward:
-// 18 us per million points from ~4 000 tiles up, 75 us at 1 024 tiles, 180 us at 256; the direct path: 25 us whatever
-// the image), while the direct path pays ~50 us more per call for its accumulators of all levels.
-constexpr int kTilePathMinTiles = 512;       // below: the direct path (256 tiles: equal on an ordered cloud, 1.7 x faster on an unordered one)
+// 18 us per million points from ~4 000 tiles up, 75 us at 1 024 tiles, 180 us at 256; the direct path: 26 us whatever
+// the image), while the direct path pays ~15 us more per call for its accumulators of all levels.
+constexpr int kTilePathMinTiles = 512;       // below: the direct path (256 tiles: 1.2 to 3 x faster from 100 k points up)
 constexpr int kTilePathEnoughTiles = 2800;   // from here on the tile path is the faster one per point
 constexpr double kTilePathUsPerMTiles = 73728.0;  // us per million points x tiles of the call
-constexpr double kDirectPathUsPerM = 25.0, kDirectPathFixedUs = 50.0;
+constexpr double kDirectPathUsPerM = 26.0, kDirectPathFixedUs = 15.0;
 constexpr int kConcurrentMaxPoints = 4000000;  // backward: full views of a larger cloud get a spatial-gradient launch each
 
 size_t max_tiles(int B, int w0, int h0)
