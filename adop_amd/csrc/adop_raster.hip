@@ -220,9 +220,10 @@ WorkspaceLayout layout(const adop_scene* s, int B, int L, int w0, int h0)
     size_t T     = max_tiles(B, w0, h0);
     w.bin_count  = o;  // followed by the row counter and the tickets of the split bins: one range to clear
     const size_t max_rows = (size_t)slice_rows(s->num_points > 0 ? s->num_points : 0, B);
-    o            = align_up(o + sizeof(uint32_t) * (T + 1 + 2 * max_rows), 256);
+    const size_t counters = T << bin_shard_shift(T);
+    o            = align_up(o + sizeof(uint32_t) * (counters + 1 + 2 * max_rows), 256);
     w.bin_offset = o;
-    o            = align_up(o + sizeof(uint32_t) * (T + 1), 256);
+    o            = align_up(o + sizeof(uint32_t) * (counters + 1), 256);
     w.bin_order  = o;
     o            = align_up(o + sizeof(uint4) * (T + max_rows), 256);
     w.bin_rows   = o;
@@ -532,8 +533,11 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
         bin.entries = (float4*)((char*)workspace + wl.bin_entries);
         bin.info    = (uint32_t*)((char*)workspace + wl.bin_info);
         const int T = bin.tiles_x * bin.tiles_y * num_views;
-        bin.row_count = bin.count + T;
-        bin.tickets   = bin.count + T + 1;
+        bin.shard_shift   = bin_shard_shift((size_t)T);
+        bin.num_tiles     = T;
+        const int counters = T << bin.shard_shift;
+        bin.row_count = bin.count + counters;
+        bin.tickets   = bin.count + counters + 1;
         bin.max_rows   = slice_rows(scene->num_points, num_views);
         bin.row_floats = slice_row_floats(scene->num_channels);
         // (read at every call: the tests split small bins)
@@ -545,7 +549,7 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
             size_t first   = (size_t)lv.pix_prefix[bin.lt] * lv.B * S;
             size_t accum_n = (size_t)lv.pix_prefix[lv.num] * lv.B * S - first;
             int grid       = pixel_grid(lv, bin.lt) > 32 ? pixel_grid(lv, bin.lt) : 32;
-            launch_clear(lv, bin.lt, grid, accum + first, S % 4 == 0 ? accum_n : 0, bin.count, T + 1 + 2 * bin.max_rows, vp, stream);
+            launch_clear(lv, bin.lt, grid, accum + first, S % 4 == 0 ? accum_n : 0, bin.count, counters + 1 + 2 * bin.max_rows, vp, stream);
             if (S % 4 != 0 && (st = fill_async(accum + first, accum_n * sizeof(float), 0, stream)) != ADOP_OK) return st;
         }
         {
@@ -554,7 +558,7 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
         }
         {
             StageScope sc("BinScatter", stream);
-            launch_tile_scan(bin, T, stream);
+            launch_tile_scan(bin, counters, stream);
             launch_bin(1, pc, dviews, lv, rp, bin, nullptr, stream);
         }
         {
@@ -1126,6 +1130,6 @@ const char* adop_version(void)
 {
     // "kernels N" names the state of the kernels' memory behaviour: it goes up whenever a change moves a kernel's bytes,
     // so that traffic figures measured for one state (rocprofv3 counters) are not quoted for another.
-    return "adop_raster 0.2 (gfx950) kernels 9";
+    return "adop_raster 0.2 (gfx950) kernels 10";
 }
 }  // extern "C"

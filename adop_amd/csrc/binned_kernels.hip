@@ -70,6 +70,11 @@ __device__ __forceinline__ void entry_tiles(const Levels& lv, const ParamArg& rp
     }
 }
 
+__device__ __forceinline__ uint32_t shard_of(uint32_t point, int shard_shift)
+{
+    return (point >> 8) & ((1u << shard_shift) - 1u);  // as bin_shard_of(): runs of 256 points take the shards in turn
+}
+
 // First pass over the points: projection (kept in the point cache) and the number of entries per tile.  A thread
 // handles PPT points whose loads are all issued before anything waits.
 template <int PPT>
@@ -199,8 +204,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(PPT > 2 
             const unsigned long long below = (1ull << lane) - 1ull;
             const unsigned long long pm    = wave_group_mask(any_in, ptile);
             const unsigned long long xm    = wave_group_mask(xtile != kNoTile, xtile);
-            if (any_in && (pm & below) == 0) atomicAdd(&bin.count[ptile], (uint32_t)__popcll(pm));
-            if (xtile != kNoTile && (xm & below) == 0) atomicAdd(&bin.count[xtile], (uint32_t)__popcll(xm));
+            const uint32_t shard = shard_of((uint32_t)i, bin.shard_shift);  // (wavefront-uniform)
+            if (any_in && (pm & below) == 0) atomicAdd(&bin.count[shard * bin.num_tiles + ptile], (uint32_t)__popcll(pm));
+            if (xtile != kNoTile && (xm & below) == 0) atomicAdd(&bin.count[shard * bin.num_tiles + xtile], (uint32_t)__popcll(xm));
         }
     }
 }
@@ -230,7 +236,8 @@ __device__ __forceinline__ void order_tiles(const BinArg& bin, int T, int g, int
         const uint32_t c = entries >> 7;
         return (uint32_t)(kOrderClasses - 1) - (c < (uint32_t)(kOrderClasses - 1) ? c : (uint32_t)(kOrderClasses - 1));  // 0 = fullest
     };
-    for (int t = g + G * tid; t < T; t += G * kBlock) atomicAdd(&s_class[class_of(bin.offset[t + 1] - bin.offset[t])], 1u);
+    const int sh = bin.shard_shift;  // (a bin: the parts of the tile's shards, one behind the other)
+    for (int t = g + G * tid; t < T; t += G * kBlock) atomicAdd(&s_class[class_of(bin.offset[(t + 1) << sh] - bin.offset[t << sh])], 1u);
     __syncthreads();
     if (tid < 64)
     {
@@ -247,7 +254,7 @@ __device__ __forceinline__ void order_tiles(const BinArg& bin, int T, int g, int
     __syncthreads();
     for (int t = g + G * tid; t < T; t += G * kBlock)
     {
-        const uint32_t start = bin.offset[t], end = bin.offset[t + 1];
+        const uint32_t start = bin.offset[t << sh], end = bin.offset[(t + 1) << sh];
         const uint32_t rank  = atomicAdd(&s_class[class_of(end - start)], 1u);
         uint32_t first_end = end, word = 0;
         const uint32_t n   = end - start;
@@ -367,12 +374,14 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels
             if (any_in && (pm[k] & below) == 0)
             {
                 const uint32_t n = (uint32_t)__popcll(pm[k]);
-                pbase[k]         = bin.offset[ptile] + atomicSub(&bin.count[ptile], n) - n;
+                const uint32_t sd = shard_of((uint32_t)(base + k * kBlock), bin.shard_shift);
+                pbase[k] = bin.offset[(ptile << bin.shard_shift) + sd] + atomicSub(&bin.count[sd * bin.num_tiles + ptile], n) - n;
             }
             if (has_x && (xm[k] & below) == 0)
             {
                 const uint32_t n = (uint32_t)__popcll(xm[k]);
-                xbase[k]         = bin.offset[xtile] + atomicSub(&bin.count[xtile], n) - n;
+                const uint32_t sd = shard_of((uint32_t)(base + k * kBlock), bin.shard_shift);
+                xbase[k] = bin.offset[(xtile << bin.shard_shift) + sd] + atomicSub(&bin.count[sd * bin.num_tiles + xtile], n) - n;
             }
         }
 #pragma unroll
@@ -398,9 +407,11 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels
 // Exclusive prefix sum of the tile counts (one workgroup): offset[0..T].  Chunks of 1024 * PER tiles; the PER counts of
 // a thread are consecutive (16-byte loads, one memory round trip per chunk).  PER = 8 covers one view of 1920 x 1080 in
 // one chunk; batches of views take PER = 32 (a chunk costs three barriers and a round trip whatever its size).
+// The counters lie shard by shard (count[shard * tiles + tile]), the offsets tile by tile with a tile's shards side by
+// side (k = (tile << shard_shift) + shard): T = tiles << shard_shift logical counters.
 template <int PER>
 __global__ __launch_bounds__(1024) void tile_scan_kernel(const uint32_t* __restrict__ count, uint32_t* __restrict__ offset,
-                                                         int T)
+                                                         int T, int shard_shift, int tiles)
 {
     __shared__ uint32_t s_wave[16];
     __shared__ uint32_t s_carry;
@@ -411,7 +422,16 @@ __global__ __launch_bounds__(1024) void tile_scan_kernel(const uint32_t* __restr
     {
         const int t0 = c0 + tid * PER;
         uint32_t v[PER];
-        if (t0 + PER <= T)  // (count is 256-byte aligned and t0 a multiple of PER)
+        if (shard_shift > 0)
+        {
+#pragma unroll
+            for (int k = 0; k < PER; ++k)
+            {
+                const int q = t0 + k;
+                v[k]        = q < T ? count[(q & ((1 << shard_shift) - 1)) * tiles + (q >> shard_shift)] : 0u;
+            }
+        }
+        else if (t0 + PER <= T)  // (count is 256-byte aligned and t0 a multiple of PER)
         {
 #pragma unroll
             for (int k = 0; k < PER; k += 4)
@@ -491,9 +511,11 @@ void launch_bin(int pass, const CloudArg& pc, const ViewConst* views, const Leve
 void launch_tile_scan(const BinArg& bin, int num_tiles, hipStream_t st)
 {
     if (num_tiles <= 8192)
-        hipLaunchKernelGGL(tile_scan_kernel<8>, dim3(1), dim3(1024), 0, st, bin.count, bin.offset, num_tiles);
+        hipLaunchKernelGGL(tile_scan_kernel<8>, dim3(1), dim3(1024), 0, st, bin.count, bin.offset, num_tiles, bin.shard_shift, bin.num_tiles);
+    else if (num_tiles <= 16384)  // (the sharded counters of a call: one chunk)
+        hipLaunchKernelGGL(tile_scan_kernel<16>, dim3(1), dim3(1024), 0, st, bin.count, bin.offset, num_tiles, bin.shard_shift, bin.num_tiles);
     else
-        hipLaunchKernelGGL(tile_scan_kernel<32>, dim3(1), dim3(1024), 0, st, bin.count, bin.offset, num_tiles);
+        hipLaunchKernelGGL(tile_scan_kernel<32>, dim3(1), dim3(1024), 0, st, bin.count, bin.offset, num_tiles, bin.shard_shift, bin.num_tiles);
 }
 
 }  // namespace adop

@@ -143,7 +143,11 @@ def check_backward(hs, refb, grads, info, stats=True):
     g_tex, g_bg, g_pts, g_pose, g_intr = grads
     cache = info.cache
     assert_close(g_tex.cpu().numpy(), refb.grad_texture, 1e-4, 1e-6, "grad_texture")
-    assert_close(g_bg.cpu().numpy(), refb.grad_background, 1e-4, 1e-5, "grad_background")
+    # the background gradient sums the upstream gradient (N(0,1) in these tests) over the empty pixels of all levels
+    # and views: a sum of n terms that cancels to O(sqrt(n)); the kernels add a handful of pixels per thread in fp32
+    # before they go on in f64, so its absolute error grows like 2^-24 sqrt(n) (1.0e-4 seen at n = 2.8 M)
+    n_pixels = hs.batch * sum(w * h for (w, h) in hs.level_sizes())
+    assert_close(g_bg.cpu().numpy(), refb.grad_background, 1e-4, max(1e-5, 2.4e-7 * np.sqrt(n_pixels)), "grad_background")
     if g_pts is not None:
         assert np.array_equal(cache.output_gradient_point_count.cpu().numpy(), refb.grad_points_count), "point count"
         # absolute bar: 1e-6 of the point's own gradient vector where that is larger than 1 (a component that cancels
