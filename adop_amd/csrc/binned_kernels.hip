@@ -424,12 +424,16 @@ __global__ __launch_bounds__(1024) void tile_scan_kernel(const uint32_t* __restr
         uint32_t v[PER];
         if (shard_shift > 0)
         {
+            // (unconditional loads of clamped indices, all in flight at once; what lies past the end counts as zero)
 #pragma unroll
             for (int k = 0; k < PER; ++k)
             {
-                const int q = t0 + k;
-                v[k]        = q < T ? count[(q & ((1 << shard_shift) - 1)) * tiles + (q >> shard_shift)] : 0u;
+                const int q = min(t0 + k, T - 1);
+                v[k]        = __builtin_nontemporal_load(count + (q & ((1 << shard_shift) - 1)) * tiles + (q >> shard_shift));
             }
+#pragma unroll
+            for (int k = 0; k < PER; ++k)
+                if (t0 + k >= T) v[k] = 0u;
         }
         else if (t0 + PER <= T)  // (count is 256-byte aligned and t0 a multiple of PER)
         {
@@ -460,13 +464,24 @@ __global__ __launch_bounds__(1024) void tile_scan_kernel(const uint32_t* __restr
         __syncthreads();
         uint32_t run = s_carry + inc - sum;
         for (int w = 0; w < (tid >> 6); ++w) run += s_wave[w];
+        // (offset is 256-byte aligned and t0 a multiple of PER: 16-byte stores, a quarter of the store instructions)
 #pragma unroll
-        for (int k = 0; k < PER; ++k)
-            if (t0 + k < T)
+        for (int k = 0; k < PER; k += 4)
+        {
+            uint4 o;
+            o.x = run, run += v[k];
+            o.y = run, run += v[k + 1];
+            o.z = run, run += v[k + 2];
+            o.w = run, run += v[k + 3];
+            if (t0 + k + 3 < T)
+                *(uint4*)(offset + t0 + k) = o;
+            else
             {
-                offset[t0 + k] = run;
-                run += v[k];
+                if (t0 + k < T) offset[t0 + k] = o.x;
+                if (t0 + k + 1 < T) offset[t0 + k + 1] = o.y;
+                if (t0 + k + 2 < T) offset[t0 + k + 2] = o.z;
             }
+        }
         __syncthreads();
         if (tid == 1023) s_carry = run;  // the last thread ends at the chunk total
         __syncthreads();
