@@ -1,5 +1,6 @@
 // launch.h — host-callable launchers of the kernels (one translation unit per kernel family).
 #pragma once
+#include <stdlib.h>
 #include "common.h"
 
 namespace adop
@@ -92,6 +93,8 @@ struct BinArg
 // in the image centre gain 15 us (config 2: 0.270 -> 0.256 ms).
 inline int bin_shard_shift(size_t tiles)
 {
+    static const int env = getenv("ADOP_BIN_SHARD_SHIFT") ? atoi(getenv("ADOP_BIN_SHARD_SHIFT")) : -1;
+    if (env >= 0 && env <= 3) return env;
     int s = 0;
     while (tiles <= 4096 && s < 3 && (tiles << (s + 1)) <= 16384) ++s;
     return s;
