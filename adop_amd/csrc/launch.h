@@ -93,8 +93,11 @@ struct BinArg
 // in the image centre gain 15 us (config 2: 0.270 -> 0.256 ms).
 inline int bin_shard_shift(size_t tiles)
 {
-    static const int env = getenv("ADOP_BIN_SHARD_SHIFT") ? atoi(getenv("ADOP_BIN_SHARD_SHIFT")) : -1;
-    if (env >= 0 && env <= 3) return env;
+    // (read at every call: the tests run every shard count on one scene; the workspace of a call is laid out with the
+    // value its size was asked with, so it must not change in between)
+    const char* e = getenv("ADOP_BIN_SHARD_SHIFT");
+    const int env = e ? atoi(e) : -1;
+    if (e && env >= 0 && env <= 3) return env;
     int s = 0;
     while (tiles <= 4096 && s < 3 && (tiles << (s + 1)) <= 16384) ++s;
     return s;

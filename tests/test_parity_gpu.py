@@ -284,6 +284,21 @@ def test_more_views_than_one_constant_chunk(oracle_mod):
     _fwd_bwd(hs, oracle_mod)
 
 
+@pytest.mark.parametrize("shift", ["0", "1", "2", "3"])
+def test_tile_counters_in_shards(oracle_mod, monkeypatch, shift, forward_path):
+    """The binning passes keep 1, 2, 4 or 8 counters per tile (runs of 256 points take them in turn; by default as many
+    as a call of up to 4 096 tiles can have within 16 384 counters): a bin is the concatenation of its shards' parts,
+    whatever their number.  Two views of 640 x 360 = 1 840 tiles."""
+    from adop_amd import scenes
+
+    if forward_path != 2:
+        pytest.skip("the tile counters belong to the tile path")
+    monkeypatch.setenv("ADOP_BIN_SHARD_SHIFT", shift)
+    announce(f"config2 300k pts B=2 640x360, ADOP_BIN_SHARD_SHIFT={shift}")
+    hs = scenes.config2(n=300_000, w=640, h=360, levels=4, batch=2, seed=8)
+    _fwd_bwd(hs, oracle_mod, collect_stats=int(shift) % 2 == 0, poison=int(shift) % 2 == 1)
+
+
 @pytest.mark.parametrize("collect_stats", [True, False], ids=["counters", "plain"])
 def test_more_views_than_bits_of_the_view_masks(oracle_mod, collect_stats):
     """70 crop windows: the runs of 64 points that miss a window are marked (and their records left unwritten) for the
