@@ -728,17 +728,15 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
                     if (vc.model == 0)
                     {
                         float kf = rp.K_gradient_factor;
-                        bo.g_k[4] *= 0.1f;
-                        bo.g_k[4] *= 0;  // :653-654
+                        bo.g_k[4] *= 0;  // the shear gradient is removed, :653-654
 #pragma unroll
                         for (int k = 0; k < 5; ++k) acc[(8 + k) * kBlock] += kf * bo.g_k[k];
                         float df = rp.distortion_gradient_factor;
+                        // float *= double literal in the reference: the product is formed in double and rounded to
+                        // float once (:664-673); 0.25 is exact either way
                         bo.g_dis[2] *= 0.25f;
-                        bo.g_dis[3] *= 0.1f;
-                        bo.g_dis[4] *= 0.1f;
-                        bo.g_dis[5] *= 0.1f;
-                        bo.g_dis[6] *= 0.1f;
-                        bo.g_dis[7] *= 0.1f;
+#pragma unroll
+                        for (int k = 3; k < 8; ++k) bo.g_dis[k] = (float)((double)bo.g_dis[k] * 0.1);
 #pragma unroll
                         for (int k = 0; k < 8; ++k) acc[(13 + k) * kBlock] += df * bo.g_dis[k];
                         acc[7 * kBlock] += 1.0f / 1024.0f;  // :680-681

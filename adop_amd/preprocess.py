@@ -171,3 +171,22 @@ def PreprocessPointCloud(position, normal=None, rank=4, block_size=256, seed=0):
     data = data[by_radius].contiguous()
     position[:, 3] = data[:, 3]
     return position, (None if normal is None else normal[order].contiguous()), data, order
+
+
+def AttachDropOutRadii(hs, rank=4, block_size=256, seed=0):
+    """Gives a host scene (``scenes.HostScene`` in the reference's point order) what the rasterizer's LOD test reads,
+    as a new scene gets it (SceneData.cpp:103-104): ``position.w`` = ComputeRadius' drop-out radius, every 256-point
+    block sorted by it; switches ``drop_out_points_by_radius`` on (the reference's default, Settings.h:36-37).  The
+    descriptors and the dropout mask of the synthetic scenes are independent random numbers per point and stay."""
+    pos = torch.from_numpy(hs.position).cuda()
+    gen = torch.Generator(device=pos.device).manual_seed(int(seed))
+    data = ComputeRadius(pos, rank, gen)
+    order = SortBlocksByRadius(data[:, 3], block_size)
+    pos = pos[order].contiguous()
+    pos[:, 3] = data[order, 3]
+    hs.position = pos.cpu().numpy()
+    if hs.normal is not None:
+        hs.normal = torch.from_numpy(hs.normal).cuda()[order].cpu().numpy()
+    hs.params.drop_out_points_by_radius = 1
+    hs.meta["lod_radius_test"] = True
+    return hs

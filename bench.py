@@ -10,7 +10,10 @@ environment-map pass on its OCam views and its texture gradient).  Prints ONE JS
 Default workload: BASELINE config 3 (10 M points, 1920x1080, 4 levels, 8 channels, forward + backward with
 descriptor / point / pose / intrinsics gradients) -> points/s.  The default run then also measures the second
 headline figure, config 4 (100 M points, 5 levels, fp16 descriptors, forward over the 300-frame orbit -> frames/s),
-and reports it under ``step.config4`` (``--no-config4`` leaves it out).
+and reports it under ``step.config4`` (``--no-config4`` leaves it out), and after it every other BASELINE
+configuration and the reference's training shape under ``step.configs``: config 1, config 2, config 5 (with its
+environment map), a training batch of 16 crops, and configs 3 and 4 once more with the cloud in random order and with
+the reference's default LOD radius test (``--headline-only`` leaves these out).
 
 ``roofline`` describes the slowest kernel of the step: algorithmic bytes of that kernel (byte model below, with
 the point-level counts V/A/G measured by the kernels' own counters in an untimed pass) divided by its average
@@ -18,11 +21,14 @@ duration measured with HIP events on the launch stream, against the 8 TB/s HBM p
 ``step.hbm_frac_measured`` use HBM bytes per launch measured with rocprofv3 counters (MEASURED_TRAFFIC below: each
 table names the profile it comes from and the kernel state it was measured on; for any other state they are null).
 ``cpu_baseline`` times the CPU checker (OpenMP build) on the host cores for the same workload (or a bounded
-sample of it).
+sample of it): one warm-up run, then the median of three; ``cpu_baseline.matches_gpu`` compares the buffers the
+checker computed in those runs with the HIP path's on the same inputs.
 """
 import argparse
 import ctypes as C
 import gc
+import hashlib
+import glob
 import json
 import os
 import sys
@@ -39,29 +45,29 @@ KERNEL_OF_STAGE = {"BinCount": "bin_count_kernel", "BinScatter": "bin_scatter_ke
                    "EnvironmentMapBackward": "env_backward_kernel"}
 
 # HBM bytes per launch (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, KiB per dispatch; FETCH_SIZE x 2.0 and WRITE_SIZE
-# x 1.0 after calibration with plain device copies of known size), per workload.  "kernels" is the state of the library
-# (the number adop_version() ends in) the profile was taken on: the figures are quoted for that state only.
+# x 1.0 after calibration with plain device copies of known size), per workload.  "sources" is kernel_sources_state() of
+# the tree the profile was taken on (python bench.py --print-sources-state): the figures are quoted for that state only.
 MEASURED_TRAFFIC = {
-    "config3": {"kernels": 10, "profile": "profiles/config3_tile_path_fwd_bwd_kernels_traffic_instructions.md",
+    "config3": {"sources": "d00cff3-state", "profile": "profiles/config3_tile_path_fwd_bwd_kernels_traffic_instructions.md",
                 "bytes": {"RenderBackward/descriptor": 860.1e6, "RenderBackward/spatial": 572.2e6, "TileBlend": 529.1e6,
                           "BinCount": 430.3e6, "CombineAndFillBackward": 220.8e6, "TileDepth": 101.5e6, "Initialize": 11.8e6,
                           "CombineAndFill": 23.5e6, "BinScatter": 197.5e6, "Post Process Gradient": 0.5e6}},
-    "config1": {"kernels": 10, "profile": "profiles/config1_direct_path_forward_kernels_traffic_instructions.md",
+    "config1": {"sources": "d00cff3-state", "profile": "profiles/config1_direct_path_forward_kernels_traffic_instructions.md",
                 "bytes": {"DepthPrepass": 13.1e6, "RenderForward": 8.5e6, "CombineAndFill": 5.6e6, "Initialize": 3.5e6}},
-    "config2": {"kernels": 10, "profile": "profiles/config2_fwd_bwd_kernels_traffic_instructions.md",
+    "config2": {"sources": "d00cff3-state", "profile": "profiles/config2_fwd_bwd_kernels_traffic_instructions.md",
                 "bytes": {"RenderBackward/descriptor": 200.8e6, "BinCount": 64.6e6, "TileBlend": 162.1e6,
                           "RenderBackward/spatial": 145.9e6, "CombineAndFillBackward": 67.2e6, "TileDepth": 37.9e6,
                           "Initialize": 3.4e6, "CombineAndFill": 6.6e6, "BinScatter": 67.4e6, "Post Process Gradient": 15.1e6}},
-    "config4": {"kernels": 10, "profile": "profiles/config4_direct_path_forward_kernels_traffic_instructions.md",
+    "config4": {"sources": "d00cff3-state", "profile": "profiles/config4_direct_path_forward_kernels_traffic_instructions.md",
                 "bytes": {"DepthPrepass": 4856.1e6, "RenderForward": 1445.6e6, "CombineAndFill": 176.8e6, "Initialize":
                           110.5e6}},
     # (the spatial-gradient stage of config5 is 8 launches, its Initialize the clear and a fill)
-    "config5": {"kernels": 10, "profile": "profiles/config5_ocam_envmap_fwd_bwd_kernels_traffic_instructions.md",
+    "config5": {"sources": "d00cff3-state", "profile": "profiles/config5_ocam_envmap_fwd_bwd_kernels_traffic_instructions.md",
                 "bytes": {"RenderBackward/spatial": 8 * 719.5e6, "EnvironmentMapBackward": 2242.8e6, "TileBlend": 5064.5e6,
                           "BinCount": 2189.5e6, "RenderBackward/descriptor": 4091.9e6, "EnvironmentMap": 3081.2e6,
                           "CombineAndFillBackward": 1872.6e6, "TileDepth": 1622.9e6, "CombineAndFill": 177.1e6, "Initialize":
                           91.5e6, "BinScatter": 3331.8e6, "Post Process Gradient": 484.7e6}},
-    "crops": {"kernels": 10, "profile": "profiles/training_batch_16_crops_fwd_bwd_kernels_traffic_instructions.md",
+    "crops": {"sources": "d00cff3-state", "profile": "profiles/training_batch_16_crops_fwd_bwd_kernels_traffic_instructions.md",
                 "bytes": {"RenderBackward/descriptor": 1579.9e6, "RenderBackward/spatial": 1242.1e6, "BinCount": 587.1e6,
                           "TileBlend": 1211.3e6, "CombineAndFillBackward": 446.2e6, "TileDepth": 249.2e6, "CombineAndFill":
                           47.9e6, "Initialize": 23.7e6, "BinScatter": 764.6e6, "Post Process Gradient": 120.3e6}},
@@ -100,10 +106,18 @@ def tile_path_model(k, N, B, C_, P_levels, V, has_dropout, lt=2):
     return k
 
 
-def kernel_state(lib):
-    """The number adop_version() ends in ("... kernels N")."""
-    words = lib.adop_version().decode().split()
-    return int(words[-1]) if len(words) >= 2 and words[-2] == "kernels" and words[-1].isdigit() else None
+def kernel_sources_state():
+    """First 12 hex digits of the SHA-256 over the sources the library is built from (adop_amd/csrc/*.hip, *.h and the
+    C header): the state of the kernels a traffic profile was taken on.  A table of MEASURED_TRAFFIC is quoted only
+    while this matches its "sources" entry, so an edited kernel can never be reported with stale measured bytes."""
+    h = hashlib.sha256()
+    files = sorted(glob.glob(os.path.join(ROOT, "adop_amd", "csrc", "*.hip")) +
+                   glob.glob(os.path.join(ROOT, "adop_amd", "csrc", "*.h")) +
+                   [os.path.join(ROOT, "include", "adop_raster.h")])
+    for f in files:
+        h.update(os.path.basename(f).encode())
+        h.update(open(f, "rb").read())
+    return h.hexdigest()[:12]
 
 
 def host_threads():
@@ -198,15 +212,100 @@ def bench_preprocess(args):
     }
 
 
-def crops_scene(args):
-    """A training batch as the reference forms it: 4 frames x 4 random crops of 512 x 512 of the config-3 scene."""
-    from adop_amd import scenes
+def make_scene(args, workload, point_order, lod):
+    """The host scene of a workload.  point_order: "morton" = the reference's stored order (Morton curve + shuffled
+    256-point blocks, SceneData.cpp:101-102), "random" = a random permutation.  lod: position.w gets the drop-out radius
+    of a new scene (4th-neighbour distance x sqrt(1/u), blocks sorted by it: SceneData.cpp:103-104; computed on the
+    device) and the LOD radius test is switched on (the reference's default, Settings.h:36-37)."""
+    from adop_amd import preprocess, scenes
+
+    import copy
 
     kw = {"n": args.points} if args.points else {}
-    return scenes.training_batch(point_order=args.point_order, **kw)
+    key = (workload, point_order, args.points)
+    if key in _scene_cache:  # (config 4 takes half a minute to generate: its LOD variant starts from the same cloud)
+        base = _scene_cache[key]
+        hs = copy.copy(base)
+        hs.params, hs.meta, hs.views = copy.copy(base.params), dict(base.meta), [copy.copy(v) for v in base.views]
+    else:
+        if workload == "config3":
+            hs = scenes.config3(point_order=point_order, **kw)
+        elif workload == "config1":
+            hs = scenes.config1(**kw)
+        elif workload == "config2":
+            hs = scenes.config2(point_order=point_order, **kw)
+        elif workload == "config4":
+            hs = scenes.config4(point_order=point_order, **kw)
+        elif workload == "crops":
+            hs = scenes.training_batch(point_order=point_order, **kw)
+        else:
+            hs = scenes.config5(point_order=point_order, **kw)
+        if workload == "config4" and point_order == "morton":
+            _scene_cache[key] = hs
+            return make_scene(args, workload, point_order, lod)
+    if lod:
+        preprocess.AttachDropOutRadii(hs)
+    return hs
 
 
-def run_workload(args, workload, steps, warmup, lib):
+_scene_cache = {}
+
+
+def compare_with_checker(lib, scene, chs, ref, refb, cgout, full):
+    """cpu_baseline.matches_gpu: the HIP path on the CPU sample's inputs (the views of ``chs`` of the resident scene)
+    against the buffers the checker computed while it was timed.  Packed depth|index, depth and weight bit for bit;
+    blended descriptors within 1e-5 relative (x sqrt(n / 1024) on a pixel of n > 1024 points, 1e-7 absolute floor: the
+    bars of tests/helpers.py).  ``full`` (the sample is the whole workload): the descriptor gradient element-wise within
+    1e-4 / 1e-6, the other gradients within 1e-4 of the tensor's largest magnitude (the checker's backward pass ran on
+    its own forward images here, whose sums differ by the order of the additions)."""
+    import numpy as np
+    import torch
+    from adop_amd import render
+
+    cache = render.PointRendererCache()
+    info = render.NeuralRenderInfo(scene=scene, images=list(chs.views), params=chs.params, num_layers=chs.num_layers,
+                                   cache=cache, train=refb is not None,
+                                   dropout_points=None if chs.dropout is None else torch.from_numpy(chs.dropout))
+
+    class Ctx:
+        def save_for_backward(self, *t):
+            self.saved_tensors = t
+
+    ctx = Ctx()
+    images, _ = render.BlendPointCloudForward(ctx, info)
+    torch.cuda.synchronize()
+    m = {"depth_index_bit_exact": True, "depth_bit_exact": True, "weight_bit_exact": True, "out_within_1e-5": True,
+         "out_max_rel_err": 0.0}
+    for l, L in enumerate(cache.layers_cuda):
+        m["depth_index_bit_exact"] &= bool(np.array_equal(L.depth_index_tensor.cpu().numpy().view(np.uint64), ref.depth_index[l]))
+        m["depth_bit_exact"] &= bool(np.array_equal(L.depth.cpu().numpy().view(np.uint32), ref.depth[l].view(np.uint32)))
+        w = L.weight.cpu().numpy()
+        m["weight_bit_exact"] &= bool(np.array_equal(w, ref.weight[l]))
+        got, want = images[l].cpu().numpy().astype(np.float64), ref.out[l].astype(np.float64)
+        err = np.abs(got - want)
+        bar = np.maximum(1e-5 * np.sqrt(np.maximum(w.astype(np.float64) / 1024.0, 1.0)) * np.abs(want), 1e-7)
+        m["out_within_1e-5"] &= bool((err <= bar).all())
+        m["out_max_rel_err"] = max(m["out_max_rel_err"], float((err / np.maximum(np.abs(want), 1e-3)).max()))
+    if refb is not None and full:
+        grads = render.BlendPointCloudBackward(ctx, info, [torch.from_numpy(g).cuda() for g in cgout])
+        torch.cuda.synchronize()
+        g_tex = grads[0].cpu().numpy().astype(np.float64)
+        want = refb.grad_texture.astype(np.float64)
+        m["grad_texture_within_1e-4"] = bool((np.abs(g_tex - want) <= np.maximum(1e-4 * np.abs(want), 1e-6)).all())
+        for name, g in zip(("grad_background", "grad_points", "grad_pose", "grad_intrinsics"), grads[1:]):
+            want = getattr(refb, name)
+            if g is not None and want is not None:
+                e = float(np.abs(g.cpu().numpy().astype(np.float64) - want).max() / max(float(np.abs(want).max()), 1e-30))
+                m[name + "_norm_err"] = e
+                m[name + "_within_1e-4"] = e <= 1e-4
+        del grads
+    m["all"] = all(v for k, v in m.items() if isinstance(v, bool))
+    del cache, info, ctx, images
+    torch.cuda.empty_cache()
+    return m
+
+
+def run_workload(args, workload, steps, warmup, lib, point_order=None, lod=False, cpu_leg=True, graph=True):
     """Measures one render workload; returns the JSON object of its bench line."""
     import numpy as np
     import torch
@@ -214,19 +313,8 @@ def run_workload(args, workload, steps, warmup, lib):
 
     dev = "cuda:0"
     t0 = time.time()
-    kw = {"n": args.points} if args.points else {}
-    if workload == "config3":
-        hs = scenes.config3(point_order=args.point_order, **kw)
-    elif workload == "config1":
-        hs = scenes.config1(**kw)
-    elif workload == "config2":
-        hs = scenes.config2(point_order=args.point_order, **kw)
-    elif workload == "config4":
-        hs = scenes.config4(point_order=args.point_order, **kw)
-    elif workload == "crops":
-        hs = crops_scene(args)
-    else:
-        hs = scenes.config5(point_order=args.point_order, **kw)
+    point_order = point_order or args.point_order
+    hs = make_scene(args, workload, point_order, lod)
     backward = workload not in ("config1", "config4")
     with_env = workload == "config5" and hs.env_texture is not None and not args.no_env
     gen_s = time.time() - t0
@@ -372,7 +460,7 @@ def run_workload(args, workload, steps, warmup, lib):
     # the same step recorded once into a HIP graph and replayed (outside the timed region above: what the host-side
     # launches cost); configuration 4 changes a host-side argument every frame and is not recorded
     graph_ms = None
-    if workload != "config4" and not args.no_graph:
+    if workload != "config4" and not args.no_graph and graph:
         side = torch.cuda.Stream()
         graph = torch.cuda.CUDAGraph()
         eager_stream = stream_of[0]
@@ -412,10 +500,10 @@ def run_workload(args, workload, steps, warmup, lib):
     # measured HBM traffic (rocprofv3 counters), for the exact workload and kernel state the profile was taken on
     measured, measured_from = {}, None
     tab = MEASURED_TRAFFIC.get(workload)
-    if (tab and not args.points and args.point_order == "morton" and not args.no_point_cache
-            and tab["kernels"] == kernel_state(lib)):
+    if (tab and not args.points and point_order == "morton" and not args.no_point_cache
+            and not lod and tab.get("sources") == kernel_sources_state()):
         measured = {k: v for k, v in tab["bytes"].items() if k in stages}
-        measured_from = {"profile": tab["profile"], "kernels": tab["kernels"]}
+        measured_from = {"profile": tab["profile"], "sources": tab["sources"]}
     step_measured = None  # every stage of the step that moves memory has a figure
     if measured and all(k in measured for k in stages if k != "Prepare Backward"):
         step_measured = sum(measured.values())
@@ -436,51 +524,60 @@ def run_workload(args, workload, steps, warmup, lib):
         value = N * B / (ms_per_step * 1e-3)
 
     cpu = None
-    if not args.no_cpu_baseline:
+    if cpu_leg and not args.no_cpu_baseline:
         import copy
         import oracle
         nthreads = host_threads()
-        chs, sample, reps = hs, "the full workload, one step", 1
+        chs, sample, full = hs, "the full workload", True
         cpu_n = args.cpu_points or 0
         if workload == "config5":
             # one of the 8 views (the others cost the same per view: stated, not measured)
             chs = copy.copy(hs)
             chs.views, chs.dropout = hs.views[:1], None if hs.dropout is None else np.ascontiguousarray(hs.dropout[:1])
-            sample = f"view 0 of {B} at the full point count and resolution, forward + backward (points/s counts that one view)"
+            sample, full = f"view 0 of {B} at the full point count and resolution, forward + backward (points/s counts that one view)", False
         if workload == "crops":
             chs = copy.copy(hs)
             chs.views, chs.dropout = hs.views[:4], np.ascontiguousarray(hs.dropout[:4])
-            sample = f"the 4 crops of frame 0 (of {B}) at the full point count, forward + backward"
+            sample, full = f"the 4 crops of frame 0 (of {B}) at the full point count, forward + backward", False
         if cpu_n and cpu_n < N:
             chs = copy.copy(chs)
             chs.position, chs.index = hs.position[:cpu_n], hs.index[:cpu_n]
             chs.normal = None if hs.normal is None else hs.normal[:cpu_n]
             chs.dropout = None if chs.dropout is None else np.ascontiguousarray(chs.dropout[:, :cpu_n])
-            sample = f"first {cpu_n} of {N} points; " + sample
-        frames_cpu = [0]
+            sample, full = f"first {cpu_n} of {N} points; " + sample, False
+        # one untimed warm-up run, then three timed ones: the median is the figure (config 4: the three runs are the
+        # orbit frames 0, 100 and 200, the warm-up is frame 50)
+        frames_cpu = [50, 0, 100, 200] if workload == "config4" else [0, 0, 0, 0]
         if workload == "config4":
-            frames_cpu, reps = [0, 100, 200], 3
-            sample = "the full cloud, orbit frames 0, 100 and 200, forward"
+            sample = "the full cloud, forward; warm-up on orbit frame 50, then frames 0, 100 and 200"
         cgout = scenes.upstream_grads(chs) if backward else None
         oracle.lib(True)  # load outside the timed region
-        tc0 = time.perf_counter()
-        for f in frames_cpu:
+        runs, matches = [], None
+        for k, f in enumerate(frames_cpu):
             if workload == "config4":
                 chs.views[0].image_index = f
+            tc0 = time.perf_counter()
             ref = oracle.forward(chs, omp=True)
-            if backward:
-                oracle.backward(chs, ref, cgout, omp=True)
-        tc = time.perf_counter() - tc0
+            refb = oracle.backward(chs, ref, cgout, omp=True) if backward else None
+            if k > 0:
+                runs.append(time.perf_counter() - tc0)
+            if k == len(frames_cpu) - 1 and not cpu_n:
+                matches = compare_with_checker(lib, scene, chs, ref, refb, cgout, full)
+                matches["sample"] = "the buffers of the last timed run" + (f" (orbit frame {f})" if workload == "config4" else "")
+            del ref, refb
+        tc = sorted(runs)[len(runs) // 2]
         if workload == "config4":
             chs.views[0].image_index = 0
         used = oracle.lib(True).oracle_num_threads()
         if workload in ("config4", "config1"):
-            cpu_val, cpu_unit = reps * (chs.num_points / N) / tc, "frames/s"
+            cpu_val, cpu_unit = (chs.num_points / N) / tc, "frames/s"
         else:
             cpu_val, cpu_unit = chs.num_points * chs.batch / tc, "points/s"
-        cpu = {"value": cpu_val, "unit": cpu_unit, "cores": used, "kind": "port", "sample": sample,
-               "seconds": round(tc, 3), "host_cpus": os.cpu_count(),
-               "threads_from": "OMP_NUM_THREADS" if os.environ.get("OMP_NUM_THREADS") else "os.cpu_count()"}
+        cpu = {"value": cpu_val, "unit": cpu_unit, "cores": used, "kind": "port",
+               "sample": sample + "; one warm-up run, median of three timed runs",
+               "seconds": round(tc, 4), "seconds_runs": [round(r, 4) for r in runs], "host_cpus": os.cpu_count(),
+               "threads_from": "OMP_NUM_THREADS" if os.environ.get("OMP_NUM_THREADS") else "os.cpu_count()",
+               "matches_gpu": matches}
         assert used == nthreads or used >= 1
 
     out = {
@@ -492,7 +589,8 @@ def run_workload(args, workload, steps, warmup, lib):
                                f"{L} levels, C={Cn}, " + ("forward+backward" if backward else "forward only") +
                                (", spherical environment map on the OCam views with its gradient" if with_env else "") +
                                (", 300-pose orbit of radius 12, 1.2 degrees per frame" if workload == "config4" else ""),
-                   "point_order": hs.meta.get("point_order", "as generated"), "lod_radius_test": False,
+                   "point_order": hs.meta.get("point_order", "as generated"),
+                   "lod_radius_test": bool(hs.params.drop_out_points_by_radius),
                    "dropout": 0.25 if hs.dropout is not None else 0.0,
                    "ghost_gradients": bool(hs.params.ghost_gradients)},
         "roofline": roofline,
@@ -503,6 +601,9 @@ def run_workload(args, workload, steps, warmup, lib):
                  "hbm_frac_measured": None if step_measured is None else round(step_measured / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                  "hbm_frac_dedup": None if dedup_bytes is None else round(dedup_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                  "measured_from": measured_from,
+                 "workspace_bytes": int(ws_n),
+                 "saved_for_backward_bytes": int((0 if cache.point_cache is None else cache.point_cache.numel() * 4) +
+                                                 (0 if cache.pixel_cache is None else cache.pixel_cache.numel() * 4)),
                  "stage_ms": {k: round(v, 4) for k, v in stages.items()},
                  "stage_GBps": {k: round(model[k] / (stages[k] * 1e-3) / 1e9, 1) for k in model if k in stages},
                  "stage_GBps_measured": {k: round(measured[k] / (stages[k] * 1e-3) / 1e9, 1) for k in measured} or None,
@@ -531,6 +632,10 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-config4", action="store_true",
                     help="default workload only: do not measure the 100 M-point orbit after config3")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="default workload only: leave out the other configurations (step.configs)")
+    ap.add_argument("--print-sources-state", action="store_true",
+                    help="print kernel_sources_state() (what a MEASURED_TRAFFIC table is keyed on) and exit")
     ap.add_argument("--no-env", action="store_true", help="config5 without the environment-map passes")
     ap.add_argument("--no-graph", action="store_true", help="do not replay the step from a HIP graph as well")
     ap.add_argument("--no-point-cache", action="store_true",
@@ -539,6 +644,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
+    if args.print_sources_state:
+        print(kernel_sources_state())
+        return
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (one process, one MI355X); "
               "a figure at several GPUs is not produced. Use --gpus 1.", file=sys.stderr)
@@ -559,17 +667,48 @@ def main():
 
     steps = args.steps or (300 if args.workload == "config4" else 20)
     out = run_workload(args, args.workload, steps, args.warmup, lib)
-    if args.workload == "config3" and not args.no_config4 and not args.points:
+
+    def brief(r):
+        """The figures of a further workload that go into step.configs of the default line."""
+        st = r["step"]
+        return {"metric": r["metric"], "value": round(r["value"], 2), "unit": r["unit"], "steps": r["steps"],
+                "ms_per_step": round(r["ms_per_step"], 4), "workload": r["config"]["workload"],
+                "point_order": r["config"]["point_order"], "lod_radius_test": r["config"]["lod_radius_test"],
+                "dtype": r["dtype"], "roofline": r["roofline"], "cpu_baseline": r["cpu_baseline"],
+                "hbm_frac": st["hbm_frac"], "hbm_frac_measured": st["hbm_frac_measured"],
+                "achieved_GBps": st["achieved_GBps"], "algorithmic_bytes": st["algorithmic_bytes"],
+                "measured_bytes": st["measured_bytes"], "workspace_bytes": st["workspace_bytes"],
+                "saved_for_backward_bytes": st["saved_for_backward_bytes"], "stage_ms": st["stage_ms"],
+                "stage_GBps": st["stage_GBps"], "scene_gen_s": st["scene_gen_s"]}
+
+    default_run = args.workload == "config3" and not args.points and args.point_order == "morton"
+    if default_run and not args.no_config4:
         # the second headline figure: forward frames/s at 100 M points over the whole 300-frame orbit
         c4 = run_workload(args, "config4", 300, args.warmup, lib)
-        out["step"]["config4"] = {
-            "metric": c4["metric"], "value": round(c4["value"], 2), "unit": c4["unit"], "frames": c4["steps"],
-            "ms_per_frame": round(c4["ms_per_step"], 4), "target_frames_per_s": 60, "workload": c4["config"]["workload"],
-            "dtype": c4["dtype"], "roofline": c4["roofline"], "cpu_baseline": c4["cpu_baseline"],
-            "hbm_frac": c4["step"]["hbm_frac"], "hbm_frac_measured": c4["step"]["hbm_frac_measured"],
-            "achieved_GBps": c4["step"]["achieved_GBps"], "stage_ms": c4["step"]["stage_ms"],
-            "stage_GBps": c4["step"]["stage_GBps"], "scene_gen_s": c4["step"]["scene_gen_s"],
-        }
+        out["step"]["config4"] = dict(brief(c4), frames=c4["steps"], ms_per_frame=round(c4["ms_per_step"], 4),
+                                      target_frames_per_s=60)
+    if default_run and not args.headline_only:
+        # Every other BASELINE configuration and the reference's training shape, and the two headline configurations
+        # once more in random point order and with the reference's default LOD radius test.  Fewer steps each, no graph
+        # replay; the CPU leg only where the work differs from a configuration already timed on the CPU.
+        cf = {}
+        few = max(5, min(steps, 10))
+        cf["config3_random_order"] = brief(run_workload(args, "config3", few, args.warmup, lib, point_order="random",
+                                                        cpu_leg=False, graph=False))
+        cf["config3_lod_radius_test"] = brief(run_workload(args, "config3", few, args.warmup, lib, lod=True, graph=False))
+        if not args.no_config4:
+            cf["config4_random_order"] = brief(run_workload(args, "config4", 100, args.warmup, lib, point_order="random",
+                                                            cpu_leg=False))
+            cf["config4_lod_radius_test"] = brief(run_workload(args, "config4", 300, args.warmup, lib, lod=True, cpu_leg=False))
+        cf["config1"] = brief(run_workload(args, "config1", 100, args.warmup, lib, graph=False))
+        cf["config2"] = brief(run_workload(args, "config2", 50, args.warmup, lib, graph=False))
+        cf["config5"] = brief(run_workload(args, "config5", few, args.warmup, lib, graph=False))
+        cf["crops"] = brief(run_workload(args, "crops", few, args.warmup, lib, graph=False))
+        out["step"]["configs"] = cf
+        # the pass line of the headline workload: bytes really moved / step time against the 8 TB/s peak, next to the
+        # fraction by algorithmic bytes
+        out["step"]["pass_line"] = {"hbm_frac_algorithmic": out["step"]["hbm_frac"],
+                                    "hbm_frac_measured": out["step"]["hbm_frac_measured"], "target": 0.60}
     print(json.dumps(out))
 
 

@@ -1021,16 +1021,14 @@ int oracle_backward(const adop_scene* s, const adop_view* views, int B, const ad
                     if (cam.model == ADOP_CAMERA_PINHOLE_DISTORTION)
                     {
                         float k_factor = rp->K_gradient_factor;
-                        bo.g_k[4] *= 0.1f;
-                        bo.g_k[4] *= 0;  // :653-654
+                        // the damping factors are double literals in the reference (float *= double: the product is
+                        // formed in double and rounded to float once), :653-673
+                        bo.g_k[4] = (float)((double)bo.g_k[4] * 0.1);
+                        bo.g_k[4] = (float)((double)bo.g_k[4] * 0);  // :653-654
                         for (int k = 0; k < 5; ++k) gi[k] += (double)(k_factor * bo.g_k[k]);
                         float df = rp->distortion_gradient_factor;
-                        bo.g_dis[2] *= 0.25f;
-                        bo.g_dis[3] *= 0.1f;
-                        bo.g_dis[4] *= 0.1f;
-                        bo.g_dis[5] *= 0.1f;
-                        bo.g_dis[6] *= 0.1f;
-                        bo.g_dis[7] *= 0.1f;
+                        bo.g_dis[2] = (float)((double)bo.g_dis[2] * 0.25);
+                        for (int k = 3; k < 8; ++k) bo.g_dis[k] = (float)((double)bo.g_dis[k] * 0.1);
                         for (int k = 0; k < 8; ++k) gi[5 + k] += (double)(df * bo.g_dis[k]);
                         l_cnt_intr[vw.camera_index] += 1.0 / 1024.0;  // :680-681
                     }

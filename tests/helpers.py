@@ -100,12 +100,53 @@ def assert_close(got, want, rel, abs_tol, what):
                              f"got {got[i]!r} want {want[i]!r}")
 
 
+# Every bar that is wider than the ones the targets state (1e-5 relative for blended descriptors; 1e-4 relative or 1e-6
+# absolute for gradients) is accounted for: the elements that pass ONLY because of the widening are counted per tensor,
+# printed per case ("[bars] ...") and held to a ceiling, so that a widened bar cannot hide a broken kernel.  The
+# ceilings are shares of the tensor's elements; `widened_log` keeps every non-zero count of the process (printed once
+# more by tests/test_zz_widened_bars.py at the end of the GPU suite).
+WIDENED_SHARE = {
+    "out": 1e-3,              # pixels of more than 1024 blended points (sqrt(n/1024) scaling) or below the 1e-7 floor
+    "grad_background": 1.0,   # C numbers, each a cancelling sum over all empty pixels
+    "grad_points": 1e-3,      # absolute bar scaled by the row's largest component
+    "grad_pose": 1.0,         # 6 numbers per frame, sums over all points with cancellation
+    "grad_intrinsics": 1.0,   # 13 numbers per camera, likewise
+}
+widened_log = []
+
+
+def assert_close_accounted(got, want, rel, abs_tol, wide_rel, wide_abs, what, kind, case=""):
+    """Holds `got` to the widened bar |got-want| <= max(wide_rel*|want|, wide_abs) and accounts for the widening: the
+    elements that miss the stated bar max(rel*|want|, abs_tol) but pass the widened one are counted, printed and held
+    to WIDENED_SHARE[kind] of the tensor (at least one element)."""
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    assert_close(got, want, wide_rel, wide_abs, what)
+    if want.size == 0:
+        return 0
+    err = np.abs(got - want)
+    only_wide = err > np.maximum(rel * np.abs(want), abs_tol)
+    n = int(only_wide.sum())
+    if n:
+        worst = float((err / np.maximum(np.abs(want), 1e-30))[only_wide].max())
+        worst_abs = float(err[only_wide].max())
+        rec = (case, what, n, int(want.size), worst, worst_abs)
+        widened_log.append(rec)
+        print(f"[bars] {case} {what}: {n} of {want.size} elements pass only under the widened bar "
+              f"(worst relative {worst:.3g}, absolute {worst_abs:.3g})", flush=True)
+        ceiling = max(1, int(WIDENED_SHARE[kind] * want.size))
+        assert n <= ceiling, f"{what}: {n} of {want.size} elements need the widened bar (ceiling {ceiling})"
+    return n
+
+
 def check_forward(hs, ref, ctx, images, masks, info, stats=True):
     """depth/index bit-exact; weight exact; blended descriptors within 1e-5 relative.  A pixel of more than 1024
     blended points gets sqrt(points / 1024) times that: the checker adds them one after the other in fp32 as the
     reference's atomics do (PointRenderer.cu:383-390), and the rounding error of such a sum grows with the root of
-    the number of terms (1.2e-5 seen on a pixel of 28 758 points, where both HIP paths agree to 1e-7)."""
+    the number of terms (1.2e-5 seen on a pixel of 28 758 points, where both HIP paths agree to 1e-7).  An absolute
+    floor of 1e-7 covers values that cancel to nothing.  Elements that need either are counted (see WIDENED_SHARE)."""
     cache = info.cache
+    case = f"{hs.name} N={hs.num_points} B={hs.batch}"
     for l in range(hs.num_layers):
         L = cache.layers_cuda[l]
         di = L.depth_index_tensor.cpu().numpy().view(np.uint64)
@@ -115,7 +156,7 @@ def check_forward(hs, ref, ctx, images, masks, info, stats=True):
         w = L.weight.cpu().numpy()
         assert np.array_equal(w, ref.weight[l]), f"level {l}: weight differs"
         rel = 1e-5 * np.sqrt(np.maximum(w.astype(np.float64) / 1024.0, 1.0))  # [B,1,h,w], broadcast over the channels
-        assert_close(images[l].cpu().numpy(), ref.out[l], rel, 1e-7, f"level {l} out")
+        assert_close_accounted(images[l].cpu().numpy(), ref.out[l], 1e-5, 0.0, rel, 1e-7, f"level {l} out", "out", case)
         if hs.params.output_background_mask:
             assert np.array_equal(masks[l].cpu().numpy(), ref.mask[l]), f"level {l}: mask differs"
     if not stats:
@@ -139,30 +180,36 @@ def count_misses(got, want, rel=1e-4, abs_tol=1e-6):
 
 
 def check_backward(hs, refb, grads, info, stats=True):
-    """gradients within 1e-4 relative or 1e-6 absolute (float atomics reorder the sums)."""
+    """gradients within 1e-4 relative or 1e-6 absolute (float atomics reorder the sums); where a bar carries a scale
+    (below), the elements that need it are counted and capped (WIDENED_SHARE)."""
     g_tex, g_bg, g_pts, g_pose, g_intr = grads
     cache = info.cache
+    case = f"{hs.name} N={hs.num_points} B={hs.batch}"
     assert_close(g_tex.cpu().numpy(), refb.grad_texture, 1e-4, 1e-6, "grad_texture")
     # the background gradient sums the upstream gradient (N(0,1) in these tests) over the empty pixels of all levels
     # and views: a sum of n terms that cancels to O(sqrt(n)); the kernels add a handful of pixels per thread in fp32
     # before they go on in f64, so its absolute error grows like 2^-24 sqrt(n) (1.0e-4 seen at n = 2.8 M)
     n_pixels = hs.batch * sum(w * h for (w, h) in hs.level_sizes())
-    assert_close(g_bg.cpu().numpy(), refb.grad_background, 1e-4, max(1e-5, 2.4e-7 * np.sqrt(n_pixels)), "grad_background")
+    assert_close_accounted(g_bg.cpu().numpy(), refb.grad_background, 1e-4, 1e-6, 1e-4,
+                           max(1e-5, 2.4e-7 * np.sqrt(n_pixels)), "grad_background", "grad_background", case)
     if g_pts is not None:
         assert np.array_equal(cache.output_gradient_point_count.cpu().numpy(), refb.grad_points_count), "point count"
         # absolute bar: 1e-6 of the point's own gradient vector where that is larger than 1 (a component that cancels
         # to 3e-3 beside components of 50, from 12 terms of that size, was off by 1.4e-6 = half a unit in the last
         # place of the terms)
         row = np.maximum(np.abs(refb.grad_points).max(axis=1, keepdims=True).astype(np.float64), 1.0)
-        assert_close(g_pts.cpu().numpy(), refb.grad_points, 1e-4, 1e-6 * row, "grad_points")
+        assert_close_accounted(g_pts.cpu().numpy(), refb.grad_points, 1e-4, 1e-6, 1e-4, 1e-6 * row, "grad_points",
+                               "grad_points", case)
     if g_pose is not None:
         assert np.array_equal(cache.output_gradient_pose_tangent_count.cpu().numpy(), refb.grad_pose_count)
         scale = np.abs(refb.grad_pose).max() + 1e-30
-        assert_close(g_pose.cpu().numpy(), refb.grad_pose, 1e-4, 1e-6 * max(scale, 1.0), "grad_pose")
+        assert_close_accounted(g_pose.cpu().numpy(), refb.grad_pose, 1e-4, 1e-6, 1e-4, 1e-6 * max(scale, 1.0),
+                               "grad_pose", "grad_pose", case)
     if g_intr is not None:
         assert np.array_equal(cache.output_gradient_intrinsics_count.cpu().numpy(), refb.grad_intrinsics_count)
         scale = np.abs(refb.grad_intrinsics).max() + 1e-30
-        assert_close(g_intr.cpu().numpy(), refb.grad_intrinsics, 1e-4, 1e-6 * max(scale, 1.0), "grad_intrinsics")
+        assert_close_accounted(g_intr.cpu().numpy(), refb.grad_intrinsics, 1e-4, 1e-6, 1e-4, 1e-6 * max(scale, 1.0),
+                               "grad_intrinsics", "grad_intrinsics", case)
     if not stats:
         return
     st = cache.read_stats()

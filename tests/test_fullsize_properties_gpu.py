@@ -1,10 +1,12 @@
 """The BASELINE configurations 3, 4 and 5 at full size (10 M points at 1920x1080 with 8 channels; 100 M points forward
-only with fp16 descriptors; 20 M points through the OCam model at 2200x1500 in 8 views): too big for the CPU checker
-inside a test, so the HIP path is held to size-independent properties of the rasterizer."""
+only with fp16 descriptors; 20 M points through the OCam model at 2200x1500 in 8 views): the HIP path against the CPU
+checker's OpenMP build (tests/test_oracle_omp.py holds that build to the pinned serial one) on config 3 with all its
+gradients, one orbit frame of config 4 and one view of config 5, with the bars of the small cases; and, for the whole
+of each configuration, size-independent properties of the rasterizer."""
 import numpy as np
 import pytest
 
-from helpers import announce, run_hip_forward
+from helpers import announce, check_backward, check_forward, download_forward, run_hip_forward
 
 pytestmark = pytest.mark.gpu
 
@@ -21,6 +23,80 @@ def full_scene(request):
 def full(request, full_scene):
     announce(f"{full_scene.name} full size: forward, forward_path={request.param}")
     return full_scene, run_hip_forward(full_scene, forward_path=request.param)
+
+
+def _against_checker(chs, backward):
+    """Both forward paths (and the backward pass on each one's saved state) against the checker's OpenMP build."""
+    import oracle
+    import torch
+    from adop_amd import render, scenes
+
+    ref = oracle.forward(chs, omp=True)
+    gout = scenes.upstream_grads(chs, 31) if backward else None
+    for path in (1, 2):
+        announce(f"{chs.name} full size against the checker: {chs.num_points} points, B={chs.batch}, forward_path={path}"
+                 f", lod={bool(chs.params.drop_out_points_by_radius)}")
+        scene, info, ctx, images, masks = run_hip_forward(chs, forward_path=path)
+        check_forward(chs, ref, ctx, images, masks, info)
+        if backward:
+            grads = render.BlendPointCloudBackward(ctx, info, [torch.from_numpy(g).cuda() for g in gout])
+            torch.cuda.synchronize()
+            refb = oracle.backward(chs, download_forward(chs, info, images, masks), gout, omp=True)
+            check_backward(chs, refb, grads, info)
+        del scene, info, ctx, images, masks
+        torch.cuda.empty_cache()
+    return ref
+
+
+def _one_view(hs, b=0):
+    import copy
+
+    chs = copy.copy(hs)
+    chs.views = [hs.views[b]]
+    chs.dropout = None if hs.dropout is None else np.ascontiguousarray(hs.dropout[b:b + 1])
+    return chs
+
+
+def test_hip_path_equals_the_checker_at_full_size(full_scene):
+    """Packed depth|index, depth, weight, mask and the counters bit for bit, blended descriptors within 1e-5, every
+    gradient within 1e-4 / 1e-6 of the checker at the sizes the targets are written for: all of config 3 (10 M points,
+    forward + backward), frame 0 of the orbit of config 4 (100 M points, fp16 descriptors), view 0 of config 5 (20 M
+    points through the OCam model, forward + backward)."""
+    hs = full_scene
+    chs = _one_view(hs) if hs.name == "config5" else hs
+    ref = _against_checker(chs, backward=hs.name != "config4")
+    L = hs.num_layers
+    assert sum(ref.stats.accepted[:L]) > 1_000_000 and ref.stats.visible[0] > 0.3 * hs.num_points
+
+
+def test_lod_radius_test_at_full_size(full_scene):
+    """The reference's default setting (drop_out_points_by_radius = true, threshold 0.6: Settings.h:36-37) with the
+    radii a new scene gets (4th-neighbour distance x sqrt(1/u), 256-point blocks sorted by radius: SceneData.cpp:103-104)
+    on config 3 (forward + backward) and on frame 0 of config 4, against the checker; the LOD test must bite (fewer
+    point-levels than without it at the coarse levels, none lost to it at level 0 beyond the points whose radius in
+    pixels is below the threshold)."""
+    import copy
+
+    from adop_amd import preprocess
+
+    hs = full_scene
+    if hs.name == "config5":
+        pytest.skip("the LOD case runs on configurations 3 and 4")
+    chs = copy.copy(hs)
+    chs.params = copy.copy(hs.params)
+    chs.meta = dict(hs.meta)
+    announce(f"{hs.name} full size: drop-out radii of {hs.num_points} points on the device")
+    preprocess.AttachDropOutRadii(chs)
+    assert float(chs.position[:, 3].min()) > 0
+    plain = __import__("oracle").forward(hs, omp=True)
+    ref = _against_checker(chs, backward=hs.name != "config4")
+    L = hs.num_layers
+    vis, vis0 = list(ref.stats.visible[:L]), list(plain.stats.visible[:L])
+    announce(f"{hs.name}: point-levels in the image with the LOD test {vis}, without {vis0}")
+    assert all(a <= b for a, b in zip(vis, vis0)) and vis[L - 1] < 0.7 * vis0[L - 1]
+    # the levels of a point stop at the first one its radius is too small for: the counts cannot grow with the level
+    # faster than without the test
+    assert all(vis[l + 1] * vis0[l] <= vis[l] * vis0[l + 1] * 1.001 for l in range(L - 1))
 
 
 def test_both_forward_paths_agree(full_scene):
