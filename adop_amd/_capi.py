@@ -121,6 +121,18 @@ class Stats(C.Structure):
     ]
 
 
+class Tuning(C.Structure):
+    """adop_tuning: the process's tuning switches (results never depend on them)."""
+    _fields_ = [(n, C.c_int32) for n in (
+        "forward_path", "tile_slice_entries", "ghost_concurrent", "bin_shard_shift", "direct_lists", "prepass_ppt",
+        "prepass_group_from", "blend_group_from", "list_block", "count_ppt", "scatter_ppt", "tile_k", "normalize_fused",
+        "normalize_by_queue")]
+
+
+WORKSPACE_POINT_CACHE_KEPT = 1
+WORKSPACE_NO_TILE_PATH = 2
+
+
 class StageTime(C.Structure):
     _fields_ = [("name", C.c_char * 32), ("total_ms", C.c_float), ("calls", C.c_int32)]
 
@@ -128,6 +140,10 @@ class StageTime(C.Structure):
 # Entry points declared in include/adop_raster.h (name -> (restype, argtypes)).
 ENTRY_POINTS = {
     "adop_workspace_size": (C.c_size_t, [C.POINTER(Scene), C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
+    "adop_workspace_size_for": (C.c_size_t, [C.POINTER(Scene), C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_uint32]),
+    "adop_tuning_defaults": (None, [C.POINTER(Tuning)]),
+    "adop_set_tuning": (C.c_int, [C.POINTER(Tuning)]),
+    "adop_get_tuning": (None, [C.POINTER(Tuning)]),
     "adop_forward": (
         C.c_int,
         [C.POINTER(Scene), C.POINTER(View), C.c_int32, C.POINTER(RenderParams), C.POINTER(ForwardBuffers),
@@ -213,3 +229,31 @@ def load_library(path=None):
     if path is None:
         _lib = lib
     return lib
+
+
+class tuning:
+    """Context manager: ``with _capi.tuning(tile_slice_entries=64): ...`` sets fields of the process's adop_tuning for
+    the calls issued inside and puts the previous set back afterwards (how the tests and the benchmark reach the
+    library's tuning switches)."""
+
+    def __init__(self, **fields):
+        self.fields = fields
+
+    def __enter__(self):
+        lib = load_library()
+        self.before = Tuning()
+        lib.adop_get_tuning(C.byref(self.before))
+        t = Tuning()
+        lib.adop_get_tuning(C.byref(t))
+        for k, v in self.fields.items():
+            if not hasattr(t, k):
+                raise AttributeError(k)
+            setattr(t, k, int(v))
+        rc = lib.adop_set_tuning(C.byref(t))
+        if rc != ADOP_OK:
+            raise ValueError(lib.adop_last_error_string().decode())
+        return t
+
+    def __exit__(self, *exc):
+        load_library().adop_set_tuning(C.byref(self.before))
+        return False

@@ -36,6 +36,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <atomic>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -71,11 +72,15 @@ struct StageEvent
     const char* name;
     hipEvent_t start, stop;
 };
+// Which calls are recorded is a switch of the calling thread; the recorded events go to one list of the process, so
+// that a thread can read what another thread's calls recorded (a framework may run the backward pass on a thread of
+// its own: torch's autograd engine does).
 thread_local bool g_profile = false;
-thread_local std::vector<StageEvent> g_stage_events;
-thread_local std::vector<hipEvent_t> g_event_pool;
+std::mutex g_stage_mutex;
+std::vector<StageEvent> g_stage_events;
+std::vector<hipEvent_t> g_event_pool;
 
-hipEvent_t take_event()
+hipEvent_t take_event()  // (g_stage_mutex held)
 {
     if (!g_event_pool.empty())
     {
@@ -95,6 +100,7 @@ struct StageScope
     StageScope(const char* name, hipStream_t s) : st(s)
     {
         if (!g_profile) return;
+        std::lock_guard<std::mutex> lock(g_stage_mutex);
         hipEvent_t a = take_event(), b = take_event();
         if (!a || !b) return;
         (void)hipEventRecord(a, st);
@@ -106,6 +112,36 @@ struct StageScope
         if (stop) (void)hipEventRecord(stop, st);
     }
 };
+
+// The process's tuning switches: one atomic word per field, so that a call being issued while another thread replaces
+// the set reads every switch whole (from the old or from the new set).
+constexpr int kTuningFields = sizeof(adop_tuning) / sizeof(int32_t);
+static_assert(sizeof(adop_tuning) == kTuningFields * sizeof(int32_t), "adop_tuning holds int32 fields only");
+constexpr adop_tuning kTuningDefaults = {/*forward_path*/ 0,    /*tile_slice_entries*/ kSliceEntries,
+                                         /*ghost_concurrent*/ -1, /*bin_shard_shift*/ -1,
+                                         /*direct_lists*/ 1,    /*prepass_ppt*/ 0,
+                                         /*prepass_group_from*/ 1, /*blend_group_from*/ 0,
+                                         /*list_block*/ 128,    /*count_ppt*/ 2,
+                                         /*scatter_ppt*/ 2,     /*tile_k*/ 1,
+                                         /*normalize_fused*/ 1, /*normalize_by_queue*/ 1};
+struct TuningStore
+{
+    std::atomic<int32_t> f[kTuningFields];
+    TuningStore()
+    {
+        const int32_t* d = (const int32_t*)&kTuningDefaults;
+        for (int k = 0; k < kTuningFields; ++k) f[k].store(d[k], std::memory_order_relaxed);
+    }
+};
+TuningStore g_tuning;
+
+adop_tuning tuning_now()
+{
+    adop_tuning t;
+    int32_t* d = (int32_t*)&t;
+    for (int k = 0; k < kTuningFields; ++k) d[k] = g_tuning.f[k].load(std::memory_order_relaxed);
+    return t;
+}
 
 struct WorkspaceLayout
 {
@@ -130,6 +166,8 @@ struct WorkspaceLayout
     size_t bin_info;    // uint32[B * N]
     size_t bin_entries; // float4[kTileLevels * B * N]
     size_t bin_cap;     // entries
+    size_t common;      // end of what every call uses (all that adop_backward needs)
+    bool has_lists, has_bins;
     size_t total;
 };
 
@@ -180,9 +218,22 @@ size_t align_up(size_t v, size_t a)
     return (v + a - 1) / a * a;
 }
 
-WorkspaceLayout layout(const adop_scene* s, int B, int L, int w0, int h0)
+// Can the tile path take a cloud of n points in B views of w0 x h0?  (Point ids need 28 bits of the bin entry, the bin
+// offsets are 32-bit with at most kTileLevels entries per point and view, the tile word holds 24 bits of tile.)
+bool can_bin(long long n, int B, int w0, int h0)
+{
+    return n > 0 && n < (1ll << 28) && (size_t)kTileLevels * (size_t)B * (size_t)n < ((size_t)1 << 32) &&
+           max_tiles(B, w0, h0) < ((size_t)1 << 24);
+}
+
+// flags: ADOP_WORKSPACE_*.  What every call uses comes first (the backward pass uses nothing else), then what a forward
+// pass without a caller's point cache uses, then the tile bins; the last two may be left out, and the bins are when
+// the tile path cannot take the cloud anyway (can_bin).
+WorkspaceLayout layout(const adop_scene* s, int B, int L, int w0, int h0, uint32_t flags = 0)
 {
     WorkspaceLayout w;
+    memset(&w, 0, sizeof(w));
+    const size_t n = (size_t)(s->num_points > 0 ? s->num_points : 0);
     size_t o     = 0;
     w.views      = o;
     o            = align_up(o + sizeof(ViewConst) * (size_t)B, 256);
@@ -201,40 +252,64 @@ WorkspaceLayout layout(const adop_scene* s, int B, int L, int w0, int h0)
     w.dw = o;
     o    = align_up(o + sizeof(float2) * (size_t)B * pyramid_pixels(L, w0, h0), 256);
     // backward work queue: workgroup k of backward_tex_kernel appends to sub-queue k % kNumQueues
-    size_t blocks = ((size_t)(s->num_points > 0 ? s->num_points : 0) + kBlock - 1) / kBlock;
+    size_t blocks = (n + kBlock - 1) / kBlock;
     w.q_cap       = (uint32_t)(((blocks + kNumQueues - 1) / kNumQueues) * kBlock);
     if (w.q_cap == 0) w.q_cap = kBlock;
     w.q_counts = o;
     o          = align_up(o + sizeof(uint32_t) * ((size_t)B * kNumQueues + 1), 256);
     w.q_items  = o;
     o          = align_up(o + sizeof(unsigned long long) * (size_t)B * kNumQueues * w.q_cap, 256);
+    w.common   = o;
     // (a view's slots are rounded up to whole prepass workgroups of at most 4 * kBlock points: list mode)
-    const size_t n_pad = (((size_t)(s->num_points > 0 ? s->num_points : 0) + 4 * kBlock - 1) / (4 * kBlock)) * (4 * kBlock);
+    const size_t n_pad = ((n + 4 * kBlock - 1) / (4 * kBlock)) * (4 * kBlock);
     w.list_stride = n_pad;
-    w.proj       = o;
-    o            = align_up(o + sizeof(float4) * (size_t)B * n_pad, 256);
-    w.list_ids   = o;
-    o            = align_up(o + sizeof(uint32_t) * (size_t)B * n_pad, 256);
-    w.list_count = o;
-    o = align_up(o + 4 * sizeof(uint32_t) * (size_t)B * (((size_t)(s->num_points > 0 ? s->num_points : 0) + kBlock - 1) / kBlock), 256);
-    size_t T     = max_tiles(B, w0, h0);
-    w.bin_count  = o;  // followed by the row counter and the tickets of the split bins: one range to clear
-    const size_t max_rows = (size_t)slice_rows(s->num_points > 0 ? s->num_points : 0, B);
-    const size_t counters = T << bin_shard_shift(T);
-    o            = align_up(o + sizeof(uint32_t) * (counters + 1 + 2 * max_rows), 256);
-    w.bin_offset = o;
-    o            = align_up(o + sizeof(uint32_t) * (counters + 1), 256);
-    w.bin_order  = o;
-    o            = align_up(o + sizeof(uint4) * (T + max_rows), 256);
-    w.bin_rows   = o;
-    o            = align_up(o + sizeof(float) * max_rows * (size_t)slice_row_floats(s->num_channels > 0 ? s->num_channels : 1), 256);
-    w.bin_cap    = (size_t)kTileLevels * (size_t)B * (size_t)(s->num_points > 0 ? s->num_points : 0);
-    w.bin_info   = o;
-    o            = align_up(o + sizeof(uint32_t) * (size_t)B * (size_t)(s->num_points > 0 ? s->num_points : 0), 256);
-    w.bin_entries = o;
-    o            = align_up(o + sizeof(float4) * w.bin_cap, 256);
+    w.has_lists   = (flags & ADOP_WORKSPACE_POINT_CACHE_KEPT) == 0;
+    if (w.has_lists)
+    {
+        w.proj       = o;
+        o            = align_up(o + sizeof(float4) * (size_t)B * n_pad, 256);
+        w.list_ids   = o;
+        o            = align_up(o + sizeof(uint32_t) * (size_t)B * n_pad, 256);
+        w.list_count = o;
+        o            = align_up(o + 4 * sizeof(uint32_t) * (size_t)B * ((n + kBlock - 1) / kBlock), 256);
+    }
+    w.has_bins = (flags & ADOP_WORKSPACE_NO_TILE_PATH) == 0 && can_bin((long long)n, B, w0, h0);
+    if (w.has_bins)
+    {
+        size_t T     = max_tiles(B, w0, h0);
+        w.bin_count  = o;  // followed by the row counter and the tickets of the split bins: one range to clear
+        const size_t max_rows = (size_t)slice_rows((long long)n, B);
+        const size_t counters = bin_counter_capacity(T);
+        o            = align_up(o + sizeof(uint32_t) * (counters + 1 + 2 * max_rows), 256);
+        w.bin_offset = o;
+        o            = align_up(o + sizeof(uint32_t) * (counters + 1), 256);
+        w.bin_order  = o;
+        o            = align_up(o + sizeof(uint4) * (T + max_rows), 256);
+        w.bin_rows   = o;
+        o            = align_up(o + sizeof(float) * max_rows * (size_t)slice_row_floats(s->num_channels > 0 ? s->num_channels : 1), 256);
+        w.bin_cap    = (size_t)kTileLevels * (size_t)B * n;
+        w.bin_info   = o;
+        o            = align_up(o + sizeof(uint32_t) * (size_t)B * n, 256);
+        w.bin_entries = o;
+        o            = align_up(o + sizeof(float4) * w.bin_cap, 256);
+    }
     w.total      = o;
     return w;
+}
+
+// The layout of the workspace a forward call was given: the largest of the four that fits (a layout without the
+// region of a forward pass that keeps no point cache only when the caller passes one).
+bool choose_layout(const adop_scene* s, int B, int L, int w0, int h0, size_t bytes, bool has_point_cache, WorkspaceLayout* out)
+{
+    const uint32_t order[4] = {0u, ADOP_WORKSPACE_POINT_CACHE_KEPT, ADOP_WORKSPACE_NO_TILE_PATH,
+                               ADOP_WORKSPACE_POINT_CACHE_KEPT | ADOP_WORKSPACE_NO_TILE_PATH};
+    for (uint32_t flags : order)
+    {
+        if ((flags & ADOP_WORKSPACE_POINT_CACHE_KEPT) && !has_point_cache) continue;
+        *out = layout(s, B, L, w0, h0, flags);
+        if (bytes >= out->total) return true;
+    }
+    return false;
 }
 
 adop_status validate(const adop_scene* s, const adop_view* views, int B, const adop_render_params* rp,
@@ -449,6 +524,51 @@ size_t adop_workspace_size(const adop_scene* scene, int32_t num_views, int32_t n
     return layout(scene, num_views, num_layers, w, h).total;
 }
 
+size_t adop_workspace_size_for(const adop_scene* scene, int32_t num_views, int32_t num_layers, int32_t w, int32_t h,
+                               uint32_t flags)
+{
+    if (!scene || num_views < 1 || num_layers < 1 || num_layers > ADOP_MAX_LAYERS || w < 1 || h < 1) return 0;
+    if (scene->num_channels < 1 || scene->num_channels > kMaxChannels) return 0;
+    if (flags & ~(ADOP_WORKSPACE_POINT_CACHE_KEPT | ADOP_WORKSPACE_NO_TILE_PATH)) return 0;
+    return layout(scene, num_views, num_layers, w, h, flags).total;
+}
+
+void adop_tuning_defaults(adop_tuning* out)
+{
+    if (out) *out = kTuningDefaults;
+}
+
+adop_status adop_set_tuning(const adop_tuning* t)
+{
+    if (!t) return fail(ADOP_INVALID_ARG, "null argument");
+    auto one_of = [](int v, std::initializer_list<int> ok) {
+        for (int k : ok)
+            if (v == k) return true;
+        return false;
+    };
+    if (t->forward_path < 0 || t->forward_path > 2) return fail(ADOP_INVALID_ARG, "tuning: forward_path must be 0, 1 or 2");
+    if (t->tile_slice_entries < 1) return fail(ADOP_INVALID_ARG, "tuning: tile_slice_entries must be positive");
+    if (t->ghost_concurrent < -1 || t->ghost_concurrent > 1) return fail(ADOP_INVALID_ARG, "tuning: ghost_concurrent must be -1, 0 or 1");
+    if (t->bin_shard_shift < -1 || t->bin_shard_shift > 3) return fail(ADOP_INVALID_ARG, "tuning: bin_shard_shift must be -1 .. 3");
+    if (!one_of(t->direct_lists, {0, 1}) || !one_of(t->normalize_fused, {0, 1}) || !one_of(t->normalize_by_queue, {0, 1}))
+        return fail(ADOP_INVALID_ARG, "tuning: direct_lists, normalize_fused and normalize_by_queue are 0 or 1");
+    if (!one_of(t->prepass_ppt, {0, 1, 2, 4}) || !one_of(t->count_ppt, {1, 2, 4}) || !one_of(t->scatter_ppt, {1, 2, 4}) ||
+        !one_of(t->tile_k, {1, 2, 4}))
+        return fail(ADOP_INVALID_ARG, "tuning: points / entries per thread must be 1, 2 or 4 (prepass_ppt: or 0)");
+    if (t->prepass_group_from < 0 || t->prepass_group_from > ADOP_MAX_LAYERS || t->blend_group_from < 0 ||
+        t->blend_group_from > ADOP_MAX_LAYERS)
+        return fail(ADOP_INVALID_ARG, "tuning: a level is 0 .. ADOP_MAX_LAYERS");
+    if (!one_of(t->list_block, {64, 128, 256})) return fail(ADOP_INVALID_ARG, "tuning: list_block must be 64, 128 or 256");
+    const int32_t* d = (const int32_t*)t;
+    for (int k = 0; k < kTuningFields; ++k) g_tuning.f[k].store(d[k], std::memory_order_relaxed);
+    return ADOP_OK;
+}
+
+void adop_get_tuning(adop_tuning* out)
+{
+    if (out) *out = tuning_now();
+}
+
 // RenderParams::render_points == false (PointRenderer.cu:1417,1433): the forward pass runs on an empty cloud (its
 // workspace layout lies inside the one the caller sized for the whole cloud).
 static const adop_scene* leave_out_points(const adop_scene* scene, adop_scene* copy)
@@ -467,8 +587,11 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
     if (st != ADOP_OK) return st;
     adop_scene without_points;
     if (params->skip_points) scene = leave_out_points(scene, &without_points);
-    WorkspaceLayout wl = layout(scene, num_views, buffers->num_layers, views[0].w, views[0].h);
-    if (!workspace || workspace_bytes < wl.total) return fail(ADOP_WORKSPACE_TOO_SMALL, "workspace too small");
+    WorkspaceLayout wl;
+    if (!workspace || !choose_layout(scene, num_views, buffers->num_layers, views[0].w, views[0].h, workspace_bytes,
+                                     buffers->point_cache != nullptr, &wl))
+        return fail(ADOP_WORKSPACE_TOO_SMALL, "workspace too small");
+    const adop_tuning tn = tuning_now();
     hipStream_t stream = (hipStream_t)hip_stream;
     ViewConst* dviews  = (ViewConst*)((char*)workspace + wl.views);
 
@@ -489,14 +612,13 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
     float* accum     = (float*)((char*)workspace + wl.pixels);
     const bool half  = scene->texture_dtype == ADOP_TEXTURE_F16;
 
-    // Tile path: point ids need 28 bits of the bin entry; a handful of points is faster through the direct path.
-    static const int env_path = getenv("ADOP_FORWARD_PATH") ? atoi(getenv("ADOP_FORWARD_PATH")) : 0;
-    int path = params->forward_path ? params->forward_path : env_path;
+    // Tile path: only where the workspace holds the bins (a caller may leave them out, and layout() does when the cloud
+    // is beyond what the bin entries can address); a handful of points is faster through the direct path.
+    int path = params->forward_path ? params->forward_path : tn.forward_path;
     if (path < 0 || path > 2) return fail(ADOP_INVALID_ARG, "forward_path must be 0, 1 or 2");
-    // (bin offsets are 32-bit: a point has at most kTileLevels entries per view)
-    const bool can_bin = scene->num_points > 0 && scene->num_points < (1 << 28) &&
-                         (size_t)kTileLevels * num_views * scene->num_points < ((size_t)1 << 32) &&
-                         max_tiles(num_views, views[0].w, views[0].h) < ((size_t)1 << 24);
+    const bool bins_possible = can_bin(scene->num_points, num_views, views[0].w, views[0].h);
+    if (path == 2 && bins_possible && !wl.has_bins)
+        return fail(ADOP_WORKSPACE_TOO_SMALL, "forward_path = 2 needs a workspace with the tile bins");
     // The tile path bins every projected point; a cloud with very many points per pixel is faster through the direct
     // path, whose early depth test drops most of them before they cost anything.
     // A batch of windows into their frames (crop offsets: the crops of a training step) counts with the share of the
@@ -517,11 +639,11 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
                    ? 2
                    : 1;
     }
-    if (path == 2 && !can_bin) path = 1;
+    if (path == 2 && !wl.has_bins) path = 1;
 
     if (path == 2)
     {
-        if (!pc.cache) pc.cache = (float4*)((char*)workspace + wl.proj);
+        if (!pc.cache) pc.cache = (float4*)((char*)workspace + wl.proj);  // (has_lists: choose_layout)
         BinArg bin;
         bin.lt      = kTileLevels < lv.num ? kTileLevels : lv.num;
         bin.tiles_x = ((views[0].w - 1) >> kTileShiftX) + 1;
@@ -533,16 +655,14 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
         bin.entries = (float4*)((char*)workspace + wl.bin_entries);
         bin.info    = (uint32_t*)((char*)workspace + wl.bin_info);
         const int T = bin.tiles_x * bin.tiles_y * num_views;
-        bin.shard_shift   = bin_shard_shift((size_t)T);
+        bin.shard_shift   = bin_shard_shift((size_t)T, tn.bin_shard_shift);
         bin.num_tiles     = T;
         const int counters = T << bin.shard_shift;
         bin.row_count = bin.count + counters;
         bin.tickets   = bin.count + counters + 1;
         bin.max_rows   = slice_rows(scene->num_points, num_views);
         bin.row_floats = slice_row_floats(scene->num_channels);
-        // (read at every call: the tests split small bins)
-        const char* env_slice = getenv("ADOP_TILE_SLICE");
-        bin.slice_entries     = env_slice && atoi(env_slice) > 0 ? (uint32_t)atoi(env_slice) : (uint32_t)kSliceEntries;
+        bin.slice_entries = (uint32_t)tn.tile_slice_entries;
         {
             StageScope sc("Initialize", stream);
             // tile counters, and for the coarse levels the packed depth and the global accumulators of the direct path
@@ -554,12 +674,12 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
         }
         {
             StageScope sc("BinCount", stream);
-            launch_bin(0, pc, dviews, lv, rp, bin, stats, stream);
+            launch_bin(0, pc, dviews, lv, rp, bin, stats, tn, stream);
         }
         {
             StageScope sc("BinScatter", stream);
             launch_tile_scan(bin, counters, stream);
-            launch_bin(1, pc, dviews, lv, rp, bin, nullptr, stream);
+            launch_bin(1, pc, dviews, lv, rp, bin, nullptr, tn, stream);
         }
         {
             StageScope sc("TileDepth", stream);
@@ -569,7 +689,7 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
             StageScope sc("TileBlend", stream);
             ADOP_HIP_CHECK(launch_tile_blend(pc, lv, rp, bin, T, half, accum, S, scene->background_color,
                                              params->output_background_mask, params->output_background_mask_value,
-                                             scene->index_is_identity, stats, stream));
+                                             scene->index_is_identity, stats, tn, stream));
         }
         if (bin.lt < lv.num)
         {
@@ -583,13 +703,14 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
 
     // Without a caller's point cache (no backward pass follows) the prepass hands the blend compacted lists of the
     // points that can still pass a depth test instead of a record per point.
-    static const int env_lists = getenv("ADOP_DIRECT_LISTS") ? atoi(getenv("ADOP_DIRECT_LISTS")) : 1;
-    if (!pc.cache && env_lists && scene->num_points > 0)
+    if (!pc.cache && !wl.has_lists)  // (choose_layout: unreachable; kept as the guard of the pointer arithmetic below)
+        return fail(ADOP_WORKSPACE_TOO_SMALL, "a forward pass without point_cache needs the full workspace");
+    if (!pc.cache && tn.direct_lists && scene->num_points > 0)
     {
         pc.cache      = (float4*)((char*)workspace + wl.proj);
         pc.list_ids   = (uint32_t*)((char*)workspace + wl.list_ids);
         pc.list_count = (uint32_t*)((char*)workspace + wl.list_count);
-        pc.list_span  = prepass_points_per_block(scene->num_points);
+        pc.list_span  = prepass_points_per_block(scene->num_points, tn.prepass_ppt);
         pc.list_stride = wl.list_stride;
     }
     size_t accum_n   = (size_t)lv.pix_prefix[lv.num] * lv.B * S;  // floats, multiple of 4 unless S < 4
@@ -605,11 +726,11 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
     }
     {
         StageScope sc("DepthPrepass", stream);
-        launch_prepass(pc, dviews, lv, rp, stats, stream);
+        launch_prepass(pc, dviews, lv, rp, stats, tn, stream);
     }
     {
         StageScope sc("RenderForward", stream);
-        launch_blend(pc, dviews, lv, rp, half, accum, S, stats, stream);
+        launch_blend(pc, dviews, lv, rp, half, accum, S, stats, tn, stream);
     }
     {
         StageScope sc("CombineAndFill", stream);
@@ -635,8 +756,11 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     if (grads->grad_pose && !grads->grad_pose_count) return fail(ADOP_INVALID_ARG, "grad_pose_count missing");
     if (grads->grad_intrinsics && !grads->grad_intrinsics_count)
         return fail(ADOP_INVALID_ARG, "grad_intrinsics_count missing");
-    WorkspaceLayout wl = layout(scene, num_views, fwd->num_layers, views[0].w, views[0].h);
+    // (the backward pass uses the first part of the workspace only, which every layout has)
+    WorkspaceLayout wl = layout(scene, num_views, fwd->num_layers, views[0].w, views[0].h,
+                                ADOP_WORKSPACE_POINT_CACHE_KEPT | ADOP_WORKSPACE_NO_TILE_PATH);
     if (!workspace || workspace_bytes < wl.total) return fail(ADOP_WORKSPACE_TOO_SMALL, "workspace too small");
+    const adop_tuning tn = tuning_now();
     hipStream_t stream = (hipStream_t)hip_stream;
     ViewConst* dviews  = (ViewConst*)((char*)workspace + wl.views);
     double* bg_partial = (double*)((char*)workspace + wl.bg_partial);
@@ -698,16 +822,14 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     // Side by side pays while a launch per view would be small or the views share few points (the crop windows of a
     // training batch; a cloud of at most kConcurrentMaxPoints points); full views of a large cloud, which share most
     // of their points, fill a launch each and need no atomics that way (8 views of 20 M points: 1.76 against 1.82 ms).
-    // ADOP_GHOST_CONCURRENT=1 forces the one launch, 0 the launch per view.
-    const char* env_conc = getenv("ADOP_GHOST_CONCURRENT");
+    // adop_tuning.ghost_concurrent = 1 forces the one launch, 0 the launch per view.
     bool windows         = num_views > 1;
     for (int b = 0; b < num_views; ++b) windows = windows && (views[b].crop_cx != 0.f || views[b].crop_cy != 0.f);
-    const bool want_conc = env_conc ? atoi(env_conc) != 0 : (windows || N <= kConcurrentMaxPoints);
+    const bool want_conc = tn.ghost_concurrent >= 0 ? tn.ghost_concurrent != 0 : (windows || N <= kConcurrentMaxPoints);
     q.concurrent         = num_views > 1 && num_views <= kConcurrentViews && want_conc ? 1 : 0;
-    // One view: the spatial-gradient kernel normalises the point gradients itself (ADOP_NORMALIZE_FUSED=0: a pass of
-    // the finalize kernel over the work queue does).
-    static const int fused_norm = getenv("ADOP_NORMALIZE_FUSED") ? atoi(getenv("ADOP_NORMALIZE_FUSED")) : 1;
-    q.normalize = (num_views == 1 && grads->grad_points && fused_norm) ? (params->normalize_mode == 0 ? 1 : 2) : 0;
+    // One view: the spatial-gradient kernel normalises the point gradients itself (adop_tuning.normalize_fused = 0: a
+    // pass of the finalize kernel does).
+    q.normalize = (num_views == 1 && grads->grad_points && tn.normalize_fused) ? (params->normalize_mode == 0 ? 1 : 2) : 0;
     if (N < 1)
     {
         // nothing writes the partial rows: clear them for finalize
@@ -736,7 +858,7 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     StageScope post("Post Process Gradient", stream);
     launch_finalize(dviews, num_views, C, bg_partial, bg_blocks, pt_partial, pt_blocks, grads, scene->num_poses,
                     scene->num_cameras, scene->intrinsics_cols, params->normalize_mode, scratch,
-                    (double*)((char*)workspace + wl.fin_mini), q.counts + (size_t)num_views * kNumQueues, N, q, stream);
+                    (double*)((char*)workspace + wl.fin_mini), q.counts + (size_t)num_views * kNumQueues, N, q, tn, stream);
     ADOP_HIP_CHECK(hipGetLastError());
     return ADOP_OK;
 }
@@ -1094,7 +1216,12 @@ adop_status adop_profile_enable(int32_t enable)
 int32_t adop_profile_read(adop_stage_time* out, int32_t max_entries)
 {
     int n = 0;
-    for (StageEvent& e : g_stage_events)
+    std::vector<StageEvent> events;
+    {
+        std::lock_guard<std::mutex> lock(g_stage_mutex);
+        events.swap(g_stage_events);
+    }
+    for (StageEvent& e : events)
     {
         float ms = 0.f;
         if (hipEventSynchronize(e.stop) == hipSuccess && hipEventElapsedTime(&ms, e.start, e.stop) == hipSuccess)
@@ -1114,10 +1241,13 @@ int32_t adop_profile_read(adop_stage_time* out, int32_t max_entries)
                 out[k].calls += 1;
             }
         }
+    }
+    std::lock_guard<std::mutex> lock(g_stage_mutex);
+    for (StageEvent& e : events)
+    {
         g_event_pool.push_back(e.start);
         g_event_pool.push_back(e.stop);
     }
-    g_stage_events.clear();
     return n;
 }
 
@@ -1128,8 +1258,6 @@ const char* adop_last_error_string(void)
 
 const char* adop_version(void)
 {
-    // "kernels N" names the state of the kernels' memory behaviour: it goes up whenever a change moves a kernel's bytes,
-    // so that traffic figures measured for one state (rocprofv3 counters) are not quoted for another.
-    return "adop_raster 0.2 (gfx950) kernels 10";
+    return "adop_raster 0.3 (gfx950)";
 }
 }  // extern "C"

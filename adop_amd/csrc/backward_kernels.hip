@@ -1302,13 +1302,13 @@ void launch_backward_ghost(const CloudArg& pc, const ViewConst* views, const Lev
 void launch_finalize(const ViewConst* views, int B, int C, const double* bg_partial, int bg_blocks,
                      const double* pt_partial, int pt_blocks, const adop_backward_buffers* g, int num_poses,
                      int num_cameras, int cols, int normalize_mode, double* scratch, double* mini, uint32_t* ticket, int n,
-                     const QueueArg& q, hipStream_t st)
+                     const QueueArg& q, const adop_tuning& tn, hipStream_t st)
 {
     FinalizeArg a{views, B, C, bg_partial, bg_blocks, pt_partial, pt_blocks, g->grad_background, g->grad_pose,
                   g->grad_pose_count, num_poses, g->grad_intrinsics, g->grad_intrinsics_count, num_cameras, cols,
                   normalize_mode, scratch, mini, ticket, nullptr, nullptr, 0};
     if (!g->grad_points || n < 1) n = 0;
-    static const int by_queue = getenv("ADOP_NORMALIZE_BY_QUEUE") ? atoi(getenv("ADOP_NORMALIZE_BY_QUEUE")) : 1;
+    const int by_queue = tn.normalize_by_queue;
     if (n == 0)
         hipLaunchKernelGGL(finalize_kernel, dim3(1), dim3(kFinalizeBlock), 0, st, a);
     else if (q.normalize)

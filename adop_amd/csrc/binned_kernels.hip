@@ -493,12 +493,12 @@ __global__ __launch_bounds__(1024) void tile_scan_kernel(const uint32_t* __restr
 // launchers
 // ------------------------------------------------------------------------------------------------
 void launch_bin(int pass, const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp,
-                const BinArg& bin, adop_stats* stats, hipStream_t st)
+                const BinArg& bin, adop_stats* stats, const adop_tuning& tn, hipStream_t st)
 {
     if (pc.n < 1) return;
     if (pass == 0)
     {
-        static const int cppt = getenv("ADOP_COUNT_PPT") ? atoi(getenv("ADOP_COUNT_PPT")) : 2;
+        const int cppt = tn.count_ppt;
         if (cppt == 2)
             hipLaunchKernelGGL((bin_count_kernel<2>), dim3((pc.n + kBlock * 2 - 1) / (kBlock * 2)), dim3(kBlock), 0, st,
                                pc, views, lv, rp, bin, stats);
@@ -512,7 +512,7 @@ void launch_bin(int pass, const CloudArg& pc, const ViewConst* views, const Leve
     }
     const int T = bin.tiles_x * bin.tiles_y * lv.B;
     const int G = order_groups(T);
-    static const int ppt = getenv("ADOP_SCATTER_PPT") ? atoi(getenv("ADOP_SCATTER_PPT")) : 2;
+    const int ppt = tn.scatter_ppt;
     if (ppt == 1)
         hipLaunchKernelGGL((bin_scatter_kernel<1>), dim3(G + (pc.n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, pc, lv, rp, bin, T, G);
     else if (ppt == 2)

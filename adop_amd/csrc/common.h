@@ -9,6 +9,15 @@
 
 #pragma clang fp contract(off)
 
+// These kernels are written for gfx950 (CDNA4) alone, and a few places lean on what that hardware does: wave64, the
+// LDS and vector instructions named in the comments, and, where partial results travel between workgroups through
+// agent-scope atomic stores and loads around a ticket (backward_kernels.hip, tile_kernels.hip), on stores being counted
+// by vmcnt, so that s_waitcnt(0) before the ticket means they have been acknowledged.  An architecture with a separate
+// store counter would need release / acquire on the ticket instead: refuse to build there rather than run wrong.
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
+#error "adop_raster's kernels are written for gfx950 only (see the comment above)"
+#endif
+
 namespace adop
 {
 constexpr int kBlock         = 256;

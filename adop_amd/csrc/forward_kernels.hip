@@ -591,21 +591,20 @@ void launch_clear(const Levels& lv, int first_level, int grid, float* accum, siz
 // their density (more loads in flight per wavefront: config 4 1.10 -> 1.04 ms), one below 2^24 points, where the
 // launch is a few workgroups per CU and the shorter chain per thread counts (1 M points in 256 x 256, unordered:
 // 0.17 -> 0.10 ms; 100 k points: 0.096 -> 0.073 ms).
-static int prepass_ppt(int n)
+static int prepass_ppt(int n, int tuned)
 {
-    static const int env = getenv("ADOP_PREPASS_PPT") ? atoi(getenv("ADOP_PREPASS_PPT")) : 0;
-    const int ppt        = env ? env : (n >= (1 << 24) ? 2 : 1);
+    const int ppt = tuned ? tuned : (n >= (1 << 24) ? 2 : 1);
     return ppt == 4 ? 4 : (ppt == 2 ? 2 : 1);
 }
 
-int prepass_points_per_block(int n) { return kBlock * prepass_ppt(n); }
+int prepass_points_per_block(int n, int tuned_ppt) { return kBlock * prepass_ppt(n, tuned_ppt); }
 
 void launch_prepass(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, adop_stats* stats,
-                    hipStream_t st)
+                    const adop_tuning& tn, hipStream_t st)
 {
     if (pc.n < 1) return;
-    static const int group_from = getenv("ADOP_PREPASS_GROUP_FROM") ? atoi(getenv("ADOP_PREPASS_GROUP_FROM")) : 1;
-    const int ppt               = prepass_ppt(pc.n);
+    const int group_from = tn.prepass_group_from;
+    const int ppt        = prepass_ppt(pc.n, tn.prepass_ppt);
     if (ppt == 4)
         hipLaunchKernelGGL((prepass_kernel<4>), dim3((pc.n + kBlock * 4 - 1) / (kBlock * 4)), dim3(kBlock), 0, st, pc,
                            views, lv, rp, group_from, stats);
@@ -619,11 +618,11 @@ void launch_prepass(const CloudArg& pc, const ViewConst* views, const Levels& lv
 
 template <int CT, bool HALF>
 static void launch_blend_t(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp,
-                           float* accum, int S, adop_stats* stats, hipStream_t st)
+                           float* accum, int S, adop_stats* stats, const adop_tuning& tn, hipStream_t st)
 {
-    static const int group_from = getenv("ADOP_BLEND_GROUP_FROM") ? atoi(getenv("ADOP_BLEND_GROUP_FROM")) : 0;  // 0: group at every level
+    const int group_from = tn.blend_group_from;  // 0: group at every level
     // list mode: one small workgroup per prepass workgroup (a few percent of the points survive in a dense cloud)
-    static const int list_block = getenv("ADOP_LIST_BLOCK") ? atoi(getenv("ADOP_LIST_BLOCK")) : 128;
+    const int list_block = tn.list_block;
     const int block = pc.list_ids ? ((list_block >= 64 && list_block <= kBlock && list_block % 64 == 0) ? list_block : 128)
                                   : kBlock;
     const int grid  = pc.list_ids ? (pc.n + pc.list_span - 1) / pc.list_span : (pc.n + kBlock - 1) / kBlock;
@@ -633,18 +632,18 @@ static void launch_blend_t(const CloudArg& pc, const ViewConst* views, const Lev
 }
 
 void launch_blend(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
-                  float* accum, int S, adop_stats* stats, hipStream_t st)
+                  float* accum, int S, adop_stats* stats, const adop_tuning& tn, hipStream_t st)
 {
     if (pc.n < 1) return;
     if (lv.C == 8)
-        half ? launch_blend_t<8, true>(pc, views, lv, rp, accum, S, stats, st)
-             : launch_blend_t<8, false>(pc, views, lv, rp, accum, S, stats, st);
+        half ? launch_blend_t<8, true>(pc, views, lv, rp, accum, S, stats, tn, st)
+             : launch_blend_t<8, false>(pc, views, lv, rp, accum, S, stats, tn, st);
     else if (lv.C == 4)
-        half ? launch_blend_t<4, true>(pc, views, lv, rp, accum, S, stats, st)
-             : launch_blend_t<4, false>(pc, views, lv, rp, accum, S, stats, st);
+        half ? launch_blend_t<4, true>(pc, views, lv, rp, accum, S, stats, tn, st)
+             : launch_blend_t<4, false>(pc, views, lv, rp, accum, S, stats, tn, st);
     else
-        half ? launch_blend_t<0, true>(pc, views, lv, rp, accum, S, stats, st)
-             : launch_blend_t<0, false>(pc, views, lv, rp, accum, S, stats, st);
+        half ? launch_blend_t<0, true>(pc, views, lv, rp, accum, S, stats, tn, st)
+             : launch_blend_t<0, false>(pc, views, lv, rp, accum, S, stats, tn, st);
 }
 
 void launch_resolve(const Levels& lv, int first_level, int grid, const float* accum, int S, const float* background,

@@ -5,6 +5,9 @@
 
 namespace adop
 {
+// The process's tuning switches as they are now (adop_set_tuning / adop_get_tuning; defined in adop_raster.hip).
+adop_tuning tuning_now();
+
 struct EnvLevels
 {
     float* uv[ADOP_MAX_LAYERS];
@@ -41,11 +44,13 @@ void launch_close_points(const float4* sorted, int n, const KnnGrid* g, const ui
                          int32_t* state, uint32_t* round_count, int round, hipStream_t st);
 void launch_morton(const float4* position, int n, const float* mn, const float* scale, unsigned long long* code,
                    hipStream_t st);
-int prepass_points_per_block(int n);  // points per workgroup of prepass_kernel on a cloud of n points (the unit of its candidate lists)
+// The launchers take the tuning switches of the call as an argument (one snapshot per call: adop_forward / adop_backward).
+// points per workgroup of prepass_kernel on a cloud of n points (the unit of its candidate lists)
+int prepass_points_per_block(int n, int tuned_ppt);
 void launch_prepass(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, adop_stats* stats,
-                    hipStream_t st);
+                    const adop_tuning& tn, hipStream_t st);
 void launch_blend(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
-                  float* accum, int S, adop_stats* stats, hipStream_t st);
+                  float* accum, int S, adop_stats* stats, const adop_tuning& tn, hipStream_t st);
 void launch_resolve(const Levels& lv, int first_level, int grid, const float* accum, int S, const float* background,
                     int write_mask, float mask_value, hipStream_t st);
 
@@ -90,17 +95,28 @@ struct BinArg
 // Shards per tile: as many as keep the counters of a call within 16 384 (the prefix sum over them is one workgroup), at
 // most 8, and none above 4 096 tiles: the second pass then looks up two lines per entry group instead of one, which a
 // view of 1920 x 1080 without hot tiles pays with 7 us (config 3), while 4 views of 512 x 512 of a cloud that piles up
-// in the image centre gain 15 us (config 2: 0.270 -> 0.256 ms).
-inline int bin_shard_shift(size_t tiles)
+// in the image centre gain 15 us (config 2: 0.270 -> 0.256 ms).  `tuned` >= 0 (adop_tuning.bin_shard_shift) asks for a
+// shift, which is lowered while the call would need more counters than the workspace holds.
+constexpr size_t kMaxShardedCounters = 65536;  // counters a call may have through an explicit shard shift
+inline int bin_shard_shift(size_t tiles, int tuned)
 {
-    // (read at every call: the tests run every shard count on one scene; the workspace of a call is laid out with the
-    // value its size was asked with, so it must not change in between)
-    const char* e = getenv("ADOP_BIN_SHARD_SHIFT");
-    const int env = e ? atoi(e) : -1;
-    if (e && env >= 0 && env <= 3) return env;
+    if (tuned >= 0)
+    {
+        int s = tuned > 3 ? 3 : tuned;
+        while (s > 0 && (tiles << s) > kMaxShardedCounters) --s;
+        return s;
+    }
     int s = 0;
     while (tiles <= 4096 && s < 3 && (tiles << (s + 1)) <= 16384) ++s;
     return s;
+}
+// counters the workspace holds for a call of `tiles` tiles: enough for every shard shift bin_shard_shift() can return
+inline size_t bin_counter_capacity(size_t tiles)
+{
+    size_t c = tiles;
+    for (int s = 1; s <= 3; ++s)
+        if ((tiles << s) <= kMaxShardedCounters) c = tiles << s;
+    return c;
 }
 inline uint32_t bin_shard_of(uint32_t point, int shard_shift) { return (point >> 8) & ((1u << shard_shift) - 1u); }
 constexpr int kMaxSlices = 1024;  // (10 bits of the slice word)
@@ -121,12 +137,13 @@ inline int slice_rows(long long n, int B)
 constexpr uint32_t kEntryIdMask  = 0x0FFFFFFFu;  // entry word: point id; bits 28..30: levels before the LOD break;
 constexpr uint32_t kEntryPrimary = 0x80000000u;  // bit 31: entry of the tile that owns the (clamped) level-0 pixel
 void launch_bin(int pass, const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp,
-                const BinArg& bin, adop_stats* stats, hipStream_t st);
+                const BinArg& bin, adop_stats* stats, const adop_tuning& tn, hipStream_t st);
 void launch_tile_scan(const BinArg& bin, int num_tiles, hipStream_t st);
 void launch_tile_depth(const Levels& lv, const BinArg& bin, int num_tiles, hipStream_t st);
 hipError_t launch_tile_blend(const CloudArg& pc, const Levels& lv, const ParamArg& rp, const BinArg& bin, int num_tiles,
                              bool half, float* accum, int S, const float* background, int write_mask,
-                             float mask_value, int identity_index, adop_stats* stats, hipStream_t st);
+                             float mask_value, int identity_index, adop_stats* stats, const adop_tuning& tn,
+                             hipStream_t st);
 
 void launch_interleave(const Levels& lv, int blocks, float* ig, float2* dw, double* partial, uint32_t* q_counts,
                        const ViewPrep& vp, hipStream_t st);
@@ -155,7 +172,7 @@ constexpr int kConcurrentViews = 24;  // views whose level masks a descriptor-pa
 void launch_finalize(const ViewConst* views, int B, int C, const double* bg_partial, int bg_blocks,
                      const double* pt_partial, int pt_blocks, const adop_backward_buffers* g, int num_poses,
                      int num_cameras, int cols, int normalize_mode, double* scratch, double* mini, uint32_t* ticket, int n,
-                     const QueueArg& q, hipStream_t st);
+                     const QueueArg& q, const adop_tuning& tn, hipStream_t st);
 
 void launch_env_sample(const ViewChunk& chunk, const double* poses, const float* intrinsics, const Levels& lv,
                        const EnvLevels& ev, const float* tex, int eh, int ew, int add_to_out, int cols, hipStream_t st);

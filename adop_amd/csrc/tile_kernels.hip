@@ -726,9 +726,8 @@ static hipError_t launch_tile_blend_k(const CloudArg& pc, const Levels& lv, cons
 template <int CT, bool HALF>
 static hipError_t launch_tile_blend_t(const CloudArg& pc, const Levels& lv, const ParamArg& rp, const BinArg& bin,
                                       int num_tiles, float* accum, int S, const float* background, int write_mask,
-                                      float mask_value, int identity_index, adop_stats* stats, hipStream_t st)
+                                      float mask_value, int identity_index, adop_stats* stats, int k, hipStream_t st)
 {
-    static const int k = getenv("ADOP_TILE_K") ? atoi(getenv("ADOP_TILE_K")) : 1;
     if (k == 1)
         return launch_tile_blend_k<CT, HALF, 1>(pc, lv, rp, bin, num_tiles, accum, S, background, write_mask, mask_value,
                                                 identity_index, stats, st);
@@ -741,10 +740,11 @@ static hipError_t launch_tile_blend_t(const CloudArg& pc, const Levels& lv, cons
 
 hipError_t launch_tile_blend(const CloudArg& pc, const Levels& lv, const ParamArg& rp, const BinArg& bin, int num_tiles,
                              bool half, float* accum, int S, const float* background, int write_mask,
-                             float mask_value, int identity_index, adop_stats* stats, hipStream_t st)
+                             float mask_value, int identity_index, adop_stats* stats, const adop_tuning& tn,
+                             hipStream_t st)
 {
 #define ADOP_TILE(CT, H) \
-    launch_tile_blend_t<CT, H>(pc, lv, rp, bin, num_tiles, accum, S, background, write_mask, mask_value, identity_index, stats, st)
+    launch_tile_blend_t<CT, H>(pc, lv, rp, bin, num_tiles, accum, S, background, write_mask, mask_value, identity_index, stats, tn.tile_k, st)
     if (lv.C == 8) return half ? ADOP_TILE(8, true) : ADOP_TILE(8, false);
     if (lv.C == 4) return half ? ADOP_TILE(4, true) : ADOP_TILE(4, false);
     return half ? ADOP_TILE(0, true) : ADOP_TILE(0, false);

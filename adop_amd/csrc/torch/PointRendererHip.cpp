@@ -81,7 +81,43 @@ void Check(adop_status st)
 {
     TORCH_CHECK(st == ADOP_OK, "adop_raster: ", adop_last_error_string());
 }
+
+// While one of these lives and a timer system is attached, the library records its stage events on this thread.
+struct StageRecording
+{
+    bool on;
+    explicit StageRecording(StageTimerSystem* t) : on(t != nullptr)
+    {
+        if (on) adop_profile_enable(1);
+    }
+    ~StageRecording()
+    {
+        if (on) adop_profile_enable(0);
+    }
+};
 }  // namespace
+
+// ---- StageTimerSystem (the role of CUDA::CudaTimerSystem behind NeuralRenderInfo::timer_system) -------------
+void StageTimerSystem::BeginFrame()
+{
+    // events of calls that ran outside a frame are dropped
+    adop_stage_time scratch[32];
+    adop_profile_read(scratch, 32);
+}
+
+void StageTimerSystem::EndFrame()
+{
+    adop_stage_time t[32];
+    const int n = adop_profile_read(t, 32);  // waits for the events of the frame's calls
+    for (int i = 0; i < n; ++i)
+    {
+        Entry& e  = stages[t[i].name];
+        e.last_ms = t[i].total_ms;
+        e.total_ms += t[i].total_ms;
+        e.calls += t[i].calls;
+        e.frames += 1;
+    }
+}
 
 // ---- NeuralPointCloudCuda ----------------------------------------------------------------------------------
 NeuralPointCloudCudaImpl::NeuralPointCloudCudaImpl(torch::Tensor position, torch::Tensor normal, torch::Tensor index)
@@ -238,8 +274,11 @@ std::pair<std::vector<torch::Tensor>, std::vector<torch::Tensor>> BlendPointClou
         pixel_cache    = torch::empty({pixels, (long)scene.num_channels}, d[0].options());
         fb.pixel_cache = pixel_cache.data_ptr<float>();
     }
-    Check(adop_forward(&scene, views.data(), (int)views.size(), &rp, &fb, cache.workspace.data_ptr(),
-                       (size_t)cache.workspace.numel(), nullptr, CurrentStream()));
+    {
+        StageRecording rec(info->timer_system);
+        Check(adop_forward(&scene, views.data(), (int)views.size(), &rp, &fb, cache.workspace.data_ptr(),
+                           (size_t)cache.workspace.numel(), nullptr, CurrentStream()));
+    }
 
     if (info->params.debug_print_num_rendered_points)  // PointRenderer.cu:1502-1512
     {
@@ -358,8 +397,11 @@ torch::autograd::variable_list BlendPointCloudBackward(torch::autograd::Autograd
         (size_t)cache.workspace.numel() < adop_workspace_size(&s, (int)views.size(), L, views[0].w, views[0].h))
         cache.workspace = torch::empty({(long)adop_workspace_size(&s, (int)views.size(), L, views[0].w, views[0].h)},
                                        f32.dtype(torch::kUInt8));
-    Check(adop_backward(&s, views.data(), (int)views.size(), &rp, &fb, &gb, cache.workspace.data_ptr(),
-                        (size_t)cache.workspace.numel(), nullptr, CurrentStream()));
+    {
+        StageRecording rec(info->timer_system);
+        Check(adop_backward(&s, views.data(), (int)views.size(), &rp, &fb, &gb, cache.workspace.data_ptr(),
+                            (size_t)cache.workspace.numel(), nullptr, CurrentStream()));
+    }
 
     torch::Tensor g_tex = cache.output_gradient_texture;
     if (scene.texture->texture.dtype() != torch::kFloat32) g_tex = g_tex.to(scene.texture->texture.dtype());
@@ -406,6 +448,110 @@ variable_list PointRender::backward(AutogradContext* ctx, variable_list grad_out
 }
 }  // namespace torch::autograd
 
+// ---- EnvironmentMapImpl::Sample + composition as an autograd function -------------------------------------------
+namespace
+{
+// The forward buffers of an environment-map call: level sizes from the tensors, `out` / `mask` as given.
+adop_forward_buffers EnvBuffers(int L, const std::vector<torch::Tensor>& images, const std::vector<torch::Tensor>& masks)
+{
+    adop_forward_buffers fb{};
+    fb.num_layers = L;
+    for (int l = 0; l < L; ++l)
+    {
+        fb.layers[l].w    = (int)images[l].size(3);
+        fb.layers[l].h    = (int)images[l].size(2);
+        fb.layers[l].out  = images[l].data_ptr<float>();
+        fb.layers[l].mask = masks.empty() ? nullptr : masks[l].data_ptr<float>();
+    }
+    return fb;
+}
+}  // namespace
+
+namespace torch::autograd
+{
+variable_list EnvironmentMapCompose::forward(AutogradContext* ctx, Variable texture, at::TensorList images_in,
+                                             at::TensorList masks_in, IValue info, bool cat_env_to_color)
+{
+    NeuralRenderInfo* nri = info.toCustomClass<NeuralRenderInfo>().get();
+    const int L           = nri->num_layers;
+    TORCH_CHECK((int)images_in.size() == L && (int)masks_in.size() == L, "one image and one mask per layer");
+    torch::Tensor tex = texture.dim() == 4 ? texture.squeeze(0) : texture;
+    TORCH_CHECK(tex.dim() == 3 && tex.dtype() == torch::kFloat32 && tex.is_cuda(), "environment map: [C,H,W] f32 on the device");
+    tex = tex.contiguous();
+    std::vector<torch::Tensor> images, masks, uv(L), outs(L);
+    for (int l = 0; l < L; ++l)
+    {
+        images.push_back(images_in[l].contiguous());
+        masks.push_back(masks_in[l].contiguous());
+        TORCH_CHECK(images[l].size(1) == tex.size(0), "environment map and images differ in channels");
+        uv[l]   = torch::empty({images[l].size(0), images[l].size(2), images[l].size(3), 2}, images[l].options());
+        outs[l] = torch::empty_like(images[l]);
+    }
+    adop_scene s = MakeScene(*nri->scene);
+    auto views   = MakeViews(nri);
+    // composed: out of place (mode 2), sampling only where mask != 1; cat: the samples of every pixel (mode 0, no mask)
+    adop_forward_buffers fb = EnvBuffers(L, images, cat_env_to_color ? std::vector<torch::Tensor>() : masks);
+    std::vector<float*> uv_ptr(L), out_ptr(L);
+    for (int l = 0; l < L; ++l)
+    {
+        uv_ptr[l]  = uv[l].data_ptr<float>();
+        out_ptr[l] = outs[l].data_ptr<float>();
+    }
+    Check(adop_env_sample(&s, views.data(), (int)views.size(), tex.data_ptr<float>(), (int)tex.size(1), (int)tex.size(2),
+                          &fb, uv_ptr.data(), out_ptr.data(), cat_env_to_color ? 0 : 2, CurrentStream()));
+    variable_list save = uv;
+    if (!cat_env_to_color) save.insert(save.end(), masks.begin(), masks.end());
+    ctx->save_for_backward(save);
+    ctx->saved_data["render_info"] = info;
+    ctx->saved_data["cat"]         = cat_env_to_color;
+    ctx->saved_data["tex_dim"]     = (int64_t)texture.dim();
+    ctx->saved_data["env_h"]       = (int64_t)tex.size(1);
+    ctx->saved_data["env_w"]       = (int64_t)tex.size(2);
+    return outs;
+}
+
+variable_list EnvironmentMapCompose::backward(AutogradContext* ctx, variable_list grad_output)
+{
+    IValue info           = ctx->saved_data["render_info"];
+    NeuralRenderInfo* nri = info.toCustomClass<NeuralRenderInfo>().get();
+    const int L           = nri->num_layers;
+    const bool cat        = ctx->saved_data["cat"].toBool();
+    const int eh = (int)ctx->saved_data["env_h"].toInt(), ew = (int)ctx->saved_data["env_w"].toInt();
+    auto saved = ctx->get_saved_variables();
+    std::vector<torch::Tensor> uv(saved.begin(), saved.begin() + L), masks;
+    if (!cat) masks.assign(saved.begin() + L, saved.begin() + 2 * L);
+    std::vector<torch::Tensor> gout(L);
+    for (int l = 0; l < L; ++l)
+    {
+        // (a level that does not reach the loss has no gradient)
+        gout[l] = grad_output[l].defined() ? grad_output[l].contiguous()
+                                           : torch::zeros({uv[l].size(0), nri->scene->texture->texture.size(0), uv[l].size(1), uv[l].size(2)},
+                                                          uv[l].options());
+    }
+    adop_scene s            = MakeScene(*nri->scene);
+    auto views              = MakeViews(nri);
+    adop_forward_buffers fb = EnvBuffers(L, gout, masks);  // (only sizes and masks are read)
+    std::vector<const float*> g_ptr(L), uv_ptr(L);
+    for (int l = 0; l < L; ++l)
+    {
+        g_ptr[l]  = gout[l].data_ptr<float>();
+        uv_ptr[l] = uv[l].data_ptr<float>();
+    }
+    torch::Tensor g_tex = torch::empty({(long)s.num_channels, (long)eh, (long)ew}, gout[0].options());
+    Check(adop_env_sample_backward(&s, views.data(), (int)views.size(), eh, ew, &fb, g_ptr.data(), uv_ptr.data(),
+                                   g_tex.data_ptr<float>(), CurrentStream()));
+    if (ctx->saved_data["tex_dim"].toInt() == 4) g_tex = g_tex.unsqueeze(0);
+    // inputs: texture, L images, L masks, info, cat.  d composed / d image = 1 (composition) or nothing (cat).
+    variable_list grads;
+    grads.push_back(g_tex);
+    for (int l = 0; l < L; ++l) grads.push_back(cat ? Variable() : grad_output[l]);
+    for (int l = 0; l < L; ++l) grads.push_back(Variable());
+    grads.push_back(Variable());
+    grads.push_back(Variable());
+    return grads;
+}
+}  // namespace torch::autograd
+
 void ApplyTangentToPose(torch::Tensor tangent, torch::Tensor pose)
 {
     TORCH_CHECK(tangent.is_contiguous() && pose.is_contiguous());
@@ -447,40 +593,16 @@ std::pair<std::vector<torch::Tensor>, std::vector<torch::Tensor>> PointRenderMod
     }
     if (nri->scene->environment_map)
     {
-        // EnvironmentMapImpl::Sample (EnvironmentMap.cu:107-157): uv from the library, sampling by torch so that
-        // autograd provides the texture gradient exactly as in the reference
+        // EnvironmentMapImpl::Sample + the composition (EnvironmentMap.cu:107-157, RenderModule.cpp:106-127) through
+        // the library's fused kernels, with the texture gradient from adop_env_sample_backward
         TORCH_CHECK(nri->params.output_background_mask);
-        auto tex = nri->scene->environment_map->texture;
-        if (tex.dim() == 3) tex = tex.unsqueeze(0);
-        adop_scene s = MakeScene(*nri->scene);
-        auto views   = MakeViews(nri);
-        adop_forward_buffers fb{};
-        fb.num_layers = nri->num_layers;
-        std::vector<torch::Tensor> uv(nri->num_layers);
-        std::vector<float*> uv_ptr(nri->num_layers);
-        int h = nri->images.front().h, w = nri->images.front().w;
+        torch::intrusive_ptr<NeuralRenderInfo> render_data = torch::make_intrusive<NeuralRenderInfo>(*nri);
+        // (the lists go in as at::TensorList: that is the type whose elements autograd takes as inputs of the node)
+        auto env = torch::autograd::EnvironmentMapCompose::apply(nri->scene->environment_map->texture,
+                                                                 at::TensorList(images), at::TensorList(point_masks),
+                                                                 torch::IValue(render_data), opt.cat_env_to_color);
         for (int i = 0; i < nri->num_layers; ++i)
-        {
-            uv[i]     = torch::empty({(long)views.size(), h, w, 2}, images[0].options());
-            uv_ptr[i] = uv[i].data_ptr<float>();
-            fb.layers[i].w = w;
-            fb.layers[i].h = h;
-            h /= 2;
-            w /= 2;
-        }
-        Check(adop_env_sample(&s, views.data(), (int)views.size(), tex.data_ptr<float>(), (int)tex.size(2),
-                              (int)tex.size(3), &fb, uv_ptr.data(), nullptr, 0, CurrentStream()));
-        namespace F = torch::nn::functional;
-        auto go     = F::GridSampleFuncOptions().align_corners(true).padding_mode(torch::kBorder).mode(torch::kBilinear);
-        auto batched = tex.repeat({(long)views.size(), 1, 1, 1});
-        for (int i = 0; i < nri->num_layers; ++i)
-        {
-            auto env = F::grid_sample(batched, uv[i], go);
-            if (opt.cat_env_to_color)
-                images[i] = torch::cat({images[i], env}, 1);
-            else
-                images[i] = images[i] + (1 - point_masks[i]) * env;
-        }
+            images[i] = opt.cat_env_to_color ? torch::cat({images[i], env[i]}, 1) : env[i];
     }
     if (opt.cat_masks_to_color)
         for (int i = 0; i < nri->num_layers; ++i) images[i] = torch::cat({images[i], point_masks[i]}, 1);

@@ -8,7 +8,9 @@
 #pragma once
 #include <torch/torch.h>
 
+#include <map>
 #include <memory>
+#include <string>
 #include <vector>
 
 #include "../../../include/adop_raster.h"
@@ -111,14 +113,40 @@ constexpr int max_layers = ADOP_MAX_LAYERS;
 
 class PointRendererCache;
 
+// Stands where saiga's CUDA::CudaTimerSystem stands in the reference (NeuralRenderInfo::timer_system,
+// PointRenderer.h:32; the SAIGA_OPTIONAL_TIME_MEASURE scopes of PointRenderer.cu:906-1610): while a render call runs with
+// a timer system attached, the library records HIP events around its stages on the call's stream
+// (adop_profile_enable); EndFrame() waits for them (adop_profile_read) and adds the stage times of the frame to the
+// table, under the reference's stage names.  Used as the reference's viewer uses its timer system
+// (RealTimeRenderer.cpp:80,196): BeginFrame(), render calls, EndFrame(), then read.
+class StageTimerSystem
+{
+   public:
+    struct Entry
+    {
+        float last_ms  = 0;  // the stage's time in the last finished frame (all its launches)
+        double total_ms = 0;
+        long calls      = 0;  // launches of the stage over all frames
+        long frames     = 0;
+    };
+    void BeginFrame();
+    void EndFrame();
+    const std::map<std::string, Entry>& Stages() const { return stages; }
+    void Reset() { stages.clear(); }
+
+   private:
+    std::map<std::string, Entry> stages;
+};
+
 class NeuralRenderInfo : public torch::CustomClassHolder
 {
    public:
     NeuralScene* scene = nullptr;
     std::vector<ReducedImageInfo> images;
     RenderParams params;
-    int num_layers            = 0;
-    PointRendererCache* cache = nullptr;
+    int num_layers                 = 0;
+    StageTimerSystem* timer_system = nullptr;  // PointRenderer.h:32
+    PointRendererCache* cache      = nullptr;
 };
 
 namespace torch::autograd
@@ -128,6 +156,20 @@ struct PointRender : public Function<PointRender>
     // returns a tensor for every layer (then a mask for every layer if params.output_background_mask)
     static variable_list forward(AutogradContext* ctx, Variable texture, Variable background_color, Variable points,
                                  Variable pose_tangents, Variable intrinsics, IValue info);
+    static variable_list backward(AutogradContext* ctx, variable_list grad_output);
+};
+// Environment map on the empty pixels (EnvironmentMapImpl::Sample, EnvironmentMap.cu:107-157, and the composition of
+// RenderModule.cpp:106-127) as one autograd function over the library's fused kernels: the forward pass samples only
+// where the composition looks (mask != 1) and writes the composed images, the backward pass sums the texture gradient
+// per tile in LDS from the texture coordinates the forward pass kept.  Same numbers as torch's grid_sample (bilinear,
+// border, align_corners) on the reference's uv followed by images + (1 - mask) * env.
+struct EnvironmentMapCompose : public Function<EnvironmentMapCompose>
+{
+    // texture [C,H,W] | [1,C,H,W]; images: L tensors [B,C,h_l,w_l]; masks: L tensors [B,1,h_l,w_l] (not differentiated);
+    // cat_env_to_color: the sampled map of every pixel is returned by itself (for torch::cat) instead of composed.
+    // Returns L tensors.  The views are info's images (pinhole, or OCam as an extension).
+    static variable_list forward(AutogradContext* ctx, Variable texture, at::TensorList images, at::TensorList masks,
+                                 IValue info, bool cat_env_to_color);
     static variable_list backward(AutogradContext* ctx, variable_list grad_output);
 };
 }  // namespace torch::autograd

@@ -11,6 +11,7 @@ struct PyScene
 {
     NeuralScene scene;
     PointRendererCache cache;
+    StageTimerSystem timer;  // what a caller hangs on NeuralRenderInfo::timer_system (render(..., timed = true))
 
     PyScene(torch::Tensor position, c10::optional<torch::Tensor> normal, torch::Tensor index, torch::Tensor texture,
             torch::Tensor background, torch::Tensor poses_se3, torch::Tensor tangent_poses, torch::Tensor intrinsics,
@@ -67,13 +68,15 @@ static RenderParams ParamsFromDict(const py::dict& d)
 using ViewTuple = std::tuple<int, int, int, int, int, float, float, float, float, float>;
 
 static std::vector<torch::Tensor> Render(PyScene& s, const std::vector<ViewTuple>& views, const py::dict& params,
-                                         int num_layers, bool training, bool through_module)
+                                         int num_layers, bool training, bool through_module, bool timed,
+                                         bool cat_env_to_color)
 {
     NeuralRenderInfo nri;
-    nri.scene      = &s.scene;
-    nri.num_layers = num_layers;
-    nri.params     = ParamsFromDict(params);
-    nri.cache      = &s.cache;
+    nri.scene        = &s.scene;
+    nri.num_layers   = num_layers;
+    nri.params       = ParamsFromDict(params);
+    nri.cache        = &s.cache;
+    nri.timer_system = timed ? &s.timer : nullptr;
     for (auto& v : views)
     {
         ReducedImageInfo i;
@@ -86,7 +89,9 @@ static std::vector<torch::Tensor> Render(PyScene& s, const std::vector<ViewTuple
         nri.images.push_back(i);
     }
     if (!through_module) return BlendPointCloud(&nri);
-    auto [images, masks] = PointRenderModuleForward(&nri, &s.cache, PointRenderModuleOptions(), training);
+    PointRenderModuleOptions opt;
+    opt.cat_env_to_color = cat_env_to_color;
+    auto [images, masks] = PointRenderModuleForward(&nri, &s.cache, opt, training);
     images.insert(images.end(), masks.begin(), masks.end());
     return images;
 }
@@ -98,9 +103,20 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
                       torch::Tensor, torch::Tensor, torch::Tensor, c10::optional<torch::Tensor>>(),
              py::arg("position"), py::arg("normal"), py::arg("index"), py::arg("texture"), py::arg("background"),
              py::arg("poses_se3"), py::arg("tangent_poses"), py::arg("intrinsics"), py::arg("env") = py::none())
-        .def("apply_tangent", [](PyScene& s) { s.scene.poses->ApplyTangent(); });
+        .def("apply_tangent", [](PyScene& s) { s.scene.poses->ApplyTangent(); })
+        // the scene's StageTimerSystem, used as the reference's viewer uses its timer system: begin_frame(), render
+        // calls with timed = true (and their backward passes), end_frame(), stage_times()
+        .def("begin_frame", [](PyScene& s) { s.timer.BeginFrame(); })
+        .def("end_frame", [](PyScene& s) { s.timer.EndFrame(); })
+        .def("stage_times", [](PyScene& s) {
+            py::dict d;
+            for (auto& [name, e] : s.timer.Stages())
+                d[py::str(name)] = py::make_tuple(e.last_ms, e.total_ms, e.calls, e.frames);
+            return d;
+        });
     m.def("render", &Render, py::arg("scene"), py::arg("views"), py::arg("params"), py::arg("num_layers"),
-          py::arg("training") = true, py::arg("through_module") = false);
+          py::arg("training") = true, py::arg("through_module") = false, py::arg("timed") = false,
+          py::arg("cat_env_to_color") = false);
     m.def("apply_tangent_to_pose", &ApplyTangentToPose);
     // point-cloud processing of a new scene (SceneDataHip.cpp)
     m.def("knn_distance", &KNearestNeighbourDistance, py::arg("position"), py::arg("n") = 4);

@@ -132,6 +132,9 @@ class NeuralRenderInfo:
     # with train: the forward pass also leaves the resolved images pixel by pixel for the backward pass (one more
     # saved tensor of the size of the images); False: the backward pass builds those records from the images itself
     keep_pixel_records: bool = True
+    # adop_workspace_size_for flags (_capi.WORKSPACE_*): a smaller workspace for a caller that always keeps the point
+    # cache (train) and / or can do without the tile-bin forward path
+    workspace_flags: int = 0
 
 
 class PointRendererCache:
@@ -166,7 +169,7 @@ class PointRendererCache:
         scene = info.scene
         dev = scene.texture.device
         new_size = (int(scene.texture.shape[0]), scene.point_cloud_cuda.Size(), info.num_layers, self.num_batches,
-                    fd.h, fd.w)
+                    fd.h, fd.w, int(info.workspace_flags))
         if new_size == self.cache_size:
             return
         B = self.num_batches
@@ -183,7 +186,7 @@ class PointRendererCache:
             h //= 2
             scale *= 0.5
         s = scene.struct()
-        nbytes = self.lib.adop_workspace_size(C.byref(s), B, info.num_layers, fd.w, fd.h)
+        nbytes = self.lib.adop_workspace_size_for(C.byref(s), B, info.num_layers, fd.w, fd.h, int(info.workspace_flags))
         self.workspace = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=dev)
         self.stats = torch.zeros(C.sizeof(_capi.Stats) // 8, dtype=torch.int64, device=dev)
         self.cache_size = new_size

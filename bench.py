@@ -636,6 +636,8 @@ def main():
                     help="default workload only: leave out the other configurations (step.configs)")
     ap.add_argument("--print-sources-state", action="store_true",
                     help="print kernel_sources_state() (what a MEASURED_TRAFFIC table is keyed on) and exit")
+    ap.add_argument("--tuning", default="",
+                    help="adop_tuning fields for the whole run, e.g. tile_k=2,count_ppt=4 (A/B runs of the library's switches)")
     ap.add_argument("--no-env", action="store_true", help="config5 without the environment-map passes")
     ap.add_argument("--no-graph", action="store_true", help="do not replay the step from a HIP graph as well")
     ap.add_argument("--no-point-cache", action="store_true",
@@ -660,6 +662,16 @@ def main():
         sys.exit(3)
     lib = _capi.load_library()
     torch.cuda.set_device(0)
+    if args.tuning:
+        t = _capi.Tuning()
+        lib.adop_get_tuning(C.byref(t))
+        for kv in args.tuning.split(","):
+            k, v = kv.split("=")
+            if not hasattr(t, k):
+                sys.exit(f"bench.py: unknown tuning field {k}")
+            setattr(t, k, int(v))
+        if lib.adop_set_tuning(C.byref(t)) != 0:
+            sys.exit("bench.py: " + lib.adop_last_error_string().decode())
     if args.workload == "preprocess":
         args.steps = args.steps or 20
         print(json.dumps(bench_preprocess(args)))

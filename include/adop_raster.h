@@ -184,8 +184,57 @@ typedef struct adop_stats
     uint64_t bad_index;                 /* texture index out of range (reference: device assert :362) */
 } adop_stats;
 
-/* Size in bytes of the workspace adop_forward / adop_backward need for B views. */
+/* Size in bytes of the workspace adop_forward / adop_backward need for B views (every path, with or without a
+ * point_cache: the size adop_workspace_size_for() returns for flags = 0).  It depends on the arguments only, never on
+ * the tuning switches below or on the environment. */
 size_t adop_workspace_size(const adop_scene* scene, int32_t num_views, int32_t num_layers, int32_t w, int32_t h);
+
+/* A smaller workspace for callers that can promise something (no counterpart in the reference, whose buffers are all
+ * torch tensors of its cache).  Per point and view the full workspace holds 8 bytes of backward work queue, 20 bytes
+ * that only a forward pass WITHOUT a caller's point_cache uses (the projected points and the candidate lists of the
+ * direct path) and 36 bytes that only the tile-bin forward path uses (a tile word and two bin entries):
+ *   ADOP_WORKSPACE_POINT_CACHE_KEPT  every adop_forward call passes buffers->point_cache (training): the 20 bytes go;
+ *   ADOP_WORKSPACE_NO_TILE_PATH      the forward pass may always take the direct path: the 36 bytes go.
+ * adop_forward lays the workspace out from workspace_bytes and from whether point_cache is NULL: the largest of the
+ * four layouts that fits and serves the call.  In a layout without tile bins it renders through the direct path (same
+ * results; forward_path = 2 is then refused with ADOP_WORKSPACE_TOO_SMALL); a call with point_cache = NULL needs the
+ * 20 bytes and is refused when not even the layout without bins has room for them.
+ * adop_backward works with every one of them.  16 crops of a 100 M-point cloud: 102 GB in full, 70 GB with the point
+ * cache kept (plus the 25.6 GB of the cache itself), 13 GB with both flags. */
+#define ADOP_WORKSPACE_POINT_CACHE_KEPT 1u
+#define ADOP_WORKSPACE_NO_TILE_PATH 2u
+size_t adop_workspace_size_for(const adop_scene* scene, int32_t num_views, int32_t num_layers, int32_t w, int32_t h,
+                               uint32_t flags);
+
+/* Tuning switches (no counterpart in the reference).  The results never depend on them, only the time a call takes;
+ * the defaults are what the measurements on MI355X chose.  One set per process: adop_set_tuning() replaces it (a call
+ * that is being issued by another thread at that moment takes every switch either from the old or from the new set),
+ * adop_get_tuning() reads it, adop_tuning_defaults() fills in the defaults.  The library reads no environment
+ * variable.  Fields set to -1 mean "the library decides". */
+typedef struct adop_tuning
+{
+    int32_t forward_path;       /* used when adop_render_params.forward_path is 0: 0 = by size (default), 1 = direct, 2 = tile bins */
+    int32_t tile_slice_entries; /* entries per slice of a split bin; a bin is split from four slices' worth on (8192) */
+    int32_t ghost_concurrent;   /* several views (at most 24): 1 = the spatial gradients of all views in one launch, 0 = one
+                                   launch per view, -1 (default) = one launch for crop windows and clouds up to 4 M points */
+    int32_t bin_shard_shift;    /* log2 of the counters per tile in the binning passes, 0..3; -1 (default) = by the tile
+                                   count (up to 8 while the call has at most 4096 tiles and 16384 counters).  A value
+                                   that would need more than 65536 counters is lowered until it does not. */
+    int32_t direct_lists;       /* direct path without a caller's point cache: 1 = candidate lists (default), 0 = a record per point */
+    int32_t prepass_ppt;        /* points per thread of the direct path's depth prepass: 1, 2, 4; 0 (default) = by the cloud size */
+    int32_t prepass_group_from; /* first level at which the depth prepass merges the lanes of a wavefront by pixel (1) */
+    int32_t blend_group_from;   /* the same for the direct path's blend (0) */
+    int32_t list_block;         /* workgroup size of the direct path's blend in list mode: 64, 128 (default), 256 */
+    int32_t count_ppt;          /* points per thread of the first binning pass: 1, 2 (default), 4 */
+    int32_t scatter_ppt;        /* points per thread of the second binning pass: 1, 2 (default), 4 */
+    int32_t tile_k;             /* entries per thread and batch of the tile blend: 1 (default), 2, 4 */
+    int32_t normalize_fused;    /* one view: 1 (default) = the spatial-gradient kernel writes the point gradients
+                                   normalised, 0 = a pass of the finalize kernel does */
+    int32_t normalize_by_queue; /* one view, normalize_fused = 0: 1 (default) = that pass walks the work queue, 0 = all points */
+} adop_tuning;
+void adop_tuning_defaults(adop_tuning* out);
+adop_status adop_set_tuning(const adop_tuning* tuning); /* ADOP_INVALID_ARG (and no change) when a field is out of range */
+void adop_get_tuning(adop_tuning* out);
 
 /* Replaces BlendPointCloudForward (PointRenderer.cu:1389-1531): InitializeData (:1039-1090),
  * DepthPrepassMulti (:203-301,1166-1203), RenderForwardMulti (:303-393,1294-1335),
@@ -303,7 +352,9 @@ typedef struct adop_stage_time
 
 adop_status adop_profile_enable(int32_t enable);
 /* Waits for the recorded events, aggregates them by stage name into out[0..max_entries) and clears the
- * recording.  Returns the number of entries written. */
+ * recording.  Returns the number of entries written.  Which calls are recorded is a switch of the thread that issues
+ * them (adop_profile_enable); what they record goes to one list of the process, which this call takes whole, whatever
+ * thread it is called from (a framework may run the backward pass on a thread of its own). */
 int32_t adop_profile_read(adop_stage_time* out, int32_t max_entries);
 
 /* Message for the last non-OK status returned on the calling thread. */

@@ -19,7 +19,8 @@ FORWARD_PATH = 0
 POISON_BITS = 0xDEADBEEF
 
 
-def run_hip_forward(hs, collect_stats=True, forward_path=None, train=True, poison=False, pixel_records=True):
+def run_hip_forward(hs, collect_stats=True, forward_path=None, train=True, poison=False, pixel_records=True,
+                    workspace_flags=0):
     import torch
     from adop_amd import render
 
@@ -29,7 +30,7 @@ def run_hip_forward(hs, collect_stats=True, forward_path=None, train=True, poiso
     cache = render.PointRendererCache()
     info = render.NeuralRenderInfo(scene=scene, images=list(hs.views), params=hs.params, num_layers=hs.num_layers,
                                    cache=cache, collect_stats=collect_stats, train=train,
-                                   keep_pixel_records=pixel_records,
+                                   keep_pixel_records=pixel_records, workspace_flags=workspace_flags,
                                    dropout_points=None if hs.dropout is None else torch.from_numpy(hs.dropout))
 
     class Ctx:

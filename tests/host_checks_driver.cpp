@@ -93,8 +93,20 @@ int main()
     {
         adop_scene big = make_scene(1 << 30, 16, 13);
         size_t a       = adop_workspace_size(&big, 64, 5, 2200, 1500);
-        // at least the bin entries (2 per point and view, 16 bytes) must fit
-        EXPECT(a > (size_t)2 * 16 * 64 * ((size_t)1 << 30), "workspace of 2^30 points x 64 views of 2200x1500x5 does not wrap");
+        // per point and view: 8 bytes of work queue, 16 of projected point, 4 of candidate list (the tile bins are left
+        // out of a cloud this size: their entries could not address it)
+        EXPECT(a > (size_t)28 * 64 * ((size_t)1 << 30), "workspace of 2^30 points x 64 views of 2200x1500x5 does not wrap");
+        EXPECT(a == adop_workspace_size_for(&big, 64, 5, 2200, 1500, ADOP_WORKSPACE_NO_TILE_PATH), "no bins at 2^30 points");
+        adop_scene binned = make_scene(1 << 27, 16, 13);
+        size_t b          = adop_workspace_size(&binned, 8, 5, 2200, 1500);
+        // with the bins: + a tile word and two entries of 16 bytes
+        EXPECT(b > (size_t)(28 + 36) * 8 * ((size_t)1 << 27), "workspace of 2^27 points x 8 views holds the tile bins");
+        EXPECT(adop_workspace_size_for(&binned, 8, 5, 2200, 1500, ADOP_WORKSPACE_NO_TILE_PATH) < b - (size_t)36 * 8 * ((size_t)1 << 27) + (64 << 20),
+               "without the bins: 36 bytes per point and view less");
+        EXPECT(adop_workspace_size_for(&binned, 8, 5, 2200, 1500, ADOP_WORKSPACE_POINT_CACHE_KEPT | ADOP_WORKSPACE_NO_TILE_PATH) <
+                   (size_t)9 * 8 * ((size_t)1 << 27) + ((size_t)8 << 30),
+               "with both flags: the work queue, the pixel arrays and little else");
+        EXPECT(adop_workspace_size_for(&binned, 8, 5, 2200, 1500, 8u) == 0, "unknown workspace flag: 0");
         adop_scene mid = make_scene(1 << 30, 16, 13);
         EXPECT(adop_workspace_size(&mid, 63, 5, 2200, 1500) < a, "fewer views, smaller workspace");
         EXPECT(adop_workspace_size(&mid, 64, 4, 2200, 1500) < a, "fewer levels, smaller workspace");

@@ -43,7 +43,7 @@ def test_struct_sizes_match_the_c_header(tmp_path):
     names = {"adop_view": _capi.View, "adop_render_params": _capi.RenderParams, "adop_scene": _capi.Scene,
              "adop_layer": _capi.Layer, "adop_forward_buffers": _capi.ForwardBuffers,
              "adop_backward_buffers": _capi.BackwardBuffers, "adop_stats": _capi.Stats,
-             "adop_stage_time": _capi.StageTime}
+             "adop_stage_time": _capi.StageTime, "adop_tuning": _capi.Tuning}
     src = tmp_path / "sizes.c"
     body = "\n".join(f'printf("{n} %zu\\n", sizeof({n}));' for n in names)
     src.write_text(f'#include <stdio.h>\n#include "{HEADER}"\nint main(void){{\n{body}\nreturn 0;}}\n')
@@ -66,6 +66,64 @@ def test_workspace_query_needs_no_gpu():
     assert n1 < n4 < 4 * n1
     assert lib.adop_workspace_size(None, 1, 4, 640, 480) == 0
     assert lib.adop_workspace_size(C.byref(s), 1, 9, 640, 480) == 0
+
+
+def test_workspace_variants_and_their_independence_of_the_tuning():
+    """adop_workspace_size_for: what a caller may leave out, per point and view; no size depends on the tuning switches
+    (the layout of a call must not move with a switch another thread sets between two calls)."""
+    lib = _capi.load_library()
+    s = _capi.Scene()
+    s.num_poses, s.num_cameras, s.intrinsics_cols, s.num_channels, s.num_points = 3, 1, 13, 8, 1_000_000
+    B, N = 4, 1_000_000
+    args = (C.byref(s), B, 4, 512, 512)
+    full = lib.adop_workspace_size(*args)
+    assert lib.adop_workspace_size_for(*args, 0) == full
+    kept = lib.adop_workspace_size_for(*args, _capi.WORKSPACE_POINT_CACHE_KEPT)
+    direct = lib.adop_workspace_size_for(*args, _capi.WORKSPACE_NO_TILE_PATH)
+    both = lib.adop_workspace_size_for(*args, _capi.WORKSPACE_POINT_CACHE_KEPT | _capi.WORKSPACE_NO_TILE_PATH)
+    slack = 1 << 20
+    assert abs((full - kept) - 20 * B * N) < slack    # projected points 16 B + candidate list 4 B per point and view
+    # tile word 4 B + two bin entries of 16 B per point and view, + counters, tile order and the rows of split bins
+    assert 36 * B * N < full - direct < 36 * B * N + 24 * slack
+    assert abs((kept - both) - (full - direct)) < slack
+    assert lib.adop_workspace_size_for(*args, 4) == 0  # unknown flag
+    # a cloud beyond what the bin entries can address: the bins are left out of every layout
+    s.num_points = (1 << 28) + 5
+    assert lib.adop_workspace_size(C.byref(s), 1, 4, 512, 512) == \
+        lib.adop_workspace_size_for(C.byref(s), 1, 4, 512, 512, _capi.WORKSPACE_NO_TILE_PATH)
+    s.num_points = N
+    with _capi.tuning(bin_shard_shift=3, tile_slice_entries=7, forward_path=1, count_ppt=4):
+        assert lib.adop_workspace_size(*args) == full
+    with _capi.tuning(bin_shard_shift=0):
+        assert lib.adop_workspace_size(*args) == full
+
+
+def test_tuning_set_get_defaults_and_range_checks():
+    lib = _capi.load_library()
+    d, t = _capi.Tuning(), _capi.Tuning()
+    lib.adop_tuning_defaults(C.byref(d))
+    lib.adop_get_tuning(C.byref(t))
+    assert bytes(d) == bytes(t)  # nothing set yet in this process (the tests put back what they change)
+    assert (d.forward_path, d.tile_slice_entries, d.ghost_concurrent, d.bin_shard_shift) == (0, 8192, -1, -1)
+    assert (d.count_ppt, d.scatter_ppt, d.tile_k, d.list_block, d.normalize_fused) == (2, 2, 1, 128, 1)
+    with _capi.tuning(tile_slice_entries=64, ghost_concurrent=0) as now:
+        lib.adop_get_tuning(C.byref(t))
+        assert t.tile_slice_entries == 64 and t.ghost_concurrent == 0 and bytes(t) == bytes(now)
+    lib.adop_get_tuning(C.byref(t))
+    assert bytes(d) == bytes(t)
+    for field, bad in (("forward_path", 3), ("tile_slice_entries", 0), ("ghost_concurrent", 2), ("bin_shard_shift", 4),
+                       ("count_ppt", 3), ("scatter_ppt", 0), ("tile_k", 8), ("list_block", 100), ("prepass_ppt", 3),
+                       ("direct_lists", 2), ("prepass_group_from", 6)):
+        with pytest.raises(ValueError, match="tuning"):
+            with _capi.tuning(**{field: bad}):
+                pass
+        lib.adop_get_tuning(C.byref(t))
+        assert bytes(d) == bytes(t), field  # a refused set changes nothing
+    assert lib.adop_set_tuning(None) != 0
+    # the library reads no environment variable
+    src = "".join(open(os.path.join(ROOT, "adop_amd", "csrc", f)).read()
+                  for f in os.listdir(os.path.join(ROOT, "adop_amd", "csrc")) if f.endswith((".hip", ".h")))
+    assert "getenv" not in src
 
 
 def test_preprocessing_entry_points_reject_bad_arguments_before_any_launch():

@@ -65,8 +65,8 @@ def test_both_forward_paths_agree_on_the_batch(batch_scene):
         assert int(L.weight.double().sum().item()) == int(sb.accepted[l]), l
 
 
-def test_backward_of_all_views_at_once_equals_view_after_view(batch_scene, monkeypatch):
-    """ADOP_GHOST_CONCURRENT=1 (the library's choice for crop windows): one spatial-gradient launch for the 16 views,
+def test_backward_of_all_views_at_once_equals_view_after_view(batch_scene):
+    """adop_tuning.ghost_concurrent = 1 (the library's choice for crop windows): one spatial-gradient launch for the 16 views,
     rows shared by views summed with atomics; 0: a launch per view, adding view after view as the reference does.
     Same forward state, so the element-wise bar of the gradients applies (1e-4 relative / 1e-6 absolute), up to the
     order of the float additions on the shared rows."""
@@ -76,12 +76,14 @@ def test_backward_of_all_views_at_once_equals_view_after_view(batch_scene, monke
     hs = batch_scene
     gout = [torch.from_numpy(g).cuda() for g in scenes.upstream_grads(hs, 7)]
     results = {}
+    from adop_amd import _capi
+
     for mode in ("1", "0"):
-        monkeypatch.setenv("ADOP_GHOST_CONCURRENT", mode)
-        announce(f"training batch: forward + backward, ADOP_GHOST_CONCURRENT={mode}")
-        scene, info, ctx, images, masks = run_hip_forward(hs, collect_stats=False, forward_path=2)
-        grads = render.BlendPointCloudBackward(ctx, info, gout, (True, True, True))
-        torch.cuda.synchronize()
+        announce(f"training batch: forward + backward, adop_tuning.ghost_concurrent={mode}")
+        with _capi.tuning(ghost_concurrent=int(mode)):
+            scene, info, ctx, images, masks = run_hip_forward(hs, collect_stats=False, forward_path=2)
+            grads = render.BlendPointCloudBackward(ctx, info, gout, (True, True, True))
+            torch.cuda.synchronize()
         results[mode] = [g.detach().clone() if g is not None else None for g in grads]
     names = ["grad_texture", "grad_background", "grad_points", "grad_pose", "grad_intrinsics"]
     for name, a, b in zip(names, results["1"], results["0"]):

@@ -285,7 +285,7 @@ def test_more_views_than_one_constant_chunk(oracle_mod):
 
 
 @pytest.mark.parametrize("shift", ["0", "1", "2", "3"])
-def test_tile_counters_in_shards(oracle_mod, monkeypatch, shift, forward_path):
+def test_tile_counters_in_shards(oracle_mod, shift, forward_path):
     """The binning passes keep 1, 2, 4 or 8 counters per tile (runs of 256 points take them in turn; by default as many
     as a call of up to 4 096 tiles can have within 16 384 counters): a bin is the concatenation of its shards' parts,
     whatever their number.  Two views of 640 x 360 = 1 840 tiles."""
@@ -293,10 +293,12 @@ def test_tile_counters_in_shards(oracle_mod, monkeypatch, shift, forward_path):
 
     if forward_path != 2:
         pytest.skip("the tile counters belong to the tile path")
-    monkeypatch.setenv("ADOP_BIN_SHARD_SHIFT", shift)
-    announce(f"config2 300k pts B=2 640x360, ADOP_BIN_SHARD_SHIFT={shift}")
+    from adop_amd import _capi
+
+    announce(f"config2 300k pts B=2 640x360, adop_tuning.bin_shard_shift={shift}")
     hs = scenes.config2(n=300_000, w=640, h=360, levels=4, batch=2, seed=8)
-    _fwd_bwd(hs, oracle_mod, collect_stats=int(shift) % 2 == 0, poison=int(shift) % 2 == 1)
+    with _capi.tuning(bin_shard_shift=int(shift)):
+        _fwd_bwd(hs, oracle_mod, collect_stats=int(shift) % 2 == 0, poison=int(shift) % 2 == 1)
 
 
 @pytest.mark.parametrize("collect_stats", [True, False], ids=["counters", "plain"])
@@ -317,18 +319,20 @@ def test_more_views_than_bits_of_the_view_masks(oracle_mod, collect_stats):
 
 @pytest.mark.parametrize("concurrent", ["0", "1"], ids=["per_view", "concurrent"])
 @pytest.mark.parametrize("batch", [2, 5, 13, 24, 25, 34])
-def test_spatial_gradients_per_view_and_of_all_views_at_once(oracle_mod, monkeypatch, concurrent, batch):
+def test_spatial_gradients_per_view_and_of_all_views_at_once(oracle_mod, concurrent, batch):
     """With several views the spatial-gradient pass runs all views side by side in one launch (up to 24 views: a point
     that several views see is summed with atomics, every other row has one owner) or once per view, in the order of
-    the views (more views, or ADOP_GHOST_CONCURRENT=0): both against the checker, with batch sizes on either side of
+    the views (more views, or adop_tuning.ghost_concurrent = 0): both against the checker, with batch sizes on either side of
     the limit and of the 32-view chunk of constants.  The views of this scene look at one small cloud, so that most
     points are shared by several views."""
     from adop_amd import scenes
 
-    monkeypatch.setenv("ADOP_GHOST_CONCURRENT", concurrent)
-    announce(f"config2 40k pts B={batch} 96x80 L3 fwd+bwd ghost, ADOP_GHOST_CONCURRENT={concurrent}")
+    from adop_amd import _capi
+
+    announce(f"config2 40k pts B={batch} 96x80 L3 fwd+bwd ghost, adop_tuning.ghost_concurrent={concurrent}")
     hs = scenes.config2(n=40_000, w=96, h=80, levels=3, batch=batch, seed=batch)
-    _fwd_bwd(hs, oracle_mod)
+    with _capi.tuning(ghost_concurrent=int(concurrent)):
+        _fwd_bwd(hs, oracle_mod)
 
 
 @pytest.mark.parametrize("mode", [0, 1])
@@ -637,10 +641,9 @@ def test_tile_path_images_are_bit_identical_from_run_to_run():
 @pytest.mark.parametrize("slice_entries", ["64", "7", "1"], ids=["slices_of_64", "slices_of_7", "no_rows_left"])
 @pytest.mark.parametrize("channels,collect_stats", [(8, True), (8, False), (4, False), (3, True)],
                          ids=["C8-counters", "C8-plain", "C4-plain", "C3-counters"])
-def test_full_bins_are_split_between_workgroups(oracle_mod, monkeypatch, forward_path, slice_entries, channels,
-                                                collect_stats):
+def test_full_bins_are_split_between_workgroups(oracle_mod, forward_path, slice_entries, channels, collect_stats):
     """A cloud that covers a few tiles only (the camera far away) puts tens of thousands of entries into one bin; bins
-    above four times ADOP_TILE_SLICE entries (8192 by default, read at every call) are split in slices of that size that
+    above four times adop_tuning.tile_slice_entries entries (8192 by default) are split in slices of that size that
     as many workgroups take, the last of which merges their rows.  Forced here on small scenes: with 64 and 7 entries
     per slice most bins are split (up to 1023 slices a bin), with 1 the rows run out and most bins stay whole.  Forward and backward
     through the tile path still equal the checker (packed depth bit for bit), with and without the counters, for the
@@ -649,14 +652,94 @@ def test_full_bins_are_split_between_workgroups(oracle_mod, monkeypatch, forward
 
     if forward_path != 2:
         pytest.skip("the tile path only")
-    monkeypatch.setenv("ADOP_TILE_SLICE", slice_entries)
-    announce(f"tile path with split bins: ADOP_TILE_SLICE={slice_entries}, C={channels}, counters={collect_stats}")
+    from adop_amd import _capi
+
+    announce(f"tile path with split bins: tile_slice_entries={slice_entries}, C={channels}, counters={collect_stats}")
     hs = scenes.config3(n=150_000, w=160, h=96, channels=channels)
-    _fwd_bwd(hs, oracle_mod, collect_stats=collect_stats, poison=not collect_stats)
-    # the camera ten times as far: the cloud lands in a handful of tiles
-    el, az = np.deg2rad(20.0), np.deg2rad(30.0)
-    hs.poses_se3 = scenes.look_at_view(30.0 * np.array([np.cos(el) * np.sin(az), np.sin(el), -np.cos(el) * np.cos(az)]))[None, :]
-    _fwd_bwd(hs, oracle_mod, collect_stats=collect_stats, poison=not collect_stats)
+    with _capi.tuning(tile_slice_entries=int(slice_entries)):
+        _fwd_bwd(hs, oracle_mod, collect_stats=collect_stats, poison=not collect_stats)
+        # the camera ten times as far: the cloud lands in a handful of tiles
+        el, az = np.deg2rad(20.0), np.deg2rad(30.0)
+        hs.poses_se3 = scenes.look_at_view(30.0 * np.array([np.cos(el) * np.sin(az), np.sin(el), -np.cos(el) * np.cos(az)]))[None, :]
+        _fwd_bwd(hs, oracle_mod, collect_stats=collect_stats, poison=not collect_stats)
+
+
+def test_smaller_workspaces(oracle_mod, forward_path):
+    """adop_workspace_size_for: a workspace without the region of a forward pass that keeps no point cache, without the
+    tile bins, or without both.  Same results; without the bins the library renders through the direct path (and
+    refuses forward_path = 2); without the other region it refuses a forward pass that passes no point cache."""
+    import torch
+    from adop_amd import _capi, render, scenes
+
+    hs = scenes.config3(n=150_000, w=256, h=144, channels=4, seed=21)
+    ref = oracle_mod.forward(hs)
+    gout = scenes.upstream_grads(hs, 9)
+    for flags in (_capi.WORKSPACE_POINT_CACHE_KEPT, _capi.WORKSPACE_NO_TILE_PATH,
+                  _capi.WORKSPACE_POINT_CACHE_KEPT | _capi.WORKSPACE_NO_TILE_PATH):
+        announce(f"workspace flags {flags}, forward_path={forward_path}")
+        no_bins = bool(flags & _capi.WORKSPACE_NO_TILE_PATH)
+        if no_bins and forward_path == 2:
+            with pytest.raises(RuntimeError, match="tile bins"):
+                run_hip_forward(hs, workspace_flags=flags)
+            continue
+        scene, info, ctx, images, masks = run_hip_forward(hs, workspace_flags=flags, poison=True)
+        check_forward(hs, ref, ctx, images, masks, info)
+        grads = render.BlendPointCloudBackward(ctx, info, _torch_grads(gout))
+        torch.cuda.synchronize()
+        refb = oracle_mod.backward(hs, download_forward(hs, info, images, masks), gout)
+        check_backward(hs, refb, grads, info)
+        # a forward pass that passes no point cache after all: refused where the workspace has no room for the
+        # projected points at all (both flags); with the bins' room instead (36 bytes per point and view where 20 are
+        # needed) the library lays the workspace out without bins and renders through the direct path
+        if flags == (_capi.WORKSPACE_POINT_CACHE_KEPT | _capi.WORKSPACE_NO_TILE_PATH):
+            with pytest.raises(RuntimeError, match="workspace too small"):
+                run_hip_forward(hs, workspace_flags=flags, train=False)
+        elif flags == _capi.WORKSPACE_POINT_CACHE_KEPT and forward_path == 2:
+            with pytest.raises(RuntimeError, match="tile bins"):
+                run_hip_forward(hs, workspace_flags=flags, train=False)
+        else:
+            got = run_hip_forward(hs, workspace_flags=flags, train=False)
+            check_forward(hs, ref, got[2], got[3], got[4], got[1])
+    # the library's own choice with a workspace that has no bins: the direct path, no error
+    import helpers
+    helpers.FORWARD_PATH = 0
+    got = run_hip_forward(hs, workspace_flags=_capi.WORKSPACE_NO_TILE_PATH)
+    check_forward(hs, ref, got[2], got[3], got[4], got[1])
+
+
+# Every kernel variant the tuning switches choose between, each on one small scene (forward without a point cache,
+# training forward and backward) against the checker.
+TUNING_VARIANTS = [dict(count_ppt=1), dict(count_ppt=4), dict(scatter_ppt=1), dict(scatter_ppt=4), dict(tile_k=2),
+                   dict(tile_k=4), dict(normalize_fused=0), dict(normalize_fused=0, normalize_by_queue=0),
+                   dict(prepass_ppt=1), dict(prepass_ppt=2), dict(prepass_ppt=4), dict(direct_lists=0),
+                   dict(prepass_group_from=0), dict(prepass_group_from=5), dict(blend_group_from=2),
+                   dict(blend_group_from=5), dict(list_block=64), dict(list_block=256),
+                   dict(bin_shard_shift=3, count_ppt=4, scatter_ppt=4), dict(forward_path=1), dict(forward_path=2)]
+
+
+@pytest.mark.parametrize("variant", TUNING_VARIANTS, ids=lambda v: ",".join(f"{k}={x}" for k, x in v.items()))
+def test_every_tuning_variant_gives_the_same_results(oracle_mod, variant, forward_path):
+    from adop_amd import _capi, scenes
+
+    tile_only = {"count_ppt", "scatter_ppt", "tile_k", "bin_shard_shift"}
+    direct_only = {"prepass_ppt", "direct_lists", "prepass_group_from", "blend_group_from", "list_block"}
+    if (forward_path == 1 and set(variant) & tile_only) or (forward_path == 2 and set(variant) & direct_only):
+        pytest.skip("a switch of the other forward path")
+    announce(f"tuning variant {variant}: 120k pts B=2 200x120 L4, forward_path={forward_path}")
+    hs = scenes.config3(n=120_000, w=200, h=120, channels=4, seed=11)
+    hs.views = [scenes.make_view(200, 120), scenes.make_view(200, 120, crop=(1.25, 1.25, -20.0, -10.0, 0.0))]
+    hs.dropout = scenes.bernoulli_mask(4, 2, hs.num_points, 0.25)
+    one = __import__("copy").copy(hs)  # (normalize_fused concerns calls with one view)
+    one.views, one.dropout = hs.views[:1], np.ascontiguousarray(hs.dropout[:1])
+    with _capi.tuning(**variant):
+        if "forward_path" in variant:
+            import helpers
+            helpers.FORWARD_PATH = 0  # the library's own choice, through the switch
+        for scene in (hs, one):
+            ref = oracle_mod.forward(scene)
+            got = run_hip_forward(scene, collect_stats=False, train=False)
+            check_forward(scene, ref, got[2], got[3], got[4], got[1], stats=False)
+            _fwd_bwd(scene, oracle_mod, collect_stats=False, poison=True)
 
 
 def test_zz_report_end_to_end_misses():

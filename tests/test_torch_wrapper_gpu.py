@@ -143,41 +143,156 @@ def test_dropout_is_drawn_like_the_reference_and_eval_disables_it(oracle_mod):
         assert_close(outs[l].detach().cpu().numpy(), ref.out[l], 1e-5, 1e-7, f"eval out {l}")
 
 
-def test_module_forward_supersampling_and_environment_map(oracle_mod):
+def _host_environment(oracle_mod, hs, env_np, ref, pooled):
+    """The reference's composition on the host (RenderModule.cpp:54-127): torch's grid_sample (bilinear, border,
+    align_corners) on the checker's uv, images + (1 - mask) * env; `pooled`: 2x2 average pool of a render at twice the
+    size first.  Returns per level (image, mask, env sample) as torch tensors with the texture in the autograd graph."""
+    import torch
+
+    tex = torch.from_numpy(env_np).clone().requires_grad_(True)
+    out = []
+    for l in range(hs.num_layers):
+        img, m = torch.from_numpy(ref.out[l]), torch.from_numpy(ref.mask[l])
+        if pooled:
+            img, m = torch.nn.functional.avg_pool2d(img, 2), torch.nn.functional.avg_pool2d(m, 2)
+        uv = torch.stack([torch.from_numpy(oracle_mod.env_uv(hs, b, l)) for b in range(hs.batch)])
+        e = torch.nn.functional.grid_sample(tex[None].expand(hs.batch, -1, -1, -1), uv, mode="bilinear",
+                                            padding_mode="border", align_corners=True)
+        out.append((img, m, e))
+    return tex, out
+
+
+@pytest.mark.parametrize("camera", ["pinhole", "ocam"])
+@pytest.mark.parametrize("super_sampling", [True, False], ids=["supersampled", "plain"])
+def test_module_forward_with_the_environment_map_and_its_gradient(oracle_mod, camera, super_sampling):
+    """PointRenderModuleForward composes the environment map through the library's fused kernels
+    (torch::autograd::EnvironmentMapCompose): the composed images, and the gradients the loss sends to the map's
+    texture and to the descriptors, against torch's grid_sample autograd on the checker's texture coordinates and the
+    checker's render.  Pinhole views as the reference, OCam views as the extension; with super-sampling the masks are
+    fractional after the 2x2 pool."""
+    import copy
+
     import torch
     from adop_amd import scenes
 
-    announce("libTorch wrapper: PointRenderModuleForward with super-sampling and the environment map")
+    announce(f"libTorch wrapper: module forward + backward with the environment map, {camera}, super_sampling={super_sampling}")
     mod = _module()
-    hs = scenes.config3(n=100_000, w=160, h=96, channels=4, levels=3)
+    if camera == "pinhole":
+        hs = scenes.config3(n=100_000, w=160, h=96, channels=4, levels=3)
+        hs.views.append(scenes.make_view(160, 96, crop=(1.5, 1.5, -40.0, -30.0, 0.0)))
+    else:
+        hs = scenes.config5(n=60_000, w=132, h=90, levels=3, batch=2, patches=60, seed=4)
     hs.dropout = None
     hs.params.ghost_gradients = 0
     hs.params.output_background_mask = 1
     env_np = scenes.rng(5).random((4, 32, 64), dtype=np.float32)
     env = torch.from_numpy(env_np).cuda().requires_grad_(True)
     s, t = _scene(mod, hs, env)
-    outs = mod.render(s, _views(hs), _params(hs, dropout=0.0, super_sampling=True), hs.num_layers, training=True,
-                      through_module=True)
+    outs = mod.render(s, _views(hs), _params(hs, dropout=0.0, super_sampling=super_sampling), hs.num_layers,
+                      training=True, through_module=True)
     L = hs.num_layers
-    assert [tuple(o.shape[2:]) for o in outs[:L]] == [(96, 160), (48, 80), (24, 40)]
-    # reference composition on the host: render at 2x, 2x2 average pool, + (1-mask)*env (RenderModule.cpp:54-127)
-    import copy
-    hs2 = copy.copy(hs)
-    v = hs.views[0]
-    hs2.views = [scenes.make_view(2 * v.w, 2 * v.h, v.image_index, v.camera_index, v.camera_model_type,
-                                  (2 * v.crop_fx, 2 * v.crop_fy, 2 * v.crop_cx, 2 * v.crop_cy, 2 * v.crop_s))]
+    assert [tuple(o.shape[2:]) for o in outs[:L]] == [(h, w) for (w, h) in hs.level_sizes()]
+    hs2 = hs
+    if super_sampling:  # render at 2x, 2x2 average pool (RenderModule.cpp:54-104)
+        hs2 = copy.copy(hs)
+        hs2.views = [scenes.make_view(2 * v.w, 2 * v.h, v.image_index, v.camera_index, v.camera_model_type,
+                                      (2 * v.crop_fx, 2 * v.crop_fy, 2 * v.crop_cx, 2 * v.crop_cy, 2 * v.crop_s))
+                     for v in hs.views]
     ref = oracle_mod.forward(hs2)
-    for l in range(L):
-        img = torch.nn.functional.avg_pool2d(torch.from_numpy(ref.out[l]), 2)
-        m = torch.nn.functional.avg_pool2d(torch.from_numpy(ref.mask[l]), 2)
-        uv = torch.from_numpy(oracle_mod.env_uv(hs, 0, l))[None]
-        e = torch.nn.functional.grid_sample(torch.from_numpy(env_np)[None], uv, mode="bilinear", padding_mode="border",
-                                            align_corners=True)
+    tex_host, levels = _host_environment(oracle_mod, hs, env_np, ref, super_sampling)
+    gout = scenes.upstream_grads(hs, 17)
+    loss_host = 0
+    for l, (img, m, e) in enumerate(levels):
         want = img + (1 - m) * e
-        assert_close(outs[l].detach().cpu().numpy(), want.numpy(), 2e-5, 2e-6, f"module out {l}")
+        assert_close(outs[l].detach().cpu().numpy(), want.detach().numpy(), 2e-5, 2e-6, f"module out {l}")
         assert_close(outs[L + l].cpu().numpy(), m.numpy(), 1e-6, 1e-7, f"module mask {l}")
-    sum(o.sum() for o in outs[:L]).backward()
-    assert env.grad is not None and float(env.grad.abs().sum()) > 0  # texture gradient through torch's grid_sample
+        loss_host = loss_host + (want * torch.from_numpy(gout[l])).sum()
+    loss_host.backward()
+    sum((o * torch.from_numpy(g).cuda()).sum() for o, g in zip(outs[:L], gout)).backward()
+    # texture gradient of the map: per-tile fixed-point sums + one float atomic per texel here, torch's scatter there
+    assert_norm_close(env.grad.cpu().numpy(), tex_host.grad.numpy(), 2e-5, "environment map gradient")
+    assert_close(env.grad.cpu().numpy(), tex_host.grad.numpy(), 1e-4, 1e-4 * float(tex_host.grad.abs().max()),
+                 "environment map gradient, element-wise")
+    # the descriptors still receive the rasterizer's gradient through the composition (d composed / d image = 1)
+    gout2 = gout
+    if super_sampling:
+        # the pool's adjoint: a quarter of the upstream gradient to each of the four pixels; a last odd row or column
+        # of the large image is dropped by the pool and receives nothing
+        gout2 = []
+        for g, (w2, h2) in zip(gout, hs2.level_sizes()):
+            big = np.zeros(g.shape[:2] + (h2, w2), np.float32)
+            big[:, :, : 2 * g.shape[2], : 2 * g.shape[3]] = np.repeat(np.repeat(g, 2, axis=2), 2, axis=3) * np.float32(0.25)
+            gout2.append(big)
+    refb = oracle_mod.backward(hs2, ref, gout2)
+    assert_close(t["texture"].grad.cpu().numpy(), refb.grad_texture, 1e-4, 1e-6, "grad texture through the composition")
+
+
+def test_module_forward_cat_env_to_color(oracle_mod):
+    """PipelineParams::cat_env_to_color (RenderModule.cpp:112-118): the sampled map of every pixel is concatenated to
+    the image instead of composed; its texture gradient then carries no (1 - mask) factor."""
+    import torch
+    from adop_amd import scenes
+
+    announce("libTorch wrapper: module forward with cat_env_to_color")
+    mod = _module()
+    hs = scenes.config3(n=60_000, w=96, h=64, channels=4, levels=2)
+    hs.dropout = None
+    hs.params.ghost_gradients = 0
+    hs.params.output_background_mask = 1
+    env_np = scenes.rng(6).random((4, 16, 32), dtype=np.float32)
+    env = torch.from_numpy(env_np).cuda().requires_grad_(True)
+    s, t = _scene(mod, hs, env)
+    outs = mod.render(s, _views(hs), _params(hs, dropout=0.0), hs.num_layers, training=True, through_module=True,
+                      cat_env_to_color=True)
+    L = hs.num_layers
+    ref = oracle_mod.forward(hs)
+    tex_host, levels = _host_environment(oracle_mod, hs, env_np, ref, False)
+    g = scenes.rng(3)
+    loss_host = 0
+    loss = 0
+    for l, (img, m, e) in enumerate(levels):
+        assert outs[l].shape[1] == 8
+        assert_close(outs[l][:, :4].detach().cpu().numpy(), img.numpy(), 1e-5, 1e-7, f"image part {l}")
+        assert_close(outs[l][:, 4:].detach().cpu().numpy(), e.detach().numpy(), 2e-5, 2e-6, f"environment part {l}")
+        go = torch.from_numpy(g.standard_normal(e.shape).astype(np.float32))
+        loss_host = loss_host + (e * go).sum()
+        loss = loss + (outs[l][:, 4:] * go.cuda()).sum()
+    loss_host.backward()
+    loss.backward()
+    assert_norm_close(env.grad.cpu().numpy(), tex_host.grad.numpy(), 2e-5, "environment map gradient (cat)")
+
+
+def test_stage_timer_system_receives_the_stage_times(oracle_mod):
+    """NeuralRenderInfo::timer_system (PointRenderer.h:32): with a timer system attached the stages of a forward and a
+    backward pass arrive under the reference's names (SAIGA_OPTIONAL_TIME_MEASURE, PointRenderer.cu:906-1610), frame by
+    frame; without one nothing is recorded."""
+    import torch
+    from adop_amd import scenes
+
+    announce("libTorch wrapper: stage timers through NeuralRenderInfo::timer_system")
+    mod = _module()
+    hs = scenes.config3(n=200_000, w=640, h=360, channels=8)
+    hs.dropout = None
+    s, t = _scene(mod, hs)
+    params = _params(hs, dropout=0.25)
+    for frame in range(3):
+        s.begin_frame()
+        outs = mod.render(s, _views(hs), params, hs.num_layers, timed=True)
+        sum(o.sum() for o in outs[: hs.num_layers]).backward()
+        s.end_frame()
+    times = s.stage_times()
+    forward = {"Initialize", "CombineAndFill"}
+    backward = {"Prepare Backward", "CombineAndFillBackward", "RenderBackward/descriptor", "RenderBackward/spatial",
+                "Post Process Gradient"}
+    assert forward | backward <= set(times), sorted(times)
+    assert ({"DepthPrepass", "RenderForward"} <= set(times)) or ({"BinCount", "BinScatter", "TileDepth", "TileBlend"} <= set(times))
+    for name, (last_ms, total_ms, calls, frames) in times.items():
+        assert frames == 3 and calls >= 3 and 0 < last_ms < 50 and total_ms >= last_ms, (name, last_ms, total_ms, calls, frames)
+    # a frame without a timer system adds nothing
+    s.begin_frame()
+    mod.render(s, _views(hs), params, hs.num_layers)
+    s.end_frame()
+    assert all(v[3] == 3 for v in s.stage_times().values())
 
 
 def test_apply_tangent(oracle_mod):

@@ -62,6 +62,26 @@ def test_static_scratch_entry_point_equals_the_workspace_one():
     # and the first input once more gives the first result
     got3, _ = _both(pos, poses, intr, frames)
     assert np.array_equal(got3.view(np.uint32), want.view(np.uint32))
+    # what the entry point is for: after the first call on the device (which looks the array's address up) a call
+    # allocates and frees no device memory.  Free memory as the driver reports it, around calls that go to buffers
+    # allocated beforehand (torch's caching allocator is not asked for anything in between).
+    import torch
+
+    s = _capi.Scene()
+    s.position, s.num_points = pos.data_ptr(), int(pos.shape[0])
+    s.poses_se3, s.num_poses = poses.data_ptr(), int(poses.shape[0])
+    s.intrinsics, s.num_cameras, s.intrinsics_cols = intr.data_ptr(), int(intr.shape[0]), 13
+    views = (_capi.View * len(frames))(*frames)
+    out = torch.empty(s.num_points, dtype=torch.float32, device=pos.device)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        rc = lib.adop_point_distance_to_camera_static(C.byref(s), views, len(frames), C.c_void_p(out.data_ptr()), stream)
+        assert rc == _capi.ADOP_OK
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before, "a call changed the free device memory"
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
 def test_static_scratch_entry_point_rejects_too_many_frames():
