@@ -121,7 +121,7 @@ constexpr adop_tuning kTuningDefaults = {/*forward_path*/ 0,    /*tile_slice_ent
                                          /*ghost_concurrent*/ -1, /*bin_shard_shift*/ -1,
                                          /*direct_lists*/ 1,    /*prepass_ppt*/ 0,
                                          /*prepass_group_from*/ 1, /*blend_group_from*/ 0,
-                                         /*list_block*/ 128,    /*count_ppt*/ 2,
+                                         /*list_block*/ 128,    /*count_ppt*/ 0,
                                          /*scatter_ppt*/ 2,     /*tile_k*/ 1,
                                          /*normalize_fused*/ 1, /*normalize_by_queue*/ 1};
 struct TuningStore
@@ -552,9 +552,9 @@ adop_status adop_set_tuning(const adop_tuning* t)
     if (t->bin_shard_shift < -1 || t->bin_shard_shift > 3) return fail(ADOP_INVALID_ARG, "tuning: bin_shard_shift must be -1 .. 3");
     if (!one_of(t->direct_lists, {0, 1}) || !one_of(t->normalize_fused, {0, 1}) || !one_of(t->normalize_by_queue, {0, 1}))
         return fail(ADOP_INVALID_ARG, "tuning: direct_lists, normalize_fused and normalize_by_queue are 0 or 1");
-    if (!one_of(t->prepass_ppt, {0, 1, 2, 4}) || !one_of(t->count_ppt, {1, 2, 4}) || !one_of(t->scatter_ppt, {1, 2, 4}) ||
+    if (!one_of(t->prepass_ppt, {0, 1, 2, 4}) || !one_of(t->count_ppt, {0, 1, 2, 4}) || !one_of(t->scatter_ppt, {1, 2, 4}) ||
         !one_of(t->tile_k, {1, 2, 4}))
-        return fail(ADOP_INVALID_ARG, "tuning: points / entries per thread must be 1, 2 or 4 (prepass_ppt: or 0)");
+        return fail(ADOP_INVALID_ARG, "tuning: points / entries per thread must be 1, 2 or 4 (prepass_ppt, count_ppt: or 0)");
     if (t->prepass_group_from < 0 || t->prepass_group_from > ADOP_MAX_LAYERS || t->blend_group_from < 0 ||
         t->blend_group_from > ADOP_MAX_LAYERS)
         return fail(ADOP_INVALID_ARG, "tuning: a level is 0 .. ADOP_MAX_LAYERS");

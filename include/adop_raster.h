@@ -225,7 +225,7 @@ typedef struct adop_tuning
     int32_t prepass_group_from; /* first level at which the depth prepass merges the lanes of a wavefront by pixel (1) */
     int32_t blend_group_from;   /* the same for the direct path's blend (0) */
     int32_t list_block;         /* workgroup size of the direct path's blend in list mode: 64, 128 (default), 256 */
-    int32_t count_ppt;          /* points per thread of the first binning pass: 1, 2 (default), 4 */
+    int32_t count_ppt;          /* points per thread of the first binning pass: 1, 2, 4; 0 (default) = 1 up to 2^22 points, 2 above */
     int32_t scatter_ppt;        /* points per thread of the second binning pass: 1, 2 (default), 4 */
     int32_t tile_k;             /* entries per thread and batch of the tile blend: 1 (default), 2, 4 */
     int32_t normalize_fused;    /* one view: 1 (default) = the spatial-gradient kernel writes the point gradients

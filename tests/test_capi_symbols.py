@@ -105,14 +105,14 @@ def test_tuning_set_get_defaults_and_range_checks():
     lib.adop_get_tuning(C.byref(t))
     assert bytes(d) == bytes(t)  # nothing set yet in this process (the tests put back what they change)
     assert (d.forward_path, d.tile_slice_entries, d.ghost_concurrent, d.bin_shard_shift) == (0, 8192, -1, -1)
-    assert (d.count_ppt, d.scatter_ppt, d.tile_k, d.list_block, d.normalize_fused) == (2, 2, 1, 128, 1)
+    assert (d.count_ppt, d.scatter_ppt, d.tile_k, d.list_block, d.normalize_fused) == (0, 2, 1, 128, 1)
     with _capi.tuning(tile_slice_entries=64, ghost_concurrent=0) as now:
         lib.adop_get_tuning(C.byref(t))
         assert t.tile_slice_entries == 64 and t.ghost_concurrent == 0 and bytes(t) == bytes(now)
     lib.adop_get_tuning(C.byref(t))
     assert bytes(d) == bytes(t)
     for field, bad in (("forward_path", 3), ("tile_slice_entries", 0), ("ghost_concurrent", 2), ("bin_shard_shift", 4),
-                       ("count_ppt", 3), ("scatter_ppt", 0), ("tile_k", 8), ("list_block", 100), ("prepass_ppt", 3),
+                       ("count_ppt", 3), ("count_ppt", -1), ("scatter_ppt", 0), ("tile_k", 8), ("list_block", 100), ("prepass_ppt", 3),
                        ("direct_lists", 2), ("prepass_group_from", 6)):
         with pytest.raises(ValueError, match="tuning"):
             with _capi.tuning(**{field: bad}):

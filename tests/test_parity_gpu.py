@@ -709,7 +709,7 @@ def test_smaller_workspaces(oracle_mod, forward_path):
 
 # Every kernel variant the tuning switches choose between, each on one small scene (forward without a point cache,
 # training forward and backward) against the checker.
-TUNING_VARIANTS = [dict(count_ppt=1), dict(count_ppt=4), dict(scatter_ppt=1), dict(scatter_ppt=4), dict(tile_k=2),
+TUNING_VARIANTS = [dict(count_ppt=1), dict(count_ppt=2), dict(count_ppt=4), dict(scatter_ppt=1), dict(scatter_ppt=4), dict(tile_k=2),
                    dict(tile_k=4), dict(normalize_fused=0), dict(normalize_fused=0, normalize_by_queue=0),
                    dict(prepass_ppt=1), dict(prepass_ppt=2), dict(prepass_ppt=4), dict(direct_lists=0),
                    dict(prepass_group_from=0), dict(prepass_group_from=5), dict(blend_group_from=2),
