@@ -53,6 +53,7 @@ class RenderParams(C.Structure):
         ("normalize_mode", C.c_int32),
         ("forward_path", C.c_int32),
         ("skip_points", C.c_int32),
+        ("workspace_flags", C.c_uint32),
     ]
 
 
@@ -131,6 +132,7 @@ class Tuning(C.Structure):
 
 WORKSPACE_POINT_CACHE_KEPT = 1
 WORKSPACE_NO_TILE_PATH = 2
+WORKSPACE_SMALL_BINS = 4
 
 
 class StageTime(C.Structure):

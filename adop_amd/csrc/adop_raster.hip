@@ -166,6 +166,7 @@ struct WorkspaceLayout
     size_t bin_info;    // uint32[B * N]
     size_t bin_entries; // float4[kTileLevels * B * N]
     size_t bin_cap;     // entries
+    size_t bin_overflow;  // uint32: set by the prefix sum when the call has more entries than bin_cap
     size_t common;      // end of what every call uses (all that adop_backward needs)
     bool has_lists, has_bins;
     size_t total;
@@ -217,6 +218,9 @@ size_t align_up(size_t v, size_t a)
 {
     return (v + a - 1) / a * a;
 }
+
+constexpr uint32_t kWorkspaceFlags =
+    ADOP_WORKSPACE_POINT_CACHE_KEPT | ADOP_WORKSPACE_NO_TILE_PATH | ADOP_WORKSPACE_SMALL_BINS;
 
 // Can the tile path take a cloud of n points in B views of w0 x h0?  (Point ids need 28 bits of the bin entry, the bin
 // offsets are 32-bit with at most kTileLevels entries per point and view, the tile word holds 24 bits of tile.)
@@ -287,7 +291,12 @@ WorkspaceLayout layout(const adop_scene* s, int B, int L, int w0, int h0, uint32
         o            = align_up(o + sizeof(uint4) * (T + max_rows), 256);
         w.bin_rows   = o;
         o            = align_up(o + sizeof(float) * max_rows * (size_t)slice_row_floats(s->num_channels > 0 ? s->num_channels : 1), 256);
-        w.bin_cap    = (size_t)kTileLevels * (size_t)B * n;
+        // every entry the call can have, or (ADOP_WORKSPACE_SMALL_BINS) one per four points and view: what views take
+        // that see a part of the cloud each; a call with more falls back to the direct path on the device
+        w.bin_cap = (size_t)kTileLevels * (size_t)B * n;
+        if (flags & ADOP_WORKSPACE_SMALL_BINS) w.bin_cap = ((size_t)B * n + 3) / 4 + 1024;
+        w.bin_overflow = o;
+        o              = align_up(o + sizeof(uint32_t), 256);
         w.bin_info   = o;
         o            = align_up(o + sizeof(uint32_t) * (size_t)B * n, 256);
         w.bin_entries = o;
@@ -295,21 +304,6 @@ WorkspaceLayout layout(const adop_scene* s, int B, int L, int w0, int h0, uint32
     }
     w.total      = o;
     return w;
-}
-
-// The layout of the workspace a forward call was given: the largest of the four that fits (a layout without the
-// region of a forward pass that keeps no point cache only when the caller passes one).
-bool choose_layout(const adop_scene* s, int B, int L, int w0, int h0, size_t bytes, bool has_point_cache, WorkspaceLayout* out)
-{
-    const uint32_t order[4] = {0u, ADOP_WORKSPACE_POINT_CACHE_KEPT, ADOP_WORKSPACE_NO_TILE_PATH,
-                               ADOP_WORKSPACE_POINT_CACHE_KEPT | ADOP_WORKSPACE_NO_TILE_PATH};
-    for (uint32_t flags : order)
-    {
-        if ((flags & ADOP_WORKSPACE_POINT_CACHE_KEPT) && !has_point_cache) continue;
-        *out = layout(s, B, L, w0, h0, flags);
-        if (bytes >= out->total) return true;
-    }
-    return false;
 }
 
 adop_status validate(const adop_scene* s, const adop_view* views, int B, const adop_render_params* rp,
@@ -529,7 +523,7 @@ size_t adop_workspace_size_for(const adop_scene* scene, int32_t num_views, int32
 {
     if (!scene || num_views < 1 || num_layers < 1 || num_layers > ADOP_MAX_LAYERS || w < 1 || h < 1) return 0;
     if (scene->num_channels < 1 || scene->num_channels > kMaxChannels) return 0;
-    if (flags & ~(ADOP_WORKSPACE_POINT_CACHE_KEPT | ADOP_WORKSPACE_NO_TILE_PATH)) return 0;
+    if (flags & ~kWorkspaceFlags) return 0;
     return layout(scene, num_views, num_layers, w, h, flags).total;
 }
 
@@ -587,10 +581,12 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
     if (st != ADOP_OK) return st;
     adop_scene without_points;
     if (params->skip_points) scene = leave_out_points(scene, &without_points);
-    WorkspaceLayout wl;
-    if (!workspace || !choose_layout(scene, num_views, buffers->num_layers, views[0].w, views[0].h, workspace_bytes,
-                                     buffers->point_cache != nullptr, &wl))
-        return fail(ADOP_WORKSPACE_TOO_SMALL, "workspace too small");
+    // (the layout the caller sized the workspace with: adop_render_params.workspace_flags)
+    if (params->workspace_flags & ~kWorkspaceFlags) return fail(ADOP_INVALID_ARG, "unknown workspace flag");
+    const WorkspaceLayout wl = layout(scene, num_views, buffers->num_layers, views[0].w, views[0].h, params->workspace_flags);
+    if (!workspace || workspace_bytes < wl.total) return fail(ADOP_WORKSPACE_TOO_SMALL, "workspace too small");
+    if (!wl.has_lists && !buffers->point_cache && !params->skip_points)
+        return fail(ADOP_INVALID_ARG, "ADOP_WORKSPACE_POINT_CACHE_KEPT: the forward pass needs point_cache");
     const adop_tuning tn = tuning_now();
     hipStream_t stream = (hipStream_t)hip_stream;
     ViewConst* dviews  = (ViewConst*)((char*)workspace + wl.views);
@@ -643,7 +639,7 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
 
     if (path == 2)
     {
-        if (!pc.cache) pc.cache = (float4*)((char*)workspace + wl.proj);  // (has_lists: choose_layout)
+        if (!pc.cache) pc.cache = (float4*)((char*)workspace + wl.proj);  // (has_lists: checked above)
         BinArg bin;
         bin.lt      = kTileLevels < lv.num ? kTileLevels : lv.num;
         bin.tiles_x = ((views[0].w - 1) >> kTileShiftX) + 1;
@@ -663,6 +659,10 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
         bin.max_rows   = slice_rows(scene->num_points, num_views);
         bin.row_floats = slice_row_floats(scene->num_channels);
         bin.slice_entries = (uint32_t)tn.tile_slice_entries;
+        // smaller bins than the call can fill: the prefix sum tells the kernels behind it whether the entries fit
+        const bool capped = wl.bin_cap < (size_t)kTileLevels * (size_t)num_views * (size_t)scene->num_points;
+        bin.overflow      = capped ? (uint32_t*)((char*)workspace + wl.bin_overflow) : nullptr;
+        bin.cap           = (uint32_t)(wl.bin_cap < 0xFFFFFFFFull ? wl.bin_cap : 0xFFFFFFFFull);
         {
             StageScope sc("Initialize", stream);
             // tile counters, and for the coarse levels the packed depth and the global accumulators of the direct path
@@ -695,7 +695,37 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
         {
             StageScope sc("CombineAndFill", stream);
             launch_resolve(lv, bin.lt, pixel_grid(lv, bin.lt), accum, S, scene->background_color,
-                           params->output_background_mask, params->output_background_mask_value, stream);
+                           params->output_background_mask, params->output_background_mask_value, stream,
+                           Gate{bin.overflow, 0u});
+        }
+        if (capped)
+        {
+            // The direct path, queued behind the tile kernels: its kernels start only when the entries did not fit (the
+            // tile kernels have then returned at once).  It renders the call from the beginning: all levels cleared,
+            // the counters counted again; the point records the first binning pass left are written once more.
+            const Gate over{bin.overflow, 1u};
+            const size_t accum_n = (size_t)lv.pix_prefix[lv.num] * lv.B * S;
+            ViewPrep none;
+            memset(&none, 0, sizeof(none));
+            {
+                StageScope sc("Initialize", stream);
+                launch_clear(lv, 0, pixel_grid(lv), accum, S % 4 == 0 ? accum_n : 0, nullptr, 0, none, stream, over, stats);
+                // (an accumulator stride that is no multiple of four floats: cleared whether needed or not)
+                if (S % 4 != 0 && (st = fill_async(accum, accum_n * sizeof(float), 0, stream)) != ADOP_OK) return st;
+            }
+            {
+                StageScope sc("DepthPrepass", stream);
+                launch_prepass(pc, dviews, lv, rp, stats, tn, stream, over);
+            }
+            {
+                StageScope sc("RenderForward", stream);
+                launch_blend(pc, dviews, lv, rp, half, accum, S, stats, tn, stream, over);
+            }
+            {
+                StageScope sc("CombineAndFill", stream);
+                launch_resolve(lv, 0, pixel_grid(lv), accum, S, scene->background_color, params->output_background_mask,
+                               params->output_background_mask_value, stream, over);
+            }
         }
         ADOP_HIP_CHECK(hipGetLastError());
         return ADOP_OK;
@@ -703,8 +733,6 @@ adop_status adop_forward(const adop_scene* scene, const adop_view* views, int32_
 
     // Without a caller's point cache (no backward pass follows) the prepass hands the blend compacted lists of the
     // points that can still pass a depth test instead of a record per point.
-    if (!pc.cache && !wl.has_lists)  // (choose_layout: unreachable; kept as the guard of the pointer arithmetic below)
-        return fail(ADOP_WORKSPACE_TOO_SMALL, "a forward pass without point_cache needs the full workspace");
     if (!pc.cache && tn.direct_lists && scene->num_points > 0)
     {
         pc.cache      = (float4*)((char*)workspace + wl.proj);
@@ -757,8 +785,8 @@ adop_status adop_backward(const adop_scene* scene, const adop_view* views, int32
     if (grads->grad_intrinsics && !grads->grad_intrinsics_count)
         return fail(ADOP_INVALID_ARG, "grad_intrinsics_count missing");
     // (the backward pass uses the first part of the workspace only, which every layout has)
-    WorkspaceLayout wl = layout(scene, num_views, fwd->num_layers, views[0].w, views[0].h,
-                                ADOP_WORKSPACE_POINT_CACHE_KEPT | ADOP_WORKSPACE_NO_TILE_PATH);
+    if (params->workspace_flags & ~kWorkspaceFlags) return fail(ADOP_INVALID_ARG, "unknown workspace flag");
+    WorkspaceLayout wl = layout(scene, num_views, fwd->num_layers, views[0].w, views[0].h, params->workspace_flags);
     if (!workspace || workspace_bytes < wl.total) return fail(ADOP_WORKSPACE_TOO_SMALL, "workspace too small");
     const adop_tuning tn = tuning_now();
     hipStream_t stream = (hipStream_t)hip_stream;

@@ -291,6 +291,7 @@ __device__ __forceinline__ void order_tiles(const BinArg& bin, int T, int g, int
 template <int PPT>
 __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels lv, ParamArg rp, BinArg bin, int T, int G)
 {
+    if (bin.overflow && *bin.overflow) return;  // more entries than the bins hold: the direct path renders the call
     if ((int)blockIdx.x < G)  // the first G workgroups order the T tiles for the tile kernels
     {
         order_tiles(bin, T, (int)blockIdx.x, G);
@@ -411,7 +412,8 @@ __global__ __launch_bounds__(kBlock) void bin_scatter_kernel(CloudArg pc, Levels
 // side (k = (tile << shard_shift) + shard): T = tiles << shard_shift logical counters.
 template <int PER>
 __global__ __launch_bounds__(1024) void tile_scan_kernel(const uint32_t* __restrict__ count, uint32_t* __restrict__ offset,
-                                                         int T, int shard_shift, int tiles)
+                                                         int T, int shard_shift, int tiles, uint32_t* __restrict__ overflow,
+                                                         uint32_t cap)
 {
     __shared__ uint32_t s_wave[16];
     __shared__ uint32_t s_carry;
@@ -486,7 +488,11 @@ __global__ __launch_bounds__(1024) void tile_scan_kernel(const uint32_t* __restr
         if (tid == 1023) s_carry = run;  // the last thread ends at the chunk total
         __syncthreads();
     }
-    if (tid == 0) offset[T] = s_carry;
+    if (tid == 0)
+    {
+        offset[T] = s_carry;
+        if (overflow) *overflow = s_carry > cap ? 1u : 0u;  // (the bins of this workspace hold `cap` entries)
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -528,11 +534,11 @@ void launch_bin(int pass, const CloudArg& pc, const ViewConst* views, const Leve
 void launch_tile_scan(const BinArg& bin, int num_tiles, hipStream_t st)
 {
     if (num_tiles <= 8192)
-        hipLaunchKernelGGL(tile_scan_kernel<8>, dim3(1), dim3(1024), 0, st, bin.count, bin.offset, num_tiles, bin.shard_shift, bin.num_tiles);
+        hipLaunchKernelGGL(tile_scan_kernel<8>, dim3(1), dim3(1024), 0, st, bin.count, bin.offset, num_tiles, bin.shard_shift, bin.num_tiles, bin.overflow, bin.cap);
     else if (num_tiles <= 16384)  // (the sharded counters of a call: one chunk)
-        hipLaunchKernelGGL(tile_scan_kernel<16>, dim3(1), dim3(1024), 0, st, bin.count, bin.offset, num_tiles, bin.shard_shift, bin.num_tiles);
+        hipLaunchKernelGGL(tile_scan_kernel<16>, dim3(1), dim3(1024), 0, st, bin.count, bin.offset, num_tiles, bin.shard_shift, bin.num_tiles, bin.overflow, bin.cap);
     else
-        hipLaunchKernelGGL(tile_scan_kernel<32>, dim3(1), dim3(1024), 0, st, bin.count, bin.offset, num_tiles, bin.shard_shift, bin.num_tiles);
+        hipLaunchKernelGGL(tile_scan_kernel<32>, dim3(1), dim3(1024), 0, st, bin.count, bin.offset, num_tiles, bin.shard_shift, bin.num_tiles, bin.overflow, bin.cap);
 }
 
 }  // namespace adop

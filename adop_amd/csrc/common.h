@@ -53,6 +53,20 @@ __device__ __forceinline__ bool depth_is_dropped(float zs)
     return (int32_t)__float_as_uint(zs) < 0;
 }
 
+// A kernel that runs only when a flag word in the workspace has a given value (flag == nullptr: always).  The flag is
+// written by an earlier launch of the same call: the first binning passes find out on the device whether the bin
+// entries of the call fit a workspace with smaller bins; if not, the tile kernels return at once and the kernels of
+// the direct path, queued behind them, run instead.
+struct Gate
+{
+    const uint32_t* flag;
+    uint32_t run_when;
+};
+__device__ __forceinline__ bool gate_closed(const Gate& g)
+{
+    return g.flag != nullptr && *g.flag != g.run_when;  // (kernel-uniform)
+}
+
 struct LevelArg
 {
     int32_t w, h;

@@ -38,9 +38,13 @@ __global__ void fill_u32_kernel(uint32_t* __restrict__ p, size_t n, uint32_t v)
 // Levels below first_level are left alone (the tile path writes them itself).
 __global__ __launch_bounds__(kBlock) void clear_kernel(Levels lv, int first_level, float4* __restrict__ accum,
                                                        size_t accum_vec4, uint32_t* __restrict__ zero_u32, int zero_n,
-                                                       ViewPrep vp)
+                                                       ViewPrep vp, Gate gate, adop_stats* zero_stats)
 {
+    if (gate_closed(gate)) return;
     prepare_views_inline(vp);
+    // (the direct path taking over from the tile path counts the point-levels again)
+    if (zero_stats && blockIdx.x == 0 && threadIdx.x < sizeof(adop_stats) / sizeof(uint64_t))
+        ((uint64_t*)zero_stats)[threadIdx.x] = 0;
     // counters of the tile bins (tile path only)
     for (int k = blockIdx.x * blockDim.x + threadIdx.x; k < zero_n; k += gridDim.x * blockDim.x) zero_u32[k] = 0;
     int r0        = lv.pix_prefix[first_level];
@@ -70,9 +74,10 @@ __global__ __launch_bounds__(kBlock) void clear_kernel(Levels lv, int first_leve
 // memory transaction whatever it carries.
 template <int PPT>
 __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const ViewConst* __restrict__ views, Levels lv,
-                                                         ParamArg rp, int group_from, adop_stats* stats)
+                                                         ParamArg rp, int group_from, adop_stats* stats, Gate gate)
 {
     __shared__ unsigned long long s_pk[kBlock];
+    if (gate_closed(gate)) return;
     __shared__ unsigned long long s_gmask[kBlock];
     __shared__ uint32_t s_gkey[kBlock];
     const bool STATS = stats != nullptr;  // counter pass (uniform branch)
@@ -278,12 +283,13 @@ __global__ __launch_bounds__(kBlock) void prepass_kernel(CloudArg pc, const View
 template <int CT, bool HALF>
 __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewConst* __restrict__ views, Levels lv,
                                                        ParamArg rp, float* __restrict__ accum, int S,
-                                                       adop_stats* stats, int group_from)
+                                                       adop_stats* stats, int group_from, Gate gate)
 {
     constexpr int CMAX = CT ? CT : kMaxChannels;
     __shared__ unsigned long long s_gmask[kBlock];
     __shared__ uint32_t s_gkey[kBlock];
     extern __shared__ float s_stage[];  // kBlock * C descriptors of the block's points
+    if (gate_closed(gate)) return;
     const bool STATS = stats != nullptr;  // counter pass (uniform branch)
     const int C      = CT ? CT : lv.C;
     const int lane   = threadIdx.x & 63;
@@ -507,9 +513,10 @@ __global__ __launch_bounds__(kBlock) void blend_kernel(CloudArg pc, const ViewCo
 template <int CT>
 __global__ __launch_bounds__(kBlock) void resolve_kernel(Levels lv, int first_level, const float* __restrict__ accum,
                                                          int S, const float* __restrict__ background, int write_mask,
-                                                         float mask_value)
+                                                         float mask_value, Gate gate)
 {
     constexpr int CMAX = CT ? CT : kMaxChannels;
+    if (gate_closed(gate)) return;
     const int C        = CT ? CT : lv.C;
     int r0             = lv.pix_prefix[first_level];
     int per_image      = lv.pix_prefix[lv.num] - r0;
@@ -581,10 +588,10 @@ void launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t st)
 }
 
 void launch_clear(const Levels& lv, int first_level, int grid, float* accum, size_t accum_floats, uint32_t* zero_u32,
-                  int zero_n, const ViewPrep& vp, hipStream_t st)
+                  int zero_n, const ViewPrep& vp, hipStream_t st, Gate gate, adop_stats* zero_stats)
 {
     hipLaunchKernelGGL(clear_kernel, dim3(grid), dim3(kBlock), 0, st, lv, first_level, (float4*)accum, accum_floats / 4,
-                       zero_u32, zero_n, vp);
+                       zero_u32, zero_n, vp, gate, zero_stats);
 }
 
 // Points per thread of prepass_kernel: two for the clouds of a hundred million points that reach the direct path by
@@ -600,25 +607,25 @@ static int prepass_ppt(int n, int tuned)
 int prepass_points_per_block(int n, int tuned_ppt) { return kBlock * prepass_ppt(n, tuned_ppt); }
 
 void launch_prepass(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, adop_stats* stats,
-                    const adop_tuning& tn, hipStream_t st)
+                    const adop_tuning& tn, hipStream_t st, Gate gate)
 {
     if (pc.n < 1) return;
     const int group_from = tn.prepass_group_from;
     const int ppt        = prepass_ppt(pc.n, tn.prepass_ppt);
     if (ppt == 4)
         hipLaunchKernelGGL((prepass_kernel<4>), dim3((pc.n + kBlock * 4 - 1) / (kBlock * 4)), dim3(kBlock), 0, st, pc,
-                           views, lv, rp, group_from, stats);
+                           views, lv, rp, group_from, stats, gate);
     else if (ppt == 2)
         hipLaunchKernelGGL((prepass_kernel<2>), dim3((pc.n + kBlock * 2 - 1) / (kBlock * 2)), dim3(kBlock), 0, st, pc,
-                           views, lv, rp, group_from, stats);
+                           views, lv, rp, group_from, stats, gate);
     else
         hipLaunchKernelGGL((prepass_kernel<1>), dim3((pc.n + kBlock - 1) / kBlock), dim3(kBlock), 0, st, pc, views, lv,
-                           rp, group_from, stats);
+                           rp, group_from, stats, gate);
 }
 
 template <int CT, bool HALF>
 static void launch_blend_t(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp,
-                           float* accum, int S, adop_stats* stats, const adop_tuning& tn, hipStream_t st)
+                           float* accum, int S, adop_stats* stats, const adop_tuning& tn, hipStream_t st, Gate gate)
 {
     const int group_from = tn.blend_group_from;  // 0: group at every level
     // list mode: one small workgroup per prepass workgroup (a few percent of the points survive in a dense cloud)
@@ -628,36 +635,36 @@ static void launch_blend_t(const CloudArg& pc, const ViewConst* views, const Lev
     const int grid  = pc.list_ids ? (pc.n + pc.list_span - 1) / pc.list_span : (pc.n + kBlock - 1) / kBlock;
     size_t lds      = sizeof(float) * (size_t)block * (size_t)lv.C;
     hipLaunchKernelGGL((blend_kernel<CT, HALF>), dim3(grid), dim3(block), lds, st, pc, views, lv, rp,
-                       accum, S, stats, group_from);
+                       accum, S, stats, group_from, gate);
 }
 
 void launch_blend(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
-                  float* accum, int S, adop_stats* stats, const adop_tuning& tn, hipStream_t st)
+                  float* accum, int S, adop_stats* stats, const adop_tuning& tn, hipStream_t st, Gate gate)
 {
     if (pc.n < 1) return;
     if (lv.C == 8)
-        half ? launch_blend_t<8, true>(pc, views, lv, rp, accum, S, stats, tn, st)
-             : launch_blend_t<8, false>(pc, views, lv, rp, accum, S, stats, tn, st);
+        half ? launch_blend_t<8, true>(pc, views, lv, rp, accum, S, stats, tn, st, gate)
+             : launch_blend_t<8, false>(pc, views, lv, rp, accum, S, stats, tn, st, gate);
     else if (lv.C == 4)
-        half ? launch_blend_t<4, true>(pc, views, lv, rp, accum, S, stats, tn, st)
-             : launch_blend_t<4, false>(pc, views, lv, rp, accum, S, stats, tn, st);
+        half ? launch_blend_t<4, true>(pc, views, lv, rp, accum, S, stats, tn, st, gate)
+             : launch_blend_t<4, false>(pc, views, lv, rp, accum, S, stats, tn, st, gate);
     else
-        half ? launch_blend_t<0, true>(pc, views, lv, rp, accum, S, stats, tn, st)
-             : launch_blend_t<0, false>(pc, views, lv, rp, accum, S, stats, tn, st);
+        half ? launch_blend_t<0, true>(pc, views, lv, rp, accum, S, stats, tn, st, gate)
+             : launch_blend_t<0, false>(pc, views, lv, rp, accum, S, stats, tn, st, gate);
 }
 
 void launch_resolve(const Levels& lv, int first_level, int grid, const float* accum, int S, const float* background,
-                    int write_mask, float mask_value, hipStream_t st)
+                    int write_mask, float mask_value, hipStream_t st, Gate gate)
 {
     if (lv.C == 8)
         hipLaunchKernelGGL((resolve_kernel<8>), dim3(grid), dim3(kBlock), 0, st, lv, first_level, accum, S, background,
-                           write_mask, mask_value);
+                           write_mask, mask_value, gate);
     else if (lv.C == 4)
         hipLaunchKernelGGL((resolve_kernel<4>), dim3(grid), dim3(kBlock), 0, st, lv, first_level, accum, S, background,
-                           write_mask, mask_value);
+                           write_mask, mask_value, gate);
     else
         hipLaunchKernelGGL((resolve_kernel<0>), dim3(grid), dim3(kBlock), 0, st, lv, first_level, accum, S, background,
-                           write_mask, mask_value);
+                           write_mask, mask_value, gate);
 }
 
 }  // namespace adop

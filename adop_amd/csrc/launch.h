@@ -19,7 +19,7 @@ void launch_prepare_views(const ViewChunk& ch, int first, int count, const doubl
                           int cols, ViewConst* out, hipStream_t st);
 void launch_fill_u32(uint32_t* p, size_t n, uint32_t v, hipStream_t st);
 void launch_clear(const Levels& lv, int first_level, int grid, float* accum, size_t accum_floats, uint32_t* zero_u32,
-                  int zero_n, const ViewPrep& vp, hipStream_t st);
+                  int zero_n, const ViewPrep& vp, hipStream_t st, Gate gate = {nullptr, 0}, adop_stats* zero_stats = nullptr);
 void launch_knn_first_grid(const float4* position, int n, const KnnGrid& box, KnnGrid* dst, hipStream_t st);
 void launch_knn_refine_grid(const float* sample, int samples, const KnnGrid* first, KnnGrid* g, uint32_t budget,
                             hipStream_t st);
@@ -48,11 +48,11 @@ void launch_morton(const float4* position, int n, const float* mn, const float* 
 // points per workgroup of prepass_kernel on a cloud of n points (the unit of its candidate lists)
 int prepass_points_per_block(int n, int tuned_ppt);
 void launch_prepass(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, adop_stats* stats,
-                    const adop_tuning& tn, hipStream_t st);
+                    const adop_tuning& tn, hipStream_t st, Gate gate = {nullptr, 0});
 void launch_blend(const CloudArg& pc, const ViewConst* views, const Levels& lv, const ParamArg& rp, bool half,
-                  float* accum, int S, adop_stats* stats, const adop_tuning& tn, hipStream_t st);
+                  float* accum, int S, adop_stats* stats, const adop_tuning& tn, hipStream_t st, Gate gate = {nullptr, 0});
 void launch_resolve(const Levels& lv, int first_level, int grid, const float* accum, int S, const float* background,
-                    int write_mask, float mask_value, hipStream_t st);
+                    int write_mask, float mask_value, hipStream_t st, Gate gate = {nullptr, 0});
 
 // Forward pass through screen-space tile bins (binned_kernels.hip, tile_kernels.hip).  A tile has kBlock level-0 pixels,
 // one per thread of a workgroup: 16 x 16 (32 x 8, with 128-byte rows in the output tensors, measured 5 % slower: more
@@ -91,6 +91,11 @@ struct BinArg
     // their own.
     int32_t shard_shift;
     int32_t num_tiles;  // tiles of all views of the call
+    // A workspace with smaller bins (ADOP_WORKSPACE_SMALL_BINS): `entries` holds `cap` entries, fewer than the call can
+    // have.  The prefix sum writes *overflow = 1 when the call has more (else 0); the second binning pass and the tile
+    // kernels then return at once.  nullptr: the bins hold every entry the call can have.
+    uint32_t* overflow;
+    uint32_t cap;
 };
 // Shards per tile: as many as keep the counters of a call within 16 384 (the prefix sum over them is one workgroup), at
 // most 8, and none above 4 096 tiles: the second pass then looks up two lines per entry group instead of one, which a

@@ -79,6 +79,7 @@ template <int LT>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) void tile_depth_kernel(Levels lv, BinArg bin, int num_tiles)
 {
     __shared__ unsigned long long s_depth[kTileMaxPixels];
+    if (bin.overflow && *bin.overflow) return;  // the bins of this workspace were too small for the call
     const int tiles_per_view = bin.tiles_x * bin.tiles_y;
     // the first max_rows workgroups take the further slices of the bins that are split (they are the longest pieces of
     // work of the launch: first, so that they do not form its tail); most calls have none
@@ -280,6 +281,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu((CT != 0
     constexpr int TX    = 1 << kTileShiftX;  // level-0 extent of the tile; TX * TY = kBlock
     constexpr int TY    = 1 << kTileShiftY;
     extern __shared__ __align__(16) unsigned char smem[];
+    if (bin.overflow && *bin.overflow) return;  // the bins of this workspace were too small for the call
     const bool STATS = stats != nullptr;
     const int C      = CT ? CT : lv.C;
     const int tid    = threadIdx.x;

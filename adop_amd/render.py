@@ -262,6 +262,7 @@ def BlendPointCloudForward(ctx, info, build=True):
     s = info.scene.struct()
     fb = cache.forward_struct()
     stats = C.c_void_p(cache.stats.data_ptr()) if info.collect_stats else None
+    info.params.workspace_flags = int(info.workspace_flags)  # (how the cache sized the workspace)
     rc = cache.lib.adop_forward(C.byref(s), cache.views_array(), cache.num_batches, C.byref(info.params), C.byref(fb),
                                 C.c_void_p(cache.workspace.data_ptr()), cache.workspace.numel(), stats, _stream_ptr())
     _check(rc, cache.lib)
@@ -339,6 +340,7 @@ def BlendPointCloudBackward(ctx, info, image_gradients, needs=(True, True, True)
     cache.info = info
     s = scene.struct()
     stats = C.c_void_p(cache.stats.data_ptr()) if info.collect_stats else None
+    info.params.workspace_flags = int(info.workspace_flags)
     rc = cache.lib.adop_backward(C.byref(s), cache.views_array(), cache.num_batches, C.byref(info.params),
                                  C.byref(fb), C.byref(gb), C.c_void_p(cache.workspace.data_ptr()),
                                  cache.workspace.numel(), stats, _stream_ptr())

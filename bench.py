@@ -323,7 +323,9 @@ def run_workload(args, workload, steps, warmup, lib, point_order=None, lod=False
     cache = render.PointRendererCache()
     info = render.NeuralRenderInfo(scene=scene, images=list(hs.views), params=hs.params, num_layers=hs.num_layers,
                                    cache=cache, train=backward and not args.no_point_cache,
+                                   workspace_flags=args.workspace_flags,
                                    dropout_points=None if hs.dropout is None else torch.from_numpy(hs.dropout))
+    hs.params.workspace_flags = args.workspace_flags
     cache.Build(info, True)
     s = scene.struct()
     fb = cache.forward_struct()
@@ -636,6 +638,8 @@ def main():
                     help="default workload only: leave out the other configurations (step.configs)")
     ap.add_argument("--print-sources-state", action="store_true",
                     help="print kernel_sources_state() (what a MEASURED_TRAFFIC table is keyed on) and exit")
+    ap.add_argument("--workspace-flags", type=int, default=0,
+                    help="adop_workspace_size_for flags: 1 point cache kept, 2 no tile path, 4 small bins")
     ap.add_argument("--tuning", default="",
                     help="adop_tuning fields for the whole run, e.g. tile_k=2,count_ppt=4 (A/B runs of the library's switches)")
     ap.add_argument("--no-env", action="store_true", help="config5 without the environment-map passes")

@@ -94,6 +94,9 @@ typedef struct adop_render_params
      * empty buffers (and ignores point_cache, which such a forward does not write).  0 (the reference's default,
      * render_points = true): rendered.  A cloud may also be empty (num_points == 0, its pointers may be NULL). */
     int32_t skip_points;
+    /* The flags the caller sized the workspace with (adop_workspace_size_for; 0 = adop_workspace_size): how
+     * adop_forward and adop_backward lay it out.  No counterpart in the reference. */
+    uint32_t workspace_flags;
 } adop_render_params;
 
 /* Inputs owned by NeuralScene: NeuralPointCloudCuda + NeuralTexture + PoseModule + IntrinsicsModule. */
@@ -194,15 +197,23 @@ size_t adop_workspace_size(const adop_scene* scene, int32_t num_views, int32_t n
  * that only a forward pass WITHOUT a caller's point_cache uses (the projected points and the candidate lists of the
  * direct path) and 36 bytes that only the tile-bin forward path uses (a tile word and two bin entries):
  *   ADOP_WORKSPACE_POINT_CACHE_KEPT  every adop_forward call passes buffers->point_cache (training): the 20 bytes go;
- *   ADOP_WORKSPACE_NO_TILE_PATH      the forward pass may always take the direct path: the 36 bytes go.
- * adop_forward lays the workspace out from workspace_bytes and from whether point_cache is NULL: the largest of the
- * four layouts that fits and serves the call.  In a layout without tile bins it renders through the direct path (same
- * results; forward_path = 2 is then refused with ADOP_WORKSPACE_TOO_SMALL); a call with point_cache = NULL needs the
- * 20 bytes and is refused when not even the layout without bins has room for them.
- * adop_backward works with every one of them.  16 crops of a 100 M-point cloud: 102 GB in full, 70 GB with the point
- * cache kept (plus the 25.6 GB of the cache itself), 13 GB with both flags. */
+ *   ADOP_WORKSPACE_NO_TILE_PATH      the forward pass may always take the direct path: the 36 bytes go;
+ *   ADOP_WORKSPACE_SMALL_BINS        tile bins for one entry per four points and view instead of two per point and view
+ *                                    (8 of the 36 bytes stay): what views take that see a part of the cloud each (the
+ *                                    crops of a training batch: 0.07 entries per point and view).  Whether a call's
+ *                                    entries fit is known on the device only, after the first binning pass: when they
+ *                                    do not, the tile kernels return at once and the direct path's kernels, which are
+ *                                    queued behind them in such a workspace (four launches that otherwise return at
+ *                                    once), render the call: same results, the time of both first passes.
+ * The same flags go into adop_render_params.workspace_flags of every call that uses the workspace: that is how
+ * adop_forward and adop_backward lay it out.  Without tile bins the forward pass renders through the direct path (same
+ * results; forward_path = 2 is then refused with ADOP_WORKSPACE_TOO_SMALL); with ADOP_WORKSPACE_POINT_CACHE_KEPT a
+ * forward call that passes no point_cache is refused (ADOP_INVALID_ARG).
+ * 16 crops of a 100 M-point cloud: 102 GB in full, 70 GB with the point cache kept, 25 GB with the cache kept and
+ * small bins, 13 GB without bins (plus the 25.6 GB of the point cache itself). */
 #define ADOP_WORKSPACE_POINT_CACHE_KEPT 1u
 #define ADOP_WORKSPACE_NO_TILE_PATH 2u
+#define ADOP_WORKSPACE_SMALL_BINS 4u
 size_t adop_workspace_size_for(const adop_scene* scene, int32_t num_views, int32_t num_layers, int32_t w, int32_t h,
                                uint32_t flags);
 

@@ -86,7 +86,9 @@ def test_workspace_variants_and_their_independence_of_the_tuning():
     # tile word 4 B + two bin entries of 16 B per point and view, + counters, tile order and the rows of split bins
     assert 36 * B * N < full - direct < 36 * B * N + 24 * slack
     assert abs((kept - both) - (full - direct)) < slack
-    assert lib.adop_workspace_size_for(*args, 4) == 0  # unknown flag
+    assert lib.adop_workspace_size_for(*args, 8) == 0  # unknown flag
+    small = lib.adop_workspace_size_for(*args, _capi.WORKSPACE_SMALL_BINS)
+    assert abs((full - small) - 28 * B * N) < slack  # two entries per point and view -> one per four: 32 -> 4 bytes
     # a cloud beyond what the bin entries can address: the bins are left out of every layout
     s.num_points = (1 << 28) + 5
     assert lib.adop_workspace_size(C.byref(s), 1, 4, 512, 512) == \

@@ -37,7 +37,8 @@ END_TO_END_MISS_SIZE = 1e-6
 end_to_end_misses = {}  # case -> {tensor: (misses, size, worst)}: printed by the last test of the file
 
 
-def _fwd_bwd(hs, oracle_mod, needs=(True, True, True), seed=5, collect_stats=True, poison=False, pixel_records=True):
+def _fwd_bwd(hs, oracle_mod, needs=(True, True, True), seed=5, collect_stats=True, poison=False, pixel_records=True,
+             workspace_flags=0):
     import torch
     from adop_amd import render, scenes
 
@@ -45,7 +46,7 @@ def _fwd_bwd(hs, oracle_mod, needs=(True, True, True), seed=5, collect_stats=Tru
 
     ref = oracle_mod.forward(hs)
     scene, info, ctx, images, masks = run_hip_forward(hs, collect_stats=collect_stats, poison=poison,
-                                                      pixel_records=pixel_records)
+                                                      pixel_records=pixel_records, workspace_flags=workspace_flags)
     check_forward(hs, ref, ctx, images, masks, info, stats=collect_stats)
     gout = scenes.upstream_grads(hs, seed)
     grads = render.BlendPointCloudBackward(ctx, info, _torch_grads(gout), needs)
@@ -665,46 +666,92 @@ def test_full_bins_are_split_between_workgroups(oracle_mod, forward_path, slice_
 
 
 def test_smaller_workspaces(oracle_mod, forward_path):
-    """adop_workspace_size_for: a workspace without the region of a forward pass that keeps no point cache, without the
-    tile bins, or without both.  Same results; without the bins the library renders through the direct path (and
-    refuses forward_path = 2); without the other region it refuses a forward pass that passes no point cache."""
+    """adop_workspace_size_for + adop_render_params.workspace_flags: a workspace without the region of a forward pass
+    that keeps no point cache, without the tile bins, with small bins, and the combinations.  Same results; without the
+    bins the library renders through the direct path (and refuses forward_path = 2); without the other region it
+    refuses a forward pass that passes no point cache."""
     import torch
     from adop_amd import _capi, render, scenes
 
     hs = scenes.config3(n=150_000, w=256, h=144, channels=4, seed=21)
     ref = oracle_mod.forward(hs)
     gout = scenes.upstream_grads(hs, 9)
-    for flags in (_capi.WORKSPACE_POINT_CACHE_KEPT, _capi.WORKSPACE_NO_TILE_PATH,
-                  _capi.WORKSPACE_POINT_CACHE_KEPT | _capi.WORKSPACE_NO_TILE_PATH):
+    KEPT, NOBINS, SMALL = _capi.WORKSPACE_POINT_CACHE_KEPT, _capi.WORKSPACE_NO_TILE_PATH, _capi.WORKSPACE_SMALL_BINS
+    lib = _capi.load_library()
+    sizes = {}
+    for flags in (0, KEPT, NOBINS, KEPT | NOBINS, SMALL, SMALL | KEPT):
         announce(f"workspace flags {flags}, forward_path={forward_path}")
-        no_bins = bool(flags & _capi.WORKSPACE_NO_TILE_PATH)
-        if no_bins and forward_path == 2:
+        if (flags & NOBINS) and forward_path == 2:
             with pytest.raises(RuntimeError, match="tile bins"):
                 run_hip_forward(hs, workspace_flags=flags)
             continue
         scene, info, ctx, images, masks = run_hip_forward(hs, workspace_flags=flags, poison=True)
+        sizes[flags] = info.cache.workspace.numel()
         check_forward(hs, ref, ctx, images, masks, info)
         grads = render.BlendPointCloudBackward(ctx, info, _torch_grads(gout))
         torch.cuda.synchronize()
         refb = oracle_mod.backward(hs, download_forward(hs, info, images, masks), gout)
         check_backward(hs, refb, grads, info)
-        # a forward pass that passes no point cache after all: refused where the workspace has no room for the
-        # projected points at all (both flags); with the bins' room instead (36 bytes per point and view where 20 are
-        # needed) the library lays the workspace out without bins and renders through the direct path
-        if flags == (_capi.WORKSPACE_POINT_CACHE_KEPT | _capi.WORKSPACE_NO_TILE_PATH):
-            with pytest.raises(RuntimeError, match="workspace too small"):
-                run_hip_forward(hs, workspace_flags=flags, train=False)
-        elif flags == _capi.WORKSPACE_POINT_CACHE_KEPT and forward_path == 2:
-            with pytest.raises(RuntimeError, match="tile bins"):
+        if flags & KEPT:  # a forward pass that passes no point cache after all
+            with pytest.raises(RuntimeError, match="point_cache"):
                 run_hip_forward(hs, workspace_flags=flags, train=False)
         else:
-            got = run_hip_forward(hs, workspace_flags=flags, train=False)
+            got = run_hip_forward(hs, workspace_flags=flags, train=False, poison=True)
             check_forward(hs, ref, got[2], got[3], got[4], got[1])
-    # the library's own choice with a workspace that has no bins: the direct path, no error
-    import helpers
-    helpers.FORWARD_PATH = 0
-    got = run_hip_forward(hs, workspace_flags=_capi.WORKSPACE_NO_TILE_PATH)
-    check_forward(hs, ref, got[2], got[3], got[4], got[1])
+    if forward_path != 2:
+        assert sizes[0] > sizes[KEPT] > sizes[NOBINS] > sizes[KEPT | NOBINS] and sizes[0] > sizes[SMALL] > sizes[SMALL | KEPT]
+    # a workspace that is too small for the flags it is called with
+    s = _capi.Scene()
+    s.num_points, s.num_channels, s.num_poses, s.num_cameras, s.intrinsics_cols = hs.num_points, 4, 1, 1, 13
+    assert lib.adop_workspace_size_for(C_byref(s), 1, 4, 256, 144, 8) == 0
+    hs.params.workspace_flags = 0
+
+
+def C_byref(x):
+    import ctypes
+
+    return ctypes.byref(x)
+
+
+@pytest.mark.parametrize("collect_stats", [True, False], ids=["counters", "plain"])
+def test_small_bins_fall_back_to_the_direct_path_on_the_device(oracle_mod, forward_path, collect_stats):
+    """ADOP_WORKSPACE_SMALL_BINS holds one bin entry per four points and view.  A view that sees the whole cloud has
+    more (a cube in front of the camera: one entry per point and a few second entries): the prefix sum of the binning
+    passes finds that out on the device, the tile kernels return at once and the direct path's kernels behind them
+    render the call, counters included.  A batch of crops fits and runs through the tile kernels.  Both against the
+    checker, forward (with and without a point cache) and backward."""
+    import torch
+    from adop_amd import _capi, render, scenes
+
+    if forward_path != 2:
+        pytest.skip("the tile path only")
+    SMALL = _capi.WORKSPACE_SMALL_BINS
+    # (a) overflow: every point of the cube is in the image
+    hs = scenes.config1(n=120_000, w=320, h=320, levels=4, seed=3, point_order="morton")
+    hs.params.ghost_gradients = 0
+    announce(f"small bins, a view that overflows them: 120k pts 320x320, counters={collect_stats}")
+    ref = oracle_mod.forward(hs)
+    assert int(ref.stats.visible[0]) > hs.num_points // 4 + 1024  # more entries than the small bins hold
+    for train in (True, False):
+        scene, info, ctx, images, masks = run_hip_forward(hs, workspace_flags=SMALL, train=train, poison=True,
+                                                          collect_stats=collect_stats)
+        check_forward(hs, ref, ctx, images, masks, info, stats=collect_stats)
+        if train:
+            gout = scenes.upstream_grads(hs, 9)
+            grads = render.BlendPointCloudBackward(ctx, info, _torch_grads(gout))
+            torch.cuda.synchronize()
+            refb = oracle_mod.backward(hs, download_forward(hs, info, images, masks), gout)
+            check_backward(hs, refb, grads, info, stats=collect_stats)
+    # (b) no overflow: four crops that see a part of the cloud each
+    hs = scenes.config3(n=200_000, w=192, h=128, channels=4, seed=13)
+    hs.views = [scenes.make_view(192, 128, crop=(3.0, 3.0, -float(x), -float(y), 0.0)) for (x, y) in
+                ((100, 60), (300, 120), (150, 200), (20, 10))]
+    hs.dropout = scenes.bernoulli_mask(5, 4, hs.num_points, 0.25)
+    announce(f"small bins, four crops that fit: 200k pts, counters={collect_stats}")
+    ref = oracle_mod.forward(hs)
+    assert sum(int(v) for v in ref.stats.visible[:1]) < hs.num_points  # well inside 4 * N / 4
+    _fwd_bwd(hs, oracle_mod, collect_stats=collect_stats, poison=True, workspace_flags=SMALL)
+    hs.params.workspace_flags = 0
 
 
 # Every kernel variant the tuning switches choose between, each on one small scene (forward without a point cache,

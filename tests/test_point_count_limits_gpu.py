@@ -1,8 +1,8 @@
 """Parity at the largest clouds the library takes, against the CPU checker: 2^28 - 1024 points through both forward
 paths (the tile path's limit: point ids have 28 bits in a bin entry), 2^28 + 1024 (the library's choice must fall
-back to the direct path) and 2^30 points (the limit of a call), forward and backward with all gradients.  The checker
-needs one to five minutes per pass at these sizes and the scenes 10 to 100 GB of host memory, so the cases run only
-when ADOP_TEST_POINT_LIMITS=1 (about 15 minutes in all); a line is printed every 30 s while they work."""
+back to the direct path) and 2^30 points (the limit of a call), forward and backward with all gradients.  The scenes
+take minutes to generate and 10 to 100 GB of host memory, so the cases run only when ADOP_TEST_POINT_LIMITS=1; a line
+is printed every 30 s while they work."""
 import os
 import threading
 import time
@@ -13,7 +13,7 @@ from helpers import announce, check_backward, check_forward, download_forward, r
 
 pytestmark = [pytest.mark.gpu,
               pytest.mark.skipif(os.environ.get("ADOP_TEST_POINT_LIMITS") != "1",
-                                 reason="takes 15 minutes and 100 GB of host memory: set ADOP_TEST_POINT_LIMITS=1")]
+                                 reason="takes several minutes and 100 GB of host memory: set ADOP_TEST_POINT_LIMITS=1")]
 
 
 @pytest.fixture
@@ -41,7 +41,7 @@ def test_largest_clouds(oracle_mod, heartbeat, n, paths):
     hs.dropout = None
     hs.params.ghost_gradients = 0  # spatial gradients of the rendered points
     announce("checker forward")
-    ref = oracle_mod.forward(hs)
+    ref = oracle_mod.forward(hs, omp=True)  # (the OpenMP build: held to the serial one by tests/test_oracle_omp.py)
     assert int(ref.stats.visible[0]) > 0.8 * n
     for path in paths:
         announce(f"{n} points, forward_path={path}: forward")
@@ -54,7 +54,7 @@ def test_largest_clouds(oracle_mod, heartbeat, n, paths):
         grads = render.BlendPointCloudBackward(ctx, info, [torch.from_numpy(g).cuda() for g in gout], (True, True, True))
         torch.cuda.synchronize()
         announce("checker backward")
-        refb = oracle_mod.backward(hs, download_forward(hs, info, images, masks), gout, True, True, True)
+        refb = oracle_mod.backward(hs, download_forward(hs, info, images, masks), gout, True, True, True, omp=True)
         check_backward(hs, refb, grads, info, stats=True)
         del grads, gout, refb, scene, info, ctx, images, masks
         torch.cuda.empty_cache()
