@@ -48,29 +48,18 @@ KERNEL_OF_STAGE = {"BinCount": "bin_count_kernel", "BinScatter": "bin_scatter_ke
 # x 1.0 after calibration with plain device copies of known size), per workload.  "sources" is kernel_sources_state() of
 # the tree the profile was taken on (python bench.py --print-sources-state): the figures are quoted for that state only.
 MEASURED_TRAFFIC = {
-    "config3": {"sources": "d00cff3-state", "profile": "profiles/config3_tile_path_fwd_bwd_kernels_traffic_instructions.md",
-                "bytes": {"RenderBackward/descriptor": 860.1e6, "RenderBackward/spatial": 572.2e6, "TileBlend": 529.1e6,
-                          "BinCount": 430.3e6, "CombineAndFillBackward": 220.8e6, "TileDepth": 101.5e6, "Initialize": 11.8e6,
-                          "CombineAndFill": 23.5e6, "BinScatter": 197.5e6, "Post Process Gradient": 0.5e6}},
-    "config1": {"sources": "d00cff3-state", "profile": "profiles/config1_direct_path_forward_kernels_traffic_instructions.md",
-                "bytes": {"DepthPrepass": 13.1e6, "RenderForward": 8.5e6, "CombineAndFill": 5.6e6, "Initialize": 3.5e6}},
-    "config2": {"sources": "d00cff3-state", "profile": "profiles/config2_fwd_bwd_kernels_traffic_instructions.md",
-                "bytes": {"RenderBackward/descriptor": 200.8e6, "BinCount": 64.6e6, "TileBlend": 162.1e6,
-                          "RenderBackward/spatial": 145.9e6, "CombineAndFillBackward": 67.2e6, "TileDepth": 37.9e6,
-                          "Initialize": 3.4e6, "CombineAndFill": 6.6e6, "BinScatter": 67.4e6, "Post Process Gradient": 15.1e6}},
-    "config4": {"sources": "d00cff3-state", "profile": "profiles/config4_direct_path_forward_kernels_traffic_instructions.md",
-                "bytes": {"DepthPrepass": 4856.1e6, "RenderForward": 1445.6e6, "CombineAndFill": 176.8e6, "Initialize":
-                          110.5e6}},
-    # (the spatial-gradient stage of config5 is 8 launches, its Initialize the clear and a fill)
-    "config5": {"sources": "d00cff3-state", "profile": "profiles/config5_ocam_envmap_fwd_bwd_kernels_traffic_instructions.md",
-                "bytes": {"RenderBackward/spatial": 8 * 719.5e6, "EnvironmentMapBackward": 2242.8e6, "TileBlend": 5064.5e6,
-                          "BinCount": 2189.5e6, "RenderBackward/descriptor": 4091.9e6, "EnvironmentMap": 3081.2e6,
-                          "CombineAndFillBackward": 1872.6e6, "TileDepth": 1622.9e6, "CombineAndFill": 177.1e6, "Initialize":
-                          91.5e6, "BinScatter": 3331.8e6, "Post Process Gradient": 484.7e6}},
-    "crops": {"sources": "d00cff3-state", "profile": "profiles/training_batch_16_crops_fwd_bwd_kernels_traffic_instructions.md",
-                "bytes": {"RenderBackward/descriptor": 1579.9e6, "RenderBackward/spatial": 1242.1e6, "BinCount": 587.1e6,
-                          "TileBlend": 1211.3e6, "CombineAndFillBackward": 446.2e6, "TileDepth": 249.2e6, "CombineAndFill":
-                          47.9e6, "Initialize": 23.7e6, "BinScatter": 764.6e6, "Post Process Gradient": 120.3e6}},
+    "config3": {"sources": "711b51ac9c49", "profile": "profiles/config3_tile_path_fwd_bwd_kernels_traffic_instructions.md",
+                "bytes": {"RenderBackward/descriptor": 860.0e6, "RenderBackward/spatial": 572.1e6, "TileBlend": 529.0e6, "BinCount": 430.3e6, "BinScatter": 197.5e6, "CombineAndFillBackward": 220.8e6, "TileDepth": 101.5e6, "Post Process Gradient": 0.5e6, "CombineAndFill": 23.5e6, "Initialize": 11.8e6}},
+    "config1": {"sources": "711b51ac9c49", "profile": "profiles/config1_direct_path_forward_kernels_traffic_instructions.md",
+                "bytes": {"DepthPrepass": 13.0e6, "RenderForward": 8.5e6, "Initialize": 3.5e6, "CombineAndFill": 5.6e6}},
+    "config2": {"sources": "711b51ac9c49", "profile": "profiles/config2_fwd_bwd_kernels_traffic_instructions.md",
+                "bytes": {"RenderBackward/descriptor": 200.8e6, "TileBlend": 161.9e6, "RenderBackward/spatial": 146.7e6, "BinScatter": 67.5e6, "BinCount": 64.5e6, "CombineAndFillBackward": 67.2e6, "TileDepth": 37.9e6, "Post Process Gradient": 15.1e6, "Initialize": 3.4e6, "CombineAndFill": 6.6e6}},
+    "config4": {"sources": "711b51ac9c49", "profile": "profiles/config4_direct_path_forward_kernels_traffic_instructions.md",
+                "bytes": {"DepthPrepass": 5080.7e6, "RenderForward": 1545.8e6, "CombineAndFill": 176.8e6, "Initialize": 110.5e6}},
+    "config5": {"sources": "711b51ac9c49", "profile": "profiles/config5_ocam_envmap_fwd_bwd_kernels_traffic_instructions.md",
+                "bytes": {"RenderBackward/spatial": 5753.6e6, "TileBlend": 5064.9e6, "EnvironmentMapBackward": 2242.8e6, "BinCount": 2189.5e6, "RenderBackward/descriptor": 4091.9e6, "EnvironmentMap": 3081.4e6, "BinScatter": 3331.6e6, "TileDepth": 1622.9e6, "CombineAndFillBackward": 1872.4e6, "Post Process Gradient": 484.7e6, "CombineAndFill": 177.1e6, "Initialize": 91.5e6}},
+    "crops": {"sources": "711b51ac9c49", "profile": "profiles/training_batch_16_crops_fwd_bwd_kernels_traffic_instructions.md",
+                "bytes": {"RenderBackward/descriptor": 1579.8e6, "RenderBackward/spatial": 1242.0e6, "BinCount": 587.1e6, "TileBlend": 1211.8e6, "BinScatter": 764.6e6, "CombineAndFillBackward": 446.2e6, "TileDepth": 249.2e6, "Post Process Gradient": 120.3e6, "CombineAndFill": 47.8e6, "Initialize": 23.7e6}},
 }
 
 
