@@ -137,3 +137,60 @@ torch::Tensor SortBlocksByRadius(torch::Tensor radius, int block_size)
     auto tail = torch::arange(nb * block_size, n, radius.options().dtype(torch::kInt64));
     return torch::cat({order.reshape({-1}), tail});
 }
+
+torch::Tensor RandomBlockShuffle(int64_t num_points, int block_size, at::Generator generator, torch::Device device)
+{
+    const int64_t nb = num_points / block_size;
+    auto i64         = torch::TensorOptions().dtype(torch::kInt64);
+    auto perm        = torch::randperm(nb, generator, i64.device(torch::kCPU)).to(device);
+    auto idx  = (perm.unsqueeze(1) * block_size + torch::arange(block_size, i64.device(device)).unsqueeze(0)).reshape({-1});
+    auto tail = torch::arange(nb * block_size, num_points, i64.device(device));
+    return torch::cat({idx, tail});
+}
+
+torch::Tensor ComputeRadius(torch::Tensor position, int n, at::Generator generator)
+{
+    position        = CheckedPosition(position);
+    const int64_t N = position.size(0);
+    auto data       = torch::zeros({N, 4}, position.options());
+    data.select(1, 0).copy_(KNearestNeighbourDistance(position, n));
+    auto u = torch::rand({N}, generator, position.options().dtype(torch::kFloat64));  // Random::sampleDouble(0, 1), :479
+    data.select(1, 2).copy_(torch::sqrt(1.0 / u.clamp_min_(1e-300)).to(torch::kFloat32));
+    data.select(1, 3).copy_(data.select(1, 0) * data.select(1, 2));
+    return data;
+}
+
+torch::Tensor FilterPointCloud(torch::Tensor position, torch::Tensor poses_se3, torch::Tensor intrinsics,
+                               const std::vector<ReducedImageInfo>& frames, int lonely_n, float lonely_th, float close_th)
+{
+    position = CheckedPosition(position);
+    auto ids = torch::arange(position.size(0), position.options().dtype(torch::kInt64));
+    // (per point: erasing other points does not change it)
+    auto cam  = PointDistanceToCamera(position, poses_se3, intrinsics, frames);
+    auto keep = RemoveLonelyPoints(position, cam, lonely_n, lonely_th);
+    position  = position.index({keep}).contiguous();
+    cam       = cam.index({keep});
+    ids       = ids.index({keep});
+    keep      = RemoveClosePoints(position, cam, close_th);
+    return ids.index({keep});
+}
+
+PreprocessedCloud PreprocessPointCloud(torch::Tensor position, torch::Tensor normal, int n, int block_size, int64_t seed)
+{
+    position      = CheckedPosition(position);
+    auto host_gen = at::detail::createCPUGenerator((uint64_t)seed);
+    auto dev_gen  = at::globalContext().defaultGenerator(position.device()).clone();
+    dev_gen.set_current_seed((uint64_t)seed);
+    auto order = ReorderMorton64(position);
+    order      = order.index({RandomBlockShuffle(position.size(0), block_size, host_gen, position.device())});
+    position   = position.index({order}).contiguous();
+    auto data  = ComputeRadius(position, n, dev_gen);
+    auto by_radius = SortBlocksByRadius(data.select(1, 3), block_size);
+    PreprocessedCloud out;
+    out.order    = order.index({by_radius});
+    out.position = position.index({by_radius}).clone();
+    out.data     = data.index({by_radius}).contiguous();
+    out.position.select(1, 3).copy_(out.data.select(1, 3));
+    if (normal.defined()) out.normal = normal.index({out.order}).contiguous();
+    return out;
+}

@@ -21,3 +21,25 @@ torch::Tensor RemoveLonelyPoints(torch::Tensor position, torch::Tensor camera_di
 torch::Tensor RemoveClosePoints(torch::Tensor position, torch::Tensor camera_distance, float dis_th = 0.00005f);
 // permutation of SceneData::SortBlocksByRadius (:671-684)
 torch::Tensor SortBlocksByRadius(torch::Tensor radius, int block_size = 256);
+// permutation of PointCloud::RandomBlockShuffle (SceneData.cpp:102): whole blocks of block_size consecutive points in
+// random order (a last, shorter block stays last); the order of the blocks is drawn on the host from `generator`.
+torch::Tensor RandomBlockShuffle(int64_t num_points, int block_size, at::Generator generator, torch::Device device);
+// SceneData::ComputeRadius (:441-484): data [N,4] with data[:,0] = distance to the n-th neighbour, data[:,2] =
+// sqrt(1 / u), u ~ U(0,1) drawn on the device from `generator`, data[:,3] = data[:,0] * data[:,2] (the drop-out radius
+// the rasterizer reads as position.w).
+torch::Tensor ComputeRadius(torch::Tensor position, int n, at::Generator generator);
+// The two filters of a new scene in the reference's order (SceneData.cpp:98-99): ids of the surviving points, ascending.
+torch::Tensor FilterPointCloud(torch::Tensor position, torch::Tensor poses_se3, torch::Tensor intrinsics,
+                               const std::vector<ReducedImageInfo>& frames, int lonely_n = 5, float lonely_th = 0.02f,
+                               float close_th = 0.00005f);
+// The initial processing of a new scene (SceneData.cpp:101-104): ReorderMorton64, RandomBlockShuffle(256), ComputeRadius,
+// SortBlocksByRadius(256).  position comes back reordered with the drop-out radius in w; order maps new to original ids.
+struct PreprocessedCloud
+{
+    torch::Tensor position;  // [N,4]
+    torch::Tensor normal;    // reordered like position, or undefined
+    torch::Tensor data;      // [N,4]
+    torch::Tensor order;     // [N] int64
+};
+PreprocessedCloud PreprocessPointCloud(torch::Tensor position, torch::Tensor normal, int n = 4, int block_size = 256,
+                                       int64_t seed = 0);

@@ -143,4 +143,27 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("remove_close_points", &RemoveClosePoints, py::arg("position"), py::arg("camera_distance"),
           py::arg("dis_th") = 0.00005f);
     m.def("sort_blocks_by_radius", &SortBlocksByRadius, py::arg("radius"), py::arg("block_size") = 256);
+    m.def("preprocess_point_cloud",
+          [](torch::Tensor position, c10::optional<torch::Tensor> normal, int n, int block_size, int64_t seed) {
+              auto r = PreprocessPointCloud(position, normal.has_value() ? *normal : torch::Tensor(), n, block_size, seed);
+              return std::make_tuple(r.position, r.normal.defined() ? c10::optional<torch::Tensor>(r.normal) : c10::nullopt,
+                                     r.data, r.order);
+          },
+          py::arg("position"), py::arg("normal") = py::none(), py::arg("n") = 4, py::arg("block_size") = 256,
+          py::arg("seed") = 0);
+    m.def("filter_point_cloud",
+          [](torch::Tensor position, torch::Tensor poses, torch::Tensor intrinsics, const std::vector<ViewTuple>& frames) {
+              std::vector<ReducedImageInfo> f;
+              for (auto& v : frames)
+              {
+                  ReducedImageInfo i;
+                  i.w                 = std::get<0>(v);
+                  i.h                 = std::get<1>(v);
+                  i.image_index       = std::get<2>(v);
+                  i.camera_index      = std::get<3>(v);
+                  i.camera_model_type = (CameraModel)std::get<4>(v);
+                  f.push_back(i);
+              }
+              return FilterPointCloud(position, poses, intrinsics, f);
+          });
 }

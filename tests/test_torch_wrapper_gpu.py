@@ -345,5 +345,13 @@ def test_scene_data_processing_in_cpp():
     assert 250 <= int((~keep).sum()) <= 320
     radius = torch.rand(n, device="cuda")
     assert torch.equal(mod.sort_blocks_by_radius(radius, 256), preprocess.SortBlocksByRadius(radius, 256))
+    # the two compositions of SceneData.cpp:98-104 in C++: the filters, and the processing of what they leave
+    assert torch.equal(mod.filter_point_cloud(pos, poses, intr, tuples), preprocess.FilterPointCloud(pos, poses, intr, frames))
+    nrm = torch.randint(0, 1 << 30, (n, 1), dtype=torch.int32, device="cuda")
+    got = mod.preprocess_point_cloud(pos, nrm, 4, 256, 3)
+    want = preprocess.PreprocessPointCloud(pos, nrm, 4, 256, 3)
+    for a, b, what in zip(got, want, ("position", "normal", "data", "order")):
+        assert torch.equal(a, b), what
+    assert bool((got[0][:, 3] > 0).all()) and sorted(got[3].tolist()) == list(range(n))
     with pytest.raises(RuntimeError):
         mod.knn_distance(pos[:3], 4)
