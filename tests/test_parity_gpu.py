@@ -3,6 +3,8 @@
 Bars: depth / index buffers and weights bit-exact; blended descriptors within 1e-5 relative; gradients within
 1e-4 relative or 1e-6 absolute.
 """
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -700,17 +702,10 @@ def test_smaller_workspaces(oracle_mod, forward_path):
             check_forward(hs, ref, got[2], got[3], got[4], got[1])
     if forward_path != 2:
         assert sizes[0] > sizes[KEPT] > sizes[NOBINS] > sizes[KEPT | NOBINS] and sizes[0] > sizes[SMALL] > sizes[SMALL | KEPT]
-    # a workspace that is too small for the flags it is called with
     s = _capi.Scene()
     s.num_points, s.num_channels, s.num_poses, s.num_cameras, s.intrinsics_cols = hs.num_points, 4, 1, 1, 13
-    assert lib.adop_workspace_size_for(C_byref(s), 1, 4, 256, 144, 8) == 0
+    assert lib.adop_workspace_size_for(ctypes.byref(s), 1, 4, 256, 144, 8) == 0  # an unknown flag
     hs.params.workspace_flags = 0
-
-
-def C_byref(x):
-    import ctypes
-
-    return ctypes.byref(x)
 
 
 @pytest.mark.parametrize("collect_stats", [True, False], ids=["counters", "plain"])
