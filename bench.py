@@ -48,17 +48,17 @@ KERNEL_OF_STAGE = {"BinCount": "bin_count_kernel", "BinScatter": "bin_scatter_ke
 # x 1.0 after calibration with plain device copies of known size), per workload.  "sources" is kernel_sources_state() of
 # the tree the profile was taken on (python bench.py --print-sources-state): the figures are quoted for that state only.
 MEASURED_TRAFFIC = {
-    "config3": {"sources": "711b51ac9c49", "profile": "profiles/config3_tile_path_fwd_bwd_kernels_traffic_instructions.md",
+    "config3": {"sources": "78604d234635", "profile": "profiles/config3_tile_path_fwd_bwd_kernels_traffic_instructions.md",
                 "bytes": {"RenderBackward/descriptor": 860.0e6, "RenderBackward/spatial": 572.1e6, "TileBlend": 529.0e6, "BinCount": 430.3e6, "BinScatter": 197.5e6, "CombineAndFillBackward": 220.8e6, "TileDepth": 101.5e6, "Post Process Gradient": 0.5e6, "CombineAndFill": 23.5e6, "Initialize": 11.8e6}},
-    "config1": {"sources": "711b51ac9c49", "profile": "profiles/config1_direct_path_forward_kernels_traffic_instructions.md",
+    "config1": {"sources": "78604d234635", "profile": "profiles/config1_direct_path_forward_kernels_traffic_instructions.md",
                 "bytes": {"DepthPrepass": 13.0e6, "RenderForward": 8.5e6, "Initialize": 3.5e6, "CombineAndFill": 5.6e6}},
-    "config2": {"sources": "711b51ac9c49", "profile": "profiles/config2_fwd_bwd_kernels_traffic_instructions.md",
+    "config2": {"sources": "78604d234635", "profile": "profiles/config2_fwd_bwd_kernels_traffic_instructions.md",
                 "bytes": {"RenderBackward/descriptor": 200.8e6, "TileBlend": 161.9e6, "RenderBackward/spatial": 146.7e6, "BinScatter": 67.5e6, "BinCount": 64.5e6, "CombineAndFillBackward": 67.2e6, "TileDepth": 37.9e6, "Post Process Gradient": 15.1e6, "Initialize": 3.4e6, "CombineAndFill": 6.6e6}},
-    "config4": {"sources": "711b51ac9c49", "profile": "profiles/config4_direct_path_forward_kernels_traffic_instructions.md",
+    "config4": {"sources": "78604d234635", "profile": "profiles/config4_direct_path_forward_kernels_traffic_instructions.md",
                 "bytes": {"DepthPrepass": 5080.7e6, "RenderForward": 1545.8e6, "CombineAndFill": 176.8e6, "Initialize": 110.5e6}},
-    "config5": {"sources": "711b51ac9c49", "profile": "profiles/config5_ocam_envmap_fwd_bwd_kernels_traffic_instructions.md",
+    "config5": {"sources": "78604d234635", "profile": "profiles/config5_ocam_envmap_fwd_bwd_kernels_traffic_instructions.md",
                 "bytes": {"RenderBackward/spatial": 5753.6e6, "TileBlend": 5064.9e6, "EnvironmentMapBackward": 2242.8e6, "BinCount": 2189.5e6, "RenderBackward/descriptor": 4091.9e6, "EnvironmentMap": 3081.4e6, "BinScatter": 3331.6e6, "TileDepth": 1622.9e6, "CombineAndFillBackward": 1872.4e6, "Post Process Gradient": 484.7e6, "CombineAndFill": 177.1e6, "Initialize": 91.5e6}},
-    "crops": {"sources": "711b51ac9c49", "profile": "profiles/training_batch_16_crops_fwd_bwd_kernels_traffic_instructions.md",
+    "crops": {"sources": "78604d234635", "profile": "profiles/training_batch_16_crops_fwd_bwd_kernels_traffic_instructions.md",
                 "bytes": {"RenderBackward/descriptor": 1579.8e6, "RenderBackward/spatial": 1242.0e6, "BinCount": 587.1e6, "TileBlend": 1211.8e6, "BinScatter": 764.6e6, "CombineAndFillBackward": 446.2e6, "TileDepth": 249.2e6, "Post Process Gradient": 120.3e6, "CombineAndFill": 47.8e6, "Initialize": 23.7e6}},
 }
 
@@ -96,16 +96,23 @@ def tile_path_model(k, N, B, C_, P_levels, V, has_dropout, lt=2):
 
 
 def kernel_sources_state():
-    """First 12 hex digits of the SHA-256 over the sources the library is built from (adop_amd/csrc/*.hip, *.h and the
-    C header): the state of the kernels a traffic profile was taken on.  A table of MEASURED_TRAFFIC is quoted only
-    while this matches its "sources" entry, so an edited kernel can never be reported with stale measured bytes."""
+    """First 12 hex digits of the SHA-256 over the code of the sources the library is built from (adop_amd/csrc/*.hip,
+    *.h and the C header; comments and white space left out): the state of the kernels a traffic profile was taken on.
+    A table of MEASURED_TRAFFIC is quoted only while this matches its "sources" entry, so an edited kernel can never be
+    reported with stale measured bytes."""
+    import re
+
     h = hashlib.sha256()
     files = sorted(glob.glob(os.path.join(ROOT, "adop_amd", "csrc", "*.hip")) +
                    glob.glob(os.path.join(ROOT, "adop_amd", "csrc", "*.h")) +
                    [os.path.join(ROOT, "include", "adop_raster.h")])
     for f in files:
+        text = open(f, encoding="utf-8").read()
+        text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)   # block comments
+        text = re.sub(r"//[^\n]*", " ", text)                # line comments (no string of these sources holds "//")
+        text = " ".join(text.split())
         h.update(os.path.basename(f).encode())
-        h.update(open(f, "rb").read())
+        h.update(text.encode())
     return h.hexdigest()[:12]
 
 

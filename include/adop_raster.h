@@ -231,7 +231,7 @@ typedef struct adop_tuning
     int32_t bin_shard_shift;    /* log2 of the counters per tile in the binning passes, 0..3; -1 (default) = by the tile
                                    count (up to 8 while the call has at most 4096 tiles and 16384 counters).  A value
                                    that would need more than 65536 counters is lowered until it does not. */
-    int32_t direct_lists;       /* direct path without a caller's point cache: 1 = candidate lists (default), 0 = a record per point */
+    int32_t direct_lists;       /* direct path without a caller's point cache: 1 = candidate lists (default), 0 = none, the blend projects again */
     int32_t prepass_ppt;        /* points per thread of the direct path's depth prepass: 1, 2, 4; 0 (default) = by the cloud size */
     int32_t prepass_group_from; /* first level at which the depth prepass merges the lanes of a wavefront by pixel (1) */
     int32_t blend_group_from;   /* the same for the direct path's blend (0) */
